@@ -1,0 +1,339 @@
+/*
+ * CPU oracle for the FP8 quantized-matmul path.  TEST INFRASTRUCTURE ONLY.
+ *
+ * Nothing in the shipped library links, loads or calls this file.  It is the checker the parity
+ * tests, the smoke test and the CPU-baseline leg of the benchmark compare the HIP kernels against.
+ *
+ * Every function is a scalar restatement of the arithmetic of the reference path (paths relative to
+ * the reference tree):
+ *   abs-max          src/kernels/quant.cu:11-28 + src/kernels/kernel_utils.cuh:17-32
+ *   scale            src/kernels/quant.cu:79-82
+ *   quantize         src/kernels/quant.cu:73-93
+ *   quantize+transp. src/kernels/quant.cu:151-164 + src/kernels/transpose_template.cuh:10-34
+ *   byte transpose   src/kernels/transpose.cu:9-32
+ *   e4m3 encode      the CUDA toolkit's fp32 -> e4m3 SATFINITE round-to-nearest-even conversion the
+ *                    reference calls at src/kernels/quant.cu:88,159 (third-party: CUDA >= 12
+ *                    cuda_fp8.hpp, not part of the reference tree); restated from the OCP FP8 format
+ *                    definition
+ *   GEMM             src/kernels/matmul.cpp:47-153 (default backend semantics: one fp32 scale factor
+ *                    sa*sb applied after accumulation, bias / beta*C added in fp32, one rounding to
+ *                    the output type)
+ *   bf16 rounding    src/testing/test_utils.h:18-26
+ *
+ * Pinning status (what independent evidence each function is checked against, in tests/):
+ *   abs-max            numpy max(abs()) on the decoded values; NaN-skip / Inf / -0 special cases
+ *   e4m3 encode        exhaustive nearest-of-256-codes search with ties-to-even, torch's CPU
+ *                      float8_e4m3fn cast after clamping, boundary closed forms (2^-10, 464, NaN)
+ *   scale              IEEE-754 division in numpy float32
+ *   quantize(+transp.) composition of the two above; identity qt(X) == transpose(q(X))
+ *   transpose          numpy .T
+ *   GEMM               numpy int64 matmul on integer-valued operands (the reference's own
+ *                      test-gemm.cpp construction), numpy float64 matmul on decoded operands
+ * The bit-level results of the CUDA conversion instruction and of cuBLASLt themselves cannot be
+ * observed here (no CUDA device or toolkit): for NaN sign/payload and for the accumulation order
+ * of the closed-source GEMM the parity is unpinned by anything the reference ships; the oracle
+ * follows the documented behaviour (canonical NaN 0x7F; any fp32 accumulation order).
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+static inline uint32_t f32_bits(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static inline float bits_f32(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+
+/* bf16 -> fp32 is exact: the 16 bits are the top half of the fp32 pattern. */
+float orc_bf16_to_f32(uint16_t h) { return bits_f32((uint32_t)h << 16); }
+
+/* fp32 -> bf16, round to nearest even (src/testing/test_utils.h:18-26); NaN stays NaN. */
+uint16_t orc_f32_to_bf16(float f) {
+    uint32_t u = f32_bits(f);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x0040u);
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+/* max_i |in[i]| as fp32; NaNs are skipped, |+-Inf| wins, result >= +0 (quant.cu:19-27). */
+float orc_abs_max_bf16(const uint16_t* in, int64_t n) {
+    float m = 0.f;
+    for (int64_t i = 0; i < n; ++i) {
+        float a = fabsf(orc_bf16_to_f32(in[i]));
+        if (a == a && a > m) m = a;   /* fmaxf semantics: the non-NaN operand */
+    }
+    return m;
+}
+
+float orc_abs_max_f32(const float* in, int64_t n) {
+    float m = 0.f;
+    for (int64_t i = 0; i < n; ++i) {
+        float a = fabsf(in[i]);
+        if (a == a && a > m) m = a;
+    }
+    return m;
+}
+
+/* fp32 -> e4m3 (OCP "fn": bias 7, 3 mantissa bits, no Inf, NaN = 0x7F), round to nearest even,
+ * saturate to +-448; NaN -> 0x7F with the sign dropped; signed zero / underflow keep the sign. */
+uint8_t orc_e4m3_encode(float y) {
+    uint32_t u = f32_bits(y);
+    uint8_t sign = (uint8_t)((u >> 31) << 7);
+    uint32_t a = u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return 0x7F;                 /* NaN, canonical */
+    if (a <= 0x3A800000u) return sign;                /* |y| <= 2^-10 (tie goes to even = 0) */
+    if (a > 0x43E80000u) return (uint8_t)(sign | 0x7E); /* |y| > 464 (Inf included) -> 448 */
+    uint32_t e = a >> 23;
+    uint32_t res;
+    if (a >= 0x3C800000u) {                           /* |y| >= 2^-6: normal in e4m3 */
+        uint32_t mant = (a >> 20) & 7u;
+        res = ((e - 127u + 7u) << 3) | mant;
+        uint32_t rem = a & 0xFFFFFu;
+        if (rem > 0x80000u || (rem == 0x80000u && (mant & 1u))) res += 1u;
+    } else {                                          /* subnormal: multiples of 2^-9 */
+        uint32_t m = (a & 0x7FFFFFu) | 0x800000u;     /* |y| = m * 2^(e-150) */
+        uint32_t sh = 141u - e;                       /* 21..24 */
+        res = m >> sh;
+        uint32_t rem = m & ((1u << sh) - 1u);
+        uint32_t half = 1u << (sh - 1u);
+        if (rem > half || (rem == half && (res & 1u))) res += 1u;
+    }
+    return (uint8_t)(sign | res);
+}
+
+/* e4m3 -> fp32 (exact). 0x7F / 0xFF decode to NaN. */
+float orc_e4m3_decode(uint8_t c) {
+    uint32_t e = (c >> 3) & 0xFu, m = c & 7u;
+    float v;
+    if (e == 0xF && m == 7) v = NAN;
+    else if (e == 0) v = ldexpf((float)m, -9);
+    else v = ldexpf((float)(8 + m), (int)e - 10);
+    return (c & 0x80) ? -v : v;
+}
+
+/* fp32 -> e5m2 (bias 15, 2 mantissa bits, max finite 57344 = 0x7B), RNE, saturate-to-finite,
+ * NaN -> canonical 0x7F with the sign dropped (the e5m2 output type of quant.cu:130-132). */
+uint8_t orc_e5m2_encode(float y) {
+    uint32_t u = f32_bits(y);
+    uint8_t sign = (uint8_t)((u >> 31) << 7);
+    uint32_t a = u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return 0x7F;
+    if (a <= 0x37000000u) return sign;                /* |y| <= 2^-17 */
+    if (a >= 0x47700000u) return (uint8_t)(sign | 0x7B); /* |y| >= 61440 = maxnorm + ulp/2 -> 57344 */
+    uint32_t e = a >> 23;
+    uint32_t res;
+    if (a >= 0x38800000u) {                           /* >= 2^-14 normal */
+        uint32_t mant = (a >> 21) & 3u;
+        res = ((e - 127u + 15u) << 2) | mant;
+        uint32_t rem = a & 0x1FFFFFu;
+        if (rem > 0x100000u || (rem == 0x100000u && (mant & 1u))) res += 1u;
+    } else {                                          /* multiples of 2^-16 */
+        uint32_t m = (a & 0x7FFFFFu) | 0x800000u;
+        uint32_t sh = 134u - e;                       /* |y| = m*2^(e-150); /2^-16 -> >> (134-e) */
+        res = m >> sh;
+        uint32_t rem = m & ((1u << sh) - 1u);
+        uint32_t half = 1u << (sh - 1u);
+        if (rem > half || (rem == half && (res & 1u))) res += 1u;
+    }
+    return (uint8_t)(sign | res);
+}
+
+float orc_e5m2_decode(uint8_t c) {
+    uint32_t e = (c >> 2) & 0x1Fu, m = c & 3u;
+    float v;
+    if (e == 0x1F) v = m ? NAN : INFINITY;
+    else if (e == 0) v = ldexpf((float)m, -16);
+    else v = ldexpf((float)(4 + m), (int)e - 17);
+    return (c & 0x80) ? -v : v;
+}
+
+/* scale = 448 / max(absmax, 1e-10); dequant = 1 / scale; two IEEE fp32 divisions (quant.cu:79-82). */
+void orc_quant_scale(float absmax, float* scale, float* dequant) {
+    volatile float a = absmax > 1e-10f ? absmax : 1e-10f;   /* fmaxf; absmax is never NaN */
+    volatile float s = 448.f / a;
+    volatile float d = 1.f / s;
+    if (scale) *scale = s;
+    if (dequant) *dequant = d;
+}
+
+/* out[i] = e4m3(scale * (float)in[i]); *scale_out = 1/scale when non-null (quant.cu:73-93). */
+void orc_quantize_e4m3_bf16(uint8_t* out, float* scale_out, const uint16_t* in, float absmax, int64_t n) {
+    float s, d;
+    orc_quant_scale(absmax, &s, &d);
+    if (scale_out) *scale_out = d;
+    for (int64_t i = 0; i < n; ++i) {
+        volatile float y = s * orc_bf16_to_f32(in[i]);     /* one fp32 multiply, no fma */
+        out[i] = orc_e4m3_encode(y);
+    }
+}
+
+/* e5m2 output uses the same 448-based scale as the reference kernel does (quant.cu:79, shared by
+ * both fp8 output types). */
+void orc_quantize_e5m2_bf16(uint8_t* out, float* scale_out, const uint16_t* in, float absmax, int64_t n) {
+    float s, d;
+    orc_quant_scale(absmax, &s, &d);
+    if (scale_out) *scale_out = d;
+    for (int64_t i = 0; i < n; ++i) {
+        volatile float y = s * orc_bf16_to_f32(in[i]);
+        out[i] = orc_e5m2_encode(y);
+    }
+}
+
+/* out[c*rows + r] = e4m3(scale * in[r*cols + c]) (quant.cu:151-164, transpose_template.cuh:21-33). */
+void orc_quantize_transpose_e4m3_bf16(uint8_t* out, float* scale_out, const uint16_t* in, float absmax,
+                                      int rows, int cols) {
+    float s, d;
+    orc_quant_scale(absmax, &s, &d);
+    if (scale_out) *scale_out = d;
+    for (int64_t r = 0; r < rows; ++r)
+        for (int64_t c = 0; c < cols; ++c) {
+            volatile float y = s * orc_bf16_to_f32(in[r * cols + c]);
+            out[c * (int64_t)rows + r] = orc_e4m3_encode(y);
+        }
+}
+
+/* dst[c*rows + r] = src[r*cols + c] (transpose.cu:9-32). */
+void orc_transpose_u8(uint8_t* dst, const uint8_t* src, int rows, int cols) {
+    for (int64_t r = 0; r < rows; ++r)
+        for (int64_t c = 0; c < cols; ++c)
+            dst[c * (int64_t)rows + r] = src[r * cols + c];
+}
+
+/*
+ * Exact TN product in the reference's matmul convention (src/kernels/matmul.cpp:80-92,
+ * src/testing/test-gemm.cpp:121-124): row-major a[M,K], b[N,K] give row-major c[N,M],
+ *   exact[n*M + m]  = sum_k dec(b[n,k]) * dec(a[m,k])        (fp64; every term and sum is exact)
+ *   sumabs[n*M + m] = sum_k |dec(b[n,k]) * dec(a[m,k])|      (for the error bound; may be NULL)
+ * Only rows n in [n0, n1) are produced (written at their absolute position).
+ */
+void orc_gemm_tn_e4m3_exact(double* exact, double* sumabs, const uint8_t* a, const uint8_t* b,
+                            int M, int N, int K, int n0, int n1) {
+    double lut[256];
+    for (int i = 0; i < 256; ++i) lut[i] = (double)orc_e4m3_decode((uint8_t)i);
+    (void)N;
+    double* arow = (double*)malloc(sizeof(double) * (size_t)K);
+    for (int64_t n = n0; n < n1; ++n) {
+        for (int k = 0; k < K; ++k) arow[k] = lut[b[n * K + k]];
+        for (int64_t m = 0; m < M; ++m) {
+            const uint8_t* am = a + m * K;
+            double s = 0.0, sa = 0.0;
+            for (int k = 0; k < K; ++k) {
+                double p = arow[k] * lut[am[k]];
+                s += p;
+                sa += fabs(p);
+            }
+            exact[n * M + m] = s;
+            if (sumabs) sumabs[n * M + m] = sa;
+        }
+    }
+    free(arow);
+}
+
+/* Same, for a list of sampled output coordinates (idx_n[i], idx_m[i]). */
+void orc_gemm_tn_e4m3_exact_sampled(double* exact, double* sumabs, const uint8_t* a, const uint8_t* b,
+                                    int M, int N, int K, const int32_t* idx_n, const int32_t* idx_m,
+                                    int64_t count) {
+    double lut[256];
+    for (int i = 0; i < 256; ++i) lut[i] = (double)orc_e4m3_decode((uint8_t)i);
+    (void)M; (void)N;
+    for (int64_t i = 0; i < count; ++i) {
+        const uint8_t* bn = b + (int64_t)idx_n[i] * K;
+        const uint8_t* am = a + (int64_t)idx_m[i] * K;
+        double s = 0.0, sa = 0.0;
+        for (int k = 0; k < K; ++k) {
+            double p = lut[bn[k]] * lut[am[k]];
+            s += p;
+            sa += fabs(p);
+        }
+        exact[i] = s;
+        if (sumabs) sumabs[i] = sa;
+    }
+}
+
+/*
+ * Epilogue of the default backend (src/kernels/matmul.cpp:59-142): with the accumulator taken as
+ * the exact sum rounded once to fp32,
+ *   t = acc * (sa * sb);  t += bias[m] (if any);  t += c_old (if accumulate);  c = round(t)
+ * all in fp32, one final rounding to the output type.  `scale` is the fp32 product sa*sb
+ * (1 for absent scales).  bias is fp32 here (bf16 biases are widened exactly by the caller).
+ */
+float orc_gemm_epilogue_f32(double exact, float scale, const float* bias_m, const float* c_old) {
+    volatile float t = (float)exact;
+    t = t * scale;
+    if (bias_m) t = t + *bias_m;
+    if (c_old) t = t + *c_old;
+    return t;
+}
+
+/* Full TN GEMM with the epilogue, bf16 or fp32 output; used for sizes the oracle finishes quickly. */
+void orc_gemm_tn_e4m3(void* c, int c_is_f32, const uint8_t* a, const uint8_t* b,
+                      const uint16_t* bias_bf16, const float* bias_f32,
+                      const float* sa, const float* sb, int M, int N, int K, int accumulate) {
+    double* ex = (double*)malloc(sizeof(double) * (size_t)M * (size_t)N);
+    orc_gemm_tn_e4m3_exact(ex, NULL, a, b, M, N, K, 0, N);
+    volatile float scale = (sa ? *sa : 1.f);
+    if (sb) scale = scale * *sb;
+    for (int64_t n = 0; n < N; ++n)
+        for (int64_t m = 0; m < M; ++m) {
+            float bias_v = 0.f, old_v = 0.f;
+            const float* bp = NULL; const float* op = NULL;
+            if (bias_bf16) { bias_v = orc_bf16_to_f32(bias_bf16[m]); bp = &bias_v; }
+            else if (bias_f32) { bias_v = bias_f32[m]; bp = &bias_v; }
+            if (accumulate) {
+                old_v = c_is_f32 ? ((float*)c)[n * M + m] : orc_bf16_to_f32(((uint16_t*)c)[n * M + m]);
+                op = &old_v;
+            }
+            float t = orc_gemm_epilogue_f32(ex[n * M + m], scale, bp, op);
+            if (c_is_f32) ((float*)c)[n * M + m] = t;
+            else ((uint16_t*)c)[n * M + m] = orc_f32_to_bf16(t);
+        }
+    free(ex);
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * Deterministic synthetic tensors: a counter-based generator (one 64-bit mix per element index),
+ * so any slice can be produced independently and the same bytes feed the CPU and the GPU side.
+ * ---------------------------------------------------------------------------------------------- */
+static inline uint64_t mix64(uint64_t x) {
+    x += 0x9E3779B97F4A7C15ull;
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+    return x ^ (x >> 31);
+}
+static inline double u01(uint64_t r) { return ((double)(r >> 11) + 0.5) * (1.0 / 9007199254740992.0); }
+
+static inline double normal_at(uint64_t key, uint64_t i) {
+    uint64_t r1 = mix64(key ^ mix64(2 * i));
+    uint64_t r2 = mix64(key ^ mix64(2 * i + 1));
+    return sqrt(-2.0 * log(u01(r1))) * cos(6.283185307179586476925 * u01(r2));
+}
+
+/* out[i] = bf16(mean + std * N(0,1)) for i in [0,n); element i depends only on (seed, stream, i). */
+void orc_fill_normal_bf16(uint16_t* out, int64_t n, uint64_t seed, uint64_t stream, float mean, float std) {
+    uint64_t key = mix64(seed * 0x100000001B3ull + stream);
+    for (int64_t i = 0; i < n; ++i)
+        out[i] = orc_f32_to_bf16((float)(mean + std * normal_at(key, (uint64_t)i)));
+}
+
+/* Student-t with 3 degrees of freedom: Z / sqrt((Z1^2+Z2^2+Z3^2)/3), scaled by `scale`. */
+void orc_fill_student_t3_bf16(uint16_t* out, int64_t n, uint64_t seed, uint64_t stream, float scale) {
+    uint64_t key = mix64(seed * 0x100000001B3ull + stream);
+    for (int64_t i = 0; i < n; ++i) {
+        double z = normal_at(key, 4 * (uint64_t)i);
+        double a = normal_at(key, 4 * (uint64_t)i + 1);
+        double b = normal_at(key, 4 * (uint64_t)i + 2);
+        double c = normal_at(key, 4 * (uint64_t)i + 3);
+        double chi = (a * a + b * b + c * c) / 3.0;
+        out[i] = orc_f32_to_bf16((float)(scale * z / sqrt(chi)));
+    }
+}
+
+/* Uniform integers in [lo, hi] stored as e4m3 codes (all |v| <= 15 are exact in e4m3), the operand
+ * construction of src/testing/test-gemm.cpp:54-85. Also returns them as int32 when vals != NULL. */
+void orc_fill_int_e4m3(uint8_t* out, int32_t* vals, int64_t n, uint64_t seed, uint64_t stream, int lo, int hi) {
+    uint64_t key = mix64(seed * 0x100000001B3ull + stream);
+    uint64_t span = (uint64_t)(hi - lo + 1);
+    for (int64_t i = 0; i < n; ++i) {
+        int v = lo + (int)(mix64(key ^ mix64((uint64_t)i)) % span);
+        out[i] = orc_e4m3_encode((float)v);
+        if (vals) vals[i] = v;
+    }
+}

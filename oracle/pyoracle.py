@@ -1,0 +1,238 @@
+"""ctypes loader for the CPU oracle (oracle/llmq_oracle.c + oracle/llmq_cpu_mt.c).
+
+Test infrastructure only.  Arrays are numpy: bf16 tensors travel as uint16 bit patterns, e4m3/e5m2
+tensors as uint8 codes.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "_build", "libllmq_oracle.so")
+_lib = None
+
+
+def build(force=False):
+    """Compile the oracle with gcc (a second or two)."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.check_call(["make", "-C", _HERE] + (["-B"] if force else []), stdout=subprocess.DEVNULL)
+    return _LIB_PATH
+
+
+def _p(arr, ctype):
+    return arr.ctypes.data_as(C.POINTER(ctype))
+
+
+def lib():
+    global _lib
+    if _lib is not None:
+        return _lib
+    build()
+    L = C.CDLL(_LIB_PATH)
+    u8p, u16p, f32p, f64p, i32p = (C.POINTER(t) for t in (C.c_uint8, C.c_uint16, C.c_float, C.c_double, C.c_int32))
+    L.orc_bf16_to_f32.restype = C.c_float
+    L.orc_bf16_to_f32.argtypes = [C.c_uint16]
+    L.orc_f32_to_bf16.restype = C.c_uint16
+    L.orc_f32_to_bf16.argtypes = [C.c_float]
+    L.orc_abs_max_bf16.restype = C.c_float
+    L.orc_abs_max_bf16.argtypes = [u16p, C.c_int64]
+    L.orc_abs_max_f32.restype = C.c_float
+    L.orc_abs_max_f32.argtypes = [f32p, C.c_int64]
+    L.orc_e4m3_encode.restype = C.c_uint8
+    L.orc_e4m3_encode.argtypes = [C.c_float]
+    L.orc_e4m3_decode.restype = C.c_float
+    L.orc_e4m3_decode.argtypes = [C.c_uint8]
+    L.orc_e5m2_encode.restype = C.c_uint8
+    L.orc_e5m2_encode.argtypes = [C.c_float]
+    L.orc_e5m2_decode.restype = C.c_float
+    L.orc_e5m2_decode.argtypes = [C.c_uint8]
+    L.orc_quant_scale.restype = None
+    L.orc_quant_scale.argtypes = [C.c_float, f32p, f32p]
+    for name in ("orc_quantize_e4m3_bf16", "orc_quantize_e5m2_bf16", "mt_quantize_e4m3_bf16"):
+        f = getattr(L, name)
+        f.restype = None
+        f.argtypes = [u8p, f32p, u16p, C.c_float, C.c_int64]
+    for name in ("orc_quantize_transpose_e4m3_bf16", "mt_quantize_transpose_e4m3_bf16"):
+        f = getattr(L, name)
+        f.restype = None
+        f.argtypes = [u8p, f32p, u16p, C.c_float, C.c_int, C.c_int]
+    for name in ("orc_transpose_u8", "mt_transpose_u8"):
+        f = getattr(L, name)
+        f.restype = None
+        f.argtypes = [u8p, u8p, C.c_int, C.c_int]
+    L.orc_gemm_tn_e4m3_exact.restype = None
+    L.orc_gemm_tn_e4m3_exact.argtypes = [f64p, f64p, u8p, u8p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
+    L.orc_gemm_tn_e4m3_exact_sampled.restype = None
+    L.orc_gemm_tn_e4m3_exact_sampled.argtypes = [f64p, f64p, u8p, u8p, C.c_int, C.c_int, C.c_int, i32p, i32p, C.c_int64]
+    L.orc_gemm_epilogue_f32.restype = C.c_float
+    L.orc_gemm_epilogue_f32.argtypes = [C.c_double, C.c_float, f32p, f32p]
+    L.orc_gemm_tn_e4m3.restype = None
+    L.orc_gemm_tn_e4m3.argtypes = [C.c_void_p, C.c_int, u8p, u8p, u16p, f32p, f32p, f32p,
+                                   C.c_int, C.c_int, C.c_int, C.c_int]
+    L.orc_fill_normal_bf16.restype = None
+    L.orc_fill_normal_bf16.argtypes = [u16p, C.c_int64, C.c_uint64, C.c_uint64, C.c_float, C.c_float]
+    L.orc_fill_student_t3_bf16.restype = None
+    L.orc_fill_student_t3_bf16.argtypes = [u16p, C.c_int64, C.c_uint64, C.c_uint64, C.c_float]
+    L.orc_fill_int_e4m3.restype = None
+    L.orc_fill_int_e4m3.argtypes = [u8p, i32p, C.c_int64, C.c_uint64, C.c_uint64, C.c_int, C.c_int]
+    L.mt_num_threads.restype = C.c_int
+    L.mt_set_num_threads.argtypes = [C.c_int]
+    L.mt_abs_max_bf16.restype = C.c_float
+    L.mt_abs_max_bf16.argtypes = [u16p, C.c_int64]
+    L.mt_gemm_tn_e4m3.restype = C.c_int
+    L.mt_gemm_tn_e4m3.argtypes = [C.c_void_p, C.c_int, u8p, u8p, u16p, f32p, f32p,
+                                  C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
+    _lib = L
+    return L
+
+
+# ---------------------------------------------------------------------------------- numpy helpers
+def bf16_to_f32(bits):
+    """uint16 bf16 patterns -> float32 (exact)."""
+    return (np.asarray(bits, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def f32_to_bf16(x):
+    """float32 -> uint16 bf16 patterns, round to nearest even (finite inputs)."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    r = u + (0x7FFF + ((u >> 16) & 1)).astype(np.uint32)
+    out = (r >> 16).astype(np.uint16)
+    nan = (u & 0x7FFFFFFF) > 0x7F800000
+    if nan.any():
+        out[nan] = ((u[nan] >> 16) | 0x40).astype(np.uint16)
+    return out
+
+
+_E4M3_TABLE = None
+
+
+def e4m3_table():
+    """float32[256] decode table of every e4m3 code (0x7F/0xFF are NaN)."""
+    global _E4M3_TABLE
+    if _E4M3_TABLE is None:
+        L = lib()
+        _E4M3_TABLE = np.array([L.orc_e4m3_decode(i) for i in range(256)], dtype=np.float32)
+    return _E4M3_TABLE
+
+
+def e4m3_decode(codes):
+    return e4m3_table()[np.asarray(codes, dtype=np.uint8)]
+
+
+def abs_max_bf16(x):
+    x = np.ascontiguousarray(x, dtype=np.uint16)
+    return float(lib().orc_abs_max_bf16(_p(x, C.c_uint16), x.size))
+
+
+def quant_scale(absmax):
+    s, d = C.c_float(), C.c_float()
+    lib().orc_quant_scale(C.c_float(absmax), C.byref(s), C.byref(d))
+    return s.value, d.value
+
+
+def quantize_e4m3(x, absmax, mt=False, fmt="e4m3"):
+    """Returns (codes uint8 like x, dequant scale float32)."""
+    x = np.ascontiguousarray(x, dtype=np.uint16)
+    out = np.empty(x.shape, dtype=np.uint8)
+    d = C.c_float()
+    name = ("mt_" if mt else "orc_") + "quantize_%s_bf16" % fmt
+    getattr(lib(), name)(_p(out, C.c_uint8), C.byref(d), _p(x, C.c_uint16), C.c_float(absmax), x.size)
+    return out, np.float32(d.value)
+
+
+def quantize_transpose_e4m3(x, absmax, mt=False):
+    x = np.ascontiguousarray(x, dtype=np.uint16)
+    rows, cols = x.shape
+    out = np.empty((cols, rows), dtype=np.uint8)
+    d = C.c_float()
+    f = lib().mt_quantize_transpose_e4m3_bf16 if mt else lib().orc_quantize_transpose_e4m3_bf16
+    f(_p(out, C.c_uint8), C.byref(d), _p(x, C.c_uint16), C.c_float(absmax), rows, cols)
+    return out, np.float32(d.value)
+
+
+def transpose_u8(x, mt=False):
+    x = np.ascontiguousarray(x, dtype=np.uint8)
+    rows, cols = x.shape
+    out = np.empty((cols, rows), dtype=np.uint8)
+    f = lib().mt_transpose_u8 if mt else lib().orc_transpose_u8
+    f(_p(out, C.c_uint8), _p(x, C.c_uint8), rows, cols)
+    return out
+
+
+def gemm_exact(a, b, rows=None):
+    """a[M,K], b[N,K] e4m3 codes -> (exact float64 [N,M], sum|terms| float64 [N,M]); rows=(n0,n1)
+    restricts the computed rows (others are left zero)."""
+    a = np.ascontiguousarray(a, dtype=np.uint8)
+    b = np.ascontiguousarray(b, dtype=np.uint8)
+    M, K = a.shape
+    N, K2 = b.shape
+    assert K == K2
+    n0, n1 = rows if rows is not None else (0, N)
+    ex = np.zeros((N, M), dtype=np.float64)
+    sa = np.zeros((N, M), dtype=np.float64)
+    lib().orc_gemm_tn_e4m3_exact(_p(ex, C.c_double), _p(sa, C.c_double), _p(a, C.c_uint8), _p(b, C.c_uint8),
+                                 M, N, K, n0, n1)
+    return ex, sa
+
+
+def gemm_exact_sampled(a, b, idx_n, idx_m):
+    a = np.ascontiguousarray(a, dtype=np.uint8)
+    b = np.ascontiguousarray(b, dtype=np.uint8)
+    M, K = a.shape
+    N, _ = b.shape
+    idx_n = np.ascontiguousarray(idx_n, dtype=np.int32)
+    idx_m = np.ascontiguousarray(idx_m, dtype=np.int32)
+    ex = np.zeros(idx_n.size, dtype=np.float64)
+    sa = np.zeros(idx_n.size, dtype=np.float64)
+    lib().orc_gemm_tn_e4m3_exact_sampled(_p(ex, C.c_double), _p(sa, C.c_double), _p(a, C.c_uint8),
+                                         _p(b, C.c_uint8), M, N, K, _p(idx_n, C.c_int32),
+                                         _p(idx_m, C.c_int32), idx_n.size)
+    return ex, sa
+
+
+def gemm_tn(a, b, sa=None, sb=None, bias=None, c_old=None, out_f32=False, mt=False):
+    """Full GEMM + epilogue.  bias: uint16 bf16 [M] or None.  c_old: previous c (accumulate) or None.
+    Returns uint16 bf16 [N,M] or float32 [N,M]."""
+    a = np.ascontiguousarray(a, dtype=np.uint8)
+    b = np.ascontiguousarray(b, dtype=np.uint8)
+    M, K = a.shape
+    N, _ = b.shape
+    dt = np.float32 if out_f32 else np.uint16
+    c = np.array(c_old, dtype=dt, copy=True).reshape(N, M) if c_old is not None else np.zeros((N, M), dtype=dt)
+    keep_a = C.c_float(sa) if sa is not None else None
+    keep_b = C.c_float(sb) if sb is not None else None
+    fsa = C.pointer(keep_a) if keep_a is not None else None
+    fsb = C.pointer(keep_b) if keep_b is not None else None
+    bp = None
+    if bias is not None:
+        bias = np.ascontiguousarray(bias, dtype=np.uint16)
+        bp = _p(bias, C.c_uint16)
+    if mt:
+        rc = lib().mt_gemm_tn_e4m3(c.ctypes.data, int(out_f32), _p(a, C.c_uint8), _p(b, C.c_uint8), bp, fsa, fsb,
+                                   M, N, K, int(c_old is not None), 0, N)
+        assert rc == 0
+    else:
+        lib().orc_gemm_tn_e4m3(c.ctypes.data, int(out_f32), _p(a, C.c_uint8), _p(b, C.c_uint8), bp, None, fsa, fsb,
+                               M, N, K, int(c_old is not None))
+    return c
+
+
+def fill_normal_bf16(n, seed, stream, mean=0.0, std=1.0):
+    out = np.empty(int(n), dtype=np.uint16)
+    lib().orc_fill_normal_bf16(_p(out, C.c_uint16), out.size, seed, stream, C.c_float(mean), C.c_float(std))
+    return out
+
+
+def fill_student_t3_bf16(n, seed, stream, scale=1.0):
+    out = np.empty(int(n), dtype=np.uint16)
+    lib().orc_fill_student_t3_bf16(_p(out, C.c_uint16), out.size, seed, stream, C.c_float(scale))
+    return out
+
+
+def fill_int_e4m3(n, seed, stream, lo=-15, hi=15):
+    out = np.empty(int(n), dtype=np.uint8)
+    vals = np.empty(int(n), dtype=np.int32)
+    lib().orc_fill_int_e4m3(_p(out, C.c_uint8), _p(vals, C.c_int32), out.size, seed, stream, lo, hi)
+    return out, vals

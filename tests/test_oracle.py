@@ -1,0 +1,262 @@
+"""Pins the CPU oracle against evidence that does not come from the oracle itself: the OCP e4m3
+format definition (nearest-code search), torch's CPU float8 casts, numpy float32/int64/float64
+arithmetic, and the constructions the reference's own tests use (src/testing/test-gemm.cpp:54-85,
+scripts/test_kernels.py:40-65,641-652,1168-1185 in the reference tree)."""
+import numpy as np
+import pytest
+import torch
+
+ALL_BF16 = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+
+
+# ------------------------------------------------------------------ independent e4m3 definitions
+def e4m3_value_of_code(c):
+    """OCP FP8 E4M3 ("fn") value of a 7-bit magnitude code, from the format definition."""
+    e, m = c >> 3, c & 7
+    if e == 0:
+        return m * 2.0 ** -9
+    return (8 + m) * 2.0 ** (e - 10)
+
+
+def e4m3_encode_search(y):
+    """Nearest-of-127-finite-codes search in float64 with ties to the even code, saturating."""
+    y = np.asarray(y, dtype=np.float32)
+    vals = np.array([e4m3_value_of_code(c) for c in range(0x7F)], dtype=np.float64)  # 0 .. 448
+    a = np.abs(y.astype(np.float64))
+    hi = np.searchsorted(vals, a, side="left")            # first code with value >= a
+    hi = np.clip(hi, 0, 0x7E)
+    lo = np.clip(hi - 1, 0, 0x7E)
+    dlo, dhi = np.abs(a - vals[lo]), np.abs(vals[hi] - a)
+    code = np.where(dlo < dhi, lo, np.where(dhi < dlo, hi, np.where(lo % 2 == 0, lo, hi)))
+    code = np.where(a >= 448.0, 0x7E, code)                # saturate-to-finite (Inf included)
+    sign = (y.view(np.uint32) >> 31).astype(np.uint8) << 7
+    out = (code.astype(np.uint8) | sign).astype(np.uint8)
+    out[np.isnan(y)] = 0x7F                                # canonical NaN, sign dropped
+    return out
+
+
+def oracle_encode(O, y):
+    y = np.ascontiguousarray(y, dtype=np.float32)
+    L = O.lib()
+    return np.array([L.orc_e4m3_encode(float(v)) if not np.isnan(v) else L.orc_e4m3_encode(float("nan"))
+                     for v in y], dtype=np.uint8)
+
+
+def encode_via_quantize(O, bits, absmax):
+    """Vectorised route into the oracle's encoder: quantize bf16 patterns with a given abs-max."""
+    q, _ = O.quantize_e4m3(bits, absmax)
+    return q
+
+
+# ------------------------------------------------------------------------------------ bf16 helpers
+def test_bf16_roundtrip_matches_torch(O):
+    rng = np.random.default_rng(1)
+    x = np.concatenate([rng.standard_normal(20000).astype(np.float32) * 10.0 ** rng.integers(-30, 30, 20000),
+                        np.array([0.0, -0.0, 1.0, 1.00390625, 1.01171875, 3.3895314e38, np.inf, -np.inf], np.float32)])
+    ours = O.f32_to_bf16(x)
+    ref = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(ours, ref)
+    L = O.lib()
+    for v in x[:2000]:
+        assert L.orc_f32_to_bf16(float(v)) == int(torch.tensor(float(v)).to(torch.bfloat16).view(torch.int16)) & 0xFFFF
+    assert np.array_equal(O.bf16_to_f32(ours), torch.from_numpy(ours.view(np.int16)).view(torch.bfloat16).float().numpy())
+
+
+# ---------------------------------------------------------------------------------------- abs-max
+def test_abs_max_matches_numpy(O):
+    # shapes of scripts/test_kernels.py:56-65 plus larger ones
+    for shape, seed in [((16, 64), 0), ((4, 128, 32), 1), ((1000, 8), 2), ((1 << 18,), 3)]:
+        x = O.fill_normal_bf16(int(np.prod(shape)), seed, 7, 0.0, 3.0)
+        assert O.abs_max_bf16(x) == np.abs(O.bf16_to_f32(x)).max()
+        assert O.lib().mt_abs_max_bf16(x.ctypes.data_as(__import__("ctypes").POINTER(__import__("ctypes").c_uint16)), x.size) \
+            == O.abs_max_bf16(x)
+
+
+def test_abs_max_special_values(O):
+    nan, snan, ninf, nzero = 0x7FC0, 0x7F81, 0xFF80, 0x8000
+    assert O.abs_max_bf16(np.array([nan, snan, 0xFFC1], np.uint16)) == 0.0          # all NaN -> 0
+    assert O.abs_max_bf16(np.array([nzero] * 8, np.uint16)) == 0.0
+    assert np.signbit(np.float32(O.abs_max_bf16(np.array([nzero] * 8, np.uint16)))) == False  # noqa: E712
+    assert O.abs_max_bf16(np.array([0x3F80, nan, 0xC000, snan], np.uint16)) == 2.0  # NaN skipped
+    assert O.abs_max_bf16(np.array([0x3F80, ninf, nan], np.uint16)) == np.inf       # |-Inf| wins
+    assert O.abs_max_bf16(np.array([0x0001, 0x8003], np.uint16)) == O.bf16_to_f32(np.array([3], np.uint16))[0]  # denormals kept
+    assert O.abs_max_bf16(np.zeros(0, np.uint16)) == 0.0
+
+
+# ------------------------------------------------------------------------------------ e4m3 encode
+def test_e4m3_decode_matches_definition_and_torch(O):
+    tab = O.e4m3_table()
+    for c in range(0x7F):
+        assert tab[c] == np.float32(e4m3_value_of_code(c))
+        assert tab[c | 0x80] == -np.float32(e4m3_value_of_code(c))
+    assert np.isnan(tab[0x7F]) and np.isnan(tab[0xFF])
+    t = torch.arange(256, dtype=torch.int32).to(torch.uint8).view(torch.float8_e4m3fn).float().numpy()
+    assert np.array_equal(np.nan_to_num(t, nan=12345.0), np.nan_to_num(tab, nan=12345.0))
+    assert np.array_equal(np.signbit(t), np.signbit(tab))
+
+
+def test_e4m3_encode_boundaries_closed_form(O):
+    L = O.lib()
+    enc = L.orc_e4m3_encode
+    assert enc(0.0) == 0x00 and enc(-0.0) == 0x80
+    assert enc(2.0 ** -10) == 0x00 and enc(-(2.0 ** -10)) == 0x80            # tie to even (zero)
+    assert enc(float(np.nextafter(np.float32(2.0 ** -10), np.float32(1)))) == 0x01
+    assert enc(2.0 ** -9) == 0x01 and enc(3 * 2.0 ** -10) == 0x02            # tie 1.5 ulp -> even (2)
+    assert enc(7.5 * 2.0 ** -9) == 0x08                                      # tie rounds up into the normals
+    assert enc(2.0 ** -6) == 0x08
+    assert enc(448.0) == 0x7E and enc(464.0) == 0x7E and enc(-464.0) == 0xFE
+    assert enc(float(np.nextafter(np.float32(464), np.float32(1e9)))) == 0x7E  # saturates
+    assert enc(1e30) == 0x7E and enc(float("inf")) == 0x7E and enc(float("-inf")) == 0xFE
+    assert enc(float("nan")) == 0x7F
+    assert enc(float(np.uint32(0xFFC00000).view(np.float32))) == 0x7F        # -NaN: sign dropped
+    assert enc(1.0) == 0x38 and enc(-1.0) == 0xB8 and enc(1.0625) == 0x38 and enc(1.1875) == 0x3A
+    assert enc(1e-45) == 0x00 and enc(-1e-45) == 0x80                        # fp32 denormal underflows
+
+
+@pytest.mark.parametrize("absmax", [448.0, 1.0, 5.15625, 0.072265625, 3.0e-5, 1e4, 0.0, 447.0, 1.7e38])
+def test_e4m3_encode_exhaustive_bf16_vs_search_and_torch(O, absmax):
+    """All 65536 bf16 inputs through scale*x, against the nearest-code search and torch's cast."""
+    s, d = O.quant_scale(absmax)
+    s32 = np.float32(s)
+    assert s32 == np.float32(448.0) / max(np.float32(absmax), np.float32(1e-10))
+    assert np.float32(d) == np.float32(1.0) / s32
+    with np.errstate(over="ignore", invalid="ignore"):
+        y = (s32 * O.bf16_to_f32(ALL_BF16)).astype(np.float32)
+    got = encode_via_quantize(O, ALL_BF16, absmax)
+    want = e4m3_encode_search(y)
+    assert np.array_equal(got, want)
+    # third opinion: torch's float8_e4m3fn cast (which does not saturate, hence the clamp)
+    finite = ~np.isnan(y)
+    t = torch.from_numpy(y[finite]).clamp(-448.0, 448.0).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert np.array_equal(got[finite], t)
+    assert np.all(got[~finite] == 0x7F)
+    # the multithreaded port agrees bit for bit
+    got_mt, d_mt = O.quantize_e4m3(ALL_BF16, absmax, mt=True)
+    assert np.array_equal(got_mt, got) and d_mt == np.float32(d)
+
+
+def test_e4m3_encode_fp32_grid_vs_search(O):
+    """Dense fp32 probes around every rounding boundary (midpoints between codes, +-1 ulp)."""
+    vals = np.array([e4m3_value_of_code(c) for c in range(0x7F)], dtype=np.float64)
+    mids = ((vals[1:] + vals[:-1]) / 2).astype(np.float32)
+    pts = np.concatenate([mids, np.nextafter(mids, np.float32(0)), np.nextafter(mids, np.float32(1e9)),
+                          vals.astype(np.float32), np.array([464, 465, 480, 1e9, 2.0 ** -10, 2.0 ** -11], np.float32)])
+    pts = np.concatenate([pts, -pts])
+    rng = np.random.default_rng(5)
+    rnd = (rng.standard_normal(20000) * 10.0 ** rng.uniform(-4, 3, 20000)).astype(np.float32)
+    pts = np.concatenate([pts, rnd])
+    assert np.array_equal(oracle_encode(O, pts), e4m3_encode_search(pts))
+
+
+def test_quantize_reference_style_checks(O):
+    # scripts/test_kernels.py:641-652: scale ~= absmax/448, dequantised values within 10 %
+    for n, seed in [(1024, 0), (8192, 1)]:
+        x = O.fill_normal_bf16(n, seed, 3)
+        am = O.abs_max_bf16(x)
+        q, d = O.quantize_e4m3(x, am)
+        assert d == pytest.approx(am / 448.0, rel=1e-6)
+        deq = O.e4m3_decode(q) * d
+        xf = O.bf16_to_f32(x)
+        big = np.abs(xf) > am * 2.0 ** -6 / 448 * 8
+        assert np.allclose(deq[big], xf[big], rtol=0.1)
+
+
+def test_zero_tensor_quantize(O):
+    x = np.array([0x0000, 0x8000] * 8, np.uint16)
+    q, d = O.quantize_e4m3(x, 0.0)
+    assert list(q[:2]) == [0x00, 0x80]
+    s, _ = O.quant_scale(0.0)
+    assert np.float32(s) == np.float32(448.0) / np.float32(1e-10)
+
+
+# -------------------------------------------------------------------------- transpose / q+transpose
+@pytest.mark.parametrize("shape", [(32, 32), (128, 256), (512, 1024), (8, 40), (72, 8)])
+def test_transpose_and_quantize_transpose(O, shape):
+    rows, cols = shape
+    x = O.fill_normal_bf16(rows * cols, 11, rows, 0.0, 2.0).reshape(rows, cols)
+    am = O.abs_max_bf16(x)
+    q, d = O.quantize_e4m3(x, am)
+    assert np.array_equal(O.transpose_u8(q), q.T)
+    assert np.array_equal(O.transpose_u8(q, mt=True), q.T)
+    qt, dt = O.quantize_transpose_e4m3(x, am)
+    assert np.array_equal(qt, q.T) and dt == d
+    qt2, _ = O.quantize_transpose_e4m3(x, am, mt=True)
+    assert np.array_equal(qt2, q.T)
+
+
+# ------------------------------------------------------------------------------------------- GEMM
+@pytest.mark.parametrize("mnk,scale", [((128, 128, 128), 4.0 / 128), ((128, 96, 768), 4.0 / 768)])
+def test_gemm_integer_known_answer(O, mnk, scale):
+    """The construction of src/testing/test-gemm.cpp: integers in [-15,15] are exact in e4m3, every
+    partial sum stays below 2^24, so the product is an exact integer matrix: numpy int64 is the truth."""
+    M, N, K = mnk
+    a, av = O.fill_int_e4m3(M * K, 12345, 0)
+    b, bv = O.fill_int_e4m3(N * K, 12345, 1)
+    a, av, b, bv = a.reshape(M, K), av.reshape(M, K), b.reshape(N, K), bv.reshape(N, K)
+    assert np.array_equal(O.e4m3_decode(a), av.astype(np.float32))
+    truth = bv.astype(np.int64) @ av.astype(np.int64).T          # [N, M]
+    ex, sabs = O.gemm_exact(a, b)
+    assert np.array_equal(ex, truth.astype(np.float64))
+    assert np.array_equal(sabs, (np.abs(bv).astype(np.int64) @ np.abs(av).astype(np.int64).T).astype(np.float64))
+    s = np.float32(np.sqrt(np.float32(scale)))
+    ss = np.float32(s * s)
+    c = O.gemm_tn(a, b, sa=float(s), sb=float(s), out_f32=True)
+    assert np.array_equal(c, truth.astype(np.float32) * ss)
+    cb = O.gemm_tn(a, b, sa=float(s), sb=float(s))
+    assert np.array_equal(cb, O.f32_to_bf16(truth.astype(np.float32) * ss))
+    # bias and accumulate (fp32 adds, single rounding)
+    _, biasv = O.fill_int_e4m3(M, 12345, 2)
+    _, oldv = O.fill_int_e4m3(N * M, 12345, 3)
+    bias = O.f32_to_bf16(biasv.astype(np.float32))
+    old = O.f32_to_bf16(oldv.astype(np.float32)).reshape(N, M)
+    want = ((truth.astype(np.float32) * ss) + biasv.astype(np.float32)[None, :]) + oldv.reshape(N, M).astype(np.float32)
+    got = O.gemm_tn(a, b, sa=float(s), sb=float(s), bias=bias, c_old=old)
+    assert np.array_equal(got, O.f32_to_bf16(want))
+    # the reference's own acceptance test (test-gemm.cpp:114-148): rel 1e-2 against the fp32 product
+    exp = truth.astype(np.float32) * s * s
+    assert np.all(np.abs(O.bf16_to_f32(cb) - exp) <= np.maximum(1e-2 * np.maximum(np.abs(exp), np.abs(O.bf16_to_f32(cb))), 1e-4))
+    # multithreaded port: exact here too (integer sums are order independent)
+    if M % 64 == 0 and N % 4 == 0:
+        assert np.array_equal(O.gemm_tn(a, b, sa=float(s), sb=float(s), mt=True), cb)
+        assert np.array_equal(O.gemm_tn(a, b, sa=float(s), sb=float(s), bias=bias, c_old=old, mt=True), got)
+
+
+def test_gemm_random_codes_vs_float64_matmul(O):
+    rng = np.random.default_rng(3)
+    M, N, K = 64, 48, 512
+    a = rng.integers(0, 256, (M, K)).astype(np.uint8)
+    b = rng.integers(0, 256, (N, K)).astype(np.uint8)
+    a[(a & 0x7F) == 0x7F] = 0x7E
+    b[(b & 0x7F) == 0x7F] = 0x7E
+    ex, sabs = O.gemm_exact(a, b)
+    ad, bd = O.e4m3_decode(a).astype(np.float64), O.e4m3_decode(b).astype(np.float64)
+    ref = bd @ ad.T
+    assert np.allclose(ex, ref, rtol=0, atol=1e-9 * np.abs(bd) @ np.abs(ad).T)
+    assert np.allclose(sabs, np.abs(bd) @ np.abs(ad).T, rtol=1e-12)
+    idx_n = rng.integers(0, N, 100).astype(np.int32)
+    idx_m = rng.integers(0, M, 100).astype(np.int32)
+    exs, sabss = O.gemm_exact_sampled(a, b, idx_n, idx_m)
+    assert np.array_equal(exs, ex[idx_n, idx_m]) and np.array_equal(sabss, sabs[idx_n, idx_m])
+    # rows subset
+    ex2, _ = O.gemm_exact(a, b, rows=(8, 16))
+    assert np.array_equal(ex2[8:16], ex[8:16]) and not ex2[:8].any()
+    # transposed-operand identity: swapping a and b transposes the result
+    ex_t, _ = O.gemm_exact(b, a)
+    assert np.array_equal(ex_t, ex.T)
+    # mt port stays within fp32 accumulation error of the exact result
+    cm = O.gemm_tn(a, b, sa=0.5, sb=0.25, out_f32=True, mt=True)
+    assert np.all(np.abs(cm - ex * 0.125) <= 2.0 ** -18 * 0.125 * sabs + 1e-30)
+
+
+# ------------------------------------------------------------------------------------- generators
+def test_generators_are_deterministic_and_sane(O):
+    x1 = O.fill_normal_bf16(1 << 16, 4, 9, 0.0, 0.02)
+    x2 = O.fill_normal_bf16(1 << 16, 4, 9, 0.0, 0.02)
+    assert np.array_equal(x1, x2)
+    assert not np.array_equal(x1, O.fill_normal_bf16(1 << 16, 4, 10, 0.0, 0.02))
+    xf = O.bf16_to_f32(x1)
+    assert abs(xf.mean()) < 5e-4 and abs(xf.std() - 0.02) < 5e-4
+    # prefix property of a counter-based stream
+    assert np.array_equal(O.fill_normal_bf16(100, 4, 9, 0.0, 0.02), x1[:100])
+    t = O.bf16_to_f32(O.fill_student_t3_bf16(1 << 16, 5, 1))
+    assert np.isfinite(t).all() and np.abs(t).max() > 8.0 and abs(np.median(t)) < 0.02
