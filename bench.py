@@ -1,0 +1,224 @@
+#!/usr/bin/env python3
+"""Benchmark of the FP8 quantized-matmul path on one MI355X.
+
+A step is one pass of the whole path over the Qwen2.5-7B MLP at 8192 tokens (configuration 4 of
+BASELINE.json): for the fused gate+up linear (3584 -> 37888) and the down linear (18944 -> 3584),
+forward + dgrad + wgrad, with every abs-max, quantize, transpose and quantize+transpose launch the
+reference's forward_qmm / backward_qmm issue (src/models/llama_model.cpp:25-47, 309-339), plus the
+per-step weight abs-max + quantize (src/models/llama_weights.cpp:207-223).  Inputs are synthetic and
+already resident in HBM when the timed region starts.
+
+One JSON line is printed:
+  value           e4m3 GEMM TFLOP/s of the whole step: 2*M*N*K summed over the six GEMMs divided by the
+                  step time (abs-max / quantize / transpose launches included in the time)
+  roofline        the GEMM kernel alone: algorithmic FLOP / mean launch duration (HIP events around
+                  each GEMM launch inside the timed steps) against the dense FP8 MFMA peak
+  quantize        abs-max + quantize (+transpose) launches: algorithmic bytes / event-timed duration
+                  against 8 TB/s
+  cpu_baseline    the multithreaded CPU port of the same path on a bounded sample (host cores of this box)
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+FP8_PEAK_TFLOPS = 5000.0   # MI355X dense FP8 MFMA peak
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
+
+BT, C, FFN = 8192, 3584, 18944
+UP = 2 * FFN  # fused gate+up output features
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="rough budget of the CPU baseline sample")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (--gpus 1); multi-GPU sharding is a design note, "
+              "not a code path", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from llmq_amd import capi, kernels as K   # fails loudly if the HIP library is missing
+
+    assert torch.cuda.is_available(), "bench.py needs the MI355X"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    gen = torch.Generator(device=dev).manual_seed(4)
+
+    def randn(shape, std):
+        return (torch.randn(shape, device=dev, generator=gen, dtype=torch.float32) * std).to(torch.bfloat16)
+
+    # ---- synthetic tensors (configuration 4) ----
+    t = {
+        "x": randn((BT, C), 1.0), "w_up": randn((UP, C), 0.015),
+        "h": randn((BT, FFN), 1.0), "w_down": randn((C, FFN), 0.015),
+        "dy_up": randn((BT, UP), 1e-4), "dy_down": randn((BT, C), 1e-4),
+    }
+    f8 = torch.float8_e4m3fn
+    e = lambda *s: torch.empty(s, dtype=f8, device=dev)
+    q = {"x": e(BT, C), "w_up": e(UP, C), "h": e(BT, FFN), "w_down": e(C, FFN), "dy_up": e(BT, UP), "dy_down": e(BT, C),
+         "w_up_t": e(C, UP), "w_down_t": e(FFN, C), "x_t": e(C, BT), "h_t": e(FFN, BT), "dy_up_t": e(UP, BT),
+         "dy_down_t": e(C, BT)}
+    stats = {k: torch.zeros(2, device=dev) for k in t}   # [abs_max, scale] pairs, as Tensor::Stats in the reference
+    out = {"y_up": torch.empty((BT, UP), dtype=torch.bfloat16, device=dev),
+           "y_down": torch.empty((BT, C), dtype=torch.bfloat16, device=dev),
+           "dh": torch.empty((BT, FFN), dtype=torch.bfloat16, device=dev),
+           "dx": torch.empty((BT, C), dtype=torch.bfloat16, device=dev),
+           "dw_up": torch.empty((UP, C), dtype=torch.bfloat16, device=dev),
+           "dw_down": torch.empty((C, FFN), dtype=torch.bfloat16, device=dev)}
+
+    timers = {}   # name -> list of (start, end, work) ; work in bytes or flop
+    record = [False]
+
+    def timed(name, work, fn):
+        if record[0]:
+            s, f = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            fn()
+            f.record()
+            timers.setdefault(name, []).append((s, f, work))
+        else:
+            fn()
+
+    def absmax_and_quantize(name):
+        n = t[name].numel()
+        timed("abs_max", 2 * n, lambda: K.abs_max(stats[name][0:1], t[name]))
+        timed("quantize", 3 * n, lambda: K.quantize_with_abs_max(q[name], stats[name][1:2], t[name], stats[name][0:1]))
+
+    def gemm(c, a, b, sa, sb, M, N, Kd):
+        timed("gemm", 2.0 * M * N * Kd, lambda: K.matmul(c, a, b, None, sa, sb, M, N, Kd))
+
+    def tr(dst, src):
+        timed("transpose", 2 * src.numel(), lambda: K.transpose(dst, src))
+
+    def qtr(dst, name):
+        timed("quantize_transpose", 3 * t[name].numel(),
+              lambda: K.quantize_and_transpose_with_abs_max(dst, None, t[name], stats[name][0:1]))
+
+    def step():
+        # weights: abs-max + quantize once per step (they change every optimizer step)
+        absmax_and_quantize("w_up")
+        absmax_and_quantize("w_down")
+        # forward gate+up, down
+        absmax_and_quantize("x")
+        gemm(out["y_up"], q["w_up"], q["x"], stats["w_up"][1:2], stats["x"][1:2], UP, BT, C)
+        absmax_and_quantize("h")
+        gemm(out["y_down"], q["w_down"], q["h"], stats["w_down"][1:2], stats["h"][1:2], C, BT, FFN)
+        # backward down: dgrad dH = dY W, wgrad dW = dY^T H
+        absmax_and_quantize("dy_down")
+        tr(q["w_down_t"], q["w_down"])
+        gemm(out["dh"], q["w_down_t"], q["dy_down"], stats["w_down"][1:2], stats["dy_down"][1:2], FFN, BT, C)
+        qtr(q["h_t"], "h")
+        tr(q["dy_down_t"], q["dy_down"])
+        gemm(out["dw_down"], q["h_t"], q["dy_down_t"], stats["h"][1:2], stats["dy_down"][1:2], FFN, C, BT)
+        # backward gate+up
+        absmax_and_quantize("dy_up")
+        tr(q["w_up_t"], q["w_up"])
+        gemm(out["dx"], q["w_up_t"], q["dy_up"], stats["w_up"][1:2], stats["dy_up"][1:2], C, BT, UP)
+        qtr(q["x_t"], "x")
+        tr(q["dy_up_t"], q["dy_up"])
+        gemm(out["dw_up"], q["x_t"], q["dy_up_t"], stats["x"][1:2], stats["dy_up"][1:2], C, UP, BT)
+
+    gemm_flop = 3 * (2.0 * UP * BT * C) + 3 * (2.0 * C * BT * FFN)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    record[0] = True
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    record[0] = False
+    step_ms = (t1 - t0) * 1e3 / args.steps
+
+    def summarize(name):
+        evs = timers.get(name, [])
+        ms = [s.elapsed_time(f) for s, f, _ in evs]
+        work = sum(w for _, _, w in evs)
+        return {"launches": len(evs), "mean_ms": sum(ms) / max(len(ms), 1), "total_ms": sum(ms), "work": work}
+
+    ks = {n: summarize(n) for n in ("gemm", "abs_max", "quantize", "quantize_transpose", "transpose")}
+    gemm_tflops_kernel = ks["gemm"]["work"] / (ks["gemm"]["total_ms"] * 1e-3) / 1e12
+    qnames = ("abs_max", "quantize", "quantize_transpose", "transpose")
+    per_kernel = {n: {"GBps": ks[n]["work"] / (ks[n]["total_ms"] * 1e-3) / 1e9,
+                      "frac_hbm": ks[n]["work"] / (ks[n]["total_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                      "mean_us": ks[n]["mean_ms"] * 1e3} for n in qnames}
+    aq_bytes = ks["abs_max"]["work"] + ks["quantize"]["work"]
+    aq_ms = ks["abs_max"]["total_ms"] + ks["quantize"]["total_ms"]
+    aq_gbs = aq_bytes / (aq_ms * 1e-3) / 1e9
+
+    result = {
+        "metric": "e4m3 GEMM TFLOP/s + % FP8 peak; quantize GB/s + % HBM (Qwen-7B MLP shape)",
+        "value": gemm_flop / (step_ms * 1e-3) / 1e12,
+        "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": step_ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "e4m3 x e4m3 -> fp32 accumulate -> bf16", "data": "synthetic",
+        "config": {"workload": "Qwen2.5-7B MLP (gate+up 3584->37888, down 18944->3584), 8192 tokens, fwd+dgrad+wgrad "
+                               "with per-tensor abs-max/quantize/transpose (BASELINE.json configs[3])",
+                   "tokens": BT, "gemm_flop_per_step": gemm_flop},
+        "roofline": {"bound": "mfma", "kernel": "gemm_tn_e4m3_kernel", "achieved": gemm_tflops_kernel,
+                     "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": gemm_tflops_kernel / FP8_PEAK_TFLOPS,
+                     "traffic": None, "mean_launch_ms": ks["gemm"]["mean_ms"], "launches": ks["gemm"]["launches"]},
+        "quantize": {"bound": "hbm", "kernels": "abs_max + quantize_with_abs_max (5 bytes/element)",
+                     "achieved": aq_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": aq_gbs / HBM_PEAK_GBS,
+                     "per_kernel": per_kernel},
+        "library": capi.version(),
+    }
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(t, np, torch, args.cpu_seconds)
+    print(json.dumps(result))
+
+
+def cpu_baseline(t, np, torch, budget_s):
+    """The multithreaded CPU port (oracle/llmq_cpu_mt.c) on a bounded sample of the same workload:
+    abs-max + quantize of X [8192x3584] and of a row-slice of W_up, then the gate+up forward GEMM for
+    that slice of output features against all 8192 tokens."""
+    import ctypes as C
+    from oracle import pyoracle as O
+    L = O.lib()
+    cores = min(L.mt_num_threads(), 16)      # the GPU box grants 16 host cores to a one-GPU job
+    L.mt_set_num_threads(cores)
+    to_bits = lambda x: x.cpu().view(torch.int16).numpy().view(np.uint16)
+    x = to_bits(t["x"])
+    # calibrate the GEMM slice: 64 weight rows first, then scale to the budget
+    w_all = t["w_up"]
+    t0 = time.perf_counter()
+    ax = float(L.mt_abs_max_bf16(x.ctypes.data_as(C.POINTER(C.c_uint16)), x.size))
+    xq, _ = O.quantize_e4m3(x, ax, mt=True)
+    t_q = time.perf_counter() - t0
+    q_gbs = 5 * x.size / t_q / 1e9
+
+    def gemm_rows(m_rows):
+        w = to_bits(w_all[:m_rows].contiguous())
+        aw = O.abs_max_bf16(w)
+        wq, _ = O.quantize_e4m3(w, aw, mt=True)
+        s = time.perf_counter()
+        O.gemm_tn(wq, xq, sa=1.0, sb=1.0, mt=True)
+        return time.perf_counter() - s
+
+    t64 = gemm_rows(64)
+    rows = int(max(64, min(UP, (budget_s / max(t64, 1e-3)) * 64)) // 64 * 64)
+    tg = gemm_rows(rows) if rows > 64 else t64
+    flop = 2.0 * rows * BT * C
+    return {"value": flop / tg / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": "gate+up forward GEMM for %d of %d output features x 8192 tokens x K=3584 (%.1f GFLOP, %.1f s); "
+                      "abs-max+quantize of X[8192x3584]: %.2f GB/s" % (rows, UP, flop / 1e9, tg, q_gbs),
+            "quantize_GBps": q_gbs}
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,113 @@
+/*
+ * llmq_fp8.h -- C ABI of the MI355X (gfx950) FP8 quantized-matmul path.
+ *
+ * One entry point per kernel entry point of the reference's src/kernels/kernels.h that lies on the
+ * path  abs-max -> scaled bf16->e4m3 quantize (plain / fused transpose) -> e4m3 x e4m3 TN GEMM.
+ * Plain pointers and sizes only; bf16 travels as uint16_t bit patterns, e4m3 as uint8_t codes.
+ *
+ * Conventions shared by every function:
+ *   - every pointer is a DEVICE pointer owned by the caller (abs-max / scale slots included);
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); work is enqueued
+ *     asynchronously on it, no host synchronisation, no allocation, legal under stream capture;
+ *   - the return value is LLMQ_OK or an error code; llmq_last_error() gives the message of the
+ *     last failure on the calling thread (the C++ shim turns codes into the reference's exception
+ *     types: std::invalid_argument / std::runtime_error);
+ *   - tensor base pointers must be 16-byte aligned (src/kernels/matmul.cpp:55-57 has the same rule).
+ */
+#ifndef LLMQ_FP8_H
+#define LLMQ_FP8_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LLMQ_OK 0
+#define LLMQ_ERR_INVALID_ARGUMENT 1 /* shape / alignment / null-pointer precondition violated */
+#define LLMQ_ERR_RUNTIME 2          /* a HIP runtime call failed (message carries hipGetErrorString) */
+
+/* Message of the last error returned on this thread ("" if none). Never NULL. */
+const char* llmq_last_error(void);
+
+/* Library version string, and the gfx target the device code was compiled for ("gfx950"). */
+const char* llmq_version(void);
+const char* llmq_target_arch(void);
+
+/*
+ * *out = max_i |in[i]| as fp32 (NaNs ignored, |+-Inf| wins, result >= +0; 0 for n == 0).
+ * The slot is reset first, then reduced into, all on `stream`.
+ * Replaces: abs_max(float*, const nv_bfloat16*, long, const cudaDeviceProp&, cudaStream_t)
+ *           src/kernels/kernels.h:247, src/kernels/quant.cu:107-109 (kernel :11-28).
+ * n may be any non-negative count (the reference requires n % 8 == 0).
+ */
+int llmq_abs_max_bf16(float* out, const uint16_t* in, int64_t n, void* stream);
+
+/* fp32 input variant.  Replaces abs_max(float*, const float*, long, ...) src/kernels/kernels.h:246,
+ * src/kernels/quant.cu:103-105. */
+int llmq_abs_max_f32(float* out, const float* in, int64_t n, void* stream);
+
+/*
+ * scale = 448.f / fmaxf(*absmax, 1e-10f); out[i] = e4m3_rn_satfinite(scale * (float)in[i]);
+ * if scale_or_null: *scale_or_null = 1.f / scale.
+ * Replaces: quantize_with_abs_max(__nv_fp8_e4m3*, float*, const nv_bfloat16*, const float*, long,
+ *           const cudaDeviceProp&, cudaStream_t)  src/kernels/kernels.h:255, src/kernels/quant.cu:127-129
+ *           (kernel :73-93).
+ */
+int llmq_quantize_e4m3_bf16(uint8_t* out, float* scale_or_null, const uint16_t* in, const float* absmax,
+                            int64_t n, void* stream);
+
+/* Same with e5m2 output codes (the gradient dtype option).  Replaces quantize_with_abs_max(
+ * __nv_fp8_e5m2*, ...) src/kernels/kernels.h:256, src/kernels/quant.cu:130-132. */
+int llmq_quantize_e5m2_bf16(uint8_t* out, float* scale_or_null, const uint16_t* in, const float* absmax,
+                            int64_t n, void* stream);
+
+/*
+ * As llmq_quantize_e4m3_bf16 on a row-major [rows, cols] input, written transposed:
+ * out[c*rows + r] = q(in[r*cols + c]).  rows % 8 == 0 and cols % 8 == 0 required.
+ * Replaces: quantize_and_transpose_with_abs_max(__nv_fp8_e4m3*, float*, const nv_bfloat16*,
+ *           const float*, int rows, int cols, const cudaDeviceProp&, cudaStream_t)
+ *           src/kernels/kernels.h:263, src/kernels/quant.cu:191-193 (kernel :151-164).
+ */
+int llmq_quantize_transpose_e4m3_bf16(uint8_t* out, float* scale_or_null, const uint16_t* in,
+                                      const float* absmax, int rows, int cols, void* stream);
+
+/*
+ * Byte transpose: dst[c*rows + r] = src[r*cols + c]  (e4m3 / e5m2 codes).  Any rows, cols >= 0.
+ * Replaces: transpose(__nv_fp8_e4m3*, const __nv_fp8_e4m3*, int rows, int cols, cudaStream_t)
+ *           src/kernels/kernels.h:267 (and the e5m2 overload :268), src/kernels/transpose.cu:38-43.
+ */
+int llmq_transpose_u8(uint8_t* dst, const uint8_t* src, int rows, int cols, void* stream);
+
+/*
+ * TN GEMM in the reference's matmul convention (column-major cuBLAS view): with ROW-MAJOR
+ * a[M,K] and b[N,K] (both e4m3, K contiguous) it writes ROW-MAJOR c[N,M]:
+ *     c[n,m] = round( (sum_k b[n,k]*a[m,k]) * (sa*sb) + bias[m] + (accumulate ? c[n,m] : 0) )
+ * fp32 accumulation, fp32 epilogue, one rounding to the output type.  sa / sb are device fp32
+ * scalars or NULL (= 1).  bias is bf16[M] or NULL.  M, N, K must be multiples of 128 (the
+ * precondition of the reference's hand-written kernel, src/kernels/gemm_mma.cu:261-263).
+ * Replaces: matmul(nv_bfloat16* c, const __nv_fp8_e4m3* a, const __nv_fp8_e4m3* b,
+ *           const nv_bfloat16* bias, const float* scale_a, const float* scale_b, cublasLtHandle_t,
+ *           std::byte* ws, size_t ws_size, int M, int N, int K, EMMTranspose::TN, bool accumulate,
+ *           cudaStream_t, EMatmulBackend)  src/kernels/kernels.h:88-90, src/kernels/matmul.cpp:216-220,
+ *           and gemm_mma_tn(...) src/kernels/gemm_mma.cu:279-284.
+ */
+int llmq_gemm_tn_e4m3_bf16(uint16_t* c, const uint8_t* a, const uint8_t* b, const uint16_t* bias_or_null,
+                           const float* sa_or_null, const float* sb_or_null, int M, int N, int K,
+                           int accumulate, void* stream);
+
+/*
+ * fp32-output variant (wgrad into fp32 gradients).  bias may be fp32[M] (bias_is_bf16 == 0) or
+ * bf16[M] (bias_is_bf16 != 0) or NULL.
+ * Replaces: matmul(float* c, const __nv_fp8_e4m3*, const __nv_fp8_e4m3*, const float* bias, ...)
+ *           src/kernels/kernels.h:72-74 and (..., const nv_bfloat16* bias, ...) :76-78,
+ *           src/kernels/matmul.cpp:198-208.
+ */
+int llmq_gemm_tn_e4m3_f32(float* c, const uint8_t* a, const uint8_t* b, const void* bias_or_null,
+                          int bias_is_bf16, const float* sa_or_null, const float* sb_or_null, int M, int N,
+                          int K, int accumulate, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LLMQ_FP8_H */

@@ -1,0 +1,59 @@
+"""ctypes binding of the C ABI declared in include/llmq_fp8.h.
+
+Raw device pointers in, status codes turned into exceptions: LLMQ_ERR_INVALID_ARGUMENT -> ValueError
+(the reference throws std::invalid_argument), LLMQ_ERR_RUNTIME -> RuntimeError.  There is no CPU
+fallback: if the library is not built the import of this module fails.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libllmq_fp8.so")
+
+EXPORTS = [
+    "llmq_last_error", "llmq_version", "llmq_target_arch",
+    "llmq_abs_max_bf16", "llmq_abs_max_f32",
+    "llmq_quantize_e4m3_bf16", "llmq_quantize_e5m2_bf16", "llmq_quantize_transpose_e4m3_bf16",
+    "llmq_transpose_u8", "llmq_gemm_tn_e4m3_bf16", "llmq_gemm_tn_e4m3_f32",
+]
+
+if not os.path.exists(LIB_PATH):
+    raise ImportError("%s is missing: build it with `python -m llmq_amd.build` (hipcc, gfx950)" % LIB_PATH)
+
+lib = C.CDLL(LIB_PATH)
+
+_vp, _i64, _int = C.c_void_p, C.c_int64, C.c_int
+lib.llmq_last_error.restype = C.c_char_p
+lib.llmq_version.restype = C.c_char_p
+lib.llmq_target_arch.restype = C.c_char_p
+lib.llmq_abs_max_bf16.argtypes = [_vp, _vp, _i64, _vp]
+lib.llmq_abs_max_f32.argtypes = [_vp, _vp, _i64, _vp]
+lib.llmq_quantize_e4m3_bf16.argtypes = [_vp, _vp, _vp, _vp, _i64, _vp]
+lib.llmq_quantize_e5m2_bf16.argtypes = [_vp, _vp, _vp, _vp, _i64, _vp]
+lib.llmq_quantize_transpose_e4m3_bf16.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _vp]
+lib.llmq_transpose_u8.argtypes = [_vp, _vp, _int, _int, _vp]
+lib.llmq_gemm_tn_e4m3_bf16.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp]
+lib.llmq_gemm_tn_e4m3_f32.argtypes = [_vp, _vp, _vp, _vp, _int, _vp, _vp, _int, _int, _int, _int, _vp]
+lib.llmq_debug_set_gemm_variant.argtypes = [_int]
+lib.llmq_debug_set_gemm_variant.restype = None
+for _name in EXPORTS[3:]:
+    getattr(lib, _name).restype = _int
+
+LLMQ_OK, LLMQ_ERR_INVALID_ARGUMENT, LLMQ_ERR_RUNTIME = 0, 1, 2
+
+
+def check(code):
+    if code == LLMQ_OK:
+        return
+    msg = lib.llmq_last_error().decode("utf-8", "replace")
+    if code == LLMQ_ERR_INVALID_ARGUMENT:
+        raise ValueError(msg)
+    raise RuntimeError(msg)
+
+
+def version():
+    return lib.llmq_version().decode()
+
+
+def target_arch():
+    return lib.llmq_target_arch().decode()

@@ -1,0 +1,143 @@
+// Per-tensor abs-max reduction for gfx950.
+//
+// Semantics follow the reference's reduce_abs_max_kernel (src/kernels/quant.cu:11-28) and
+// handle_absmax_reduction (src/kernels/kernel_utils.cuh:17-32): *result = max_i |in[i]| as fp32,
+// NaNs ignored, result >= +0, slot reset before the reduction.  The result is order independent, so
+// it is bit exact by construction.
+//
+// Design: HBM-bound streaming read (2 bytes per element).  Each lane issues UNROLL independent
+// 128-bit loads per trip (grid-stride, every wave instruction covers 1 KiB contiguous), folds them
+// with packed 16-bit integer ops, then wave shuffle -> LDS -> one global atomic per workgroup.
+//
+// The fold works on bit patterns: for a bf16 pattern p, a = p & 0x7FFF is |x|'s pattern and
+// y = 0x7F80 - a (mod 2^16) is <= 0x7F80 for every non-NaN value and >= 0xFF81 for every NaN.
+// min over y therefore ignores NaNs and finds the largest |x|; the start value 0x7F80 encodes 0.
+#include "common.hpp"
+
+namespace llmq {
+
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t fold_bf16x2(uint32_t acc, uint32_t w) {
+    u16x2 a = __builtin_bit_cast(u16x2, w & 0x7FFF7FFFu);
+    u16x2 y = (u16x2)(0x7F80) - a;
+    u16x2 m = __builtin_elementwise_min(__builtin_bit_cast(u16x2, acc), y);
+    return __builtin_bit_cast(uint32_t, m);
+}
+
+__device__ __forceinline__ uint32_t fold_vec(uint32_t acc, const uint4& v) {
+    acc = fold_bf16x2(acc, v.x);
+    acc = fold_bf16x2(acc, v.y);
+    acc = fold_bf16x2(acc, v.z);
+    acc = fold_bf16x2(acc, v.w);
+    return acc;
+}
+
+// Block-level finish shared by the bf16 and fp32 kernels: `y` is "limit - |x| pattern" (smaller is
+// larger |x|), `limit` the pattern of +Inf in that width, `shift` moves it to fp32 bit positions.
+__device__ __forceinline__ void block_min_to_atomic_max(unsigned* result, uint32_t y, uint32_t limit, int shift) {
+    __shared__ uint32_t wave_min[16];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        uint32_t o = __shfl_xor(y, off, kWave);
+        y = o < y ? o : y;
+    }
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    if (lane == 0) wave_min[wave] = y;
+    __syncthreads();
+    if (wave == 0) {
+        const int nw = blockDim.x / kWave;
+        y = lane < nw ? wave_min[lane] : limit;
+#pragma unroll
+        for (int off = 8; off > 0; off >>= 1) {
+            uint32_t o = __shfl_xor(y, off, kWave);
+            y = o < y ? o : y;
+        }
+        if (lane == 0) {
+            uint32_t bits = (limit - y) << shift;
+            if (bits != 0) atomicMax(result, bits);  // non-negative floats order like their bit patterns
+        }
+    }
+}
+
+template <int UNROLL>
+__global__ __launch_bounds__(256) void absmax_bf16_kernel(unsigned* __restrict__ result,
+                                                          const uint4* __restrict__ in, int64_t nvec,
+                                                          const uint16_t* __restrict__ tail, int ntail) {
+    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    uint32_t acc = 0x7F807F80u;
+    int64_t i = tid;
+    for (; i + (UNROLL - 1) * stride < nvec; i += UNROLL * stride) {
+        uint4 v[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) v[u] = in[i + u * stride];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) acc = fold_vec(acc, v[u]);
+    }
+    for (; i < nvec; i += stride) acc = fold_vec(acc, in[i]);
+    if (tid < ntail) acc = fold_bf16x2(acc, (uint32_t)tail[tid]);
+    uint32_t lo = acc & 0xFFFFu, hi = acc >> 16;
+    block_min_to_atomic_max(result, lo < hi ? lo : hi, 0x7F80u, 16);
+}
+
+template <int UNROLL>
+__global__ __launch_bounds__(256) void absmax_f32_kernel(unsigned* __restrict__ result,
+                                                         const uint4* __restrict__ in, int64_t nvec,
+                                                         const uint32_t* __restrict__ tail, int ntail) {
+    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    uint32_t acc = 0x7F800000u;
+    auto fold = [&](uint32_t w) {
+        uint32_t y = 0x7F800000u - (w & 0x7FFFFFFFu);  // wraps to a huge value for NaN
+        acc = y < acc ? y : acc;
+    };
+    int64_t i = tid;
+    for (; i + (UNROLL - 1) * stride < nvec; i += UNROLL * stride) {
+        uint4 v[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) v[u] = in[i + u * stride];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) { fold(v[u].x); fold(v[u].y); fold(v[u].z); fold(v[u].w); }
+    }
+    for (; i < nvec; i += stride) { uint4 v = in[i]; fold(v.x); fold(v.y); fold(v.z); fold(v.w); }
+    if (tid < ntail) fold(tail[tid]);
+    block_min_to_atomic_max(result, acc, 0x7F800000u, 0);
+}
+
+__global__ void reset_slot_kernel(unsigned* slot) { *slot = 0u; }
+
+template <typename Kernel, typename Elem>
+static int launch_absmax(Kernel kernel, float* out, const Elem* in, int64_t n, int elems_per_vec, int unroll,
+                         hipStream_t stream) {
+    LLMQ_REQUIRE(out != nullptr, "abs_max: result pointer is null");
+    LLMQ_REQUIRE(n >= 0, "abs_max: negative element count %lld", (long long)n);
+    LLMQ_REQUIRE(n == 0 || in != nullptr, "abs_max: input pointer is null");
+    LLMQ_REQUIRE(aligned16(in), "abs_max: input pointer must be 16-byte aligned");
+    // A one-lane fill kernel rather than a memset node: safe to record into a HIP graph.
+    hipLaunchKernelGGL(reset_slot_kernel, dim3(1), dim3(1), 0, stream, reinterpret_cast<unsigned*>(out));
+    LLMQ_HIP_TRY(hipGetLastError());
+    if (n == 0) return LLMQ_OK;
+    const int64_t nvec = n / elems_per_vec;
+    const int ntail = (int)(n - nvec * elems_per_vec);
+    const int64_t per_block = 256LL * unroll;
+    int64_t blocks = (nvec + per_block - 1) / per_block;
+    const int64_t max_blocks = (int64_t)cu_count() * 8;
+    if (blocks > max_blocks) blocks = max_blocks;
+    if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), 0, stream, reinterpret_cast<unsigned*>(out),
+                       reinterpret_cast<const uint4*>(in), nvec, in + nvec * elems_per_vec, ntail);
+    LLMQ_HIP_TRY(hipGetLastError());
+    return LLMQ_OK;
+}
+
+}  // namespace llmq
+
+extern "C" int llmq_abs_max_bf16(float* out, const uint16_t* in, int64_t n, void* stream) {
+    return llmq::launch_absmax(llmq::absmax_bf16_kernel<4>, out, in, n, 8, 4, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int llmq_abs_max_f32(float* out, const float* in, int64_t n, void* stream) {
+    return llmq::launch_absmax(llmq::absmax_f32_kernel<4>, out, reinterpret_cast<const uint32_t*>(in), n, 4, 4,
+                               static_cast<hipStream_t>(stream));
+}

@@ -1,0 +1,49 @@
+// Shared host/device helpers of the gfx950 FP8 path.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstdio>
+
+#include "llmq_fp8.h"
+
+namespace llmq {
+
+// Records a message for llmq_last_error() and returns `code`.
+int set_error(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+inline int hip_fail(hipError_t e, const char* what) {
+    (void)hipGetLastError();  // clear the sticky error, as the reference's CUDA_CHECK does
+    return set_error(LLMQ_ERR_RUNTIME, "%s: %s", what, hipGetErrorString(e));
+}
+
+#define LLMQ_HIP_TRY(expr)                                           \
+    do {                                                             \
+        hipError_t _e = (expr);                                      \
+        if (_e != hipSuccess) return ::llmq::hip_fail(_e, #expr);    \
+    } while (0)
+
+#define LLMQ_REQUIRE(cond, ...)                                                    \
+    do {                                                                           \
+        if (!(cond)) return ::llmq::set_error(LLMQ_ERR_INVALID_ARGUMENT, __VA_ARGS__); \
+    } while (0)
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Number of compute units of the current device (cached per device id).
+int cu_count();
+
+constexpr int kWave = 64;
+
+// ---- device helpers -----------------------------------------------------------------------------
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xFFFF0000u); }
+
+// scale = 448 / max(absmax, 1e-10) with an IEEE-correct fp32 division (src/kernels/quant.cu:79).
+__device__ __forceinline__ float quant_scale(float absmax) {
+    float a = (absmax > 1e-10f) ? absmax : 1e-10f;  // fmaxf semantics incl. NaN -> 1e-10
+    return __fdiv_rn(448.f, a);
+}
+
+}  // namespace llmq

@@ -1,0 +1,225 @@
+// Scaled bf16 -> fp8 quantization (plain and with fused transpose) for gfx950.
+//
+// Semantics follow the reference's quantize_with_abs_max_kernel (src/kernels/quant.cu:73-93) and
+// quantize_and_transpose_with_abs_max_kernel (src/kernels/quant.cu:151-164):
+//   scale = 448.f / fmaxf(*abs_max, 1e-10f);  out = fp8_rn_satfinite(scale * (float)in);
+//   *scale_ptr = 1.f / scale  (written by one lane when the pointer is non-null).
+// The conversion the reference calls is the CUDA toolkit's saturating round-to-nearest-even one:
+// NaN -> 0x7F (sign dropped), |y| above the largest finite value (and +-Inf) -> +-max, zero and
+// underflow keep their sign.  Here the gfx950 packed conversion instruction (OCP formats) does the
+// rounding; saturation is made explicit with a median-of-three clamp and NaNs are patched in a
+// rarely-taken branch, so the bytes do not depend on the instruction's overflow/NaN conventions.
+//
+// Both kernels are HBM bound (2 bytes read + 1 byte written per element): every global access is a
+// 128-bit (or 64-bit for the plain kernel's stores) per-lane access that is contiguous across the
+// wave; the transposing kernel stages a [64 or 128 cols] x [256 rows] tile of fp8 codes in LDS
+// (row stride 65 dwords: conflict-free for both the dword writes and the dword reads) so that the
+// stores along the transposed rows are 256-byte contiguous per 16 lanes.
+#include "common.hpp"
+
+namespace llmq {
+
+enum Fp8Format { kE4M3 = 0, kE5M2 = 1 };
+
+template <int FMT>
+__device__ __forceinline__ float clamp_finite(float y) {
+    constexpr float lim = FMT == kE4M3 ? 448.f : 57344.f;
+    return __builtin_amdgcn_fmed3f(y, -lim, lim);  // +-Inf and overflow -> +-max finite
+}
+
+// Packs fp8(a), fp8(b) into the low (hi == false) or high half of `old`.
+template <int FMT>
+__device__ __forceinline__ uint32_t cvt_pk(float a, float b, uint32_t old, bool hi) {
+    if constexpr (FMT == kE4M3) {
+        return hi ? (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, (int)old, true)
+                  : (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, (int)old, false);
+    } else {
+        return hi ? (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(a, b, (int)old, true)
+                  : (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(a, b, (int)old, false);
+    }
+}
+
+// Four scaled values -> one dword of four codes (y0 in the lowest byte).
+template <int FMT>
+__device__ __forceinline__ uint32_t encode4(float y0, float y1, float y2, float y3) {
+    uint32_t w = cvt_pk<FMT>(clamp_finite<FMT>(y0), clamp_finite<FMT>(y1), 0u, false);
+    w = cvt_pk<FMT>(clamp_finite<FMT>(y2), clamp_finite<FMT>(y3), w, true);
+    if (__builtin_expect((y0 != y0) | (y1 != y1) | (y2 != y2) | (y3 != y3), 0)) {
+        if (y0 != y0) w = (w & 0xFFFFFF00u) | 0x0000007Fu;
+        if (y1 != y1) w = (w & 0xFFFF00FFu) | 0x00007F00u;
+        if (y2 != y2) w = (w & 0xFF00FFFFu) | 0x007F0000u;
+        if (y3 != y3) w = (w & 0x00FFFFFFu) | 0x7F000000u;
+    }
+    return w;
+}
+
+template <int FMT>
+__device__ __forceinline__ uint2 encode8(const uint4& v, float s) {
+    uint2 r;
+    r.x = encode4<FMT>(s * bf16_lo(v.x), s * bf16_hi(v.x), s * bf16_lo(v.y), s * bf16_hi(v.y));
+    r.y = encode4<FMT>(s * bf16_lo(v.z), s * bf16_hi(v.z), s * bf16_lo(v.w), s * bf16_hi(v.w));
+    return r;
+}
+
+template <int FMT, int UNROLL>
+__global__ __launch_bounds__(256) void quantize_kernel(uint2* __restrict__ out, float* __restrict__ scale_ptr,
+                                                       const uint4* __restrict__ in,
+                                                       const float* __restrict__ absmax, int64_t nvec,
+                                                       const uint16_t* __restrict__ tail_in,
+                                                       uint8_t* __restrict__ tail_out, int ntail) {
+    const float s = quant_scale(*absmax);
+    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    if (tid == 0 && scale_ptr) *scale_ptr = __fdiv_rn(1.f, s);
+    int64_t i = tid;
+    for (; i + (UNROLL - 1) * stride < nvec; i += UNROLL * stride) {
+        uint4 v[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) v[u] = in[i + u * stride];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) out[i + u * stride] = encode8<FMT>(v[u], s);
+    }
+    for (; i < nvec; i += stride) out[i] = encode8<FMT>(in[i], s);
+    if (tid < ntail) {
+        float y = s * __uint_as_float((uint32_t)tail_in[tid] << 16);
+        tail_out[tid] = (uint8_t)(encode4<FMT>(y, 0.f, 0.f, 0.f) & 0xFFu);
+    }
+}
+
+// ---- quantize + transpose -------------------------------------------------------------------------
+constexpr int kQtRows = 256;       // tile extent along the input rows (= contiguous bytes of the output)
+constexpr int kQtStride = 65;      // LDS row stride in dwords (64 dwords of payload + 1 pad)
+
+// NCH = number of 8-column chunks per tile: the tile is [kQtRows rows] x [8*NCH cols].
+template <int NCH>
+__global__ __launch_bounds__(256) void quantize_transpose_kernel(uint8_t* __restrict__ out,
+                                                                 float* __restrict__ scale_ptr,
+                                                                 const uint16_t* __restrict__ in,
+                                                                 const float* __restrict__ absmax, int rows,
+                                                                 int cols, int rows_mult16) {
+    constexpr int TC = 8 * NCH;
+    constexpr int QPP = 256 / NCH;            // row quads per pass
+    constexpr int PASSES = (kQtRows / 4) / QPP;
+    __shared__ uint32_t tile[TC * kQtStride];
+
+    const float s = quant_scale(*absmax);
+    const int t = threadIdx.x;
+    if (t == 0 && blockIdx.x == 0 && blockIdx.y == 0 && scale_ptr) *scale_ptr = __fdiv_rn(1.f, s);
+
+    const int r0 = blockIdx.y * kQtRows;
+    const int c0 = blockIdx.x * TC;
+    const int chunk = t % NCH;
+    const int q = t / NCH;
+    const int col = c0 + 8 * chunk;
+
+    uint4 v[PASSES][4];
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+        const int rq = q + QPP * p;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int row = r0 + 4 * rq + j;
+            if (row < rows && col < cols) {
+                v[p][j] = *reinterpret_cast<const uint4*>(in + (int64_t)row * cols + col);
+            } else {
+                v[p][j] = make_uint4(0, 0, 0, 0);
+            }
+        }
+    }
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+        const int rq = q + QPP * p;
+        const uint32_t w[4][4] = {{v[p][0].x, v[p][0].y, v[p][0].z, v[p][0].w},
+                                  {v[p][1].x, v[p][1].y, v[p][1].z, v[p][1].w},
+                                  {v[p][2].x, v[p][2].y, v[p][2].z, v[p][2].w},
+                                  {v[p][3].x, v[p][3].y, v[p][3].z, v[p][3].w}};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {  // word k holds columns 2k (low half) and 2k+1 (high half)
+            const uint32_t even = encode4<kE4M3>(s * bf16_lo(w[0][k]), s * bf16_lo(w[1][k]),
+                                                 s * bf16_lo(w[2][k]), s * bf16_lo(w[3][k]));
+            const uint32_t odd = encode4<kE4M3>(s * bf16_hi(w[0][k]), s * bf16_hi(w[1][k]),
+                                                s * bf16_hi(w[2][k]), s * bf16_hi(w[3][k]));
+            tile[(8 * chunk + 2 * k) * kQtStride + rq] = even;
+            tile[(8 * chunk + 2 * k + 1) * kQtStride + rq] = odd;
+        }
+    }
+    __syncthreads();
+
+    constexpr int ITEMS = TC * (kQtRows / 16);  // 16-byte pieces in the tile
+#pragma unroll
+    for (int it = 0; it < ITEMS / 256; ++it) {
+        const int item = t + 256 * it;
+        const int c = item / 16, p = item % 16;
+        const int r = r0 + 16 * p;
+        if (c0 + c < cols && r < rows) {
+            const uint32_t* src = &tile[c * kQtStride + 4 * p];
+            uint8_t* dst = out + (int64_t)(c0 + c) * rows + r;
+            if (rows_mult16) {
+                *reinterpret_cast<uint4*>(dst) = make_uint4(src[0], src[1], src[2], src[3]);
+            } else {
+                *reinterpret_cast<uint2*>(dst) = make_uint2(src[0], src[1]);
+                if (r + 8 < rows) *reinterpret_cast<uint2*>(dst + 8) = make_uint2(src[2], src[3]);
+            }
+        }
+    }
+}
+
+template <int FMT>
+static int launch_quantize(uint8_t* out, float* scale_ptr, const uint16_t* in, const float* absmax, int64_t n,
+                           hipStream_t stream) {
+    LLMQ_REQUIRE(n >= 0, "quantize_with_abs_max: negative element count %lld", (long long)n);
+    LLMQ_REQUIRE(absmax != nullptr, "quantize_with_abs_max: abs_max pointer is null");
+    LLMQ_REQUIRE(n == 0 || (out != nullptr && in != nullptr), "quantize_with_abs_max: null tensor pointer");
+    LLMQ_REQUIRE(aligned16(in) && aligned16(out), "quantize_with_abs_max: tensors must be 16-byte aligned");
+    constexpr int UNROLL = 4;
+    const int64_t nvec = n / 8;
+    const int ntail = (int)(n - nvec * 8);
+    int64_t blocks = (nvec + 256 * UNROLL - 1) / (256 * UNROLL);
+    const int64_t max_blocks = (int64_t)cu_count() * 8;
+    if (blocks > max_blocks) blocks = max_blocks;
+    if (blocks < 1) blocks = 1;  // still writes the scale for n == 0
+    hipLaunchKernelGGL((quantize_kernel<FMT, UNROLL>), dim3((unsigned)blocks), dim3(256), 0, stream,
+                       reinterpret_cast<uint2*>(out), scale_ptr, reinterpret_cast<const uint4*>(in), absmax, nvec,
+                       in + nvec * 8, out + nvec * 8, ntail);
+    LLMQ_HIP_TRY(hipGetLastError());
+    return LLMQ_OK;
+}
+
+}  // namespace llmq
+
+extern "C" int llmq_quantize_e4m3_bf16(uint8_t* out, float* scale_or_null, const uint16_t* in,
+                                       const float* absmax, int64_t n, void* stream) {
+    return llmq::launch_quantize<llmq::kE4M3>(out, scale_or_null, in, absmax, n, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int llmq_quantize_e5m2_bf16(uint8_t* out, float* scale_or_null, const uint16_t* in,
+                                       const float* absmax, int64_t n, void* stream) {
+    return llmq::launch_quantize<llmq::kE5M2>(out, scale_or_null, in, absmax, n, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int llmq_quantize_transpose_e4m3_bf16(uint8_t* out, float* scale_or_null, const uint16_t* in,
+                                                 const float* absmax, int rows, int cols, void* stream) {
+    using namespace llmq;
+    LLMQ_REQUIRE(rows >= 0 && cols >= 0, "quantize_and_transpose_with_abs_max: negative shape %d x %d", rows, cols);
+    LLMQ_REQUIRE(rows % 8 == 0 && cols % 8 == 0,
+                 "quantize_and_transpose_with_abs_max: rows (%d) and cols (%d) must be multiples of 8", rows, cols);
+    LLMQ_REQUIRE(absmax != nullptr, "quantize_and_transpose_with_abs_max: abs_max pointer is null");
+    const bool empty = rows == 0 || cols == 0;
+    LLMQ_REQUIRE(empty || (out != nullptr && in != nullptr), "quantize_and_transpose_with_abs_max: null tensor pointer");
+    LLMQ_REQUIRE(aligned16(in) && aligned16(out), "quantize_and_transpose_with_abs_max: tensors must be 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int rows_mult16 = rows % 16 == 0;
+    const unsigned gy = empty ? 1u : (unsigned)((rows + kQtRows - 1) / kQtRows);
+    // Wide tiles (256-byte row segments on the read side) once there are enough of them to fill the chip.
+    const int64_t wide_tiles = (int64_t)((cols + 127) / 128) * gy;
+    if (!empty && cols >= 128 && wide_tiles >= 2LL * cu_count()) {
+        hipLaunchKernelGGL(quantize_transpose_kernel<16>, dim3((unsigned)((cols + 127) / 128), gy), dim3(256), 0, st,
+                           out, scale_or_null, in, absmax, rows, cols, rows_mult16);
+    } else {
+        const unsigned gx = empty ? 1u : (unsigned)((cols + 63) / 64);
+        hipLaunchKernelGGL(quantize_transpose_kernel<8>, dim3(gx, gy), dim3(256), 0, st, out, scale_or_null, in,
+                           absmax, empty ? 0 : rows, empty ? 0 : cols, rows_mult16);
+    }
+    LLMQ_HIP_TRY(hipGetLastError());
+    return LLMQ_OK;
+}

@@ -1,0 +1,102 @@
+"""Host-side mirror of the reference's per-kernel Python entry points for the FP8 path
+(reference: src/binding/python/kernels.py:121-165, src/binding/kernel_binding.cpp:393-509), on torch
+tensors that live on the MI355X.  torch is used only for device memory and streams; every call goes
+through the C ABI (llmq_amd.capi) into the hand-written gfx950 kernels.
+
+Names, argument order and in-place "out first" convention are the reference's:
+    abs_max(scale, x, stream=0)
+    quantize_with_abs_max(out, scale, x, abs_max, stream=0)
+    quantize_and_transpose_with_abs_max(out, scale, x, abs_max, stream=0)
+    transpose(dst, src, stream=0)
+    matmul(c, a, b, bias, scale_a, scale_b, M, N, K, accumulate=False, stream=0)   [kernels.h convention]
+`stream` is a raw hipStream_t handle (0 = torch's current stream).
+"""
+import torch
+
+from . import capi
+
+_FP8 = (torch.float8_e4m3fn, torch.float8_e5m2, torch.uint8)
+
+
+def _stream(stream):
+    return stream if stream else torch.cuda.current_stream().cuda_stream
+
+
+def _dev(t, name, dtypes=None, optional=False):
+    if t is None:
+        if optional:
+            return None
+        raise ValueError("%s must not be None" % name)
+    if not t.is_cuda:
+        raise ValueError("%s must be a device tensor" % name)
+    if not t.is_contiguous():
+        raise ValueError("%s must be contiguous" % name)
+    if dtypes is not None and t.dtype not in dtypes:
+        raise ValueError("%s: unsupported dtype %s" % (name, t.dtype))
+    return t.data_ptr()
+
+
+def abs_max(scale, x, stream=0):
+    """scale[0] = max |x| (fp32).  x: bf16 or fp32 device tensor."""
+    out = _dev(scale, "scale", (torch.float32,))
+    ptr = _dev(x, "x", (torch.bfloat16, torch.float32))
+    f = capi.lib.llmq_abs_max_bf16 if x.dtype == torch.bfloat16 else capi.lib.llmq_abs_max_f32
+    capi.check(f(out, ptr, x.numel(), _stream(stream)))
+
+
+def quantize_with_abs_max(out, scale, x, abs_max, stream=0):
+    """out = fp8(448/abs_max * x); scale[0] = abs_max/448 (as 1/(448/abs_max)).  scale may be None."""
+    o = _dev(out, "out", _FP8)
+    s = _dev(scale, "scale", (torch.float32,), optional=True)
+    i = _dev(x, "x", (torch.bfloat16,))
+    a = _dev(abs_max, "abs_max", (torch.float32,))
+    if out.numel() != x.numel():
+        raise ValueError("out and x must have the same number of elements")
+    f = capi.lib.llmq_quantize_e5m2_bf16 if out.dtype == torch.float8_e5m2 else capi.lib.llmq_quantize_e4m3_bf16
+    capi.check(f(o, s, i, a, x.numel(), _stream(stream)))
+
+
+def quantize_and_transpose_with_abs_max(out, scale, x, abs_max, stream=0):
+    """x: [rows, cols] bf16 -> out: [cols, rows] e4m3."""
+    if x.dim() != 2 or out.dim() != 2 or out.shape[0] != x.shape[1] or out.shape[1] != x.shape[0]:
+        raise ValueError("x must be [rows, cols] and out [cols, rows]")
+    o = _dev(out, "out", (torch.float8_e4m3fn, torch.uint8))
+    s = _dev(scale, "scale", (torch.float32,), optional=True)
+    i = _dev(x, "x", (torch.bfloat16,))
+    a = _dev(abs_max, "abs_max", (torch.float32,))
+    capi.check(capi.lib.llmq_quantize_transpose_e4m3_bf16(o, s, i, a, x.shape[0], x.shape[1], _stream(stream)))
+
+
+def transpose(dst, src, stream=0):
+    """src: [rows, cols] fp8 codes -> dst: [cols, rows]."""
+    if src.dim() != 2 or dst.dim() != 2 or dst.shape[0] != src.shape[1] or dst.shape[1] != src.shape[0]:
+        raise ValueError("src must be [rows, cols] and dst [cols, rows]")
+    if dst.dtype != src.dtype:
+        raise ValueError("dst and src must have the same dtype")
+    d = _dev(dst, "dst", _FP8)
+    s = _dev(src, "src", _FP8)
+    capi.check(capi.lib.llmq_transpose_u8(d, s, src.shape[0], src.shape[1], _stream(stream)))
+
+
+def matmul(c, a, b, bias, scale_a, scale_b, M, N, K, accumulate=False, stream=0):
+    """TN matmul in the convention of the reference's kernels.h: row-major a[M,K], b[N,K] (e4m3) give
+    row-major c[N,M] = (b @ a.T) * scale_a * scale_b (+ bias[M]) (+ c).  c: bf16 or fp32."""
+    pa = _dev(a, "a", (torch.float8_e4m3fn, torch.uint8))
+    pb = _dev(b, "b", (torch.float8_e4m3fn, torch.uint8))
+    pc = _dev(c, "c", (torch.bfloat16, torch.float32))
+    if a.numel() != M * K or b.numel() != N * K or c.numel() != N * M:
+        raise ValueError("operand sizes do not match M, N, K")
+    sa = _dev(scale_a, "scale_a", (torch.float32,), optional=True)
+    sb = _dev(scale_b, "scale_b", (torch.float32,), optional=True)
+    if c.dtype == torch.bfloat16:
+        pbias = _dev(bias, "bias", (torch.bfloat16,), optional=True)
+        if bias is not None and bias.numel() != M:
+            raise ValueError("bias must have M elements")
+        capi.check(capi.lib.llmq_gemm_tn_e4m3_bf16(pc, pa, pb, pbias, sa, sb, M, N, K, int(accumulate), _stream(stream)))
+    else:
+        pbias = _dev(bias, "bias", (torch.bfloat16, torch.float32), optional=True)
+        if bias is not None and bias.numel() != M:
+            raise ValueError("bias must have M elements")
+        is_bf16 = int(bias is not None and bias.dtype == torch.bfloat16)
+        capi.check(capi.lib.llmq_gemm_tn_e4m3_f32(pc, pa, pb, pbias, is_bf16, sa, sb, M, N, K, int(accumulate),
+                                                  _stream(stream)))

@@ -1,0 +1,52 @@
+"""Helpers shared by the GPU parity tests: host<->device moves of raw bit patterns and the GEMM
+tolerance of the path (stated once, here)."""
+import numpy as np
+import torch
+
+
+def dev_bf16(bits):
+    """uint16 bf16 patterns (numpy) -> bf16 device tensor with the same bits."""
+    return torch.from_numpy(np.ascontiguousarray(bits).view(np.int16)).view(torch.bfloat16).cuda()
+
+
+def dev_u8(codes):
+    return torch.from_numpy(np.ascontiguousarray(codes, dtype=np.uint8)).cuda()
+
+
+def host_bits(t):
+    """device tensor -> numpy array of raw patterns (uint16 for bf16, uint8 for fp8/uint8, fp32 as is)."""
+    t = t.detach().cpu()
+    if t.dtype == torch.bfloat16:
+        return t.view(torch.int16).numpy().view(np.uint16)
+    if t.dtype in (torch.float8_e4m3fn, torch.float8_e5m2):
+        return t.view(torch.uint8).numpy()
+    return t.numpy()
+
+
+def dev_scalar(v):
+    return torch.tensor([v], dtype=torch.float32, device="cuda")
+
+
+# GEMM tolerance versus the exact (fp64) product of the same e4m3 operands times the fp32 factor sa*sb:
+#   bf16 output:  |err| <= 2^-8 * |ref| + 2^-20 * (sa*sb) * sum_k |a_k b_k|     and rel-Frobenius <= 2.5e-3
+#   fp32 output:  |err| <= 2^-18 * (sa*sb) * sum_k |a_k b_k|                    and rel-Frobenius <= 5e-5
+# (2^-8 is half a bf16 ulp of the result; the second term bounds fp32 accumulation in any order.)
+def gemm_check(got_f32, exact, sumabs, scale, out_is_bf16, extra=None):
+    """got_f32: decoded device result; exact/sumabs: oracle fp64 arrays of the same shape; extra: fp64
+    array added after scaling (bias + old c).  Returns (max_abs_err, rel_frobenius); asserts the bounds."""
+    ref = exact * float(scale)
+    if extra is not None:
+        ref = ref + extra
+    err = np.abs(got_f32.astype(np.float64) - ref)
+    mag = np.abs(float(scale)) * sumabs + (np.abs(extra) if extra is not None else 0.0)
+    if out_is_bf16:
+        bound = 2.0 ** -8 * np.abs(ref) + 2.0 ** -20 * mag + 1e-38
+        fro_lim = 2.5e-3
+    else:
+        bound = 2.0 ** -18 * mag + 1e-38
+        fro_lim = 5e-5
+    worst = float((err / bound).max())
+    assert worst <= 1.0, "GEMM element error exceeds the stated bound by x%.3f" % worst
+    fro = float(np.sqrt((err ** 2).sum()) / max(np.sqrt((ref ** 2).sum()), 1e-300))
+    assert fro <= fro_lim, "relative Frobenius error %.3e > %.1e" % (fro, fro_lim)
+    return float(err.max()), fro

@@ -1,0 +1,268 @@
+"""GPU parity tests: every call goes through the C ABI (llmq_amd.capi via llmq_amd.kernels) and is
+compared with the CPU oracle on identical inputs.  abs-max, scales and fp8 bytes must be bit exact;
+GEMM results must meet the tolerance stated in tests/gpu_util.py."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import dev_bf16, dev_scalar, dev_u8, gemm_check, host_bits
+
+pytestmark = pytest.mark.gpu
+
+ALL_BF16 = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+
+
+@pytest.fixture(scope="module")
+def K():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from llmq_amd import kernels
+    return kernels
+
+
+def gpu_abs_max(K, bits):
+    out = torch.full((1,), 123.0, dtype=torch.float32, device="cuda")   # stale value must be overwritten
+    K.abs_max(out, dev_bf16(bits))
+    return out.cpu().numpy()[0]
+
+
+def gpu_quantize(K, bits, absmax, fmt=torch.float8_e4m3fn, with_scale=True):
+    x = dev_bf16(bits)
+    out = torch.empty(x.shape, dtype=fmt, device="cuda")
+    scale = torch.full((1,), -1.0, dtype=torch.float32, device="cuda") if with_scale else None
+    K.quantize_with_abs_max(out, scale, x, dev_scalar(absmax))
+    return host_bits(out), (scale.cpu().numpy()[0] if with_scale else None)
+
+
+# ------------------------------------------------------------------------------------------ abs-max
+@pytest.mark.parametrize("n", [8, 64, 1000, 1024, 16 * 64, 4 * 128 * 32, 1 << 20, (1 << 20) + 8, 3 * 1000 * 1000 + 5, 7])
+def test_abs_max_bit_exact(K, O, n):
+    x = O.fill_normal_bf16(n, 100 + n % 97, 1, 0.0, 2.5)
+    assert gpu_abs_max(K, x).view(np.uint32) == np.float32(O.abs_max_bf16(x)).view(np.uint32)
+
+
+def test_abs_max_special_values(K, O):
+    cases = [
+        np.array([0x7FC0, 0x7F81, 0xFFC1, 0xFFFF] * 2, np.uint16),                 # all NaN -> 0
+        np.array([0x8000] * 16, np.uint16),                                         # -0 -> +0
+        np.array([0x3F80, 0x7FC0, 0xC000, 0x7F81, 0, 0, 0, 0], np.uint16),          # NaN skipped -> 2
+        np.array([0x3F80, 0xFF80, 0x7FC0, 0, 0, 0, 0, 0], np.uint16),               # -Inf wins
+        np.array([0x0001, 0x8003, 0, 0, 0, 0, 0, 0], np.uint16),                    # denormals kept
+        np.array([0x7F7F, 0xFF7F] + [0] * 6, np.uint16),                            # max finite
+        np.zeros(0, np.uint16),                                                     # empty -> 0
+    ]
+    for c in cases:
+        got, want = gpu_abs_max(K, c), np.float32(O.abs_max_bf16(c))
+        assert got.view(np.uint32) == want.view(np.uint32), (c, got, want)
+    # maximum hidden at every position of a block-sized tensor's tail
+    base = O.fill_normal_bf16(1 << 16, 5, 5)
+    for pos in [0, 1, 7, 8, 65535, 65528, 4099]:
+        x = base.copy()
+        x[pos] = 0xC2C8  # -100
+        assert gpu_abs_max(K, x) == 100.0
+
+
+def test_abs_max_f32(K):
+    g = torch.Generator(device="cuda").manual_seed(3)
+    x = torch.randn(1000003, device="cuda", generator=g) * 7
+    x[12345] = float("nan")
+    out = torch.zeros(1, device="cuda")
+    K.abs_max(out, x)
+    assert out.item() == torch.nan_to_num(x, nan=0.0).abs().max().item()
+
+
+# ----------------------------------------------------------------------------------------- quantize
+@pytest.mark.parametrize("absmax", [448.0, 1.0, 5.15625, 0.072265625, 3.0e-5, 1e4, 0.0, 447.0, 1.7e38, float("inf")])
+def test_quantize_exhaustive_all_bf16_inputs(K, O, absmax):
+    got, scale = gpu_quantize(K, ALL_BF16, absmax)
+    want, d = O.quantize_e4m3(ALL_BF16, absmax)
+    bad = np.nonzero(got != want)[0]
+    assert bad.size == 0, [(hex(int(ALL_BF16[i])), hex(int(got[i])), hex(int(want[i]))) for i in bad[:10]]
+    assert np.float32(scale).view(np.uint32) == np.float32(d).view(np.uint32)
+
+
+@pytest.mark.parametrize("absmax", [448.0, 57344.0, 1.0, 3.0e-5, 0.0])
+def test_quantize_e5m2_exhaustive(K, O, absmax):
+    got, scale = gpu_quantize(K, ALL_BF16, absmax, fmt=torch.float8_e5m2)
+    want, d = O.quantize_e4m3(ALL_BF16, absmax, fmt="e5m2")
+    bad = np.nonzero(got != want)[0]
+    assert bad.size == 0, [(hex(int(ALL_BF16[i])), hex(int(got[i])), hex(int(want[i]))) for i in bad[:10]]
+    assert np.float32(scale).view(np.uint32) == np.float32(d).view(np.uint32)
+
+
+@pytest.mark.parametrize("n", [8, 1024, 8192, 8200, 1 << 20, 4096 * 896, 13])
+def test_quantize_random_tensors(K, O, n):
+    x = O.fill_normal_bf16(n, 7, n % 11)
+    am = O.abs_max_bf16(x)
+    got, scale = gpu_quantize(K, x, am)
+    want, d = O.quantize_e4m3(x, am, mt=True)
+    assert np.array_equal(got, want) and np.float32(scale) == d
+    got2, none = gpu_quantize(K, x, am, with_scale=False)      # null scale pointer
+    assert np.array_equal(got2, want) and none is None
+
+
+def test_quantize_stale_absmax_saturates(K, O):
+    x = O.fill_normal_bf16(1 << 16, 9, 9, 0.0, 10.0)
+    got, _ = gpu_quantize(K, x, 1.0)              # abs-max far too small: values clamp at +-448
+    want, _ = O.quantize_e4m3(x, 1.0)
+    assert np.array_equal(got, want) and (got == 0x7E).any() and (got == 0xFE).any()
+
+
+# ------------------------------------------------------------------------- quantize + transpose, transpose
+QT_SHAPES = [(32, 32), (128, 256), (512, 1024), (8, 8), (8, 72), (72, 8), (264, 136), (256, 64), (1000, 24),
+             (4096, 896), (520, 1160), (2048, 4864)]
+
+
+@pytest.mark.parametrize("shape", QT_SHAPES)
+def test_quantize_transpose_bit_exact(K, O, shape):
+    rows, cols = shape
+    x = O.fill_normal_bf16(rows * cols, 21, rows + cols).reshape(rows, cols)
+    am = O.abs_max_bf16(x)
+    want, d = O.quantize_e4m3(x, am, mt=True)
+    xd = dev_bf16(x)
+    out = torch.empty((cols, rows), dtype=torch.float8_e4m3fn, device="cuda")
+    scale = torch.zeros(1, device="cuda")
+    K.quantize_and_transpose_with_abs_max(out, scale, xd, dev_scalar(am))
+    assert np.array_equal(host_bits(out), want.T)
+    assert scale.item() == d
+    out2 = torch.empty((cols, rows), dtype=torch.float8_e4m3fn, device="cuda")
+    K.quantize_and_transpose_with_abs_max(out2, None, xd, dev_scalar(am))   # null scale as at llama_model.cpp:328
+    assert np.array_equal(host_bits(out2), want.T)
+
+
+@pytest.mark.parametrize("shape", QT_SHAPES + [(1, 1), (3, 5), (17, 33), (100, 7), (64, 65), (4864, 896), (16, 4096)])
+def test_transpose_bit_exact(K, shape):
+    rows, cols = shape
+    rng = np.random.default_rng(rows * 131 + cols)
+    src = rng.integers(0, 256, (rows, cols)).astype(np.uint8)
+    d = torch.empty((cols, rows), dtype=torch.uint8, device="cuda")
+    K.transpose(d, dev_u8(src))
+    assert np.array_equal(d.cpu().numpy(), src.T)
+
+
+# --------------------------------------------------------------------------------------------- GEMM
+def set_variant(v):
+    from llmq_amd import capi
+    capi.lib.llmq_debug_set_gemm_variant(v)
+
+
+VARIANTS = [0, 1, 2, 3, 4, 5]
+
+
+def run_gemm(K, a, b, M, N, Kd, sa, sb, bias_bits=None, old=None, out_f32=False):
+    dt = torch.float32 if out_f32 else torch.bfloat16
+    if old is not None:
+        c = (torch.from_numpy(old).cuda() if out_f32 else dev_bf16(old)).reshape(N, M).clone()
+    else:
+        c = torch.full((N, M), float("nan"), dtype=dt, device="cuda")
+    bias = dev_bf16(bias_bits) if bias_bits is not None else None
+    K.matmul(c, dev_u8(a), dev_u8(b), bias, dev_scalar(sa) if sa is not None else None,
+             dev_scalar(sb) if sb is not None else None, M, N, Kd, accumulate=old is not None)
+    torch.cuda.synchronize()
+    return c
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("mnk", [(128, 128, 128), (256, 256, 256), (512, 768, 384), (256, 512, 1024)])
+def test_gemm_integer_known_answer_exact(K, O, variant, mnk):
+    """Construction of src/testing/test-gemm.cpp:54-85: integer operands, exact fp32 sums -> the bf16
+    output must equal the oracle bit for bit (set / bias / accumulate)."""
+    M, N, Kd = mnk
+    if variant in (1, 2, 5) and (M % 256 or N % 256):
+        pytest.skip("256-tile variants need multiples of 256")
+    a, _ = O.fill_int_e4m3(M * Kd, 12345, 0)
+    b, _ = O.fill_int_e4m3(N * Kd, 12345, 1)
+    a, b = a.reshape(M, Kd), b.reshape(N, Kd)
+    s = float(np.sqrt(np.float32(4.0 / Kd)))
+    _, biasv = O.fill_int_e4m3(M, 12345, 2)
+    _, oldv = O.fill_int_e4m3(N * M, 12345, 3)
+    bias = O.f32_to_bf16(biasv.astype(np.float32))
+    old = O.f32_to_bf16(oldv.astype(np.float32)).reshape(N, M)
+    set_variant(variant)
+    try:
+        for use_bias, use_old in [(False, False), (True, False), (False, True), (True, True)]:
+            want = O.gemm_tn(a, b, sa=s, sb=s, bias=bias if use_bias else None, c_old=old if use_old else None, mt=True)
+            got = run_gemm(K, a, b, M, N, Kd, s, s, bias if use_bias else None, old if use_old else None)
+            assert np.array_equal(host_bits(got), want), (use_bias, use_old)
+        want32 = O.gemm_tn(a, b, sa=s, sb=s, out_f32=True, mt=True)
+        got32 = run_gemm(K, a, b, M, N, Kd, s, s, out_f32=True)
+        assert np.array_equal(got32.cpu().numpy(), want32)
+    finally:
+        set_variant(0)
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("out_f32", [False, True])
+def test_gemm_random_codes_within_tolerance(K, O, variant, out_f32):
+    M, N, Kd = 512, 256, 896
+    rng = np.random.default_rng(17)
+    a = rng.integers(0, 256, (M, Kd)).astype(np.uint8)
+    b = rng.integers(0, 256, (N, Kd)).astype(np.uint8)
+    a[(a & 0x7F) == 0x7F] ^= 1      # no NaN codes
+    b[(b & 0x7F) == 0x7F] ^= 1
+    sa, sb = 0.37, 1.0 / 448
+    exact, sumabs = O.gemm_exact(a, b)
+    scale = np.float32(np.float32(sa) * np.float32(sb))
+    set_variant(variant)
+    try:
+        got = run_gemm(K, a, b, M, N, Kd, sa, sb, out_f32=out_f32)
+        g32 = got.float().cpu().numpy()
+        gemm_check(g32, exact, sumabs, scale, not out_f32)
+        # no scales at all (null pointers)
+        got1 = run_gemm(K, a, b, M, N, Kd, None, None, out_f32=True)
+        gemm_check(got1.cpu().numpy(), exact, sumabs, 1.0, False)
+        # bias + accumulate on top
+        bias = O.fill_normal_bf16(M, 3, 3, 0.0, 50.0)
+        old = O.bf16_to_f32(O.fill_normal_bf16(N * M, 3, 4, 0.0, 100.0)).reshape(N, M)
+        oldp = old if out_f32 else O.f32_to_bf16(old)
+        got2 = run_gemm(K, a, b, M, N, Kd, sa, sb, bias, oldp, out_f32=out_f32)
+        extra = O.bf16_to_f32(bias).astype(np.float64)[None, :] + old.astype(np.float64)
+        gemm_check(got2.float().cpu().numpy(), exact, sumabs, scale, not out_f32, extra=extra)
+    finally:
+        set_variant(0)
+
+
+def test_gemm_matches_swapped_operand_transpose(K, O):
+    """c(a,b)^T == c(b,a): a size-independent identity that catches row/column mix-ups."""
+    M, N, Kd = 384, 640, 256
+    rng = np.random.default_rng(2)
+    a = rng.integers(0, 0x7E, (M, Kd)).astype(np.uint8) | (rng.integers(0, 2, (M, Kd)).astype(np.uint8) << 7)
+    b = rng.integers(0, 0x7E, (N, Kd)).astype(np.uint8) | (rng.integers(0, 2, (N, Kd)).astype(np.uint8) << 7)
+    c1 = run_gemm(K, a, b, M, N, Kd, 0.01, 0.5, out_f32=True)
+    c2 = run_gemm(K, b, a, N, M, Kd, 0.5, 0.01, out_f32=True)
+    assert torch.allclose(c1, c2.T, rtol=1e-5, atol=1e-4)
+
+
+# ----------------------------------------------------------------------- configuration 1, end to end
+def test_config1_forward_pipeline(K, O):
+    """X[4096x896]~N(0,1), W[4864x896]~N(0,0.02), seed 0: abs-max, quantize both, Y = X W^T (bf16)."""
+    BT, C, OC = 4096, 896, 4864
+    x = O.fill_normal_bf16(BT * C, 0, 1, 0.0, 1.0).reshape(BT, C)
+    w = O.fill_normal_bf16(OC * C, 0, 2, 0.0, 0.02).reshape(OC, C)
+    xd, wd = dev_bf16(x), dev_bf16(w)
+    stats = torch.zeros(4, device="cuda")          # [x absmax, x scale, w absmax, w scale]
+    xq = torch.empty((BT, C), dtype=torch.float8_e4m3fn, device="cuda")
+    wq = torch.empty((OC, C), dtype=torch.float8_e4m3fn, device="cuda")
+    y = torch.empty((BT, OC), dtype=torch.bfloat16, device="cuda")
+    K.abs_max(stats[0:1], xd)
+    K.abs_max(stats[2:3], wd)
+    K.quantize_with_abs_max(xq, stats[1:2], xd, stats[0:1])
+    K.quantize_with_abs_max(wq, stats[3:4], wd, stats[2:3])
+    K.matmul(y, wq, xq, None, stats[3:4], stats[1:2], OC, BT, C)       # forward_qmm call, llama_model.cpp:44
+    torch.cuda.synchronize()
+    st = stats.cpu().numpy()
+    ax, aw = O.abs_max_bf16(x), O.abs_max_bf16(w)
+    xq_o, dx = O.quantize_e4m3(x, ax, mt=True)
+    wq_o, dw = O.quantize_e4m3(w, aw, mt=True)
+    assert st[0] == np.float32(ax) and st[2] == np.float32(aw) and st[1] == dx and st[3] == dw
+    assert np.array_equal(host_bits(xq), xq_o) and np.array_equal(host_bits(wq), wq_o)
+    rng = np.random.default_rng(0)
+    idx_n = np.concatenate([rng.integers(0, BT, 60000), np.full(OC, 4095), np.arange(BT)]).astype(np.int32)
+    idx_m = np.concatenate([rng.integers(0, OC, 60000), np.arange(OC), np.full(BT, 4863)]).astype(np.int32)
+    ex, sabs = O.gemm_exact_sampled(wq_o, xq_o, idx_n, idx_m)
+    got = y.float().cpu().numpy()[idx_n, idx_m]
+    scale = np.float32(dw * dx)
+    max_abs, fro = gemm_check(got, ex, sabs, scale, True)
+    # closeness to the unquantised product, as a sanity check of the whole path (fp8 noise ~ 3-4 %)
+    ref = (O.bf16_to_f32(x)[idx_n[:2000]].astype(np.float64) * O.bf16_to_f32(w)[idx_m[:2000]].astype(np.float64)).sum(1)
+    rel = np.linalg.norm(got[:2000] - ref) / np.linalg.norm(ref)
+    assert rel < 0.08, rel
