@@ -187,7 +187,7 @@ def cpu_baseline(t, np, torch, budget_s):
     """The multithreaded CPU port (oracle/llmq_cpu_mt.c) on a bounded sample of the same workload:
     abs-max + quantize of X [8192x3584] and of a row-slice of W_up, then the gate+up forward GEMM for
     that slice of output features against all 8192 tokens."""
-    import ctypes as C
+    import ctypes
     from oracle import pyoracle as O
     L = O.lib()
     cores = min(L.mt_num_threads(), 16)      # the GPU box grants 16 host cores to a one-GPU job
@@ -197,7 +197,7 @@ def cpu_baseline(t, np, torch, budget_s):
     # calibrate the GEMM slice: 64 weight rows first, then scale to the budget
     w_all = t["w_up"]
     t0 = time.perf_counter()
-    ax = float(L.mt_abs_max_bf16(x.ctypes.data_as(C.POINTER(C.c_uint16)), x.size))
+    ax = float(L.mt_abs_max_bf16(x.ctypes.data_as(ctypes.POINTER(ctypes.c_uint16)), x.size))
     xq, _ = O.quantize_e4m3(x, ax, mt=True)
     t_q = time.perf_counter() - t0
     q_gbs = 5 * x.size / t_q / 1e9

@@ -7,6 +7,10 @@ fallback: if the library is not built the import of this module fails.
 import ctypes as C
 import os
 
+# torch bundles its own HIP runtime (same SONAME as /opt/rocm's, requested under a different file
+# name): whichever copy is loaded first must serve the whole process, so torch goes first.
+import torch  # noqa: F401
+
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libllmq_fp8.so")
 

@@ -28,9 +28,18 @@ def dev_scalar(v):
 
 
 # GEMM tolerance versus the exact (fp64) product of the same e4m3 operands times the fp32 factor sa*sb:
-#   bf16 output:  |err| <= 2^-8 * |ref| + 2^-20 * (sa*sb) * sum_k |a_k b_k|     and rel-Frobenius <= 2.5e-3
-#   fp32 output:  |err| <= 2^-18 * (sa*sb) * sum_k |a_k b_k|                    and rel-Frobenius <= 5e-5
-# (2^-8 is half a bf16 ulp of the result; the second term bounds fp32 accumulation in any order.)
+#   bf16 output:  |err| <= 2^-8 * |ref| + 2^-11 * (sa*sb) * sum_k |a_k b_k|     and rel-Frobenius <= 2.5e-3
+#   fp32 output:  |err| <= 2^-11 * (sa*sb) * sum_k |a_k b_k|                    and rel-Frobenius <= 2e-4
+# 2^-8 is half a bf16 ulp of the result.  The second term is the accumulation error of the gfx950 FP8
+# matrix instruction itself, measured with one-hot probes on the device: inside each group of 8
+# consecutive K positions the products are aligned to the group's largest product and truncated
+# (towards zero) 14 bits below its leading bit, so a group loses less than 7 * 2^-14 of its largest
+# term; summed over groups that is below 7 * 2^-14 * sum|a b| < 2^-11 * sum|a b|.  (Across groups and
+# into the fp32 accumulator the window is 27 bits, negligible next to it.)  Integer-valued operands
+# with |product| < 2^14 are unaffected, which is why the known-answer tests are bit exact.
+ACC_TERM = 2.0 ** -11
+
+
 def gemm_check(got_f32, exact, sumabs, scale, out_is_bf16, extra=None):
     """got_f32: decoded device result; exact/sumabs: oracle fp64 arrays of the same shape; extra: fp64
     array added after scaling (bias + old c).  Returns (max_abs_err, rel_frobenius); asserts the bounds."""
@@ -40,11 +49,11 @@ def gemm_check(got_f32, exact, sumabs, scale, out_is_bf16, extra=None):
     err = np.abs(got_f32.astype(np.float64) - ref)
     mag = np.abs(float(scale)) * sumabs + (np.abs(extra) if extra is not None else 0.0)
     if out_is_bf16:
-        bound = 2.0 ** -8 * np.abs(ref) + 2.0 ** -20 * mag + 1e-38
+        bound = 2.0 ** -8 * np.abs(ref) + ACC_TERM * mag + 1e-38
         fro_lim = 2.5e-3
     else:
-        bound = 2.0 ** -18 * mag + 1e-38
-        fro_lim = 5e-5
+        bound = ACC_TERM * mag + 1e-38
+        fro_lim = 2e-4
     worst = float((err / bound).max())
     assert worst <= 1.0, "GEMM element error exceeds the stated bound by x%.3f" % worst
     fro = float(np.sqrt((err ** 2).sum()) / max(np.sqrt((ref ** 2).sum()), 1e-300))
