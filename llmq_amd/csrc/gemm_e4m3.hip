@@ -21,6 +21,8 @@
 //   * the linear workgroup id is remapped so that each of the 8 XCDs (workgroups are dealt to XCDs
 //     round-robin) works on a contiguous range of tiles, walked in column-major groups of `group`
 //     tile-rows for L2 reuse of both operands.
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace llmq {
@@ -237,6 +239,230 @@ __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_kernel(GemmArgs 
     }
 }
 
+// ---- software-pipelined variant ---------------------------------------------------------------------
+// Same tiling, LDS layout and epilogue as above, with the K loop written as an explicit software
+// pipeline over half-steps (K = 64, one matrix instruction deep).  Within a half-step the matrix
+// instructions run row by row (a-fragment i against all b-fragments); as soon as row i has been
+// issued its a-fragment registers are refilled from LDS for the next half-step, and the b-fragments
+// of the next half-step go into a second small buffer.  LDS reads therefore stream under the matrix
+// instructions with (NI + 2 NJ) fragment registers instead of a full double buffer.  The single
+// workgroup barrier per K-step sits in the second half-step right after its first row has been
+// queued: at that point every wave has finished reading the stage the next direct-to-LDS copies
+// overwrite, and the stage fetched one step earlier has landed.
+template <int MASK, int N>
+__device__ __forceinline__ void sched_group() {
+    if constexpr (N > 0) __builtin_amdgcn_sched_group_barrier(MASK, N, 0);
+}
+
+template <int BLK_N, int BLK_M, int WV_N, int WV_M, typename OutT>
+__global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(GemmArgs g) {
+    constexpr int T = WV_N * WV_M * 64;
+    constexpr int WT_N = BLK_N / WV_N, WT_M = BLK_M / WV_M;
+    constexpr int NI = WT_N / 32, NJ = WT_M / 32;
+    constexpr int P_BYTES = BLK_N * kBK, Q_BYTES = BLK_M * kBK, STAGE = P_BYTES + Q_BYTES;
+    constexpr int P_ITERS = BLK_N * 8 / T, Q_ITERS = BLK_M * 8 / T, LOADS = P_ITERS + Q_ITERS;
+    static_assert(T / 8 % 32 == 0 && (NJ == 1 || NJ == 2 || NJ == 4) && NI >= 2, "tile configuration");
+
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * STAGE];
+
+    const int tid = threadIdx.x;
+    const int lane = tid % 64;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
+    const int wn = wave / WV_M, wm = wave % WV_M;
+    const int l32 = lane % 32, kg = lane / 32;
+
+    const int tiles_n = g.N / BLK_N, tiles_m = g.M / BLK_M;
+    int tile_n, tile_m;
+    {
+        const int nwg = gridDim.x, wg = blockIdx.x;
+        const int xcd = wg % 8, idx = wg / 8;
+        const int q = nwg / 8, r = nwg % 8;
+        const int logical = xcd * q + (xcd < r ? xcd : r) + idx;
+        const int per_group = g.group * tiles_m;
+        const int gid = logical / per_group;
+        const int first_n = gid * g.group;
+        const int gsz = (tiles_n - first_n) < g.group ? (tiles_n - first_n) : g.group;
+        const int in_group = logical % per_group;
+        tile_n = first_n + in_group % gsz;
+        tile_m = in_group / gsz;
+    }
+    const int n_blk = tile_n * BLK_N, m_blk = tile_m * BLK_M;
+
+    const int ld_row = tid / 8;
+    const int ld_chunk = (tid & 7) ^ ((ld_row >> 1) & 7);
+    const uint8_t* p_src = g.b + (int64_t)n_blk * g.K + (int64_t)ld_row * g.K + ld_chunk * 16;
+    const uint8_t* q_src[Q_ITERS];
+#pragma unroll
+    for (int it = 0; it < Q_ITERS; ++it) {
+        const int rho = it * (T / 8) + ld_row;
+        const int w = rho / WT_M, rw = rho % WT_M;
+        const int grow = w * WT_M + NJ * (rw % 32) + rw / 32;
+        q_src[it] = g.a + (int64_t)m_blk * g.K + (int64_t)grow * g.K + ld_chunk * 16;
+    }
+    auto issue_loads = [&](int stage, int k0) {
+        uint8_t* base = lds + stage * STAGE + wave * 1024;
+#pragma unroll
+        for (int it = 0; it < P_ITERS; ++it)
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(p_src + (int64_t)it * (T / 8) * g.K + k0),
+                (__attribute__((address_space(3))) void*)(base + it * T * 16), 16, 0, 0);
+#pragma unroll
+        for (int it = 0; it < Q_ITERS; ++it)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(q_src[it] + k0),
+                                             (__attribute__((address_space(3))) void*)(base + P_BYTES + it * T * 16), 16,
+                                             0, 0);
+    };
+
+    const int sw = (l32 >> 1) & 7;
+    const int p_frag = (wn * WT_N + l32) * kBK;
+    const int q_frag = P_BYTES + (wm * WT_M + l32) * kBK;
+    // byte offsets of the two 16-byte chunks a lane reads in half-step 0 / 1
+    const int cofs[2][2] = {{((2 * kg) ^ sw) * 16, ((2 * kg + 1) ^ sw) * 16},
+                            {((4 + 2 * kg) ^ sw) * 16, ((4 + 2 * kg + 1) ^ sw) * 16}};
+
+    auto read_frag = [&](const uint8_t* row, int h) -> v8i {
+        const v4i lo = *reinterpret_cast<const v4i*>(row + cofs[h][0]);
+        const v4i hi = *reinterpret_cast<const v4i*>(row + cofs[h][1]);
+        return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    };
+
+    v16f acc[NI][NJ];
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    const int KT = g.K / kBK;
+    issue_loads(0, 0);
+    if (KT > 1) {
+        issue_loads(1, kBK);
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LOADS) : "memory");
+    } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __syncthreads();
+
+    v8i fa[NI], fb[2][NJ];
+#pragma unroll
+    for (int i = 0; i < NI; ++i) fa[i] = read_frag(lds + p_frag + i * 32 * kBK, 0);
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) fb[0][j] = read_frag(lds + q_frag + j * 32 * kBK, 0);
+
+    // One half-step.  H: which half (selects the b-fragment buffer); NEXT: another half-step follows
+    // and its fragments are read from `next`; SYNC: barrier after the first row (the following
+    // half-step lives in the other LDS stage); REFILL: start the direct-to-LDS copies of the stage
+    // after that one into the stage just released.
+    auto half_step = [&](auto h_tag, auto next_tag, auto sync_tag, auto refill_tag, const uint8_t* next,
+                         int refill_stage, int refill_k0) {
+        constexpr int H = decltype(h_tag)::value;
+        constexpr bool NEXT = decltype(next_tag)::value;
+        constexpr bool SYNC = decltype(sync_tag)::value;
+        constexpr bool REFILL = decltype(refill_tag)::value;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[H][j], acc[i][j], 0, 0, 0, 0, 0, 0);
+            if (i == 0) {
+                if constexpr (SYNC) {
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    __syncthreads();
+                    if constexpr (REFILL) issue_loads(refill_stage, refill_k0);
+                }
+                if constexpr (NEXT) {
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j) fb[H ^ 1][j] = read_frag(next + q_frag + j * 32 * kBK, H ^ 1);
+                }
+            }
+            if constexpr (NEXT) fa[i] = read_frag(next + p_frag + i * 32 * kBK, H ^ 1);
+        }
+        // issue order inside the half-step: NJ matrix instructions, then the LDS reads (and a share of
+        // the global->LDS loads) written after them
+        if constexpr (NEXT && !SYNC) {
+            sched_group<0x008, NJ>();
+            sched_group<0x100, 2 * NJ + 2>();
+#pragma unroll
+            for (int i = 1; i < NI; ++i) {
+                sched_group<0x008, NJ>();
+                sched_group<0x100, 2>();
+            }
+        } else if constexpr (NEXT && SYNC) {
+            constexpr int LD = REFILL ? LOADS : 0;
+            constexpr int L0 = LD - (LD / NI) * (NI - 1);
+            sched_group<0x020, L0>();
+            sched_group<0x100, 2 * NJ + 2>();
+#pragma unroll
+            for (int i = 1; i < NI; ++i) {
+                sched_group<0x008, NJ>();
+                sched_group<0x100, 2>();
+                sched_group<0x020, LD / NI>();
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    using std::integral_constant;
+    constexpr integral_constant<int, 0> H0{};
+    constexpr integral_constant<int, 1> H1{};
+    constexpr integral_constant<bool, true> Y{};
+    constexpr integral_constant<bool, false> NO{};
+    int kt = 0;
+    for (; kt + 2 < KT; ++kt) {  // steady state: a next stage exists and one more can be fetched
+        half_step(H0, Y, NO, NO, lds + (kt & 1) * STAGE, 0, 0);
+        half_step(H1, Y, Y, Y, lds + ((kt + 1) & 1) * STAGE, kt & 1, (kt + 2) * kBK);
+    }
+    if (kt + 1 < KT) {           // second to last stage: nothing left to fetch
+        half_step(H0, Y, NO, NO, lds + (kt & 1) * STAGE, 0, 0);
+        half_step(H1, Y, Y, NO, lds + ((kt + 1) & 1) * STAGE, 0, 0);
+        ++kt;
+    }
+    half_step(H0, Y, NO, NO, lds + (kt & 1) * STAGE, 0, 0);   // last stage
+    half_step(H1, NO, NO, NO, lds, 0, 0);
+
+    float scale = g.sa ? *g.sa : 1.f;
+    if (g.sb) scale = scale * *g.sb;
+    OutT* c = reinterpret_cast<OutT*>(g.c);
+    const int m_lane = m_blk + wm * WT_M + NJ * l32;
+    float bias_v[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        bias_v[j] = 0.f;
+        if (g.bias) {
+            bias_v[j] = g.bias_is_bf16
+                            ? __uint_as_float((uint32_t) reinterpret_cast<const uint16_t*>(g.bias)[m_lane + j] << 16)
+                            : reinterpret_cast<const float*>(g.bias)[m_lane + j];
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int n = n_blk + wn * WT_N + i * 32 + 8 * (r / 4) + 4 * kg + (r % 4);
+            OutT* dst = c + (int64_t)n * g.M + m_lane;
+            Pack<NJ, OutT> old, out;
+            if (g.accumulate) old = *reinterpret_cast<const Pack<NJ, OutT>*>(dst);
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                float t = acc[i][j][r] * scale;
+                if (g.bias) t = t + bias_v[j];
+                if (g.accumulate) t = t + OutIo<OutT>::load(&old.v[j]);
+                out.v[j] = OutIo<OutT>::cvt(t);
+            }
+            *reinterpret_cast<Pack<NJ, OutT>*>(dst) = out;
+        }
+    }
+}
+
+template <int BLK_N, int BLK_M, int WV_N, int WV_M, typename OutT>
+static int launch_pipe(const GemmArgs& g, hipStream_t stream) {
+    const int tiles = (g.N / BLK_N) * (g.M / BLK_M);
+    hipLaunchKernelGGL((gemm_tn_e4m3_pipe_kernel<BLK_N, BLK_M, WV_N, WV_M, OutT>), dim3((unsigned)tiles),
+                       dim3(WV_N * WV_M * 64), 0, stream, g);
+    LLMQ_HIP_TRY(hipGetLastError());
+    return LLMQ_OK;
+}
+
 // ---- host side ------------------------------------------------------------------------------------
 template <int BLK_N, int BLK_M, int WV_N, int WV_M, bool DMA, typename OutT>
 static int launch_cfg(const GemmArgs& g, hipStream_t stream) {
@@ -264,7 +490,7 @@ static int gemm_dispatch(GemmArgs g, hipStream_t stream) {
     if (variant == 0) {
         const bool n256 = g.N % 256 == 0, m256 = g.M % 256 == 0;
         const int64_t tiles256 = (int64_t)(g.N / 256) * (g.M / 256);
-        if (n256 && m256 && tiles256 >= cu_count()) variant = 1;
+        if (n256 && m256 && tiles256 >= cu_count()) variant = 6;
         else variant = 3;
     }
     switch (variant) {
@@ -273,6 +499,9 @@ static int gemm_dispatch(GemmArgs g, hipStream_t stream) {
         case 3: return launch_cfg<128, 128, 2, 2, true, OutT>(g, stream);
         case 4: return launch_cfg<128, 128, 2, 2, false, OutT>(g, stream);
         case 5: return launch_cfg<256, 256, 2, 2, true, OutT>(g, stream);
+        case 6: return launch_pipe<256, 256, 2, 4, OutT>(g, stream);
+        case 7: return launch_pipe<256, 256, 2, 2, OutT>(g, stream);
+        case 8: return launch_pipe<128, 128, 2, 2, OutT>(g, stream);
         default: return set_error(LLMQ_ERR_INVALID_ARGUMENT, "matmul: unknown kernel variant %d", variant);
     }
 }
