@@ -1,0 +1,258 @@
+// llmq_kernels.hpp -- C++20 host shim over the C ABI (llmq_fp8.h) that keeps the names, argument
+// order and error behaviour of the reference's kernel entry points for the FP8 quantized-matmul path
+// (reference: src/kernels/kernels.h:22-23, 72-98, 246-270; Tensor overloads src/kernels/kernels.cpp:
+// 224-236, 258-310, 332-374).  A caller written against the reference's kernels.h compiles against this
+// header after the type substitutions
+//     nv_bfloat16 -> __hip_bfloat16        __nv_fp8_e4m3 -> __hip_fp8_e4m3     __nv_fp8_e5m2 -> __hip_fp8_e5m2
+//     cudaStream_t -> hipStream_t          cudaDeviceProp -> hipDeviceProp_t   cublasLtHandle_t -> llmqBlasHandle_t
+// The device-property, handle and workspace arguments are accepted and ignored (the gfx950 kernels
+// need neither a library handle nor a workspace).  Errors surface as the reference's exception types:
+// std::invalid_argument for shape / dtype / argument errors, std::runtime_error for runtime failures.
+#ifndef LLMQ_KERNELS_HPP
+#define LLMQ_KERNELS_HPP
+
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp8.h>
+#include <hip/hip_runtime_api.h>
+
+#include <array>
+#include <cstddef>
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "llmq_fp8.h"
+
+// ---- boundary types (reference: src/utilities/dtype.h:16-71, src/utilities/tensor.h:23-132) ----------
+enum class ETensorDType : int { FP32, BF16, FP16, INT32, INT8, FP8_E4M3, FP8_E5M2, BYTE };
+
+constexpr int get_dtype_size(ETensorDType t) {
+    switch (t) {
+        case ETensorDType::FP32: case ETensorDType::INT32: return 4;
+        case ETensorDType::BF16: case ETensorDType::FP16: return 2;
+        default: return 1;
+    }
+}
+
+inline const char* dtype_to_str(ETensorDType t) {
+    switch (t) {
+        case ETensorDType::FP32: return "FP32";
+        case ETensorDType::BF16: return "BF16";
+        case ETensorDType::FP16: return "FP16";
+        case ETensorDType::INT32: return "INT32";
+        case ETensorDType::INT8: return "INT8";
+        case ETensorDType::FP8_E4M3: return "FP8_E4M3";
+        case ETensorDType::FP8_E5M2: return "FP8_E5M2";
+        default: return "BYTE";
+    }
+}
+
+template <class T> constexpr ETensorDType dtype_from_type = ETensorDType::BYTE;
+template <> inline constexpr ETensorDType dtype_from_type<float> = ETensorDType::FP32;
+template <> inline constexpr ETensorDType dtype_from_type<__hip_bfloat16> = ETensorDType::BF16;
+template <> inline constexpr ETensorDType dtype_from_type<__hip_fp8_e4m3> = ETensorDType::FP8_E4M3;
+template <> inline constexpr ETensorDType dtype_from_type<__hip_fp8_e5m2> = ETensorDType::FP8_E5M2;
+template <> inline constexpr ETensorDType dtype_from_type<std::int8_t> = ETensorDType::INT8;
+template <> inline constexpr ETensorDType dtype_from_type<std::int32_t> = ETensorDType::INT32;
+
+constexpr int MAX_TENSOR_DIM = 5;
+
+// A contiguous typed view of device memory; Stats points at two consecutive device floats
+// [abs_max, scale] when the tensor takes part in quantization.
+struct Tensor {
+    ETensorDType DType = ETensorDType::BYTE;
+    std::array<long, MAX_TENSOR_DIM> Sizes{};
+    std::byte* Data = nullptr;
+    float* Stats = nullptr;
+    int Rank = 0;
+    int Device = -1;
+
+    [[nodiscard]] constexpr bool empty() const { return Data == nullptr; }
+    [[nodiscard]] constexpr std::size_t nelem() const {
+        std::size_t sz = 1;
+        for (int i = 0; i < Rank; ++i) sz *= (std::size_t)Sizes[i];
+        return sz;
+    }
+    [[nodiscard]] constexpr std::size_t bytes() const { return nelem() * (std::size_t)get_dtype_size(DType); }
+    constexpr explicit operator bool() const { return !empty(); }
+
+    template <class T> T* get() {
+        check<T>();
+        return reinterpret_cast<T*>(Data);
+    }
+    template <class T> const T* get() const {
+        check<T>();
+        return reinterpret_cast<const T*>(Data);
+    }
+    template <class T> const T* get_optional() const { return empty() ? nullptr : get<T>(); }
+
+    float* abs_max() { return Stats; }
+    float* scale() { return Stats ? Stats + 1 : nullptr; }
+    const float* abs_max() const { return Stats; }
+    const float* scale() const { return Stats ? Stats + 1 : nullptr; }
+
+    template <typename Container>
+    static Tensor from_pointer(std::byte* ptr, int device, ETensorDType dtype, const Container& shape) {
+        if (shape.size() > (std::size_t)MAX_TENSOR_DIM) throw std::runtime_error("Tensor rank too large");
+        Tensor t;
+        t.DType = dtype;
+        t.Sizes.fill(1);
+        std::size_t i = 0;
+        for (auto s : shape) t.Sizes[i++] = (long)s;
+        t.Data = ptr;
+        t.Rank = (int)shape.size();
+        t.Device = device;
+        return t;
+    }
+
+  private:
+    template <class T> void check() const {
+        if constexpr (!std::is_same_v<T, std::byte>) {
+            if (dtype_from_type<T> != DType)
+                throw std::logic_error(std::string("DType mismatch: requested ") + dtype_to_str(dtype_from_type<T>) +
+                                       ", tensor is " + dtype_to_str(DType));
+        }
+    }
+};
+
+struct QuantizableTensor {  // reference: src/models/llama_run_state.h:19-24
+    Tensor Value;
+    Tensor Quant = Tensor{};
+};
+
+enum class EMMTranspose { TT, TN, NT, NN };
+enum class EMatmulBackend { CuBLAS, Custom };
+typedef struct llmqBlasContext* llmqBlasHandle_t;  // stands in for cublasLtHandle_t; always ignored
+
+namespace llmq_detail {
+inline void check(int code) {
+    if (code == LLMQ_OK) return;
+    if (code == LLMQ_ERR_INVALID_ARGUMENT) throw std::invalid_argument(llmq_last_error());
+    throw std::runtime_error(llmq_last_error());
+}
+inline void require_tn(EMMTranspose mode) {
+    if (mode != EMMTranspose::TN)
+        throw std::invalid_argument("matmul: FP8 operands are only supported in TN layout (both K-contiguous)");
+}
+template <class... T> [[noreturn]] void unsupported(const char* func, const T&... t) {
+    std::string msg = std::string(func) + ": unsupported dtypes. Got [";
+    ((msg += (t.empty() ? std::string("<null>") : std::string(dtype_to_str(t.DType))) + ", "), ...);
+    throw std::invalid_argument(msg + "]");
+}
+inline const uint16_t* u16(const __hip_bfloat16* p) { return reinterpret_cast<const uint16_t*>(p); }
+inline uint16_t* u16(__hip_bfloat16* p) { return reinterpret_cast<uint16_t*>(p); }
+template <class F8> const uint8_t* u8(const F8* p) { return reinterpret_cast<const uint8_t*>(p); }
+template <class F8> uint8_t* u8(F8* p) { return reinterpret_cast<uint8_t*>(p); }
+}  // namespace llmq_detail
+
+// ---- quantization (reference: src/kernels/kernels.h:246-264) -----------------------------------------
+inline void abs_max(float* scale, const float* in, long N, const hipDeviceProp_t&, hipStream_t stream) {
+    llmq_detail::check(llmq_abs_max_f32(scale, in, N, stream));
+}
+inline void abs_max(float* scale, const __hip_bfloat16* in, long N, const hipDeviceProp_t&, hipStream_t stream) {
+    llmq_detail::check(llmq_abs_max_bf16(scale, llmq_detail::u16(in), N, stream));
+}
+inline void abs_max(float* scale, const Tensor& in, long N, const hipDeviceProp_t& dp, hipStream_t stream) {
+    if (in.DType == ETensorDType::FP32) abs_max(scale, in.get<float>(), N, dp, stream);
+    else if (in.DType == ETensorDType::BF16) abs_max(scale, in.get<__hip_bfloat16>(), N, dp, stream);
+    else llmq_detail::unsupported(__func__, in);
+}
+
+inline void quantize_with_abs_max(__hip_fp8_e4m3* out, float* scale_ptr, const __hip_bfloat16* in, const float* abs_max,
+                                  long N, const hipDeviceProp_t&, hipStream_t stream) {
+    llmq_detail::check(llmq_quantize_e4m3_bf16(llmq_detail::u8(out), scale_ptr, llmq_detail::u16(in), abs_max, N, stream));
+}
+inline void quantize_with_abs_max(__hip_fp8_e5m2* out, float* scale_ptr, const __hip_bfloat16* in, const float* abs_max,
+                                  long N, const hipDeviceProp_t&, hipStream_t stream) {
+    llmq_detail::check(llmq_quantize_e5m2_bf16(llmq_detail::u8(out), scale_ptr, llmq_detail::u16(in), abs_max, N, stream));
+}
+inline void quantize_with_abs_max(Tensor& out, float* scale_ptr, const Tensor& in, const float* abs_max, long N,
+                                  const hipDeviceProp_t& dp, hipStream_t stream) {
+    if (in.DType == ETensorDType::BF16 && out.DType == ETensorDType::FP8_E4M3)
+        quantize_with_abs_max(out.get<__hip_fp8_e4m3>(), scale_ptr, in.get<__hip_bfloat16>(), abs_max, N, dp, stream);
+    else if (in.DType == ETensorDType::BF16 && out.DType == ETensorDType::FP8_E5M2)
+        quantize_with_abs_max(out.get<__hip_fp8_e5m2>(), scale_ptr, in.get<__hip_bfloat16>(), abs_max, N, dp, stream);
+    else llmq_detail::unsupported(__func__, out, in);
+}
+
+inline void quantize_and_transpose_with_abs_max(__hip_fp8_e4m3* out, float* scale_ptr, const __hip_bfloat16* in,
+                                                const float* abs_max, int rows, int cols, const hipDeviceProp_t&,
+                                                hipStream_t stream) {
+    llmq_detail::check(llmq_quantize_transpose_e4m3_bf16(llmq_detail::u8(out), scale_ptr, llmq_detail::u16(in), abs_max,
+                                                         rows, cols, stream));
+}
+inline void quantize_and_transpose_with_abs_max(Tensor& out, float* scale_ptr, const Tensor& in, const float* abs_max,
+                                                int rows, int cols, const hipDeviceProp_t& dp, hipStream_t stream) {
+    if (out.DType == ETensorDType::FP8_E4M3 && in.DType == ETensorDType::BF16)
+        quantize_and_transpose_with_abs_max(out.get<__hip_fp8_e4m3>(), scale_ptr, in.get<__hip_bfloat16>(), abs_max, rows,
+                                            cols, dp, stream);
+    else llmq_detail::unsupported(__func__, out, in);
+}
+
+// ---- transpose (reference: src/kernels/kernels.h:266-270) --------------------------------------------
+inline void transpose(__hip_fp8_e4m3* dst, const __hip_fp8_e4m3* src, int rows, int cols, hipStream_t stream) {
+    llmq_detail::check(llmq_transpose_u8(llmq_detail::u8(dst), llmq_detail::u8(src), rows, cols, stream));
+}
+inline void transpose(__hip_fp8_e5m2* dst, const __hip_fp8_e5m2* src, int rows, int cols, hipStream_t stream) {
+    llmq_detail::check(llmq_transpose_u8(llmq_detail::u8(dst), llmq_detail::u8(src), rows, cols, stream));
+}
+inline void transpose(Tensor& dst, const Tensor& src, int rows, int cols, hipStream_t stream) {
+    if (dst.DType != src.DType) llmq_detail::unsupported(__func__, dst, src);
+    if (src.DType == ETensorDType::FP8_E4M3)
+        transpose(dst.get<__hip_fp8_e4m3>(), src.get<__hip_fp8_e4m3>(), rows, cols, stream);
+    else if (src.DType == ETensorDType::FP8_E5M2)
+        transpose(dst.get<__hip_fp8_e5m2>(), src.get<__hip_fp8_e5m2>(), rows, cols, stream);
+    else llmq_detail::unsupported(__func__, dst, src);
+}
+
+// ---- matmul (reference: src/kernels/kernels.h:72-78, 88-90, 96-98) --------------------------------------
+// Row-major a[M,K], b[N,K] -> row-major c[N,M] = (b . a^T) * (*scale_a * *scale_b) (+ bias[M]) (+ c).
+inline void matmul(__hip_bfloat16* c, const __hip_fp8_e4m3* a, const __hip_fp8_e4m3* b, const __hip_bfloat16* bias,
+                   const float* scale_a, const float* scale_b, llmqBlasHandle_t, std::byte*, std::size_t, int M, int N,
+                   int K, EMMTranspose mode, bool accumulate, hipStream_t stream,
+                   EMatmulBackend = EMatmulBackend::Custom) {
+    llmq_detail::require_tn(mode);
+    llmq_detail::check(llmq_gemm_tn_e4m3_bf16(llmq_detail::u16(c), llmq_detail::u8(a), llmq_detail::u8(b),
+                                              llmq_detail::u16(bias), scale_a, scale_b, M, N, K, accumulate, stream));
+}
+inline void matmul(float* c, const __hip_fp8_e4m3* a, const __hip_fp8_e4m3* b, const float* bias, const float* scale_a,
+                   const float* scale_b, llmqBlasHandle_t, std::byte*, std::size_t, int M, int N, int K,
+                   EMMTranspose mode, bool accumulate, hipStream_t stream, EMatmulBackend = EMatmulBackend::Custom) {
+    llmq_detail::require_tn(mode);
+    llmq_detail::check(llmq_gemm_tn_e4m3_f32(c, llmq_detail::u8(a), llmq_detail::u8(b), bias, 0, scale_a, scale_b, M, N, K,
+                                             accumulate, stream));
+}
+inline void matmul(float* c, const __hip_fp8_e4m3* a, const __hip_fp8_e4m3* b, const __hip_bfloat16* bias,
+                   const float* scale_a, const float* scale_b, llmqBlasHandle_t, std::byte*, std::size_t, int M, int N,
+                   int K, EMMTranspose mode, bool accumulate, hipStream_t stream,
+                   EMatmulBackend = EMatmulBackend::Custom) {
+    llmq_detail::require_tn(mode);
+    llmq_detail::check(llmq_gemm_tn_e4m3_f32(c, llmq_detail::u8(a), llmq_detail::u8(b), bias, 1, scale_a, scale_b, M, N, K,
+                                             accumulate, stream));
+}
+inline void matmul(Tensor& c, const Tensor& a, const Tensor& b, const Tensor& bias, const float* scale_a,
+                   const float* scale_b, llmqBlasHandle_t handle, Tensor& workspace, int M, int N, int K,
+                   EMMTranspose mode, bool accumulate, hipStream_t stream,
+                   EMatmulBackend backend = EMatmulBackend::Custom) {
+    std::byte* ws = workspace.Data;
+    const std::size_t ws_size = workspace.empty() ? 0 : workspace.bytes();
+    if (a.DType != ETensorDType::FP8_E4M3 || b.DType != ETensorDType::FP8_E4M3)
+        llmq_detail::unsupported(__func__, c, a, b, bias, workspace);
+    if (c.DType == ETensorDType::FP32) {
+        if (!bias.empty() && bias.DType == ETensorDType::BF16)
+            matmul(c.get<float>(), a.get<__hip_fp8_e4m3>(), b.get<__hip_fp8_e4m3>(), bias.get<__hip_bfloat16>(), scale_a,
+                   scale_b, handle, ws, ws_size, M, N, K, mode, accumulate, stream, backend);
+        else
+            matmul(c.get<float>(), a.get<__hip_fp8_e4m3>(), b.get<__hip_fp8_e4m3>(), bias.get_optional<float>(), scale_a,
+                   scale_b, handle, ws, ws_size, M, N, K, mode, accumulate, stream, backend);
+    } else if (c.DType == ETensorDType::BF16) {
+        matmul(c.get<__hip_bfloat16>(), a.get<__hip_fp8_e4m3>(), b.get<__hip_fp8_e4m3>(),
+               bias.get_optional<__hip_bfloat16>(), scale_a, scale_b, handle, ws, ws_size, M, N, K, mode, accumulate, stream,
+               backend);
+    } else {
+        llmq_detail::unsupported(__func__, c, a, b, bias, workspace);
+    }
+}
+
+#endif  // LLMQ_KERNELS_HPP

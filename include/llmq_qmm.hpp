@@ -1,0 +1,96 @@
+// llmq_qmm.hpp -- host glue that issues the kernel call sequence of one FP8 linear layer, forward and
+// backward, the way the reference's forward_qmm / backward_qmm do (src/models/llama_model.cpp:25-47,
+// 280-340, FP8 branches).  The reference passes its whole LLamaRunState into backward_qmm; here the
+// part of it the path needs (a LIFO device stack for temporaries, the device properties and the
+// gradient dtype, src/training/model.cpp:129-143, src/utilities/stack.cpp:13-25) is QmmRunState.
+#ifndef LLMQ_QMM_HPP
+#define LLMQ_QMM_HPP
+
+#include "llmq_kernels.hpp"
+
+// LIFO bump allocator over one device arena: temp_alloc / temp_free are host pointer arithmetic only,
+// so the sequence stays legal under stream capture.  Blocks are rounded up to 4096 bytes.
+struct QmmRunState {
+    std::byte* Arena = nullptr;
+    std::size_t Capacity = 0;
+    std::size_t Top = 0;
+    std::size_t HighWater = 0;
+    int Device = 0;
+    hipDeviceProp_t DeviceProp{};
+    ETensorDType GradDType = ETensorDType::FP8_E4M3;
+    llmqBlasHandle_t BlasHandle = nullptr;
+    Tensor Workspace{};
+    EMatmulBackend MatmulBackend = EMatmulBackend::Custom;
+    std::vector<std::byte*> Live;
+
+    Tensor temp_alloc(ETensorDType dtype, const std::vector<long>& shape) {
+        Tensor t = Tensor::from_pointer(nullptr, Device, dtype, shape);
+        const std::size_t need = (t.bytes() + 4095) / 4096 * 4096;
+        if (Top + need > Capacity) throw std::runtime_error("QmmRunState: temporary stack exhausted");
+        t.Data = Arena + Top;
+        Top += need;
+        if (Top > HighWater) HighWater = Top;
+        Live.push_back(t.Data);
+        return t;
+    }
+    void temp_free(Tensor& t) {
+        if (Live.empty() || Live.back() != t.Data) throw std::logic_error("QmmRunState: temp_free out of LIFO order");
+        Live.pop_back();
+        Top = (std::size_t)(t.Data - Arena);
+        t.Data = nullptr;
+    }
+    // Bytes of stack backward_qmm needs for one layer (the dry run of llama_run_state.cpp:362-390).
+    static std::size_t backward_temp_bytes(int B, int T, int C, int OC) {
+        auto up = [](std::size_t b) { return (b + 4095) / 4096 * 4096; };
+        const std::size_t wt = up((std::size_t)C * OC), at = up((std::size_t)C * B * T), gt = up((std::size_t)OC * B * T);
+        return wt > at + gt ? wt : at + gt;
+    }
+};
+
+// out[B*T, OC] = inp[B*T, C] . weight[OC, C]^T (+ bias).  weight is already e4m3 with valid Stats.
+inline void forward_qmm(Tensor& out, QuantizableTensor& inp, Tensor& weight, const Tensor& bias,
+                        llmqBlasHandle_t handle, Tensor& workspace, int B, int T, int C, int OC,
+                        const hipDeviceProp_t& dp, bool reuse_inp_quant, hipStream_t stream, EMatmulBackend backend) {
+    if (weight.DType != ETensorDType::FP8_E4M3)
+        throw std::invalid_argument("forward_qmm: this build implements the FP8 (e4m3 weight) branch only");
+    if (!reuse_inp_quant) {
+        quantize_with_abs_max(inp.Quant, inp.Quant.scale(), inp.Value, inp.Quant.abs_max(), (long)B * T * C, dp, stream);
+    }
+    matmul(out, weight, inp.Quant, bias, weight.scale(), inp.Quant.scale(), handle, workspace, OC, B * T, C,
+           EMMTranspose::TN, false, stream, backend);
+}
+
+// dinp[B*T, C] = dout . weight ;  dweight[OC, C] (+)= dout^T . inp.
+inline void backward_qmm(Tensor& dinp, Tensor& dweight, QuantizableTensor& dout, QuantizableTensor& inp,
+                         Tensor& weight, bool accumulate_gradient, QmmRunState& rs, int B, int T, int C, int OC,
+                         bool reuse_inp, hipStream_t stream) {
+    if (weight.DType != ETensorDType::FP8_E4M3)
+        throw std::invalid_argument("backward_qmm: this build implements the FP8 (e4m3 weight) branch only");
+    quantize_with_abs_max(dout.Quant, dout.Quant.scale(), dout.Value, dout.Quant.abs_max(), (long)B * T * OC,
+                          rs.DeviceProp, stream);
+
+    auto& inp_q = inp.Quant;
+    Tensor weight_tp = rs.temp_alloc(inp_q.DType, {C, OC});
+    transpose(weight_tp, weight, OC, C, stream);
+    Tensor no_bias{};
+    matmul(dinp, weight_tp, dout.Quant, no_bias, weight.scale(), dout.Quant.scale(), rs.BlasHandle, rs.Workspace, C,
+           B * T, OC, EMMTranspose::TN, false, stream, rs.MatmulBackend);
+    rs.temp_free(weight_tp);
+
+    Tensor activation_tp = rs.temp_alloc(inp_q.DType, {C, (long)B * T});
+    Tensor grad_tp = rs.temp_alloc(rs.GradDType, {OC, (long)B * T});
+    if (reuse_inp) {
+        transpose(activation_tp, inp_q, B * T, C, stream);
+    } else {
+        // a stack temporary carries no Stats, so no scale is written here (llama_model.cpp:328)
+        quantize_and_transpose_with_abs_max(activation_tp, activation_tp.scale(), inp.Value, inp.Quant.abs_max(),
+                                            B * T, C, rs.DeviceProp, stream);
+    }
+    transpose(grad_tp, dout.Quant, B * T, OC, stream);
+    matmul(dweight, activation_tp, grad_tp, no_bias, inp_q.scale(), dout.Quant.scale(), rs.BlasHandle, rs.Workspace, C,
+           OC, B * T, EMMTranspose::TN, accumulate_gradient, stream, rs.MatmulBackend);
+    rs.temp_free(grad_tp);
+    rs.temp_free(activation_tp);
+}
+
+#endif  // LLMQ_QMM_HPP

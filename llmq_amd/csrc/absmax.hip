@@ -54,12 +54,16 @@ __device__ __forceinline__ void block_min_to_atomic_max(unsigned* result, uint32
             y = o < y ? o : y;
         }
         if (lane == 0) {
+            // Non-negative floats order like their bit patterns.  The slot only ever grows, so a block
+            // whose maximum does not exceed the value already there skips the (serialising) atomic.
             uint32_t bits = (limit - y) << shift;
-            if (bits != 0) atomicMax(result, bits);  // non-negative floats order like their bit patterns
+            if (bits > __atomic_load_n(result, __ATOMIC_RELAXED)) atomicMax(result, bits);
         }
     }
 }
 
+// Every lane keeps UNROLL independent 128-bit loads in flight; out-of-range slots of the last trip are
+// predicated to zero instead of falling into a serial tail loop.
 template <int UNROLL>
 __global__ __launch_bounds__(256) void absmax_bf16_kernel(unsigned* __restrict__ result,
                                                           const uint4* __restrict__ in, int64_t nvec,
@@ -67,15 +71,16 @@ __global__ __launch_bounds__(256) void absmax_bf16_kernel(unsigned* __restrict__
     const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     uint32_t acc = 0x7F807F80u;
-    int64_t i = tid;
-    for (; i + (UNROLL - 1) * stride < nvec; i += UNROLL * stride) {
+    for (int64_t i = tid; i < nvec; i += UNROLL * stride) {
         uint4 v[UNROLL];
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) v[u] = in[i + u * stride];
+        for (int u = 0; u < UNROLL; ++u) {
+            const int64_t idx = i + u * stride;
+            v[u] = idx < nvec ? in[idx] : make_uint4(0, 0, 0, 0);
+        }
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) acc = fold_vec(acc, v[u]);
     }
-    for (; i < nvec; i += stride) acc = fold_vec(acc, in[i]);
     if (tid < ntail) acc = fold_bf16x2(acc, (uint32_t)tail[tid]);
     uint32_t lo = acc & 0xFFFFu, hi = acc >> 16;
     block_min_to_atomic_max(result, lo < hi ? lo : hi, 0x7F80u, 16);
@@ -92,15 +97,16 @@ __global__ __launch_bounds__(256) void absmax_f32_kernel(unsigned* __restrict__ 
         uint32_t y = 0x7F800000u - (w & 0x7FFFFFFFu);  // wraps to a huge value for NaN
         acc = y < acc ? y : acc;
     };
-    int64_t i = tid;
-    for (; i + (UNROLL - 1) * stride < nvec; i += UNROLL * stride) {
+    for (int64_t i = tid; i < nvec; i += UNROLL * stride) {
         uint4 v[UNROLL];
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) v[u] = in[i + u * stride];
+        for (int u = 0; u < UNROLL; ++u) {
+            const int64_t idx = i + u * stride;
+            v[u] = idx < nvec ? in[idx] : make_uint4(0, 0, 0, 0);
+        }
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) { fold(v[u].x); fold(v[u].y); fold(v[u].z); fold(v[u].w); }
     }
-    for (; i < nvec; i += stride) { uint4 v = in[i]; fold(v.x); fold(v.y); fold(v.z); fold(v.w); }
     if (tid < ntail) fold(tail[tid]);
     block_min_to_atomic_max(result, acc, 0x7F800000u, 0);
 }
@@ -121,9 +127,10 @@ static int launch_absmax(Kernel kernel, float* out, const Elem* in, int64_t n, i
     const int64_t nvec = n / elems_per_vec;
     const int ntail = (int)(n - nvec * elems_per_vec);
     const int64_t per_block = 256LL * unroll;
+    // One trip per lane (`unroll` independent 16-byte loads each): on this chip a plain grid with many
+    // short workgroups sustains more HBM bandwidth than a persistent grid-stride loop.
     int64_t blocks = (nvec + per_block - 1) / per_block;
-    const int64_t max_blocks = (int64_t)cu_count() * 8;
-    if (blocks > max_blocks) blocks = max_blocks;
+    if (blocks > 0x7FFFFFFF) blocks = 0x7FFFFFFF;
     if (blocks < 1) blocks = 1;
     hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), 0, stream, reinterpret_cast<unsigned*>(out),
                        reinterpret_cast<const uint4*>(in), nvec, in + nvec * elems_per_vec, ntail);
@@ -134,10 +141,10 @@ static int launch_absmax(Kernel kernel, float* out, const Elem* in, int64_t n, i
 }  // namespace llmq
 
 extern "C" int llmq_abs_max_bf16(float* out, const uint16_t* in, int64_t n, void* stream) {
-    return llmq::launch_absmax(llmq::absmax_bf16_kernel<4>, out, in, n, 8, 4, static_cast<hipStream_t>(stream));
+    return llmq::launch_absmax(llmq::absmax_bf16_kernel<8>, out, in, n, 8, 8, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int llmq_abs_max_f32(float* out, const float* in, int64_t n, void* stream) {
-    return llmq::launch_absmax(llmq::absmax_f32_kernel<4>, out, reinterpret_cast<const uint32_t*>(in), n, 4, 4,
+    return llmq::launch_absmax(llmq::absmax_f32_kernel<8>, out, reinterpret_cast<const uint32_t*>(in), n, 4, 8,
                                static_cast<hipStream_t>(stream));
 }

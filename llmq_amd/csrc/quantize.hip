@@ -71,15 +71,19 @@ __global__ __launch_bounds__(256) void quantize_kernel(uint2* __restrict__ out, 
     const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     if (tid == 0 && scale_ptr) *scale_ptr = __fdiv_rn(1.f, s);
-    int64_t i = tid;
-    for (; i + (UNROLL - 1) * stride < nvec; i += UNROLL * stride) {
+    for (int64_t i = tid; i < nvec; i += UNROLL * stride) {
         uint4 v[UNROLL];
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) v[u] = in[i + u * stride];
+        for (int u = 0; u < UNROLL; ++u) {
+            const int64_t idx = i + u * stride;
+            v[u] = idx < nvec ? in[idx] : make_uint4(0, 0, 0, 0);
+        }
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) out[i + u * stride] = encode8<FMT>(v[u], s);
+        for (int u = 0; u < UNROLL; ++u) {
+            const int64_t idx = i + u * stride;
+            if (idx < nvec) out[idx] = encode8<FMT>(v[u], s);
+        }
     }
-    for (; i < nvec; i += stride) out[i] = encode8<FMT>(in[i], s);
     if (tid < ntail) {
         float y = s * __uint_as_float((uint32_t)tail_in[tid] << 16);
         tail_out[tid] = (uint8_t)(encode4<FMT>(y, 0.f, 0.f, 0.f) & 0xFFu);
@@ -91,7 +95,7 @@ constexpr int kQtRows = 256;       // tile extent along the input rows (= contig
 constexpr int kQtStride = 65;      // LDS row stride in dwords (64 dwords of payload + 1 pad)
 
 // NCH = number of 8-column chunks per tile: the tile is [kQtRows rows] x [8*NCH cols].
-template <int NCH>
+template <int NCH, bool ROW_MAJOR_GRID>
 __global__ __launch_bounds__(256) void quantize_transpose_kernel(uint8_t* __restrict__ out,
                                                                  float* __restrict__ scale_ptr,
                                                                  const uint16_t* __restrict__ in,
@@ -106,8 +110,8 @@ __global__ __launch_bounds__(256) void quantize_transpose_kernel(uint8_t* __rest
     const int t = threadIdx.x;
     if (t == 0 && blockIdx.x == 0 && blockIdx.y == 0 && scale_ptr) *scale_ptr = __fdiv_rn(1.f, s);
 
-    const int r0 = blockIdx.y * kQtRows;
-    const int c0 = blockIdx.x * TC;
+    const int r0 = (ROW_MAJOR_GRID ? blockIdx.x : blockIdx.y) * kQtRows;
+    const int c0 = (ROW_MAJOR_GRID ? blockIdx.y : blockIdx.x) * TC;
     const int chunk = t % NCH;
     const int q = t / NCH;
     const int col = c0 + 8 * chunk;
@@ -164,6 +168,8 @@ __global__ __launch_bounds__(256) void quantize_transpose_kernel(uint8_t* __rest
     }
 }
 
+int g_qt_row_major_grid = 1;
+
 template <int FMT>
 static int launch_quantize(uint8_t* out, float* scale_ptr, const uint16_t* in, const float* absmax, int64_t n,
                            hipStream_t stream) {
@@ -171,12 +177,13 @@ static int launch_quantize(uint8_t* out, float* scale_ptr, const uint16_t* in, c
     LLMQ_REQUIRE(absmax != nullptr, "quantize_with_abs_max: abs_max pointer is null");
     LLMQ_REQUIRE(n == 0 || (out != nullptr && in != nullptr), "quantize_with_abs_max: null tensor pointer");
     LLMQ_REQUIRE(aligned16(in) && aligned16(out), "quantize_with_abs_max: tensors must be 16-byte aligned");
-    constexpr int UNROLL = 4;
+    constexpr int UNROLL = 8;
     const int64_t nvec = n / 8;
     const int ntail = (int)(n - nvec * 8);
+    // One trip per lane (UNROLL independent 16-byte loads, then UNROLL 8-byte stores): many short
+    // workgroups sustain more HBM bandwidth here than a persistent grid-stride loop.
     int64_t blocks = (nvec + 256 * UNROLL - 1) / (256 * UNROLL);
-    const int64_t max_blocks = (int64_t)cu_count() * 8;
-    if (blocks > max_blocks) blocks = max_blocks;
+    if (blocks > 0x7FFFFFFF) blocks = 0x7FFFFFFF;
     if (blocks < 1) blocks = 1;  // still writes the scale for n == 0
     hipLaunchKernelGGL((quantize_kernel<FMT, UNROLL>), dim3((unsigned)blocks), dim3(256), 0, stream,
                        reinterpret_cast<uint2*>(out), scale_ptr, reinterpret_cast<const uint4*>(in), absmax, nvec,
@@ -197,6 +204,8 @@ extern "C" int llmq_quantize_e5m2_bf16(uint8_t* out, float* scale_or_null, const
     return llmq::launch_quantize<llmq::kE5M2>(out, scale_or_null, in, absmax, n, static_cast<hipStream_t>(stream));
 }
 
+extern "C" void llmq_debug_set_qt_order(int v) { llmq::g_qt_row_major_grid = v; }
+
 extern "C" int llmq_quantize_transpose_e4m3_bf16(uint8_t* out, float* scale_or_null, const uint16_t* in,
                                                  const float* absmax, int rows, int cols, void* stream) {
     using namespace llmq;
@@ -212,13 +221,23 @@ extern "C" int llmq_quantize_transpose_e4m3_bf16(uint8_t* out, float* scale_or_n
     const unsigned gy = empty ? 1u : (unsigned)((rows + kQtRows - 1) / kQtRows);
     // Wide tiles (256-byte row segments on the read side) once there are enough of them to fill the chip.
     const int64_t wide_tiles = (int64_t)((cols + 127) / 128) * gy;
+    const bool rm = g_qt_row_major_grid != 0;
     if (!empty && cols >= 128 && wide_tiles >= 2LL * cu_count()) {
-        hipLaunchKernelGGL(quantize_transpose_kernel<16>, dim3((unsigned)((cols + 127) / 128), gy), dim3(256), 0, st,
-                           out, scale_or_null, in, absmax, rows, cols, rows_mult16);
+        const unsigned gx = (unsigned)((cols + 127) / 128);
+        if (rm && gx <= 65535u)
+            hipLaunchKernelGGL((quantize_transpose_kernel<16, true>), dim3(gy, gx), dim3(256), 0, st, out, scale_or_null,
+                               in, absmax, rows, cols, rows_mult16);
+        else
+            hipLaunchKernelGGL((quantize_transpose_kernel<16, false>), dim3(gx, gy), dim3(256), 0, st, out, scale_or_null,
+                               in, absmax, rows, cols, rows_mult16);
     } else {
         const unsigned gx = empty ? 1u : (unsigned)((cols + 63) / 64);
-        hipLaunchKernelGGL(quantize_transpose_kernel<8>, dim3(gx, gy), dim3(256), 0, st, out, scale_or_null, in,
-                           absmax, empty ? 0 : rows, empty ? 0 : cols, rows_mult16);
+        if (rm && gx <= 65535u)
+            hipLaunchKernelGGL((quantize_transpose_kernel<8, true>), dim3(gy, gx), dim3(256), 0, st, out, scale_or_null, in,
+                               absmax, empty ? 0 : rows, empty ? 0 : cols, rows_mult16);
+        else
+            hipLaunchKernelGGL((quantize_transpose_kernel<8, false>), dim3(gx, gy), dim3(256), 0, st, out, scale_or_null, in,
+                               absmax, empty ? 0 : rows, empty ? 0 : cols, rows_mult16);
     }
     LLMQ_HIP_TRY(hipGetLastError());
     return LLMQ_OK;

@@ -30,12 +30,15 @@ __device__ __forceinline__ void transpose4x4(uint32_t a, uint32_t b, uint32_t c,
     out[3] = __builtin_amdgcn_perm(u1, t1, 0x07060302u);
 }
 
+// ROW_MAJOR_GRID: consecutive workgroups walk along the input rows (so concurrently running groups
+// write neighbouring 256-byte segments of the same output rows) instead of along the input columns.
+template <bool ROW_MAJOR_GRID>
 __global__ __launch_bounds__(256) void transpose_u8_kernel(uint8_t* __restrict__ dst,
                                                            const uint8_t* __restrict__ src, int rows, int cols) {
     __shared__ uint32_t tile[kTrCols * kTrStride];
     const int t = threadIdx.x;
-    const int r0 = blockIdx.y * kTrRows;
-    const int c0 = blockIdx.x * kTrCols;
+    const int r0 = (ROW_MAJOR_GRID ? blockIdx.x : blockIdx.y) * kTrRows;
+    const int c0 = (ROW_MAJOR_GRID ? blockIdx.y : blockIdx.x) * kTrCols;
     const int chunk = t % 8;  // 16-column chunk
     const int q = t / 8;      // row quad within a pass (32 per pass, 2 passes)
     const int col = c0 + 16 * chunk;
@@ -100,7 +103,11 @@ __global__ __launch_bounds__(256) void transpose_u8_generic_kernel(uint8_t* __re
     }
 }
 
+int g_transpose_row_major_grid = 1;
+
 }  // namespace llmq
+
+extern "C" void llmq_debug_set_transpose_order(int v) { llmq::g_transpose_row_major_grid = v; }
 
 extern "C" int llmq_transpose_u8(uint8_t* dst, const uint8_t* src, int rows, int cols, void* stream) {
     using namespace llmq;
@@ -110,8 +117,12 @@ extern "C" int llmq_transpose_u8(uint8_t* dst, const uint8_t* src, int rows, int
     LLMQ_REQUIRE(dst != src, "transpose: in-place transpose is not supported");
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (rows % 16 == 0 && cols % 16 == 0 && aligned16(src) && aligned16(dst)) {
-        dim3 grid((unsigned)((cols + kTrCols - 1) / kTrCols), (unsigned)((rows + kTrRows - 1) / kTrRows));
-        hipLaunchKernelGGL(transpose_u8_kernel, grid, dim3(256), 0, st, dst, src, rows, cols);
+        const unsigned gc = (unsigned)((cols + kTrCols - 1) / kTrCols), gr = (unsigned)((rows + kTrRows - 1) / kTrRows);
+        if (g_transpose_row_major_grid && gc <= 65535u) {
+            hipLaunchKernelGGL(transpose_u8_kernel<true>, dim3(gr, gc), dim3(256), 0, st, dst, src, rows, cols);
+        } else {
+            hipLaunchKernelGGL(transpose_u8_kernel<false>, dim3(gc, gr), dim3(256), 0, st, dst, src, rows, cols);
+        }
     } else {
         dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64));
         hipLaunchKernelGGL(transpose_u8_generic_kernel, grid, dim3(256), 0, st, dst, src, rows, cols);

@@ -1,0 +1,148 @@
+// C++ harness: replays forward_qmm / backward_qmm (include/llmq_qmm.hpp) for one linear layer on the
+// GPU through the C++ shim and compares every result with the CPU oracle (oracle/llmq_oracle.c, linked
+// into this test binary only).  Also exercises the shim's exception behaviour.
+//   usage: qmm_harness BT C OC [reuse_inp]
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "llmq_qmm.hpp"
+
+extern "C" {
+float orc_abs_max_bf16(const uint16_t* in, int64_t n);
+float orc_bf16_to_f32(uint16_t h);
+void orc_quantize_e4m3_bf16(uint8_t* out, float* scale_out, const uint16_t* in, float absmax, int64_t n);
+void orc_transpose_u8(uint8_t* dst, const uint8_t* src, int rows, int cols);
+void orc_gemm_tn_e4m3_exact_sampled(double* exact, double* sumabs, const uint8_t* a, const uint8_t* b, int M, int N, int K,
+                                    const int32_t* idx_n, const int32_t* idx_m, int64_t count);
+void orc_fill_normal_bf16(uint16_t* out, int64_t n, uint64_t seed, uint64_t stream, float mean, float std);
+}
+
+#define HIP_OK(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) { std::printf("HIP error %s at line %d\n", hipGetErrorString(e_), __LINE__); return 2; } } while (0)
+
+static int failures = 0;
+#define EXPECT(cond, ...) do { if (!(cond)) { ++failures; std::printf("FAIL: " __VA_ARGS__); std::printf("\n"); } } while (0)
+
+template <class T> static T* dalloc(std::size_t n) { void* p = nullptr; if (hipMalloc(&p, n * sizeof(T) + 16) != hipSuccess) std::abort(); return (T*)p; }
+
+static Tensor make(ETensorDType dt, void* p, std::vector<long> shape, float* stats = nullptr) {
+    Tensor t = Tensor::from_pointer((std::byte*)p, 0, dt, shape);
+    t.Stats = stats;
+    return t;
+}
+
+static void check_gemm(const char* name, const std::vector<uint16_t>& got_bf16, const std::vector<float>& got_f32, int N, int M,
+                       const uint8_t* a, const uint8_t* b, int K, float scale) {
+    const int S = 20000;
+    std::vector<int32_t> in(S), im(S);
+    uint64_t s = 88172645463325252ull;
+    for (int i = 0; i < S; ++i) { s ^= s << 13; s ^= s >> 7; s ^= s << 17; in[i] = (int32_t)(s % N); im[i] = (int32_t)((s >> 32) % M); }
+    std::vector<double> ex(S), sa(S);
+    orc_gemm_tn_e4m3_exact_sampled(ex.data(), sa.data(), a, b, M, N, K, in.data(), im.data(), S);
+    double worst = 0, e2 = 0, r2 = 0, maxabs = 0;
+    const bool bf16 = !got_bf16.empty();
+    for (int i = 0; i < S; ++i) {
+        const std::size_t o = (std::size_t)in[i] * M + im[i];
+        const double g = bf16 ? (double)orc_bf16_to_f32(got_bf16[o]) : (double)got_f32[o];
+        const double ref = ex[i] * scale, err = std::fabs(g - ref);
+        const double bound = (bf16 ? std::ldexp(std::fabs(ref), -8) : 0.0) + std::ldexp(scale * sa[i], -11) + 1e-38;
+        worst = std::fmax(worst, err / bound); maxabs = std::fmax(maxabs, err); e2 += err * err; r2 += ref * ref;
+    }
+    const double fro = std::sqrt(e2 / r2);
+    std::printf("%-10s [%d x %d] K=%d: max-abs err %.3e, rel-Frobenius %.3e, worst/bound %.3f\n", name, N, M, K, maxabs, fro, worst);
+    EXPECT(worst <= 1.0, "%s exceeds the element bound", name);
+    EXPECT(fro <= (bf16 ? 2.5e-3 : 2e-4), "%s exceeds the Frobenius bound", name);
+}
+
+int main(int argc, char** argv) {
+    const int BT = argc > 1 ? std::atoi(argv[1]) : 1024, C = argc > 2 ? std::atoi(argv[2]) : 896, OC = argc > 3 ? std::atoi(argv[3]) : 1152;
+    const bool reuse_inp = argc > 4 && std::atoi(argv[4]) != 0;
+    const int B = 1, T = BT;
+    std::printf("qmm_harness BT=%d C=%d OC=%d reuse_inp=%d\n", BT, C, OC, (int)reuse_inp);
+    hipStream_t stream; HIP_OK(hipStreamCreate(&stream));
+    QmmRunState rs; HIP_OK(hipGetDeviceProperties(&rs.DeviceProp, 0));
+    rs.Capacity = QmmRunState::backward_temp_bytes(B, T, C, OC);
+    rs.Arena = dalloc<std::byte>(rs.Capacity);
+
+    std::vector<uint16_t> hx((std::size_t)BT * C), hw((std::size_t)OC * C), hdy((std::size_t)BT * OC);
+    orc_fill_normal_bf16(hx.data(), hx.size(), 7, 1, 0.f, 1.f);
+    orc_fill_normal_bf16(hw.data(), hw.size(), 7, 2, 0.f, 0.02f);
+    orc_fill_normal_bf16(hdy.data(), hdy.size(), 7, 3, 0.f, 1e-3f);
+    auto* dx = dalloc<uint16_t>(hx.size()); auto* dw = dalloc<uint16_t>(hw.size()); auto* ddy = dalloc<uint16_t>(hdy.size());
+    HIP_OK(hipMemcpy(dx, hx.data(), hx.size() * 2, hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(dw, hw.data(), hw.size() * 2, hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(ddy, hdy.data(), hdy.size() * 2, hipMemcpyHostToDevice));
+    float* stats = dalloc<float>(8);   // [x: absmax, scale][w][dy]
+    HIP_OK(hipMemset(stats, 0, 32));
+
+    QuantizableTensor inp{make(ETensorDType::BF16, dx, {BT, C}), make(ETensorDType::FP8_E4M3, dalloc<uint8_t>(hx.size()), {BT, C}, stats)};
+    QuantizableTensor dout{make(ETensorDType::BF16, ddy, {BT, OC}), make(ETensorDType::FP8_E4M3, dalloc<uint8_t>(hdy.size()), {BT, OC}, stats + 4)};
+    Tensor w_master = make(ETensorDType::BF16, dw, {OC, C});
+    Tensor weight = make(ETensorDType::FP8_E4M3, dalloc<uint8_t>(hw.size()), {OC, C}, stats + 2);
+    Tensor out = make(ETensorDType::BF16, dalloc<uint16_t>((std::size_t)BT * OC), {BT, OC});
+    Tensor dinp = make(ETensorDType::BF16, dalloc<uint16_t>((std::size_t)BT * C), {BT, C});
+    Tensor dweight = make(ETensorDType::FP32, dalloc<float>((std::size_t)OC * C), {OC, C});
+    Tensor no_bias{}, workspace{};
+
+    // producers' abs-max epilogues are replaced by the standalone kernel; weights as llama_weights.cpp:207-223
+    abs_max(inp.Quant.abs_max(), inp.Value, (long)BT * C, rs.DeviceProp, stream);
+    abs_max(weight.abs_max(), w_master, (long)OC * C, rs.DeviceProp, stream);
+    abs_max(dout.Quant.abs_max(), dout.Value, (long)BT * OC, rs.DeviceProp, stream);
+    quantize_with_abs_max(weight, weight.scale(), w_master, weight.abs_max(), (long)OC * C, rs.DeviceProp, stream);
+    forward_qmm(out, inp, weight, no_bias, nullptr, workspace, B, T, C, OC, rs.DeviceProp, false, stream, EMatmulBackend::Custom);
+    backward_qmm(dinp, dweight, dout, inp, weight, false, rs, B, T, C, OC, reuse_inp, stream);
+    HIP_OK(hipStreamSynchronize(stream));
+    EXPECT(rs.Top == 0 && rs.Live.empty(), "temporary stack not unwound");
+    EXPECT(rs.HighWater == rs.Capacity, "backward_temp_bytes (%zu) != high-water mark (%zu)", rs.Capacity, rs.HighWater);
+
+    // ---- oracle side ----
+    float hstats[8]; HIP_OK(hipMemcpy(hstats, stats, 32, hipMemcpyDeviceToHost));
+    const float ax = orc_abs_max_bf16(hx.data(), hx.size()), aw = orc_abs_max_bf16(hw.data(), hw.size()), ag = orc_abs_max_bf16(hdy.data(), hdy.size());
+    std::vector<uint8_t> xq(hx.size()), wq(hw.size()), gq(hdy.size());
+    float sx, sw, sg;
+    orc_quantize_e4m3_bf16(xq.data(), &sx, hx.data(), ax, hx.size());
+    orc_quantize_e4m3_bf16(wq.data(), &sw, hw.data(), aw, hw.size());
+    orc_quantize_e4m3_bf16(gq.data(), &sg, hdy.data(), ag, hdy.size());
+    EXPECT(std::memcmp(&hstats[0], &ax, 4) == 0 && std::memcmp(&hstats[2], &aw, 4) == 0 && std::memcmp(&hstats[4], &ag, 4) == 0, "abs-max mismatch");
+    EXPECT(std::memcmp(&hstats[1], &sx, 4) == 0 && std::memcmp(&hstats[3], &sw, 4) == 0 && std::memcmp(&hstats[5], &sg, 4) == 0, "scale mismatch");
+    std::vector<uint8_t> got(std::max({xq.size(), wq.size(), gq.size()}));
+    HIP_OK(hipMemcpy(got.data(), inp.Quant.Data, xq.size(), hipMemcpyDeviceToHost));
+    EXPECT(std::memcmp(got.data(), xq.data(), xq.size()) == 0, "x quantized bytes differ");
+    HIP_OK(hipMemcpy(got.data(), weight.Data, wq.size(), hipMemcpyDeviceToHost));
+    EXPECT(std::memcmp(got.data(), wq.data(), wq.size()) == 0, "w quantized bytes differ");
+    HIP_OK(hipMemcpy(got.data(), dout.Quant.Data, gq.size(), hipMemcpyDeviceToHost));
+    EXPECT(std::memcmp(got.data(), gq.data(), gq.size()) == 0, "dy quantized bytes differ");
+
+    std::vector<uint16_t> hy((std::size_t)BT * OC), hdx((std::size_t)BT * C); std::vector<float> hdw((std::size_t)OC * C);
+    HIP_OK(hipMemcpy(hy.data(), out.Data, hy.size() * 2, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(hdx.data(), dinp.Data, hdx.size() * 2, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(hdw.data(), dweight.Data, hdw.size() * 4, hipMemcpyDeviceToHost));
+    std::vector<uint8_t> wqt(wq.size()), xqt(xq.size()), gqt(gq.size());
+    orc_transpose_u8(wqt.data(), wq.data(), OC, C);
+    orc_transpose_u8(xqt.data(), xq.data(), BT, C);
+    orc_transpose_u8(gqt.data(), gq.data(), BT, OC);
+    check_gemm("forward", hy, {}, BT, OC, wq.data(), xq.data(), C, sw * sx);
+    check_gemm("dgrad", hdx, {}, BT, C, wqt.data(), gq.data(), OC, sw * sg);
+    check_gemm("wgrad", {}, hdw, OC, C, xqt.data(), gqt.data(), BT, sx * sg);
+
+    // ---- error behaviour of the shim (reference: gemm_mma.cu:261-263, kernels.cpp:18-24) ----
+    bool threw = false;
+    try { matmul(out, weight, inp.Quant, no_bias, nullptr, nullptr, nullptr, workspace, OC, BT, C + 64, EMMTranspose::TN, false, stream); }
+    catch (const std::invalid_argument&) { threw = true; }
+    EXPECT(threw, "matmul with K %% 128 != 0 must throw std::invalid_argument");
+    threw = false;
+    try { matmul(out, weight, inp.Quant, no_bias, nullptr, nullptr, nullptr, workspace, OC, BT, C, EMMTranspose::NN, false, stream); }
+    catch (const std::invalid_argument&) { threw = true; }
+    EXPECT(threw, "non-TN FP8 matmul must throw std::invalid_argument");
+    threw = false;
+    try { quantize_with_abs_max(out, nullptr, inp.Value, stats, 8, rs.DeviceProp, stream); }
+    catch (const std::invalid_argument&) { threw = true; }
+    EXPECT(threw, "unsupported dtype combination must throw std::invalid_argument");
+
+    std::printf(failures ? "RESULT: FAIL (%d)\n" : "RESULT: PASS\n", failures);
+    return failures ? 1 : 0;
+}

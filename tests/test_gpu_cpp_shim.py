@@ -1,0 +1,19 @@
+"""Runs the C++ harness (tests/cpp/qmm_harness.cpp): forward_qmm / backward_qmm through the C++20
+shim that mirrors the reference's kernels.h, checked against the CPU oracle inside the harness."""
+import os
+import subprocess
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+HERE = os.path.dirname(os.path.abspath(__file__))
+BIN = os.path.join(HERE, "cpp", "build", "qmm_harness")
+
+
+@pytest.mark.parametrize("args", [("1024", "896", "1152", "0"), ("2048", "896", "896", "1"), ("512", "4864", "896", "0"),
+                                  ("4096", "1536", "1792", "0")])
+def test_qmm_harness(args):
+    assert os.path.exists(BIN), "build it with `make -C tests/cpp` (done by __graft_entry__.build())"
+    r = subprocess.run([BIN, *args], capture_output=True, text=True, timeout=150)
+    print(r.stdout[-3000:], r.stderr[-2000:])
+    assert r.returncode == 0 and "RESULT: PASS" in r.stdout
