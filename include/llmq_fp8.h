@@ -17,6 +17,7 @@
 #ifndef LLMQ_FP8_H
 #define LLMQ_FP8_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -91,10 +92,14 @@ int llmq_transpose_u8(uint8_t* dst, const uint8_t* src, int rows, int cols, void
  *           std::byte* ws, size_t ws_size, int M, int N, int K, EMMTranspose::TN, bool accumulate,
  *           cudaStream_t, EMatmulBackend)  src/kernels/kernels.h:88-90, src/kernels/matmul.cpp:216-220,
  *           and gemm_mma_tn(...) src/kernels/gemm_mma.cu:279-284.
+ * workspace: device scratch like the reference's matmul workspace (32 MiB in src/training/model.cpp:69),
+ * or NULL with size 0.  It is only used when the output has too few tiles to fill the chip: K is
+ * then split, fp32 partial results (N*M*4 bytes per split) go to the workspace and are added in a
+ * fixed order, so results are deterministic.  Calls that share a workspace must be stream ordered.
  */
 int llmq_gemm_tn_e4m3_bf16(uint16_t* c, const uint8_t* a, const uint8_t* b, const uint16_t* bias_or_null,
-                           const float* sa_or_null, const float* sb_or_null, int M, int N, int K,
-                           int accumulate, void* stream);
+                           const float* sa_or_null, const float* sb_or_null, void* workspace_or_null,
+                           size_t workspace_bytes, int M, int N, int K, int accumulate, void* stream);
 
 /*
  * fp32-output variant (wgrad into fp32 gradients).  bias may be fp32[M] (bias_is_bf16 == 0) or
@@ -104,8 +109,9 @@ int llmq_gemm_tn_e4m3_bf16(uint16_t* c, const uint8_t* a, const uint8_t* b, cons
  *           src/kernels/matmul.cpp:198-208.
  */
 int llmq_gemm_tn_e4m3_f32(float* c, const uint8_t* a, const uint8_t* b, const void* bias_or_null,
-                          int bias_is_bf16, const float* sa_or_null, const float* sb_or_null, int M, int N,
-                          int K, int accumulate, void* stream);
+                          int bias_is_bf16, const float* sa_or_null, const float* sb_or_null,
+                          void* workspace_or_null, size_t workspace_bytes, int M, int N, int K, int accumulate,
+                          void* stream);
 
 #ifdef __cplusplus
 }

@@ -5,8 +5,9 @@
 // header after the type substitutions
 //     nv_bfloat16 -> __hip_bfloat16        __nv_fp8_e4m3 -> __hip_fp8_e4m3     __nv_fp8_e5m2 -> __hip_fp8_e5m2
 //     cudaStream_t -> hipStream_t          cudaDeviceProp -> hipDeviceProp_t   cublasLtHandle_t -> llmqBlasHandle_t
-// The device-property, handle and workspace arguments are accepted and ignored (the gfx950 kernels
-// need neither a library handle nor a workspace).  Errors surface as the reference's exception types:
+// The device-property and handle arguments are accepted and ignored.  The matmul workspace is passed
+// through: the gfx950 GEMM uses it for split-K partial sums when the output has too few tiles to fill
+// the chip, and works without one.  Errors surface as the reference's exception types:
 // std::invalid_argument for shape / dtype / argument errors, std::runtime_error for runtime failures.
 #ifndef LLMQ_KERNELS_HPP
 #define LLMQ_KERNELS_HPP
@@ -209,27 +210,29 @@ inline void transpose(Tensor& dst, const Tensor& src, int rows, int cols, hipStr
 // ---- matmul (reference: src/kernels/kernels.h:72-78, 88-90, 96-98) --------------------------------------
 // Row-major a[M,K], b[N,K] -> row-major c[N,M] = (b . a^T) * (*scale_a * *scale_b) (+ bias[M]) (+ c).
 inline void matmul(__hip_bfloat16* c, const __hip_fp8_e4m3* a, const __hip_fp8_e4m3* b, const __hip_bfloat16* bias,
-                   const float* scale_a, const float* scale_b, llmqBlasHandle_t, std::byte*, std::size_t, int M, int N,
-                   int K, EMMTranspose mode, bool accumulate, hipStream_t stream,
-                   EMatmulBackend = EMatmulBackend::Custom) {
+                   const float* scale_a, const float* scale_b, llmqBlasHandle_t, std::byte* workspace,
+                   std::size_t workspace_size, int M, int N, int K, EMMTranspose mode, bool accumulate,
+                   hipStream_t stream, EMatmulBackend = EMatmulBackend::Custom) {
     llmq_detail::require_tn(mode);
     llmq_detail::check(llmq_gemm_tn_e4m3_bf16(llmq_detail::u16(c), llmq_detail::u8(a), llmq_detail::u8(b),
-                                              llmq_detail::u16(bias), scale_a, scale_b, M, N, K, accumulate, stream));
+                                              llmq_detail::u16(bias), scale_a, scale_b, workspace, workspace_size, M, N,
+                                              K, accumulate, stream));
 }
 inline void matmul(float* c, const __hip_fp8_e4m3* a, const __hip_fp8_e4m3* b, const float* bias, const float* scale_a,
-                   const float* scale_b, llmqBlasHandle_t, std::byte*, std::size_t, int M, int N, int K,
-                   EMMTranspose mode, bool accumulate, hipStream_t stream, EMatmulBackend = EMatmulBackend::Custom) {
-    llmq_detail::require_tn(mode);
-    llmq_detail::check(llmq_gemm_tn_e4m3_f32(c, llmq_detail::u8(a), llmq_detail::u8(b), bias, 0, scale_a, scale_b, M, N, K,
-                                             accumulate, stream));
-}
-inline void matmul(float* c, const __hip_fp8_e4m3* a, const __hip_fp8_e4m3* b, const __hip_bfloat16* bias,
-                   const float* scale_a, const float* scale_b, llmqBlasHandle_t, std::byte*, std::size_t, int M, int N,
-                   int K, EMMTranspose mode, bool accumulate, hipStream_t stream,
+                   const float* scale_b, llmqBlasHandle_t, std::byte* workspace, std::size_t workspace_size, int M,
+                   int N, int K, EMMTranspose mode, bool accumulate, hipStream_t stream,
                    EMatmulBackend = EMatmulBackend::Custom) {
     llmq_detail::require_tn(mode);
-    llmq_detail::check(llmq_gemm_tn_e4m3_f32(c, llmq_detail::u8(a), llmq_detail::u8(b), bias, 1, scale_a, scale_b, M, N, K,
-                                             accumulate, stream));
+    llmq_detail::check(llmq_gemm_tn_e4m3_f32(c, llmq_detail::u8(a), llmq_detail::u8(b), bias, 0, scale_a, scale_b,
+                                             workspace, workspace_size, M, N, K, accumulate, stream));
+}
+inline void matmul(float* c, const __hip_fp8_e4m3* a, const __hip_fp8_e4m3* b, const __hip_bfloat16* bias,
+                   const float* scale_a, const float* scale_b, llmqBlasHandle_t, std::byte* workspace,
+                   std::size_t workspace_size, int M, int N, int K, EMMTranspose mode, bool accumulate,
+                   hipStream_t stream, EMatmulBackend = EMatmulBackend::Custom) {
+    llmq_detail::require_tn(mode);
+    llmq_detail::check(llmq_gemm_tn_e4m3_f32(c, llmq_detail::u8(a), llmq_detail::u8(b), bias, 1, scale_a, scale_b,
+                                             workspace, workspace_size, M, N, K, accumulate, stream));
 }
 inline void matmul(Tensor& c, const Tensor& a, const Tensor& b, const Tensor& bias, const float* scale_a,
                    const float* scale_b, llmqBlasHandle_t handle, Tensor& workspace, int M, int N, int K,

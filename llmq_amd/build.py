@@ -20,6 +20,7 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++20", "-fPIC",
     "-ffp-contract=off",                       # the epilogue and the quantize multiply are defined op by op
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-mllvm", "-enable-post-misched=0",       # keep the hand-specified interleave of the GEMM K loop
     "-Wall", "-Wextra", "-Wno-unused-parameter", "-Wno-unknown-warning-option",
     "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
 ]

@@ -7,20 +7,33 @@
 //
 // Kernel design (nothing here is derived from the reference's mma.sync kernel):
 //   * one workgroup computes a BLK_N x BLK_M tile of c, K is walked in steps of 128 bytes;
-//   * both operand tiles are staged in LDS, double buffered; with DMA == true the global->LDS copies
-//     are 16-byte-per-lane direct-to-LDS loads (no VGPR staging), issued one K-step ahead;
+//   * both operand tiles are staged in LDS, double buffered, by 16-byte-per-lane direct-to-LDS loads
+//     (no VGPR staging) issued one K-step ahead;
 //   * LDS rows are 128 bytes (one K-step) and the eight 16-byte chunks of a row are XOR-swizzled
 //     with (row >> 1) & 7, which makes the 128-bit fragment reads of 16 consecutive rows hit all 64
 //     banks exactly once; the swizzle is applied on the global side (each lane picks its source chunk)
 //     because direct-to-LDS loads land linearly (lane i -> base + 16 i);
 //   * the matrix instruction is v_mfma_f32_32x32x64_f8f6f4 (fp8 x fp8, K = 64 per instruction, two per
 //     K-step); both operands use the same lane->K mapping, so any consistent mapping is correct;
-//   * rows of the a-tile (the m / column index of c) are permuted on their way into LDS so that the NJ
-//     accumulators a lane holds for one c row are NJ consecutive columns: the epilogue then stores
-//     NJ packed outputs per lane and 32 lanes cover a contiguous row segment (256 B for bf16, NJ = 4);
+//   * rows of the a-tile (the m / column index of c) are permuted on their way into LDS so that the two
+//     accumulators a lane holds for one c row are consecutive columns: the epilogue stores packed
+//     pairs and 32 lanes cover a contiguous row segment;
+//   * the K loop is an explicit software pipeline over half-steps (K = 64, one matrix instruction
+//     deep).  Within a half-step the matrix instructions run row by row (b-rows fragment i against all
+//     a-rows fragments); as soon as row i has been issued its fragment registers are refilled from LDS
+//     for the next half-step, and the other operand's fragments of the next half-step go into a second
+//     small buffer.  LDS reads therefore stream under the matrix instructions with (NI + 2 NJ)
+//     fragment registers instead of a full double buffer.  The single workgroup barrier per K-step sits
+//     in the second half-step right after its first row has been queued: at that point every wave has
+//     finished reading the stage the next direct-to-LDS copies overwrite, and the stage fetched one
+//     step earlier has landed;
 //   * the linear workgroup id is remapped so that each of the 8 XCDs (workgroups are dealt to XCDs
 //     round-robin) works on a contiguous range of tiles, walked in column-major groups of `group`
-//     tile-rows for L2 reuse of both operands.
+//     tile-rows for L2 reuse of both operands;
+//   * shapes with too few output tiles to fill the chip (weight gradients of small layers) split K
+//     over gridDim.y: every split writes its raw fp32 accumulators to a slice of the caller's
+//     workspace, and a second kernel adds the slices in a fixed order and applies the epilogue, so the
+//     result does not depend on scheduling.
 #include <type_traits>
 
 #include "common.hpp"
@@ -30,27 +43,10 @@ namespace llmq {
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
 
 constexpr int kBK = 128;  // bytes (= e4m3 elements) of K per LDS stage
-
-__device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x0040u);
-    u += 0x7FFFu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
-}
-
-template <typename OutT> struct OutIo;
-template <> struct OutIo<uint16_t> {
-    static __device__ __forceinline__ float load(const uint16_t* p) { return __uint_as_float((uint32_t)*p << 16); }
-    static __device__ __forceinline__ uint16_t cvt(float v) { return f32_to_bf16_rne(v); }
-};
-template <> struct OutIo<float> {
-    static __device__ __forceinline__ float load(const float* p) { return *p; }
-    static __device__ __forceinline__ float cvt(float v) { return v; }
-};
-
-template <int NJ, typename OutT> struct Pack { OutT v[NJ]; } __attribute__((aligned(sizeof(OutT) * NJ)));
 
 struct GemmArgs {
     void* c;
@@ -62,206 +58,54 @@ struct GemmArgs {
     int M, N, K;
     int bias_is_bf16;
     int accumulate;
-    int group;  // tile-rows per rasterisation group
+    int group;       // tile-rows per rasterisation group
+    float* partial;  // split-K only: [splits][N][M] raw accumulators
+    int k_len;       // split-K only: K elements per split (multiple of 128)
 };
 
-template <int BLK_N, int BLK_M, int WV_N, int WV_M, bool DMA, typename OutT>
-__global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_kernel(GemmArgs g) {
-    constexpr int T = WV_N * WV_M * 64;
-    constexpr int WT_N = BLK_N / WV_N, WT_M = BLK_M / WV_M;
-    constexpr int NI = WT_N / 32, NJ = WT_M / 32;
-    constexpr int P_BYTES = BLK_N * kBK, Q_BYTES = BLK_M * kBK, STAGE = P_BYTES + Q_BYTES;
-    constexpr int P_ITERS = BLK_N * 8 / T, Q_ITERS = BLK_M * 8 / T;
-    static_assert(BLK_N * 8 % T == 0 && BLK_M * 8 % T == 0, "tile chunks must divide evenly over the lanes");
-    static_assert(T / 8 % 32 == 0, "row permutation assumes whole 32-row groups per load iteration");
-    static_assert(NJ == 1 || NJ == 2 || NJ == 4, "packed epilogue width");
-
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * STAGE];
-
-    const int tid = threadIdx.x;
-    const int lane = tid % 64, wave = tid / 64;
-    const int wn = wave / WV_M, wm = wave % WV_M;
-    const int l32 = lane % 32, kg = lane / 32;
-
-    // ---- workgroup -> tile (XCD-contiguous, grouped column-major walk) ----
-    const int tiles_n = g.N / BLK_N, tiles_m = g.M / BLK_M;
-    int tile_n, tile_m;
-    {
-        const int nwg = gridDim.x, wg = blockIdx.x;
-        const int xcd = wg % 8, idx = wg / 8;
-        const int q = nwg / 8, r = nwg % 8;
-        const int logical = xcd * q + (xcd < r ? xcd : r) + idx;
-        const int per_group = g.group * tiles_m;
-        const int gid = logical / per_group;
-        const int first_n = gid * g.group;
-        const int gsz = (tiles_n - first_n) < g.group ? (tiles_n - first_n) : g.group;
-        const int in_group = logical % per_group;
-        tile_n = first_n + in_group % gsz;
-        tile_m = in_group / gsz;
+// Output pair store: y = v (+ old value when accumulating), one rounding to the output type.
+template <typename OutT> struct PairIo;
+template <> struct PairIo<uint16_t> {
+    static __device__ __forceinline__ void load(const uint16_t* p, float& v0, float& v1) {
+        const uint32_t old = *reinterpret_cast<const uint32_t*>(p);
+        v0 = __uint_as_float(old << 16);
+        v1 = __uint_as_float(old & 0xFFFF0000u);
     }
-    const int n_blk = tile_n * BLK_N, m_blk = tile_m * BLK_M;
-
-    // ---- global -> LDS copy plan: chunk id = it*T + tid, LDS offset = 16 * chunk id (linear) ----
-    const int ld_row = tid / 8;                         // + it * (T/8)
-    const int ld_chunk = (tid & 7) ^ ((ld_row >> 1) & 7);  // logical 16-byte chunk this lane fetches
-    const uint8_t* p_src = g.b + (int64_t)n_blk * g.K + (int64_t)ld_row * g.K + ld_chunk * 16;
-    // a-tile row permutation: LDS row rho (within wave column w) holds global row NJ*(rho%32) + rho/32
-    const uint8_t* q_src[Q_ITERS];
-#pragma unroll
-    for (int it = 0; it < Q_ITERS; ++it) {
-        const int rho = it * (T / 8) + ld_row;
-        const int w = rho / WT_M, rw = rho % WT_M;
-        const int grow = w * WT_M + NJ * (rw % 32) + rw / 32;
-        q_src[it] = g.a + (int64_t)m_blk * g.K + (int64_t)grow * g.K + ld_chunk * 16;
+    static __device__ __forceinline__ void store(uint16_t* p, float v0, float v1) {
+        const f32x2_t v = {v0, v1};
+        *reinterpret_cast<bf16x2_t*>(p) = __builtin_convertvector(v, bf16x2_t);  // v_cvt_pk_bf16_f32, RNE
     }
-
-    auto issue_loads = [&](int stage, int k0, uint4* regs) {
-        uint8_t* base = lds + stage * STAGE;
-#pragma unroll
-        for (int it = 0; it < P_ITERS; ++it) {
-            const uint8_t* src = p_src + (int64_t)it * (T / 8) * g.K + k0;
-            if constexpr (DMA) {
-                __builtin_amdgcn_global_load_lds(
-                    (const __attribute__((address_space(1))) void*)src,
-                    (__attribute__((address_space(3))) void*)(base + (it * T + wave * 64) * 16), 16, 0, 0);
-            } else {
-                regs[it] = *reinterpret_cast<const uint4*>(src);
-            }
-        }
-#pragma unroll
-        for (int it = 0; it < Q_ITERS; ++it) {
-            const uint8_t* src = q_src[it] + k0;
-            if constexpr (DMA) {
-                __builtin_amdgcn_global_load_lds(
-                    (const __attribute__((address_space(1))) void*)src,
-                    (__attribute__((address_space(3))) void*)(base + P_BYTES + (it * T + wave * 64) * 16), 16, 0, 0);
-            } else {
-                regs[P_ITERS + it] = *reinterpret_cast<const uint4*>(src);
-            }
-        }
-    };
-    auto commit_loads = [&](int stage, const uint4* regs) {
-        if constexpr (!DMA) {
-            uint8_t* base = lds + stage * STAGE;
-#pragma unroll
-            for (int it = 0; it < P_ITERS; ++it)
-                *reinterpret_cast<uint4*>(base + (it * T + tid) * 16) = regs[it];
-#pragma unroll
-            for (int it = 0; it < Q_ITERS; ++it)
-                *reinterpret_cast<uint4*>(base + P_BYTES + (it * T + tid) * 16) = regs[P_ITERS + it];
-        }
-    };
-
-    // ---- fragment read plan ----
-    const int sw = (l32 >> 1) & 7;
-    const int p_frag = (wn * WT_N + l32) * kBK;            // + ti*32*kBK
-    const int q_frag = P_BYTES + (wm * WT_M + l32) * kBK;  // + tj*32*kBK
-
-    v16f acc[NI][NJ];
-#pragma unroll
-    for (int i = 0; i < NI; ++i)
-#pragma unroll
-        for (int j = 0; j < NJ; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
-    uint4 regs[DMA ? 1 : (P_ITERS + Q_ITERS)];
-    const int KT = g.K / kBK;
-
-    issue_loads(0, 0, regs);
-    commit_loads(0, regs);
-    if constexpr (DMA) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-
-    for (int kt = 0; kt < KT; ++kt) {
-        const int cur = kt & 1;
-        if (kt + 1 < KT) issue_loads(cur ^ 1, (kt + 1) * kBK, regs);
-        const uint8_t* st = lds + cur * STAGE;
-#pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            const int c0 = ((4 * s + 2 * kg) ^ sw) * 16, c1 = ((4 * s + 2 * kg + 1) ^ sw) * 16;
-            v8i fa[NI], fb[NJ];
-#pragma unroll
-            for (int i = 0; i < NI; ++i) {
-                const v4i lo = *reinterpret_cast<const v4i*>(st + p_frag + i * 32 * kBK + c0);
-                const v4i hi = *reinterpret_cast<const v4i*>(st + p_frag + i * 32 * kBK + c1);
-                fa[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-            }
-#pragma unroll
-            for (int j = 0; j < NJ; ++j) {
-                const v4i lo = *reinterpret_cast<const v4i*>(st + q_frag + j * 32 * kBK + c0);
-                const v4i hi = *reinterpret_cast<const v4i*>(st + q_frag + j * 32 * kBK + c1);
-                fb[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-            }
-#pragma unroll
-            for (int i = 0; i < NI; ++i)
-#pragma unroll
-                for (int j = 0; j < NJ; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[j], acc[i][j], 0, 0, 0, 0, 0, 0);
-        }
-        if (kt + 1 < KT) commit_loads(cur ^ 1, regs);
-        if constexpr (DMA) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
+};
+template <> struct PairIo<float> {
+    static __device__ __forceinline__ void load(const float* p, float& v0, float& v1) {
+        const float2 old = *reinterpret_cast<const float2*>(p);
+        v0 = old.x;
+        v1 = old.y;
     }
+    static __device__ __forceinline__ void store(float* p, float v0, float v1) {
+        *reinterpret_cast<float2*>(p) = make_float2(v0, v1);
+    }
+};
 
-    // ---- epilogue: acc * (sa*sb) (+ bias[m]) (+ c) -> one rounding -> packed stores ----
-    float scale = g.sa ? *g.sa : 1.f;
-    if (g.sb) scale = scale * *g.sb;
-    OutT* c = reinterpret_cast<OutT*>(g.c);
-    const int m_lane = m_blk + wm * WT_M + NJ * l32;
-    float bias_v[NJ];
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-        bias_v[j] = 0.f;
-        if (g.bias) {
-            bias_v[j] = g.bias_is_bf16
-                            ? __uint_as_float((uint32_t) reinterpret_cast<const uint16_t*>(g.bias)[m_lane + j] << 16)
-                            : reinterpret_cast<const float*>(g.bias)[m_lane + j];
-        }
-    }
-#pragma unroll
-    for (int i = 0; i < NI; ++i) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int n = n_blk + wn * WT_N + i * 32 + 8 * (r / 4) + 4 * kg + (r % 4);
-            OutT* dst = c + (int64_t)n * g.M + m_lane;
-            Pack<NJ, OutT> old, out;
-            if (g.accumulate) old = *reinterpret_cast<const Pack<NJ, OutT>*>(dst);
-#pragma unroll
-            for (int j = 0; j < NJ; ++j) {
-                float t = acc[i][j][r] * scale;
-                if (g.bias) t = t + bias_v[j];
-                if (g.accumulate) t = t + OutIo<OutT>::load(&old.v[j]);
-                out.v[j] = OutIo<OutT>::cvt(t);
-            }
-            *reinterpret_cast<Pack<NJ, OutT>*>(dst) = out;
-        }
-    }
+__device__ __forceinline__ float load_bias(const void* bias, int is_bf16, int m) {
+    return is_bf16 ? __uint_as_float((uint32_t) reinterpret_cast<const uint16_t*>(bias)[m] << 16)
+                   : reinterpret_cast<const float*>(bias)[m];
 }
 
-// ---- software-pipelined variant ---------------------------------------------------------------------
-// Same tiling, LDS layout and epilogue as above, with the K loop written as an explicit software
-// pipeline over half-steps (K = 64, one matrix instruction deep).  Within a half-step the matrix
-// instructions run row by row (a-fragment i against all b-fragments); as soon as row i has been
-// issued its a-fragment registers are refilled from LDS for the next half-step, and the b-fragments
-// of the next half-step go into a second small buffer.  LDS reads therefore stream under the matrix
-// instructions with (NI + 2 NJ) fragment registers instead of a full double buffer.  The single
-// workgroup barrier per K-step sits in the second half-step right after its first row has been
-// queued: at that point every wave has finished reading the stage the next direct-to-LDS copies
-// overwrite, and the stage fetched one step earlier has landed.
 template <int MASK, int N>
 __device__ __forceinline__ void sched_group() {
     if constexpr (N > 0) __builtin_amdgcn_sched_group_barrier(MASK, N, 0);
 }
 
-template <int BLK_N, int BLK_M, int WV_N, int WV_M, typename OutT>
+// SPLIT: blockIdx.y selects a K range of g.k_len elements and the raw accumulators go to g.partial.
+template <int BLK_N, int BLK_M, int WV_N, int WV_M, typename OutT, bool SPLIT>
 __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(GemmArgs g) {
     constexpr int T = WV_N * WV_M * 64;
     constexpr int WT_N = BLK_N / WV_N, WT_M = BLK_M / WV_M;
     constexpr int NI = WT_N / 32, NJ = WT_M / 32;
     constexpr int P_BYTES = BLK_N * kBK, Q_BYTES = BLK_M * kBK, STAGE = P_BYTES + Q_BYTES;
     constexpr int P_ITERS = BLK_N * 8 / T, Q_ITERS = BLK_M * 8 / T, LOADS = P_ITERS + Q_ITERS;
-    static_assert(T / 8 % 32 == 0 && (NJ == 1 || NJ == 2 || NJ == 4) && NI >= 2, "tile configuration");
+    static_assert(T / 8 % 32 == 0 && NJ == 2 && NI >= 2, "tile configuration");
 
     __shared__ __attribute__((aligned(16))) uint8_t lds[2 * STAGE];
 
@@ -288,29 +132,38 @@ __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(Gemm
     }
     const int n_blk = tile_n * BLK_N, m_blk = tile_m * BLK_M;
 
+    int k_begin = 0, k_count = g.K;
+    if constexpr (SPLIT) {
+        k_begin = blockIdx.y * g.k_len;
+        k_count = (g.K - k_begin) < g.k_len ? (g.K - k_begin) : g.k_len;
+    }
+
     const int ld_row = tid / 8;
     const int ld_chunk = (tid & 7) ^ ((ld_row >> 1) & 7);
-    const uint8_t* p_src = g.b + (int64_t)n_blk * g.K + (int64_t)ld_row * g.K + ld_chunk * 16;
+    const uint8_t* p_src = g.b + (int64_t)n_blk * g.K + (int64_t)ld_row * g.K + ld_chunk * 16 + k_begin;
     const uint8_t* q_src[Q_ITERS];
 #pragma unroll
     for (int it = 0; it < Q_ITERS; ++it) {
         const int rho = it * (T / 8) + ld_row;
         const int w = rho / WT_M, rw = rho % WT_M;
         const int grow = w * WT_M + NJ * (rw % 32) + rw / 32;
-        q_src[it] = g.a + (int64_t)m_blk * g.K + (int64_t)grow * g.K + ld_chunk * 16;
+        q_src[it] = g.a + (int64_t)m_blk * g.K + (int64_t)grow * g.K + ld_chunk * 16 + k_begin;
     }
     auto issue_loads = [&](int stage, int k0) {
         uint8_t* base = lds + stage * STAGE + wave * 1024;
 #pragma unroll
-        for (int it = 0; it < P_ITERS; ++it)
-            __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(p_src + (int64_t)it * (T / 8) * g.K + k0),
-                (__attribute__((address_space(3))) void*)(base + it * T * 16), 16, 0, 0);
+        for (int it = 0; it < P_ITERS; ++it) {
+            const uint8_t* src = p_src + (int64_t)it * (T / 8) * g.K + k0;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                             (__attribute__((address_space(3))) void*)(base + it * T * 16), 16, 0, 0);
+        }
 #pragma unroll
-        for (int it = 0; it < Q_ITERS; ++it)
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(q_src[it] + k0),
+        for (int it = 0; it < Q_ITERS; ++it) {
+            const uint8_t* src = q_src[it] + k0;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                              (__attribute__((address_space(3))) void*)(base + P_BYTES + it * T * 16), 16,
                                              0, 0);
+        }
     };
 
     const int sw = (l32 >> 1) & 7;
@@ -334,7 +187,7 @@ __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(Gemm
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    const int KT = g.K / kBK;
+    const int KT = k_count / kBK;
     issue_loads(0, 0);
     if (KT > 1) {
         issue_loads(1, kBK);
@@ -350,10 +203,10 @@ __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(Gemm
 #pragma unroll
     for (int j = 0; j < NJ; ++j) fb[0][j] = read_frag(lds + q_frag + j * 32 * kBK, 0);
 
-    // One half-step.  H: which half (selects the b-fragment buffer); NEXT: another half-step follows
-    // and its fragments are read from `next`; SYNC: barrier after the first row (the following
-    // half-step lives in the other LDS stage); REFILL: start the direct-to-LDS copies of the stage
-    // after that one into the stage just released.
+    // One half-step.  H: which half (selects the second operand's fragment buffer); NEXT: another
+    // half-step follows and its fragments are read from `next`; SYNC: barrier after the first row (the
+    // following half-step lives in the other LDS stage); REFILL: start the direct-to-LDS copies of the
+    // stage after that one into the stage just released.
     auto half_step = [&](auto h_tag, auto next_tag, auto sync_tag, auto refill_tag, const uint8_t* next,
                          int refill_stage, int refill_k0) {
         constexpr int H = decltype(h_tag)::value;
@@ -420,107 +273,175 @@ __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(Gemm
     half_step(H0, Y, NO, NO, lds + (kt & 1) * STAGE, 0, 0);   // last stage
     half_step(H1, NO, NO, NO, lds, 0, 0);
 
-    float scale = g.sa ? *g.sa : 1.f;
-    if (g.sb) scale = scale * *g.sb;
-    OutT* c = reinterpret_cast<OutT*>(g.c);
+    // Epilogue.  Accumulator register r of fragment (i, j) is c row 8*(r/4) + 4*kg + r%4 of the
+    // fragment; thanks to the a-tile row permutation the lane's two j values are adjacent columns.
     const int m_lane = m_blk + wm * WT_M + NJ * l32;
-    float bias_v[NJ];
+    if constexpr (SPLIT) {
+        float* part = g.partial + (int64_t)blockIdx.y * g.N * g.M;
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-        bias_v[j] = 0.f;
-        if (g.bias) {
-            bias_v[j] = g.bias_is_bf16
-                            ? __uint_as_float((uint32_t) reinterpret_cast<const uint16_t*>(g.bias)[m_lane + j] << 16)
-                            : reinterpret_cast<const float*>(g.bias)[m_lane + j];
-        }
-    }
+        for (int i = 0; i < NI; ++i) {
 #pragma unroll
-    for (int i = 0; i < NI; ++i) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int n = n_blk + wn * WT_N + i * 32 + 8 * (r / 4) + 4 * kg + (r % 4);
-            OutT* dst = c + (int64_t)n * g.M + m_lane;
-            Pack<NJ, OutT> old, out;
-            if (g.accumulate) old = *reinterpret_cast<const Pack<NJ, OutT>*>(dst);
-#pragma unroll
-            for (int j = 0; j < NJ; ++j) {
-                float t = acc[i][j][r] * scale;
-                if (g.bias) t = t + bias_v[j];
-                if (g.accumulate) t = t + OutIo<OutT>::load(&old.v[j]);
-                out.v[j] = OutIo<OutT>::cvt(t);
+            for (int r = 0; r < 16; ++r) {
+                const int n = n_blk + wn * WT_N + i * 32 + 8 * (r / 4) + 4 * kg + (r % 4);
+                PairIo<float>::store(part + (int64_t)n * g.M + m_lane, acc[i][0][r], acc[i][1][r]);
             }
-            *reinterpret_cast<Pack<NJ, OutT>*>(dst) = out;
+        }
+    } else {
+        float scale = g.sa ? *g.sa : 1.f;
+        if (g.sb) scale = scale * *g.sb;
+        OutT* c = reinterpret_cast<OutT*>(g.c);
+        float bias0 = 0.f, bias1 = 0.f;
+        if (g.bias) {
+            bias0 = load_bias(g.bias, g.bias_is_bf16, m_lane);
+            bias1 = load_bias(g.bias, g.bias_is_bf16, m_lane + 1);
+        }
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int n = n_blk + wn * WT_N + i * 32 + 8 * (r / 4) + 4 * kg + (r % 4);
+                OutT* dst = c + (int64_t)n * g.M + m_lane;
+                float v0 = acc[i][0][r] * scale, v1 = acc[i][1][r] * scale;
+                if (g.bias) {
+                    v0 = v0 + bias0;
+                    v1 = v1 + bias1;
+                }
+                if (g.accumulate) {
+                    float o0, o1;
+                    PairIo<OutT>::load(dst, o0, o1);
+                    v0 = v0 + o0;
+                    v1 = v1 + o1;
+                }
+                PairIo<OutT>::store(dst, v0, v1);
+            }
         }
     }
 }
 
-template <int BLK_N, int BLK_M, int WV_N, int WV_M, typename OutT>
-static int launch_pipe(const GemmArgs& g, hipStream_t stream) {
-    const int tiles = (g.N / BLK_N) * (g.M / BLK_M);
-    hipLaunchKernelGGL((gemm_tn_e4m3_pipe_kernel<BLK_N, BLK_M, WV_N, WV_M, OutT>), dim3((unsigned)tiles),
-                       dim3(WV_N * WV_M * 64), 0, stream, g);
-    LLMQ_HIP_TRY(hipGetLastError());
-    return LLMQ_OK;
+// Second pass of the split-K path: c = round((sum_s partial[s]) * scale + bias + old), slices added in
+// index order.  One lane handles two adjacent columns; HBM-bound elementwise work.
+template <typename OutT>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs g, int splits) {
+    const int64_t pairs = (int64_t)g.N * g.M / 2;
+    const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (p >= pairs) return;
+    const int64_t e = 2 * p;
+    const int64_t slice = (int64_t)g.N * g.M;
+    float v0 = 0.f, v1 = 0.f;
+    for (int s = 0; s < splits; ++s) {
+        const float2 t = *reinterpret_cast<const float2*>(g.partial + s * slice + e);
+        v0 = v0 + t.x;
+        v1 = v1 + t.y;
+    }
+    float scale = g.sa ? *g.sa : 1.f;
+    if (g.sb) scale = scale * *g.sb;
+    v0 = v0 * scale;
+    v1 = v1 * scale;
+    if (g.bias) {
+        const int m = (int)(e % g.M);
+        v0 = v0 + load_bias(g.bias, g.bias_is_bf16, m);
+        v1 = v1 + load_bias(g.bias, g.bias_is_bf16, m + 1);
+    }
+    OutT* dst = reinterpret_cast<OutT*>(g.c) + e;
+    if (g.accumulate) {
+        float o0, o1;
+        PairIo<OutT>::load(dst, o0, o1);
+        v0 = v0 + o0;
+        v1 = v1 + o1;
+    }
+    PairIo<OutT>::store(dst, v0, v1);
 }
 
 // ---- host side ------------------------------------------------------------------------------------
-template <int BLK_N, int BLK_M, int WV_N, int WV_M, bool DMA, typename OutT>
-static int launch_cfg(const GemmArgs& g, hipStream_t stream) {
+template <int BLK_N, int BLK_M, int WV_N, int WV_M, typename OutT>
+static int launch_pipe(const GemmArgs& g, int splits, hipStream_t stream) {
     const int tiles = (g.N / BLK_N) * (g.M / BLK_M);
-    hipLaunchKernelGGL((gemm_tn_e4m3_kernel<BLK_N, BLK_M, WV_N, WV_M, DMA, OutT>), dim3((unsigned)tiles),
-                       dim3(WV_N * WV_M * 64), 0, stream, g);
+    if (splits > 1) {
+        hipLaunchKernelGGL((gemm_tn_e4m3_pipe_kernel<BLK_N, BLK_M, WV_N, WV_M, OutT, true>),
+                           dim3((unsigned)tiles, (unsigned)splits), dim3(WV_N * WV_M * 64), 0, stream, g);
+        LLMQ_HIP_TRY(hipGetLastError());
+        const int64_t pairs = (int64_t)g.N * g.M / 2;
+        hipLaunchKernelGGL((splitk_reduce_kernel<OutT>), dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, stream,
+                           g, splits);
+    } else {
+        hipLaunchKernelGGL((gemm_tn_e4m3_pipe_kernel<BLK_N, BLK_M, WV_N, WV_M, OutT, false>), dim3((unsigned)tiles),
+                           dim3(WV_N * WV_M * 64), 0, stream, g);
+    }
     LLMQ_HIP_TRY(hipGetLastError());
     return LLMQ_OK;
 }
 
-// Variant selector: 0 = automatic.  Non-zero values pick one instantiation explicitly (used by the
-// tuning harness and the tests to cover every instantiation).
-int g_gemm_variant = 0;
+// Tuning / test hooks: 0 = automatic.  tile: 1 = 256 x 256 tile with 8 waves, 2 = 128 x 128 tile with
+// 4 waves.  splits: forced number of K splits (needs a workspace).
+int g_gemm_tile = 0;
+int g_gemm_splits = 0;
 
 template <typename OutT>
-static int gemm_dispatch(GemmArgs g, hipStream_t stream) {
+static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     LLMQ_REQUIRE(g.M > 0 && g.N > 0 && g.K > 0, "matmul: M, N, K must be positive (got %d, %d, %d)", g.M, g.N, g.K);
     LLMQ_REQUIRE(g.M % 128 == 0 && g.N % 128 == 0 && g.K % 128 == 0,
                  "matmul: M, N, K must be divisible by 128 (got %d, %d, %d)", g.M, g.N, g.K);
     LLMQ_REQUIRE(g.a && g.b && g.c, "matmul: null operand pointer");
-    LLMQ_REQUIRE(aligned16(g.a) && aligned16(g.b) && aligned16(g.c) && aligned16(g.bias),
+    LLMQ_REQUIRE(aligned16(g.a) && aligned16(g.b) && aligned16(g.c) && aligned16(g.bias) && aligned16(workspace),
                  "matmul: all pointers must be 16-byte aligned");
+    LLMQ_REQUIRE(workspace != nullptr || workspace_bytes == 0, "matmul: workspace size given without a workspace");
     g.group = 8;
-    int variant = g_gemm_variant;
-    if (variant == 0) {
-        const bool n256 = g.N % 256 == 0, m256 = g.M % 256 == 0;
-        const int64_t tiles256 = (int64_t)(g.N / 256) * (g.M / 256);
-        if (n256 && m256 && tiles256 >= cu_count()) variant = 6;
-        else variant = 3;
+    const int cus = cu_count();
+    int tile = g_gemm_tile;
+    LLMQ_REQUIRE(tile >= 0 && tile <= 2, "matmul: unknown tile selector %d", tile);
+    const bool fits256 = g.N % 256 == 0 && g.M % 256 == 0;
+    LLMQ_REQUIRE(tile != 1 || fits256, "matmul: the 256 x 256 tile needs M and N divisible by 256");
+    if (tile == 0) tile = (fits256 && (int64_t)(g.N / 256) * (g.M / 256) >= cus) ? 1 : 2;
+
+    // Split K when the tiles alone leave most of the chip idle: aim at about one workgroup per compute
+    // unit, keep at least 512 elements of K per split, and stay inside the caller's workspace.
+    const int64_t tiles = tile == 1 ? (int64_t)(g.N / 256) * (g.M / 256) : (int64_t)(g.N / 128) * (g.M / 128);
+    const int64_t slice_bytes = (int64_t)g.N * g.M * 4;
+    const int64_t ws_splits = (int64_t)(workspace_bytes / (size_t)slice_bytes);
+    int splits = g_gemm_splits;
+    LLMQ_REQUIRE(splits >= 0, "matmul: negative split count %d", splits);
+    if (splits == 0) {
+        splits = 1;
+        if (2 * tiles <= cus && ws_splits >= 2) {
+            int64_t want = cus / tiles;
+            if (want > g.K / 512) want = g.K / 512;
+            if (want > ws_splits) want = ws_splits;
+            if (want > 1) splits = (int)want;
+        }
+    } else if (splits > 1) {
+        LLMQ_REQUIRE(splits <= g.K / kBK, "matmul: %d splits for K = %d", splits, g.K);
+        LLMQ_REQUIRE(ws_splits >= splits, "matmul: workspace of %zu bytes is too small for %d splits", workspace_bytes,
+                     splits);
     }
-    switch (variant) {
-        case 1: return launch_cfg<256, 256, 2, 4, true, OutT>(g, stream);
-        case 2: return launch_cfg<256, 256, 2, 4, false, OutT>(g, stream);
-        case 3: return launch_cfg<128, 128, 2, 2, true, OutT>(g, stream);
-        case 4: return launch_cfg<128, 128, 2, 2, false, OutT>(g, stream);
-        case 5: return launch_cfg<256, 256, 2, 2, true, OutT>(g, stream);
-        case 6: return launch_pipe<256, 256, 2, 4, OutT>(g, stream);
-        case 7: return launch_pipe<256, 256, 2, 2, OutT>(g, stream);
-        case 8: return launch_pipe<128, 128, 2, 2, OutT>(g, stream);
-        default: return set_error(LLMQ_ERR_INVALID_ARGUMENT, "matmul: unknown kernel variant %d", variant);
+    if (splits > 1) {
+        const int steps = g.K / kBK;
+        g.k_len = ((steps + splits - 1) / splits) * kBK;
+        splits = (g.K + g.k_len - 1) / g.k_len;  // no empty split
+        g.partial = reinterpret_cast<float*>(workspace);
     }
+    if (tile == 1) return launch_pipe<256, 256, 2, 4, OutT>(g, splits, stream);
+    return launch_pipe<128, 128, 2, 2, OutT>(g, splits, stream);
 }
 
 }  // namespace llmq
 
 extern "C" int llmq_gemm_tn_e4m3_bf16(uint16_t* c, const uint8_t* a, const uint8_t* b, const uint16_t* bias_or_null,
-                                      const float* sa_or_null, const float* sb_or_null, int M, int N, int K,
-                                      int accumulate, void* stream) {
-    llmq::GemmArgs g{c, a, b, bias_or_null, sa_or_null, sb_or_null, M, N, K, 1, accumulate, 8};
-    return llmq::gemm_dispatch<uint16_t>(g, static_cast<hipStream_t>(stream));
+                                      const float* sa_or_null, const float* sb_or_null, void* workspace_or_null,
+                                      size_t workspace_bytes, int M, int N, int K, int accumulate, void* stream) {
+    llmq::GemmArgs g{c, a, b, bias_or_null, sa_or_null, sb_or_null, M, N, K, 1, accumulate, 8, nullptr, 0};
+    return llmq::gemm_dispatch<uint16_t>(g, workspace_or_null, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int llmq_gemm_tn_e4m3_f32(float* c, const uint8_t* a, const uint8_t* b, const void* bias_or_null,
-                                     int bias_is_bf16, const float* sa_or_null, const float* sb_or_null, int M, int N,
-                                     int K, int accumulate, void* stream) {
-    llmq::GemmArgs g{c, a, b, bias_or_null, sa_or_null, sb_or_null, M, N, K, bias_is_bf16, accumulate, 8};
-    return llmq::gemm_dispatch<float>(g, static_cast<hipStream_t>(stream));
+                                     int bias_is_bf16, const float* sa_or_null, const float* sb_or_null,
+                                     void* workspace_or_null, size_t workspace_bytes, int M, int N, int K,
+                                     int accumulate, void* stream) {
+    llmq::GemmArgs g{c, a, b, bias_or_null, sa_or_null, sb_or_null, M, N, K, bias_is_bf16, accumulate, 8, nullptr, 0};
+    return llmq::gemm_dispatch<float>(g, workspace_or_null, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
-// Tuning / test hook (not part of the drop-in surface): force a kernel instantiation, 0 = automatic.
-extern "C" void llmq_debug_set_gemm_variant(int v) { llmq::g_gemm_variant = v; }
+// Tuning / test hooks (not part of the drop-in surface).
+extern "C" void llmq_debug_set_gemm_variant(int tile, int splits) {
+    llmq::g_gemm_tile = tile;
+    llmq::g_gemm_splits = splits;
+}

@@ -78,9 +78,15 @@ def transpose(dst, src, stream=0):
     capi.check(capi.lib.llmq_transpose_u8(d, s, src.shape[0], src.shape[1], _stream(stream)))
 
 
-def matmul(c, a, b, bias, scale_a, scale_b, M, N, K, accumulate=False, stream=0):
+def matmul(c, a, b, bias, scale_a, scale_b, M, N, K, accumulate=False, stream=0, workspace=None):
     """TN matmul in the convention of the reference's kernels.h: row-major a[M,K], b[N,K] (e4m3) give
-    row-major c[N,M] = (b @ a.T) * scale_a * scale_b (+ bias[M]) (+ c).  c: bf16 or fp32."""
+    row-major c[N,M] = (b @ a.T) * scale_a * scale_b (+ bias[M]) (+ c).  c: bf16 or fp32.
+    workspace: optional device byte tensor (the reference passes a 32 MiB one); it enables the
+    split-K path for outputs with too few tiles to fill the chip."""
+    pws, ws_bytes = None, 0
+    if workspace is not None:
+        pws = _dev(workspace, "workspace", (torch.uint8, torch.int8, torch.float32))
+        ws_bytes = workspace.numel() * workspace.element_size()
     pa = _dev(a, "a", (torch.float8_e4m3fn, torch.uint8))
     pb = _dev(b, "b", (torch.float8_e4m3fn, torch.uint8))
     pc = _dev(c, "c", (torch.bfloat16, torch.float32))
@@ -92,11 +98,12 @@ def matmul(c, a, b, bias, scale_a, scale_b, M, N, K, accumulate=False, stream=0)
         pbias = _dev(bias, "bias", (torch.bfloat16,), optional=True)
         if bias is not None and bias.numel() != M:
             raise ValueError("bias must have M elements")
-        capi.check(capi.lib.llmq_gemm_tn_e4m3_bf16(pc, pa, pb, pbias, sa, sb, M, N, K, int(accumulate), _stream(stream)))
+        capi.check(capi.lib.llmq_gemm_tn_e4m3_bf16(pc, pa, pb, pbias, sa, sb, pws, ws_bytes, M, N, K, int(accumulate),
+                                                   _stream(stream)))
     else:
         pbias = _dev(bias, "bias", (torch.bfloat16, torch.float32), optional=True)
         if bias is not None and bias.numel() != M:
             raise ValueError("bias must have M elements")
         is_bf16 = int(bias is not None and bias.dtype == torch.bfloat16)
-        capi.check(capi.lib.llmq_gemm_tn_e4m3_f32(pc, pa, pb, pbias, is_bf16, sa, sb, M, N, K, int(accumulate),
-                                                  _stream(stream)))
+        capi.check(capi.lib.llmq_gemm_tn_e4m3_f32(pc, pa, pb, pbias, is_bf16, sa, sb, pws, ws_bytes, M, N, K,
+                                                  int(accumulate), _stream(stream)))

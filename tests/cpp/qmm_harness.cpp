@@ -86,7 +86,10 @@ int main(int argc, char** argv) {
     Tensor out = make(ETensorDType::BF16, dalloc<uint16_t>((std::size_t)BT * OC), {BT, OC});
     Tensor dinp = make(ETensorDType::BF16, dalloc<uint16_t>((std::size_t)BT * C), {BT, C});
     Tensor dweight = make(ETensorDType::FP32, dalloc<float>((std::size_t)OC * C), {OC, C});
-    Tensor no_bias{}, workspace{};
+    Tensor no_bias{};
+    // matmul workspace sized like the reference's (src/training/model.cpp:69)
+    Tensor workspace = make(ETensorDType::BYTE, dalloc<uint8_t>(32u << 20), {32L << 20});
+    rs.Workspace = workspace;
 
     // producers' abs-max epilogues are replaced by the standalone kernel; weights as llama_weights.cpp:207-223
     abs_max(inp.Quant.abs_max(), inp.Value, (long)BT * C, rs.DeviceProp, stream);

@@ -50,13 +50,16 @@ def test_invalid_arguments_are_rejected_without_a_gpu(capi):
     assert L.llmq_transpose_u8(None, p, 16, 16, None) == INV
     assert L.llmq_transpose_u8(p, p, 0, 16, None) == capi.LLMQ_OK            # empty: nothing to do
     # GEMM: the 128-divisibility rule of the reference's custom kernel (gemm_mma.cu:261-263)
-    assert L.llmq_gemm_tn_e4m3_bf16(p, p, p, None, None, None, 128, 128, 64, 0, None) == INV
+    assert L.llmq_gemm_tn_e4m3_bf16(p, p, p, None, None, None, None, 0, 128, 128, 64, 0, None) == INV
     assert b"divisible by 128" in L.llmq_last_error()
-    assert L.llmq_gemm_tn_e4m3_bf16(p, p, p, None, None, None, 100, 128, 128, 0, None) == INV
-    assert L.llmq_gemm_tn_e4m3_bf16(p, None, p, None, None, None, 128, 128, 128, 0, None) == INV
-    assert L.llmq_gemm_tn_e4m3_bf16(p, p + 8, p, None, None, None, 128, 128, 128, 0, None) == INV
+    assert L.llmq_gemm_tn_e4m3_bf16(p, p, p, None, None, None, None, 0, 100, 128, 128, 0, None) == INV
+    assert L.llmq_gemm_tn_e4m3_bf16(p, None, p, None, None, None, None, 0, 128, 128, 128, 0, None) == INV
+    assert L.llmq_gemm_tn_e4m3_bf16(p, p + 8, p, None, None, None, None, 0, 128, 128, 128, 0, None) == INV
     assert b"aligned" in L.llmq_last_error()
-    assert L.llmq_gemm_tn_e4m3_f32(p, p, p, None, 0, None, None, 0, 128, 128, 0, None) == INV
+    assert L.llmq_gemm_tn_e4m3_f32(p, p, p, None, 0, None, None, None, 0, 0, 128, 128, 0, None) == INV
+    assert L.llmq_gemm_tn_e4m3_bf16(p, p, p, None, None, None, None, 4096, 128, 128, 128, 0, None) == INV
+    assert b"workspace" in L.llmq_last_error()
+    assert L.llmq_gemm_tn_e4m3_bf16(p, p, p, None, None, None, p + 4, 4096, 128, 128, 128, 0, None) == INV
     with pytest.raises(ValueError):
         capi.check(INV)
     with pytest.raises(RuntimeError):

@@ -56,16 +56,26 @@ class QT:
         return self.stats[1:2]
 
 
+_WS = {}
+
+
+def workspace():
+    """Matmul workspace sized like the reference's (src/training/model.cpp:69)."""
+    if "ws" not in _WS:
+        _WS["ws"] = torch.empty(32 << 20, dtype=torch.uint8, device="cuda")
+    return _WS["ws"]
+
+
 def forward_qmm(K, out, inp, weight_q, weight_scale, BT, C, OC):
     K.quantize_with_abs_max(inp.quant, inp.scale, inp.value, inp.abs_max)
-    K.matmul(out, weight_q, inp.quant, None, weight_scale, inp.scale, OC, BT, C)
+    K.matmul(out, weight_q, inp.quant, None, weight_scale, inp.scale, OC, BT, C, workspace=workspace())
 
 
 def backward_qmm(K, dinp, dweight, dout, inp, weight_q, weight_scale, BT, C, OC, reuse_inp, accumulate=False):
     K.quantize_with_abs_max(dout.quant, dout.scale, dout.value, dout.abs_max)
     weight_tp = torch.empty((C, OC), dtype=F8, device="cuda")
     K.transpose(weight_tp, weight_q)
-    K.matmul(dinp, weight_tp, dout.quant, None, weight_scale, dout.scale, C, BT, OC)
+    K.matmul(dinp, weight_tp, dout.quant, None, weight_scale, dout.scale, C, BT, OC, workspace=workspace())
     act_tp = torch.empty((C, BT), dtype=F8, device="cuda")
     grad_tp = torch.empty((OC, BT), dtype=F8, device="cuda")
     if reuse_inp:
@@ -73,7 +83,8 @@ def backward_qmm(K, dinp, dweight, dout, inp, weight_q, weight_scale, BT, C, OC,
     else:
         K.quantize_and_transpose_with_abs_max(act_tp, None, inp.value, inp.abs_max)
     K.transpose(grad_tp, dout.quant)
-    K.matmul(dweight, act_tp, grad_tp, None, inp.scale, dout.scale, C, OC, BT, accumulate=accumulate)
+    K.matmul(dweight, act_tp, grad_tp, None, inp.scale, dout.scale, C, OC, BT, accumulate=accumulate,
+             workspace=workspace())
     return weight_tp, act_tp, grad_tp
 
 
@@ -136,7 +147,8 @@ def run_linear_fwd_bwd(K, O, BT, C, OC, x, w, dy, seed, backward=True, reuse_inp
     check_gemm(O, dweight, np.ascontiguousarray(xc.T), np.ascontiguousarray(gc.T), dx_s, dg_s, seed + 2, "wgrad dw")
     # accumulate into an existing gradient (second micro-step of gradient accumulation)
     old = dweight.float().cpu().numpy()
-    K.matmul(dweight, a_tp, g_tp, None, inp.scale, dout.scale, C, OC, BT, accumulate=True)
+    K.matmul(dweight, a_tp, g_tp, None, inp.scale, dout.scale, C, OC, BT, accumulate=True,
+             workspace=workspace())
     torch.cuda.synchronize()
     check_gemm(O, dweight, np.ascontiguousarray(xc.T), np.ascontiguousarray(gc.T), dx_s, dg_s, seed + 2, "wgrad dw +=", c_old=old)
 

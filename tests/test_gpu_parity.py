@@ -141,11 +141,26 @@ def test_transpose_bit_exact(K, shape):
 
 # --------------------------------------------------------------------------------------------- GEMM
 def set_variant(v):
+    """v = (tile, splits): tile 0 = automatic, 1 = 256 x 256, 2 = 128 x 128; splits 0 = automatic."""
     from llmq_amd import capi
-    capi.lib.llmq_debug_set_gemm_variant(v)
+    capi.lib.llmq_debug_set_gemm_variant(v[0], v[1])
 
 
-VARIANTS = [0, 1, 2, 3, 4, 5, 6, 7, 8]
+VARIANTS = [(0, 0), (1, 0), (2, 0), (1, 2), (2, 2), (2, 3)]
+_WORKSPACE = {}
+
+
+def workspace():
+    if "ws" not in _WORKSPACE:
+        _WORKSPACE["ws"] = torch.empty(32 << 20, dtype=torch.uint8, device="cuda")
+    return _WORKSPACE["ws"]
+
+
+def skip_unsupported(variant, M, N, Kd):
+    if variant[0] == 1 and (M % 256 or N % 256):
+        pytest.skip("the 256 x 256 tile needs multiples of 256")
+    if variant[1] > Kd // 128:
+        pytest.skip("more splits than K-steps")
 
 
 def run_gemm(K, a, b, M, N, Kd, sa, sb, bias_bits=None, old=None, out_f32=False):
@@ -156,7 +171,7 @@ def run_gemm(K, a, b, M, N, Kd, sa, sb, bias_bits=None, old=None, out_f32=False)
         c = torch.full((N, M), float("nan"), dtype=dt, device="cuda")
     bias = dev_bf16(bias_bits) if bias_bits is not None else None
     K.matmul(c, dev_u8(a), dev_u8(b), bias, dev_scalar(sa) if sa is not None else None,
-             dev_scalar(sb) if sb is not None else None, M, N, Kd, accumulate=old is not None)
+             dev_scalar(sb) if sb is not None else None, M, N, Kd, accumulate=old is not None, workspace=workspace())
     torch.cuda.synchronize()
     return c
 
@@ -167,8 +182,7 @@ def test_gemm_integer_known_answer_exact(K, O, variant, mnk):
     """Construction of src/testing/test-gemm.cpp:54-85: integer operands, exact fp32 sums -> the bf16
     output must equal the oracle bit for bit (set / bias / accumulate)."""
     M, N, Kd = mnk
-    if variant in (1, 2, 5, 6, 7) and (M % 256 or N % 256):
-        pytest.skip("256-tile variants need multiples of 256")
+    skip_unsupported(variant, M, N, Kd)
     a, _ = O.fill_int_e4m3(M * Kd, 12345, 0)
     b, _ = O.fill_int_e4m3(N * Kd, 12345, 1)
     a, b = a.reshape(M, Kd), b.reshape(N, Kd)
@@ -187,13 +201,14 @@ def test_gemm_integer_known_answer_exact(K, O, variant, mnk):
         got32 = run_gemm(K, a, b, M, N, Kd, s, s, out_f32=True)
         assert np.array_equal(got32.cpu().numpy(), want32)
     finally:
-        set_variant(0)
+        set_variant((0, 0))
 
 
 @pytest.mark.parametrize("variant", VARIANTS)
 @pytest.mark.parametrize("out_f32", [False, True])
 def test_gemm_random_codes_within_tolerance(K, O, variant, out_f32):
     M, N, Kd = 512, 256, 896
+    skip_unsupported(variant, M, N, Kd)
     rng = np.random.default_rng(17)
     a = rng.integers(0, 256, (M, Kd)).astype(np.uint8)
     b = rng.integers(0, 256, (N, Kd)).astype(np.uint8)
@@ -218,7 +233,32 @@ def test_gemm_random_codes_within_tolerance(K, O, variant, out_f32):
         extra = O.bf16_to_f32(bias).astype(np.float64)[None, :] + old.astype(np.float64)
         gemm_check(got2.float().cpu().numpy(), exact, sumabs, scale, not out_f32, extra=extra)
     finally:
-        set_variant(0)
+        set_variant((0, 0))
+
+
+@pytest.mark.parametrize("mnk", [(128, 128, 4096), (256, 384, 2048), (896, 896, 8192)])
+def test_gemm_automatic_split_k(K, O, mnk):
+    """Few-tile shapes with a workspace take the split-K path on their own; integer operands keep
+    every partial sum exact, so the result must still equal the oracle bit for bit, and repeated
+    calls must agree (fixed summation order)."""
+    M, N, Kd = mnk
+    a, _ = O.fill_int_e4m3(M * Kd, 777, 0)
+    b, _ = O.fill_int_e4m3(N * Kd, 777, 1)
+    a, b = a.reshape(M, Kd), b.reshape(N, Kd)
+    s = float(np.sqrt(np.float32(4.0 / Kd)))
+    _, biasv = O.fill_int_e4m3(M, 777, 2)
+    bias = O.f32_to_bf16(biasv.astype(np.float32))
+    want = O.gemm_tn(a, b, sa=s, sb=s, bias=bias, mt=True)
+    got = run_gemm(K, a, b, M, N, Kd, s, s, bias)
+    assert np.array_equal(host_bits(got), want)
+    rng = np.random.default_rng(5)
+    ar = rng.integers(0, 0x7E, (M, Kd)).astype(np.uint8)
+    br = rng.integers(0, 0x7E, (N, Kd)).astype(np.uint8) | 0x80
+    c1 = run_gemm(K, ar, br, M, N, Kd, 0.01, 0.02, out_f32=True)
+    c2 = run_gemm(K, ar, br, M, N, Kd, 0.01, 0.02, out_f32=True)
+    assert torch.equal(c1, c2)
+    exact, sumabs = O.gemm_exact(ar, br)
+    gemm_check(c1.cpu().numpy(), exact, sumabs, np.float32(np.float32(0.01) * np.float32(0.02)), False)
 
 
 def test_gemm_matches_swapped_operand_transpose(K, O):
