@@ -39,6 +39,8 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch one plain 1 GiB copy kernel (reference point for hardware traffic counters)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="rough budget of the CPU baseline sample")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -142,7 +144,29 @@ def main():
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     record[0] = False
+    if args.calibrate_copy:
+        src = torch.randint(0, 255, (1 << 30,), dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        capi.check(capi.lib.llmq_debug_copy_u8(dst.data_ptr(), src.data_ptr(), src.numel(),
+                                               torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
     step_ms = (t1 - t0) * 1e3 / args.steps
+
+    # What the matrix cores sustain with no memory traffic at all: a register-only MFMA loop on random
+    # fp8 operands (the chip lowers its clock under that load), about 0.3 s of it.
+    scratch = torch.empty(256 * 512, dtype=torch.float32, device=dev)
+    st = torch.cuda.current_stream().cuda_stream
+    ceiling = {}
+    for label, rnd in (("constant_operands", 0), ("random_operands", 1)):
+        capi.check(capi.lib.llmq_debug_mfma_ceiling(scratch.data_ptr(), 256, 20000, rnd, st))
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+        reps, iters = 6, 100000
+        for _ in range(reps):
+            capi.check(capi.lib.llmq_debug_mfma_ceiling(scratch.data_ptr(), 256, iters, rnd, st))
+        ev1.record()
+        torch.cuda.synchronize()
+        ceiling[label] = 256.0 * 8 * iters * 4 * 131072.0 * reps / (ev0.elapsed_time(ev1) * 1e-3) / 1e12
 
     def summarize(name):
         evs = timers.get(name, [])
@@ -172,7 +196,9 @@ def main():
                    "tokens": BT, "gemm_flop_per_step": gemm_flop},
         "roofline": {"bound": "mfma", "kernel": "gemm_tn_e4m3_pipe_kernel", "achieved": gemm_tflops_kernel,
                      "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": gemm_tflops_kernel / FP8_PEAK_TFLOPS,
-                     "traffic": None, "mean_launch_ms": ks["gemm"]["mean_ms"], "launches": ks["gemm"]["launches"]},
+                     "traffic": measured_traffic(), "mfma_only_ceiling_TFLOPs": ceiling,
+                     "frac_of_mfma_only_ceiling": gemm_tflops_kernel / ceiling["random_operands"],
+                     "mean_launch_ms": ks["gemm"]["mean_ms"], "launches": ks["gemm"]["launches"]},
         "quantize": {"bound": "hbm", "kernels": "abs_max + quantize_with_abs_max (5 bytes/element)",
                      "achieved": aq_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": aq_gbs / HBM_PEAK_GBS,
                      "per_kernel": per_kernel},
@@ -182,6 +208,19 @@ def main():
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(t, np, torch, args.cpu_seconds)
     print(json.dumps(result))
+
+
+def measured_traffic():
+    """HBM-side bytes per GEMM launch (L2 fetch + write-back) from the hardware-counter summary kept
+    under profiles/ for this same workload; None when that file is absent."""
+    path = os.path.join(ROOT, "profiles", "gemm_tn_e4m3_pipe_kernel__bench_qwen7b_mlp__traffic.txt")
+    try:
+        for line in open(path):
+            if line.startswith("traffic_bytes_per_launch"):
+                return float(line.split("=")[1].split()[0])
+    except OSError:
+        pass
+    return None
 
 
 def cpu_baseline(t, np, torch, budget_s):

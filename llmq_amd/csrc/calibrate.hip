@@ -1,0 +1,93 @@
+// Calibration kernels for measurements (not part of the drop-in surface).
+//
+//  * llmq_debug_copy_u8: a plain streaming copy whose HBM bytes are known exactly (n read + n
+//    written); hardware traffic counters of the real kernels are scaled by what they read for it.
+//  * llmq_debug_mfma_ceiling: a loop of v_mfma_f32_32x32x64_f8f6f4 on register operands with no
+//    memory traffic at all, 8 waves per compute unit.  With constant operands it runs at the nominal
+//    clock; with random fp8 operands that change every iteration (what a real K loop feeds the matrix
+//    cores) the chip lowers its clock under power, and the rate it sustains is the practical ceiling
+//    any fp8 GEMM on this part is measured against.
+#include "common.hpp"
+
+namespace llmq {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+__global__ __launch_bounds__(256) void copy_calibration_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src,
+                                                               int64_t nvec) {
+    const int64_t base = ((int64_t)blockIdx.x * 256 + threadIdx.x);
+    const int64_t stride = (int64_t)gridDim.x * 256;
+#pragma unroll 4
+    for (int u = 0; u < 4; ++u) {
+        const int64_t i = base + u * stride;
+        if (i < nvec) dst[i] = src[i];
+    }
+}
+
+__device__ __forceinline__ uint32_t mix32(uint32_t x) {
+    x ^= x >> 16; x *= 0x7feb352dU; x ^= x >> 15; x *= 0x846ca68bU; x ^= x >> 16;
+    return x;
+}
+
+template <bool RANDOM>
+__global__ __launch_bounds__(512) void mfma_ceiling_kernel(float* out, int iters) {
+    v8i a[2], b[2];
+    for (int s = 0; s < 2; ++s)
+        for (int i = 0; i < 8; ++i) {
+            if (!RANDOM) {
+                a[s][i] = 0x38383838;  // 1.0 in every byte
+                b[s][i] = 0x38383838;
+            } else {
+                const uint32_t ra = mix32(threadIdx.x * 64 + i + 17 * s + blockIdx.x * 77777u), rb = mix32(ra + 12345u);
+                a[s][i] = ra & 0xBFBFBFBFu;  // bit 6 of every byte cleared: no NaN code, magnitudes below 2
+                b[s][i] = rb & 0xBFBFBFBFu;
+            }
+        }
+    v16f acc[4];
+    for (int n = 0; n < 4; ++n)
+        for (int i = 0; i < 16; ++i) acc[n][i] = 0.f;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int n = 0; n < 4; ++n)
+            acc[n] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[n & 1], b[(n >> 1) & 1], acc[n], 0, 0, 0, 0, 0, 0);
+        if (RANDOM) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                a[0][i] ^= 0x15150a0a;
+                b[1][i] ^= 0x0a0a1515;
+            }
+        }
+    }
+    float s = 0;
+    for (int n = 0; n < 4; ++n)
+        for (int i = 0; i < 16; ++i) s += acc[n][i];
+    out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
+}  // namespace llmq
+
+extern "C" int llmq_debug_copy_u8(uint8_t* dst, const uint8_t* src, int64_t n, void* stream) {
+    using namespace llmq;
+    LLMQ_REQUIRE(dst && src && n > 0 && n % 16 == 0, "copy: need non-null pointers and a positive multiple of 16 bytes");
+    LLMQ_REQUIRE(aligned16(dst) && aligned16(src), "copy: pointers must be 16-byte aligned");
+    const int64_t nvec = n / 16;
+    const int64_t blocks = (nvec + 1023) / 1024;
+    LLMQ_REQUIRE(blocks <= 0x7FFFFFFF, "copy: too large");
+    hipLaunchKernelGGL(copy_calibration_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       reinterpret_cast<uint4*>(dst), reinterpret_cast<const uint4*>(src), nvec);
+    LLMQ_HIP_TRY(hipGetLastError());
+    return LLMQ_OK;
+}
+
+// Launches one ceiling kernel: `blocks` workgroups of 512 lanes, `iters` iterations of 4 matrix
+// instructions per wave (= blocks * 8 * iters * 4 * 131072 flop).  scratch: blocks * 512 floats.
+extern "C" int llmq_debug_mfma_ceiling(float* scratch, int blocks, int iters, int random_operands, void* stream) {
+    using namespace llmq;
+    LLMQ_REQUIRE(scratch != nullptr && blocks > 0 && iters > 0, "mfma_ceiling: bad arguments");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (random_operands) hipLaunchKernelGGL(mfma_ceiling_kernel<true>, dim3((unsigned)blocks), dim3(512), 0, st, scratch, iters);
+    else hipLaunchKernelGGL(mfma_ceiling_kernel<false>, dim3((unsigned)blocks), dim3(512), 0, st, scratch, iters);
+    LLMQ_HIP_TRY(hipGetLastError());
+    return LLMQ_OK;
+}

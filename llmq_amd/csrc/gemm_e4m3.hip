@@ -391,7 +391,14 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
     LLMQ_REQUIRE(tile >= 0 && tile <= 2, "matmul: unknown tile selector %d", tile);
     const bool fits256 = g.N % 256 == 0 && g.M % 256 == 0;
     LLMQ_REQUIRE(tile != 1 || fits256, "matmul: the 256 x 256 tile needs M and N divisible by 256");
-    if (tile == 0) tile = (fits256 && (int64_t)(g.N / 256) * (g.M / 256) >= cus) ? 1 : 2;
+    if (tile == 0) {
+        // Rounds of workgroups the chip needs: one 256 x 256 tile per compute unit and round (four units
+        // of work), or two co-resident 128 x 128 tiles (two units, at about 0.8 of the rate per unit).
+        const int64_t t256 = (int64_t)(g.N / 256) * (g.M / 256), t128 = (int64_t)(g.N / 128) * (g.M / 128);
+        const double cost256 = 4.0 * (double)((t256 + cus - 1) / cus);
+        const double cost128 = 2.0 * 1.25 * (double)((t128 + 2 * cus - 1) / (2 * cus));
+        tile = (fits256 && t256 >= cus && cost256 <= cost128) ? 1 : 2;
+    }
 
     // Split K when the tiles alone leave most of the chip idle: aim at about one workgroup per compute
     // unit, keep at least 512 elements of K per split, and stay inside the caller's workspace.
