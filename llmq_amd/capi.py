@@ -40,6 +40,8 @@ lib.llmq_gemm_tn_e4m3_bf16.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, C.c_si
 lib.llmq_gemm_tn_e4m3_f32.argtypes = [_vp, _vp, _vp, _vp, _int, _vp, _vp, _vp, C.c_size_t, _int, _int, _int, _int, _vp]
 lib.llmq_debug_set_gemm_variant.argtypes = [_int, _int]
 lib.llmq_debug_set_gemm_variant.restype = None
+lib.llmq_debug_set_gemm_persist.argtypes = [_int]
+lib.llmq_debug_set_gemm_persist.restype = None
 lib.llmq_debug_copy_u8.argtypes = [_vp, _vp, _i64, _vp]
 lib.llmq_debug_copy_u8.restype = _int
 lib.llmq_debug_mfma_ceiling.argtypes = [_vp, _int, _int, _int, _vp]

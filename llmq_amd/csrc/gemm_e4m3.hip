@@ -92,13 +92,24 @@ __device__ __forceinline__ float load_bias(const void* bias, int is_bf16, int m)
                    : reinterpret_cast<const float*>(bias)[m];
 }
 
+// Hides a value from loop-invariant code motion: lane-derived constants that are only needed between
+// tiles are recomputed from the lane id there instead of occupying registers across the K loop.
+__device__ __forceinline__ int opaque(int x) {
+    asm volatile("" : "+v"(x));
+    return x;
+}
+
 template <int MASK, int N>
 __device__ __forceinline__ void sched_group() {
     if constexpr (N > 0) __builtin_amdgcn_sched_group_barrier(MASK, N, 0);
 }
 
 // SPLIT: blockIdx.y selects a K range of g.k_len elements and the raw accumulators go to g.partial.
-template <int BLK_N, int BLK_M, int WV_N, int WV_M, typename OutT, bool SPLIT>
+// PERSIST: the grid has one workgroup per compute unit and every workgroup walks a list of tiles.  The
+// operand stream then runs across tile boundaries: the copies of the next tile's first two K-steps are
+// issued during the last two K-steps of the current tile, so the epilogue of a tile overlaps with the
+// fetch of the next one and no pipeline fill or workgroup launch sits between tiles.  Needs K >= 256.
+template <int BLK_N, int BLK_M, int WV_N, int WV_M, typename OutT, bool SPLIT, bool PERSIST>
 __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(GemmArgs g) {
     constexpr int T = WV_N * WV_M * 64;
     constexpr int WT_N = BLK_N / WV_N, WT_M = BLK_M / WV_M;
@@ -106,6 +117,7 @@ __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(Gemm
     constexpr int P_BYTES = BLK_N * kBK, Q_BYTES = BLK_M * kBK, STAGE = P_BYTES + Q_BYTES;
     constexpr int P_ITERS = BLK_N * 8 / T, Q_ITERS = BLK_M * 8 / T, LOADS = P_ITERS + Q_ITERS;
     static_assert(T / 8 % 32 == 0 && NJ == 2 && NI >= 2, "tile configuration");
+    static_assert(!(SPLIT && PERSIST), "split-K tiles are not walked persistently");
 
     __shared__ __attribute__((aligned(16))) uint8_t lds[2 * STAGE];
 
@@ -116,21 +128,31 @@ __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(Gemm
     const int l32 = lane % 32, kg = lane / 32;
 
     const int tiles_n = g.N / BLK_N, tiles_m = g.M / BLK_M;
-    int tile_n, tile_m;
-    {
-        const int nwg = gridDim.x, wg = blockIdx.x;
-        const int xcd = wg % 8, idx = wg / 8;
-        const int q = nwg / 8, r = nwg % 8;
-        const int logical = xcd * q + (xcd < r ? xcd : r) + idx;
+    // Tile order: XCD x (workgroups are dealt to XCDs round-robin) owns a contiguous range of the
+    // "logical" tile sequence, which walks column-major groups of g.group tile-rows.
+    const int total = tiles_n * tiles_m;
+    const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
+    const int xq = (PERSIST ? total : (int)gridDim.x) / 8, xr = (PERSIST ? total : (int)gridDim.x) % 8;
+    const int xcd_first = xcd * xq + (xcd < xr ? xcd : xr);
+    auto decode = [&](int logical, int& n_blk, int& m_blk) {
         const int per_group = g.group * tiles_m;
         const int gid = logical / per_group;
         const int first_n = gid * g.group;
         const int gsz = (tiles_n - first_n) < g.group ? (tiles_n - first_n) : g.group;
         const int in_group = logical % per_group;
-        tile_n = first_n + in_group % gsz;
-        tile_m = in_group / gsz;
+        n_blk = (first_n + in_group % gsz) * BLK_N;
+        m_blk = (in_group / gsz) * BLK_M;
+    };
+    int my_tiles = 1, tile_stride = 0;
+    if constexpr (PERSIST) {
+        const int xcd_count = xq + (xcd < xr ? 1 : 0);
+        tile_stride = gridDim.x / 8;
+        my_tiles = slot < xcd_count ? (xcd_count - slot + tile_stride - 1) / tile_stride : 0;
+        if (my_tiles == 0) return;  // uniform for the whole workgroup, before any barrier
     }
-    const int n_blk = tile_n * BLK_N, m_blk = tile_m * BLK_M;
+    int logical = xcd_first + slot;
+    int n_blk, m_blk;
+    decode(logical, n_blk, m_blk);
 
     int k_begin = 0, k_count = g.K;
     if constexpr (SPLIT) {
@@ -138,19 +160,25 @@ __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(Gemm
         k_count = (g.K - k_begin) < g.k_len ? (g.K - k_begin) : g.k_len;
     }
 
-    const int ld_row = tid / 8;
-    const int ld_chunk = (tid & 7) ^ ((ld_row >> 1) & 7);
-    const uint8_t* p_src = g.b + (int64_t)n_blk * g.K + (int64_t)ld_row * g.K + ld_chunk * 16 + k_begin;
+    // global source of every direct-to-LDS copy this lane issues for one K-step
+    const uint8_t* p_src;
     const uint8_t* q_src[Q_ITERS];
+    auto set_sources = [&](int nb, int mb) {
+        const int t_id = PERSIST ? opaque(threadIdx.x) : tid;
+        const int ld_row = t_id / 8;
+        const int ld_chunk = (t_id & 7) ^ ((ld_row >> 1) & 7);
+        p_src = g.b + (int64_t)nb * g.K + (int64_t)ld_row * g.K + ld_chunk * 16 + k_begin;
 #pragma unroll
-    for (int it = 0; it < Q_ITERS; ++it) {
-        const int rho = it * (T / 8) + ld_row;
-        const int w = rho / WT_M, rw = rho % WT_M;
-        const int grow = w * WT_M + NJ * (rw % 32) + rw / 32;
-        q_src[it] = g.a + (int64_t)m_blk * g.K + (int64_t)grow * g.K + ld_chunk * 16 + k_begin;
-    }
-    auto issue_loads = [&](int stage, int k0) {
-        uint8_t* base = lds + stage * STAGE + wave * 1024;
+        for (int it = 0; it < Q_ITERS; ++it) {
+            const int rho = it * (T / 8) + ld_row;
+            const int w = rho / WT_M, rw = rho % WT_M;
+            const int grow = w * WT_M + NJ * (rw % 32) + rw / 32;
+            q_src[it] = g.a + (int64_t)mb * g.K + (int64_t)grow * g.K + ld_chunk * 16 + k_begin;
+        }
+    };
+    set_sources(n_blk, m_blk);
+    auto issue_loads = [&](int stage_ofs, int k0) {
+        uint8_t* base = lds + stage_ofs + wave * 1024;
 #pragma unroll
         for (int it = 0; it < P_ITERS; ++it) {
             const uint8_t* src = p_src + (int64_t)it * (T / 8) * g.K + k0;
@@ -180,17 +208,20 @@ __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(Gemm
     };
 
     v16f acc[NI][NJ];
+    auto clear_acc = [&]() {
 #pragma unroll
-    for (int i = 0; i < NI; ++i)
+        for (int i = 0; i < NI; ++i)
 #pragma unroll
-        for (int j = 0; j < NJ; ++j)
+            for (int j = 0; j < NJ; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    };
+    clear_acc();
 
     const int KT = k_count / kBK;
     issue_loads(0, 0);
     if (KT > 1) {
-        issue_loads(1, kBK);
+        issue_loads(STAGE, kBK);
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LOADS) : "memory");
     } else {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -208,7 +239,7 @@ __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(Gemm
     // following half-step lives in the other LDS stage); REFILL: start the direct-to-LDS copies of the
     // stage after that one into the stage just released.
     auto half_step = [&](auto h_tag, auto next_tag, auto sync_tag, auto refill_tag, const uint8_t* next,
-                         int refill_stage, int refill_k0) {
+                         int refill_ofs, int refill_k0) {
         constexpr int H = decltype(h_tag)::value;
         constexpr bool NEXT = decltype(next_tag)::value;
         constexpr bool SYNC = decltype(sync_tag)::value;
@@ -222,7 +253,7 @@ __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(Gemm
                 if constexpr (SYNC) {
                     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                     __syncthreads();
-                    if constexpr (REFILL) issue_loads(refill_stage, refill_k0);
+                    if constexpr (REFILL) issue_loads(refill_ofs, refill_k0);
                 }
                 if constexpr (NEXT) {
 #pragma unroll
@@ -255,66 +286,113 @@ __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(Gemm
         }
         __builtin_amdgcn_sched_barrier(0);
     };
+
+    // Epilogue.  Accumulator register r of fragment (i, j) is c row 8*(r/4) + 4*kg + r%4 of the
+    // fragment; thanks to the a-tile row permutation the lane's two j values are adjacent columns.
+    auto epilogue = [&](int nb, int mb) {
+        const int e_lane = PERSIST ? opaque(threadIdx.x) % 64 : lane;
+        const int l32 = e_lane % 32, kg = e_lane / 32;
+        const int m_lane = mb + wm * WT_M + NJ * l32;
+        if constexpr (SPLIT) {
+            float* part = g.partial + (int64_t)blockIdx.y * g.N * g.M;
+#pragma unroll
+            for (int i = 0; i < NI; ++i) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int n = nb + wn * WT_N + i * 32 + 8 * (r / 4) + 4 * kg + (r % 4);
+                    PairIo<float>::store(part + (int64_t)n * g.M + m_lane, acc[i][0][r], acc[i][1][r]);
+                }
+            }
+        } else {
+            float scale = g.sa ? *g.sa : 1.f;
+            if (g.sb) scale = scale * *g.sb;
+            OutT* c = reinterpret_cast<OutT*>(g.c);
+            float bias0 = 0.f, bias1 = 0.f;
+            if (g.bias) {
+                bias0 = load_bias(g.bias, g.bias_is_bf16, m_lane);
+                bias1 = load_bias(g.bias, g.bias_is_bf16, m_lane + 1);
+            }
+#pragma unroll
+            for (int i = 0; i < NI; ++i) {
+                // all 16 old values of this fragment row are requested before the first one is used
+                float o0[16], o1[16];
+                if (g.accumulate) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int n = nb + wn * WT_N + i * 32 + 8 * (r / 4) + 4 * kg + (r % 4);
+                        PairIo<OutT>::load(c + (int64_t)n * g.M + m_lane, o0[r], o1[r]);
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int n = nb + wn * WT_N + i * 32 + 8 * (r / 4) + 4 * kg + (r % 4);
+                    OutT* dst = c + (int64_t)n * g.M + m_lane;
+                    float v0 = acc[i][0][r] * scale, v1 = acc[i][1][r] * scale;
+                    if (g.bias) {
+                        v0 = v0 + bias0;
+                        v1 = v1 + bias1;
+                    }
+                    if (g.accumulate) {
+                        v0 = v0 + o0[r];
+                        v1 = v1 + o1[r];
+                    }
+                    PairIo<OutT>::store(dst, v0, v1);
+                }
+            }
+        }
+    };
+
     using std::integral_constant;
     constexpr integral_constant<int, 0> H0{};
     constexpr integral_constant<int, 1> H1{};
     constexpr integral_constant<bool, true> Y{};
     constexpr integral_constant<bool, false> NO{};
-    int kt = 0;
-    for (; kt + 2 < KT; ++kt) {  // steady state: a next stage exists and one more can be fetched
-        half_step(H0, Y, NO, NO, lds + (kt & 1) * STAGE, 0, 0);
-        half_step(H1, Y, Y, Y, lds + ((kt + 1) & 1) * STAGE, kt & 1, (kt + 2) * kBK);
-    }
-    if (kt + 1 < KT) {           // second to last stage: nothing left to fetch
-        half_step(H0, Y, NO, NO, lds + (kt & 1) * STAGE, 0, 0);
-        half_step(H1, Y, Y, NO, lds + ((kt + 1) & 1) * STAGE, 0, 0);
-        ++kt;
-    }
-    half_step(H0, Y, NO, NO, lds + (kt & 1) * STAGE, 0, 0);   // last stage
-    half_step(H1, NO, NO, NO, lds, 0, 0);
-
-    // Epilogue.  Accumulator register r of fragment (i, j) is c row 8*(r/4) + 4*kg + r%4 of the
-    // fragment; thanks to the a-tile row permutation the lane's two j values are adjacent columns.
-    const int m_lane = m_blk + wm * WT_M + NJ * l32;
-    if constexpr (SPLIT) {
-        float* part = g.partial + (int64_t)blockIdx.y * g.N * g.M;
-#pragma unroll
-        for (int i = 0; i < NI; ++i) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int n = n_blk + wn * WT_N + i * 32 + 8 * (r / 4) + 4 * kg + (r % 4);
-                PairIo<float>::store(part + (int64_t)n * g.M + m_lane, acc[i][0][r], acc[i][1][r]);
-            }
+    if constexpr (!PERSIST) {
+        int kt = 0;
+        for (; kt + 2 < KT; ++kt) {  // steady state: a next stage exists and one more can be fetched
+            half_step(H0, Y, NO, NO, lds + (kt & 1) * STAGE, 0, 0);
+            half_step(H1, Y, Y, Y, lds + ((kt + 1) & 1) * STAGE, (kt & 1) * STAGE, (kt + 2) * kBK);
         }
+        if (kt + 1 < KT) {           // second to last stage: nothing left to fetch
+            half_step(H0, Y, NO, NO, lds + (kt & 1) * STAGE, 0, 0);
+            half_step(H1, Y, Y, NO, lds + ((kt + 1) & 1) * STAGE, 0, 0);
+            ++kt;
+        }
+        half_step(H0, Y, NO, NO, lds + (kt & 1) * STAGE, 0, 0);   // last stage
+        half_step(H1, NO, NO, NO, lds, 0, 0);
+        epilogue(n_blk, m_blk);
     } else {
-        float scale = g.sa ? *g.sa : 1.f;
-        if (g.sb) scale = scale * *g.sb;
-        OutT* c = reinterpret_cast<OutT*>(g.c);
-        float bias0 = 0.f, bias1 = 0.f;
-        if (g.bias) {
-            bias0 = load_bias(g.bias, g.bias_is_bf16, m_lane);
-            bias1 = load_bias(g.bias, g.bias_is_bf16, m_lane + 1);
-        }
-#pragma unroll
-        for (int i = 0; i < NI; ++i) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int n = n_blk + wn * WT_N + i * 32 + 8 * (r / 4) + 4 * kg + (r % 4);
-                OutT* dst = c + (int64_t)n * g.M + m_lane;
-                float v0 = acc[i][0][r] * scale, v1 = acc[i][1][r] * scale;
-                if (g.bias) {
-                    v0 = v0 + bias0;
-                    v1 = v1 + bias1;
-                }
-                if (g.accumulate) {
-                    float o0, o1;
-                    PairIo<OutT>::load(dst, o0, o1);
-                    v0 = v0 + o0;
-                    v1 = v1 + o1;
-                }
-                PairIo<OutT>::store(dst, v0, v1);
+        int cur = 0;  // byte offset of the LDS stage the current K-step lives in
+        for (int t = 0; t < my_tiles; ++t) {
+            for (int kt = 0; kt + 2 < KT; ++kt) {
+                half_step(H0, Y, NO, NO, lds + cur, 0, 0);
+                half_step(H1, Y, Y, Y, lds + (STAGE - cur), cur, (kt + 2) * kBK);
+                cur = STAGE - cur;
             }
+            // The copy stream moves on to the next tile (after the last tile it re-reads the first
+            // K-steps of that same tile: harmless, and the loop body stays free of branches).
+            const int cur_n = n_blk, cur_m = m_blk;
+            if (t + 1 < my_tiles) {
+                logical += tile_stride;
+                decode(logical, n_blk, m_blk);
+            }
+            set_sources(n_blk, m_blk);
+            half_step(H0, Y, NO, NO, lds + cur, 0, 0);                      // K-step KT-2
+            half_step(H1, Y, Y, Y, lds + (STAGE - cur), cur, 0);
+            cur = STAGE - cur;
+            half_step(H0, Y, NO, NO, lds + cur, 0, 0);                      // K-step KT-1
+            half_step(H1, NO, Y, Y, lds, cur, kBK);
+            cur = STAGE - cur;
+            epilogue(cur_n, cur_m);
+            clear_acc();
+            // first fragments of the next tile (its first K-step landed before the barrier above); they
+            // are read only now so that the epilogue has the fragment registers to itself
+#pragma unroll
+            for (int i = 0; i < NI; ++i) fa[i] = read_frag(lds + cur + p_frag + i * 32 * kBK, 0);
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) fb[0][j] = read_frag(lds + cur + q_frag + j * 32 * kBK, 0);
         }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the surplus copies of the last tile
     }
 }
 
@@ -354,18 +432,21 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs g, int spli
 
 // ---- host side ------------------------------------------------------------------------------------
 template <int BLK_N, int BLK_M, int WV_N, int WV_M, typename OutT>
-static int launch_pipe(const GemmArgs& g, int splits, hipStream_t stream) {
+static int launch_pipe(const GemmArgs& g, int splits, int persistent_grid, hipStream_t stream) {
     const int tiles = (g.N / BLK_N) * (g.M / BLK_M);
     if (splits > 1) {
-        hipLaunchKernelGGL((gemm_tn_e4m3_pipe_kernel<BLK_N, BLK_M, WV_N, WV_M, OutT, true>),
+        hipLaunchKernelGGL((gemm_tn_e4m3_pipe_kernel<BLK_N, BLK_M, WV_N, WV_M, OutT, true, false>),
                            dim3((unsigned)tiles, (unsigned)splits), dim3(WV_N * WV_M * 64), 0, stream, g);
         LLMQ_HIP_TRY(hipGetLastError());
         const int64_t pairs = (int64_t)g.N * g.M / 2;
         hipLaunchKernelGGL((splitk_reduce_kernel<OutT>), dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, stream,
                            g, splits);
+    } else if (persistent_grid > 0) {
+        hipLaunchKernelGGL((gemm_tn_e4m3_pipe_kernel<BLK_N, BLK_M, WV_N, WV_M, OutT, false, true>),
+                           dim3((unsigned)persistent_grid), dim3(WV_N * WV_M * 64), 0, stream, g);
     } else {
-        hipLaunchKernelGGL((gemm_tn_e4m3_pipe_kernel<BLK_N, BLK_M, WV_N, WV_M, OutT, false>), dim3((unsigned)tiles),
-                           dim3(WV_N * WV_M * 64), 0, stream, g);
+        hipLaunchKernelGGL((gemm_tn_e4m3_pipe_kernel<BLK_N, BLK_M, WV_N, WV_M, OutT, false, false>),
+                           dim3((unsigned)tiles), dim3(WV_N * WV_M * 64), 0, stream, g);
     }
     LLMQ_HIP_TRY(hipGetLastError());
     return LLMQ_OK;
@@ -375,6 +456,7 @@ static int launch_pipe(const GemmArgs& g, int splits, hipStream_t stream) {
 // 4 waves.  splits: forced number of K splits (needs a workspace).
 int g_gemm_tile = 0;
 int g_gemm_splits = 0;
+int g_gemm_persist = -1;  // -1 = automatic, 0 = never, 1 = whenever possible
 
 template <typename OutT>
 static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hipStream_t stream) {
@@ -426,8 +508,13 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
         splits = (g.K + g.k_len - 1) / g.k_len;  // no empty split
         g.partial = reinterpret_cast<float*>(workspace);
     }
-    if (tile == 1) return launch_pipe<256, 256, 2, 4, OutT>(g, splits, stream);
-    return launch_pipe<128, 128, 2, 2, OutT>(g, splits, stream);
+    // Persistent walk (one workgroup per compute unit) for the large tile when there is more than one
+    // round of tiles; its cross-tile copy stream needs at least two K-steps.
+    int persistent_grid = 0;
+    const bool can_persist = tile == 1 && splits == 1 && g.K >= 2 * kBK && cus % 8 == 0;
+    if (can_persist && (g_gemm_persist == 1 || (g_gemm_persist < 0 && tiles > cus))) persistent_grid = cus;
+    if (tile == 1) return launch_pipe<256, 256, 2, 4, OutT>(g, splits, persistent_grid, stream);
+    return launch_pipe<128, 128, 2, 2, OutT>(g, splits, 0, stream);
 }
 
 }  // namespace llmq
@@ -452,3 +539,4 @@ extern "C" void llmq_debug_set_gemm_variant(int tile, int splits) {
     llmq::g_gemm_tile = tile;
     llmq::g_gemm_splits = splits;
 }
+extern "C" void llmq_debug_set_gemm_persist(int v) { llmq::g_gemm_persist = v; }

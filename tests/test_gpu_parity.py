@@ -141,12 +141,14 @@ def test_transpose_bit_exact(K, shape):
 
 # --------------------------------------------------------------------------------------------- GEMM
 def set_variant(v):
-    """v = (tile, splits): tile 0 = automatic, 1 = 256 x 256, 2 = 128 x 128; splits 0 = automatic."""
+    """v = (tile, splits[, persistent]): tile 0 = automatic, 1 = 256 x 256, 2 = 128 x 128; splits 0 =
+    automatic; persistent -1 = automatic, 0 = one workgroup per tile, 1 = persistent tile walk."""
     from llmq_amd import capi
     capi.lib.llmq_debug_set_gemm_variant(v[0], v[1])
+    capi.lib.llmq_debug_set_gemm_persist(v[2] if len(v) > 2 else -1)
 
 
-VARIANTS = [(0, 0), (1, 0), (2, 0), (1, 2), (2, 2), (2, 3)]
+VARIANTS = [(0, 0), (1, 0, 0), (1, 1, 1), (2, 0), (1, 2), (2, 2), (2, 3)]
 _WORKSPACE = {}
 
 
@@ -161,6 +163,8 @@ def skip_unsupported(variant, M, N, Kd):
         pytest.skip("the 256 x 256 tile needs multiples of 256")
     if variant[1] > Kd // 128:
         pytest.skip("more splits than K-steps")
+    if len(variant) > 2 and variant[2] == 1 and Kd < 256:
+        pytest.skip("the persistent walk needs two K-steps")
 
 
 def run_gemm(K, a, b, M, N, Kd, sa, sb, bias_bits=None, old=None, out_f32=False):
@@ -232,6 +236,35 @@ def test_gemm_random_codes_within_tolerance(K, O, variant, out_f32):
         got2 = run_gemm(K, a, b, M, N, Kd, sa, sb, bias, oldp, out_f32=out_f32)
         extra = O.bf16_to_f32(bias).astype(np.float64)[None, :] + old.astype(np.float64)
         gemm_check(got2.float().cpu().numpy(), exact, sumabs, scale, not out_f32, extra=extra)
+    finally:
+        set_variant((0, 0))
+
+
+@pytest.mark.parametrize("mnk", [(4352, 4352, 384), (4608, 4096, 256), (8192, 4864, 512)])
+def test_gemm_persistent_tile_walk(K, O, mnk):
+    """More tiles than compute units: workgroups walk several tiles each and the operand stream crosses
+    tile boundaries (odd and even numbers of K-steps flip the LDS stage parity differently).  Integer
+    operands -> bit-exact against the oracle, with bias and accumulation, bf16 and fp32 outputs."""
+    M, N, Kd = mnk
+    a, _ = O.fill_int_e4m3(M * Kd, 4242, 0)
+    b, _ = O.fill_int_e4m3(N * Kd, 4242, 1)
+    a, b = a.reshape(M, Kd), b.reshape(N, Kd)
+    s = float(np.sqrt(np.float32(4.0 / Kd)))
+    _, biasv = O.fill_int_e4m3(M, 4242, 2)
+    _, oldv = O.fill_int_e4m3(N * M, 4242, 3)
+    bias = O.f32_to_bf16(biasv.astype(np.float32))
+    old = O.f32_to_bf16(oldv.astype(np.float32)).reshape(N, M)
+    set_variant((1, 1, 1))
+    try:
+        want = O.gemm_tn(a, b, sa=s, sb=s, mt=True)
+        got = run_gemm(K, a, b, M, N, Kd, s, s)
+        assert np.array_equal(host_bits(got), want)
+        want = O.gemm_tn(a, b, sa=s, sb=s, bias=bias, c_old=old, mt=True)
+        got = run_gemm(K, a, b, M, N, Kd, s, s, bias, old)
+        assert np.array_equal(host_bits(got), want)
+        want32 = O.gemm_tn(a, b, sa=s, sb=s, out_f32=True, mt=True)
+        got32 = run_gemm(K, a, b, M, N, Kd, s, s, out_f32=True)
+        assert np.array_equal(got32.cpu().numpy(), want32)
     finally:
         set_variant((0, 0))
 
