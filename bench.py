@@ -39,6 +39,7 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay of the step")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain 1 GiB copy kernel (reference point for hardware traffic counters)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="rough budget of the CPU baseline sample")
@@ -144,6 +145,21 @@ def main():
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     record[0] = False
+
+    # The same step recorded once into a HIP graph and replayed (the reference replays its transformer
+    # block from a graph as well, src/models/llama_model.cpp:49-71): removes the launch gaps.
+    graph_ms = None
+    if not args.no_graph:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        graph.replay()
+        torch.cuda.synchronize()
+        g0 = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        graph_ms = (time.perf_counter() - g0) * 1e3 / args.steps
     if args.calibrate_copy:
         src = torch.randint(0, 255, (1 << 30,), dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
@@ -202,6 +218,8 @@ def main():
         "quantize": {"bound": "hbm", "kernels": "abs_max + quantize_with_abs_max (5 bytes/element)",
                      "achieved": aq_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": aq_gbs / HBM_PEAK_GBS,
                      "per_kernel": per_kernel},
+        "hip_graph_replay": None if graph_ms is None else {"ms_per_step": graph_ms,
+                                                           "value": gemm_flop / (graph_ms * 1e-3) / 1e12},
         "library": capi.version(),
     }
 

@@ -203,3 +203,59 @@ def test_config5_outlier_stress(K, O, name, C, OC):
     assert zero_frac > 1e-3, "expected a visible underflow-to-zero fraction"
     assert sub_frac > 0.05, "expected many subnormal codes"
     run_linear_fwd_bwd(K, O, BT, C, OC, x, w, dy.to(torch.bfloat16), seed=500 + OC % 100)
+
+
+def test_hip_graph_replay_matches_eager(K, O):
+    """The whole call sequence of one linear layer (abs-max, quantize, forward, backward with split-K
+    wgrad) recorded into a HIP graph, as the reference records a transformer block
+    (src/models/llama_model.cpp:49-71): every replay, with new inputs and eager work in between, must
+    reproduce the eager result bit for bit."""
+    BT, C, OC = 2048, 896, 1152
+    x = torch.empty((BT, C), dtype=torch.bfloat16, device="cuda")
+    w = torch.empty((OC, C), dtype=torch.bfloat16, device="cuda")
+    dy = torch.empty((BT, OC), dtype=torch.bfloat16, device="cuda")
+    inp, wq, dout = QT(x), QT(w), QT(dy)
+    y = torch.empty((BT, OC), dtype=torch.bfloat16, device="cuda")
+    dinp = torch.empty((BT, C), dtype=torch.bfloat16, device="cuda")
+    dweight = torch.empty((OC, C), dtype=torch.float32, device="cuda")
+    workspace()                                    # allocate outside the capture
+
+    def fill(seed):
+        x.copy_(dev_bf16(O.fill_normal_bf16(BT * C, seed, 1).reshape(BT, C)))
+        w.copy_(dev_bf16(O.fill_normal_bf16(OC * C, seed, 2, 0.0, 0.02).reshape(OC, C)))
+        dy.copy_(dev_bf16(O.fill_normal_bf16(BT * OC, seed, 3, 0.0, 1e-3).reshape(BT, OC)))
+
+    def sequence():
+        K.abs_max(inp.abs_max, inp.value)
+        K.abs_max(wq.abs_max, wq.value)
+        K.abs_max(dout.abs_max, dout.value)
+        K.quantize_with_abs_max(wq.quant, wq.scale, wq.value, wq.abs_max)
+        forward_qmm(K, y, inp, wq.quant, wq.scale, BT, C, OC)
+        backward_qmm(K, dinp, dweight, dout, inp, wq.quant, wq.scale, BT, C, OC, reuse_inp=False)
+
+    def snapshot():
+        torch.cuda.synchronize()
+        return [t.clone() for t in (inp.stats, wq.stats, dout.stats, inp.quant.view(torch.uint8), y, dinp, dweight)]
+
+    fill(50)
+    sequence()                                     # warm-up (also creates the transposed temporaries' pool)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        sequence()
+        with torch.cuda.graph(graph, stream=side):
+            sequence()
+    torch.cuda.current_stream().wait_stream(side)
+    for seed in (51, 52, 53):
+        fill(seed)
+        sequence()
+        want = snapshot()
+        for t in (y, dinp, dweight):
+            t.fill_(float("nan"))
+        inp.stats.zero_()
+        graph.replay()
+        got = snapshot()
+        for a, b in zip(want, got):
+            assert torch.equal(a.view(torch.uint8) if a.dtype != torch.uint8 else a,
+                               b.view(torch.uint8) if b.dtype != torch.uint8 else b), "replay for seed %d differs" % seed
