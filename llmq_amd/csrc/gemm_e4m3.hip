@@ -63,27 +63,30 @@ struct GemmArgs {
     int k_len;       // split-K only: K elements per split (multiple of 128)
 };
 
-// Output pair store: y = v (+ old value when accumulating), one rounding to the output type.
+#define LLMQ_GLOBAL __attribute__((address_space(1)))
+
+// Pair of adjacent outputs in global memory: load as fp32, store with one rounding to the output type.
 template <typename OutT> struct PairIo;
 template <> struct PairIo<uint16_t> {
-    static __device__ __forceinline__ void load(const uint16_t* p, float& v0, float& v1) {
-        const uint32_t old = *reinterpret_cast<const uint32_t*>(p);
+    static __device__ __forceinline__ void load(const LLMQ_GLOBAL void* p, float& v0, float& v1) {
+        const uint32_t old = *(const LLMQ_GLOBAL uint32_t*)p;
         v0 = __uint_as_float(old << 16);
         v1 = __uint_as_float(old & 0xFFFF0000u);
     }
-    static __device__ __forceinline__ void store(uint16_t* p, float v0, float v1) {
+    static __device__ __forceinline__ void store(LLMQ_GLOBAL void* p, float v0, float v1) {
         const f32x2_t v = {v0, v1};
-        *reinterpret_cast<bf16x2_t*>(p) = __builtin_convertvector(v, bf16x2_t);  // v_cvt_pk_bf16_f32, RNE
+        *(LLMQ_GLOBAL bf16x2_t*)p = __builtin_convertvector(v, bf16x2_t);  // v_cvt_pk_bf16_f32, RNE
     }
 };
 template <> struct PairIo<float> {
-    static __device__ __forceinline__ void load(const float* p, float& v0, float& v1) {
-        const float2 old = *reinterpret_cast<const float2*>(p);
-        v0 = old.x;
-        v1 = old.y;
+    static __device__ __forceinline__ void load(const LLMQ_GLOBAL void* p, float& v0, float& v1) {
+        const f32x2_t old = *(const LLMQ_GLOBAL f32x2_t*)p;
+        v0 = old[0];
+        v1 = old[1];
     }
-    static __device__ __forceinline__ void store(float* p, float v0, float v1) {
-        *reinterpret_cast<float2*>(p) = make_float2(v0, v1);
+    static __device__ __forceinline__ void store(LLMQ_GLOBAL void* p, float v0, float v1) {
+        const f32x2_t v = {v0, v1};
+        *(LLMQ_GLOBAL f32x2_t*)p = v;
     }
 };
 
@@ -97,6 +100,13 @@ __device__ __forceinline__ float load_bias(const void* bias, int is_bf16, int m)
 __device__ __forceinline__ int opaque(int x) {
     asm volatile("" : "+v"(x));
     return x;
+}
+
+// Pins a wave-uniform pointer in scalar registers, so that "pointer + 32-bit lane offset" selects the
+// scalar-base addressing form instead of a 64-bit vector add per access.
+__device__ __forceinline__ LLMQ_GLOBAL char* scalar_ptr(LLMQ_GLOBAL char* p) {
+    asm volatile("" : "+s"(p));
+    return p;
 }
 
 template <int MASK, int N>
@@ -119,7 +129,9 @@ __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(Gemm
     static_assert(T / 8 % 32 == 0 && NJ == 2 && NI >= 2, "tile configuration");
     static_assert(!(SPLIT && PERSIST), "split-K tiles are not walked persistently");
 
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * STAGE];
+    // two operand stages + 4 KiB per wave for the staged bf16 epilogue
+    constexpr int EPI_BYTES = 4096;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * STAGE + WV_N * WV_M * EPI_BYTES];
 
     const int tid = threadIdx.x;
     const int lane = tid % 64;
@@ -289,55 +301,120 @@ __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(Gemm
 
     // Epilogue.  Accumulator register r of fragment (i, j) is c row 8*(r/4) + 4*kg + r%4 of the
     // fragment; thanks to the a-tile row permutation the lane's two j values are adjacent columns.
-    auto epilogue = [&](int nb, int mb) {
+    // Addresses are "wave-uniform row pointer + one 32-bit lane offset", and the bias / accumulate
+    // cases are separate straight-line instances, so the common case is 2 multiplies, 1 convert and
+    // 1 store per output pair.
+    auto epilogue_rows = [&](auto bias_tag, auto acc_tag, auto* out, float scale, int nb, int mb) {
+        constexpr bool BIAS = decltype(bias_tag)::value;
+        constexpr bool ACC = decltype(acc_tag)::value;
+        using T = std::remove_pointer_t<decltype(out)>;
         const int e_lane = PERSIST ? opaque(threadIdx.x) % 64 : lane;
-        const int l32 = e_lane % 32, kg = e_lane / 32;
-        const int m_lane = mb + wm * WT_M + NJ * l32;
-        if constexpr (SPLIT) {
-            float* part = g.partial + (int64_t)blockIdx.y * g.N * g.M;
+        const int el32 = e_lane % 32, ekg = e_lane / 32;
+        const int m_lane = mb + wm * WT_M + NJ * el32;
+        // byte offset of the lane inside a group of rows; below 2^32 (4 rows of at most 2^27 elements)
+        const uint32_t lane_bytes = ((uint32_t)(4 * ekg) * (uint32_t)g.M + (uint32_t)m_lane) * (uint32_t)sizeof(T);
+        float bias0 = 0.f, bias1 = 0.f;
+        if constexpr (BIAS) {
+            bias0 = load_bias(g.bias, g.bias_is_bf16, m_lane);
+            bias1 = load_bias(g.bias, g.bias_is_bf16, m_lane + 1);
+        }
+        const int row0 = nb + wn * WT_N;  // wave-uniform
 #pragma unroll
-            for (int i = 0; i < NI; ++i) {
+        for (int i = 0; i < NI; ++i) {
+            float o0[16], o1[16];
+            if constexpr (ACC) {  // all 16 old values of this fragment row are requested before the first use
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    const int n = nb + wn * WT_N + i * 32 + 8 * (r / 4) + 4 * kg + (r % 4);
-                    PairIo<float>::store(part + (int64_t)n * g.M + m_lane, acc[i][0][r], acc[i][1][r]);
+                    LLMQ_GLOBAL char* row = scalar_ptr((LLMQ_GLOBAL char*)(out + (int64_t)(row0 + i * 32 + 8 * (r / 4) + (r % 4)) * g.M));
+                    PairIo<T>::load(row + lane_bytes, o0[r], o1[r]);
                 }
             }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                LLMQ_GLOBAL char* row = scalar_ptr((LLMQ_GLOBAL char*)(out + (int64_t)(row0 + i * 32 + 8 * (r / 4) + (r % 4)) * g.M));
+                float v0 = acc[i][0][r] * scale, v1 = acc[i][1][r] * scale;
+                if constexpr (BIAS) {
+                    v0 = v0 + bias0;
+                    v1 = v1 + bias1;
+                }
+                if constexpr (ACC) {
+                    v0 = v0 + o0[r];
+                    v1 = v1 + o1[r];
+                }
+                PairIo<T>::store(row + lane_bytes, v0, v1);
+            }
+        }
+    };
+    // bf16 output without accumulation: every 32 x 64 fragment row of the wave tile goes through a
+    // private 4 KiB LDS tile (row stride 128 B; rows 4 apart swap places pairwise so that the two lane
+    // halves of a write hit different bank halves) and leaves as 16-byte pieces, eight lanes per 128-byte
+    // row segment: 16 store instructions of 1 KiB per wave instead of 64 of 256 B.
+    auto epilogue_staged = [&](auto bias_tag, uint16_t* out, float scale, int nb, int mb) {
+        constexpr bool BIAS = decltype(bias_tag)::value;
+        const int e_lane = PERSIST ? opaque(threadIdx.x) % 64 : lane;
+        const int el32 = e_lane % 32, ekg = e_lane / 32;
+        const int m_wave = mb + wm * WT_M;
+        float bias0 = 0.f, bias1 = 0.f;
+        if constexpr (BIAS) {
+            bias0 = load_bias(g.bias, g.bias_is_bf16, m_wave + NJ * el32);
+            bias1 = load_bias(g.bias, g.bias_is_bf16, m_wave + NJ * el32 + 1);
+        }
+        uint8_t* tile = lds + 2 * STAGE + wave * EPI_BYTES;
+        // register r of a fragment is tile row 8*(r/4) + 4*kg + r%4, stored at row position (row ^ kg)
+        uint8_t* w_even = tile + (4 * ekg) * 128 + el32 * 4 + ekg * 128;   // r % 4 even: position r%4 + kg
+        uint8_t* w_odd = tile + (4 * ekg) * 128 + el32 * 4 - ekg * 128;    // r % 4 odd:  position r%4 - kg
+        const int r_row = e_lane / 8, r_chunk = e_lane % 8;               // read side: position, 16-byte chunk
+        const uint8_t* r_src = tile + r_row * 128 + r_chunk * 16;
+        const uint32_t lane_bytes =
+            ((uint32_t)(r_row ^ ekg) * (uint32_t)g.M + (uint32_t)(m_wave + r_chunk * 8)) * 2u;  // row = position ^ kg
+        const int row0 = nb + wn * WT_N;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float v0 = acc[i][0][r] * scale, v1 = acc[i][1][r] * scale;
+                if constexpr (BIAS) {
+                    v0 = v0 + bias0;
+                    v1 = v1 + bias1;
+                }
+                const f32x2_t v = {v0, v1};
+                uint8_t* dst = ((r % 4) % 2 == 0 ? w_even : w_odd) + (8 * (r / 4) + (r % 4)) * 128;
+                *reinterpret_cast<bf16x2_t*>(dst) = __builtin_convertvector(v, bf16x2_t);
+            }
+            v4i piece[4];
+#pragma unroll
+            for (int p = 0; p < 4; ++p) piece[p] = *reinterpret_cast<const v4i*>(r_src + p * 8 * 128);
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                LLMQ_GLOBAL char* row = scalar_ptr((LLMQ_GLOBAL char*)(out + (int64_t)(row0 + i * 32 + p * 8) * g.M));
+                *(LLMQ_GLOBAL v4i*)(row + lane_bytes) = piece[p];
+            }
+        }
+    };
+    auto epilogue = [&](int nb, int mb) {
+        constexpr std::true_type yes{};
+        constexpr std::false_type no{};
+        if constexpr (!SPLIT && std::is_same_v<OutT, uint16_t>) {
+            if (!g.accumulate) {
+                float scale = g.sa ? *g.sa : 1.f;
+                if (g.sb) scale = scale * *g.sb;
+                if (g.bias) epilogue_staged(yes, reinterpret_cast<uint16_t*>(g.c), scale, nb, mb);
+                else epilogue_staged(no, reinterpret_cast<uint16_t*>(g.c), scale, nb, mb);
+                return;
+            }
+        }
+        if constexpr (SPLIT) {
+            epilogue_rows(no, no, g.partial + (int64_t)blockIdx.y * g.N * g.M, 1.f, nb, mb);
         } else {
             float scale = g.sa ? *g.sa : 1.f;
             if (g.sb) scale = scale * *g.sb;
             OutT* c = reinterpret_cast<OutT*>(g.c);
-            float bias0 = 0.f, bias1 = 0.f;
             if (g.bias) {
-                bias0 = load_bias(g.bias, g.bias_is_bf16, m_lane);
-                bias1 = load_bias(g.bias, g.bias_is_bf16, m_lane + 1);
-            }
-#pragma unroll
-            for (int i = 0; i < NI; ++i) {
-                // all 16 old values of this fragment row are requested before the first one is used
-                float o0[16], o1[16];
-                if (g.accumulate) {
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int n = nb + wn * WT_N + i * 32 + 8 * (r / 4) + 4 * kg + (r % 4);
-                        PairIo<OutT>::load(c + (int64_t)n * g.M + m_lane, o0[r], o1[r]);
-                    }
-                }
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int n = nb + wn * WT_N + i * 32 + 8 * (r / 4) + 4 * kg + (r % 4);
-                    OutT* dst = c + (int64_t)n * g.M + m_lane;
-                    float v0 = acc[i][0][r] * scale, v1 = acc[i][1][r] * scale;
-                    if (g.bias) {
-                        v0 = v0 + bias0;
-                        v1 = v1 + bias1;
-                    }
-                    if (g.accumulate) {
-                        v0 = v0 + o0[r];
-                        v1 = v1 + o1[r];
-                    }
-                    PairIo<OutT>::store(dst, v0, v1);
-                }
+                if (g.accumulate) epilogue_rows(yes, yes, c, scale, nb, mb);
+                else epilogue_rows(yes, no, c, scale, nb, mb);
+            } else {
+                if (g.accumulate) epilogue_rows(no, yes, c, scale, nb, mb);
+                else epilogue_rows(no, no, c, scale, nb, mb);
             }
         }
     };
@@ -407,9 +484,10 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs g, int spli
     const int64_t slice = (int64_t)g.N * g.M;
     float v0 = 0.f, v1 = 0.f;
     for (int s = 0; s < splits; ++s) {
-        const float2 t = *reinterpret_cast<const float2*>(g.partial + s * slice + e);
-        v0 = v0 + t.x;
-        v1 = v1 + t.y;
+        float t0, t1;
+        PairIo<float>::load((const LLMQ_GLOBAL float*)(g.partial + s * slice + e), t0, t1);
+        v0 = v0 + t0;
+        v1 = v1 + t1;
     }
     float scale = g.sa ? *g.sa : 1.f;
     if (g.sb) scale = scale * *g.sb;
@@ -423,11 +501,11 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs g, int spli
     OutT* dst = reinterpret_cast<OutT*>(g.c) + e;
     if (g.accumulate) {
         float o0, o1;
-        PairIo<OutT>::load(dst, o0, o1);
+        PairIo<OutT>::load((const LLMQ_GLOBAL OutT*)dst, o0, o1);
         v0 = v0 + o0;
         v1 = v1 + o1;
     }
-    PairIo<OutT>::store(dst, v0, v1);
+    PairIo<OutT>::store((LLMQ_GLOBAL OutT*)dst, v0, v1);
 }
 
 // ---- host side ------------------------------------------------------------------------------------
