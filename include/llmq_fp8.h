@@ -113,6 +113,21 @@ int llmq_gemm_tn_e4m3_f32(float* c, const uint8_t* a, const uint8_t* b, const vo
                           void* workspace_or_null, size_t workspace_bytes, int M, int N, int K, int accumulate,
                           void* stream);
 
+/*
+ * Mixed-format variants for the e5m2 gradient dtype: a is e4m3 (weights / activations), b is e5m2 (the
+ * quantized output gradient); everything else as above.
+ * Replaces: matmul(nv_bfloat16* c, const __nv_fp8_e4m3* a, const __nv_fp8_e5m2* b, const nv_bfloat16* bias, ...)
+ *           src/kernels/kernels.h:92-94, src/kernels/matmul.cpp:222-226, and the fp32-output declaration
+ *           src/kernels/kernels.h:80-82.
+ */
+int llmq_gemm_tn_e4m3_e5m2_bf16(uint16_t* c, const uint8_t* a, const uint8_t* b_e5m2, const uint16_t* bias_or_null,
+                                const float* sa_or_null, const float* sb_or_null, void* workspace_or_null,
+                                size_t workspace_bytes, int M, int N, int K, int accumulate, void* stream);
+int llmq_gemm_tn_e4m3_e5m2_f32(float* c, const uint8_t* a, const uint8_t* b_e5m2, const void* bias_or_null,
+                               int bias_is_bf16, const float* sa_or_null, const float* sb_or_null,
+                               void* workspace_or_null, size_t workspace_bytes, int M, int N, int K, int accumulate,
+                               void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -234,12 +234,41 @@ inline void matmul(float* c, const __hip_fp8_e4m3* a, const __hip_fp8_e4m3* b, c
     llmq_detail::check(llmq_gemm_tn_e4m3_f32(c, llmq_detail::u8(a), llmq_detail::u8(b), bias, 1, scale_a, scale_b,
                                              workspace, workspace_size, M, N, K, accumulate, stream));
 }
+// e4m3 x e5m2 (gradient dtype option; reference: src/kernels/kernels.h:80-82, 92-94)
+inline void matmul(__hip_bfloat16* c, const __hip_fp8_e4m3* a, const __hip_fp8_e5m2* b, const __hip_bfloat16* bias,
+                   const float* scale_a, const float* scale_b, llmqBlasHandle_t, std::byte* workspace,
+                   std::size_t workspace_size, int M, int N, int K, EMMTranspose mode, bool accumulate,
+                   hipStream_t stream, EMatmulBackend = EMatmulBackend::Custom) {
+    llmq_detail::require_tn(mode);
+    llmq_detail::check(llmq_gemm_tn_e4m3_e5m2_bf16(llmq_detail::u16(c), llmq_detail::u8(a), llmq_detail::u8(b),
+                                                   llmq_detail::u16(bias), scale_a, scale_b, workspace, workspace_size,
+                                                   M, N, K, accumulate, stream));
+}
+inline void matmul(float* c, const __hip_fp8_e4m3* a, const __hip_fp8_e5m2* b, const __hip_bfloat16* bias,
+                   const float* scale_a, const float* scale_b, llmqBlasHandle_t, std::byte* workspace,
+                   std::size_t workspace_size, int M, int N, int K, EMMTranspose mode, bool accumulate,
+                   hipStream_t stream, EMatmulBackend = EMatmulBackend::Custom) {
+    llmq_detail::require_tn(mode);
+    llmq_detail::check(llmq_gemm_tn_e4m3_e5m2_f32(c, llmq_detail::u8(a), llmq_detail::u8(b), bias, 1, scale_a, scale_b,
+                                                  workspace, workspace_size, M, N, K, accumulate, stream));
+}
 inline void matmul(Tensor& c, const Tensor& a, const Tensor& b, const Tensor& bias, const float* scale_a,
                    const float* scale_b, llmqBlasHandle_t handle, Tensor& workspace, int M, int N, int K,
                    EMMTranspose mode, bool accumulate, hipStream_t stream,
                    EMatmulBackend backend = EMatmulBackend::Custom) {
     std::byte* ws = workspace.Data;
     const std::size_t ws_size = workspace.empty() ? 0 : workspace.bytes();
+    if (a.DType == ETensorDType::FP8_E4M3 && b.DType == ETensorDType::FP8_E5M2) {
+        if (c.DType == ETensorDType::BF16)
+            matmul(c.get<__hip_bfloat16>(), a.get<__hip_fp8_e4m3>(), b.get<__hip_fp8_e5m2>(),
+                   bias.get_optional<__hip_bfloat16>(), scale_a, scale_b, handle, ws, ws_size, M, N, K, mode, accumulate,
+                   stream, backend);
+        else if (c.DType == ETensorDType::FP32)
+            matmul(c.get<float>(), a.get<__hip_fp8_e4m3>(), b.get<__hip_fp8_e5m2>(), bias.get_optional<__hip_bfloat16>(),
+                   scale_a, scale_b, handle, ws, ws_size, M, N, K, mode, accumulate, stream, backend);
+        else llmq_detail::unsupported(__func__, c, a, b, bias, workspace);
+        return;
+    }
     if (a.DType != ETensorDType::FP8_E4M3 || b.DType != ETensorDType::FP8_E4M3)
         llmq_detail::unsupported(__func__, c, a, b, bias, workspace);
     if (c.DType == ETensorDType::FP32) {

@@ -18,7 +18,7 @@ EXPORTS = [
     "llmq_last_error", "llmq_version", "llmq_target_arch",
     "llmq_abs_max_bf16", "llmq_abs_max_f32",
     "llmq_quantize_e4m3_bf16", "llmq_quantize_e5m2_bf16", "llmq_quantize_transpose_e4m3_bf16",
-    "llmq_transpose_u8", "llmq_gemm_tn_e4m3_bf16", "llmq_gemm_tn_e4m3_f32",
+    "llmq_transpose_u8", "llmq_gemm_tn_e4m3_bf16", "llmq_gemm_tn_e4m3_f32", "llmq_gemm_tn_e4m3_e5m2_bf16", "llmq_gemm_tn_e4m3_e5m2_f32",
 ]
 
 if not os.path.exists(LIB_PATH):
@@ -38,6 +38,8 @@ lib.llmq_quantize_transpose_e4m3_bf16.argtypes = [_vp, _vp, _vp, _vp, _int, _int
 lib.llmq_transpose_u8.argtypes = [_vp, _vp, _int, _int, _vp]
 lib.llmq_gemm_tn_e4m3_bf16.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, C.c_size_t, _int, _int, _int, _int, _vp]
 lib.llmq_gemm_tn_e4m3_f32.argtypes = [_vp, _vp, _vp, _vp, _int, _vp, _vp, _vp, C.c_size_t, _int, _int, _int, _int, _vp]
+lib.llmq_gemm_tn_e4m3_e5m2_bf16.argtypes = lib.llmq_gemm_tn_e4m3_bf16.argtypes
+lib.llmq_gemm_tn_e4m3_e5m2_f32.argtypes = lib.llmq_gemm_tn_e4m3_f32.argtypes
 lib.llmq_debug_set_gemm_variant.argtypes = [_int, _int]
 lib.llmq_debug_set_gemm_variant.restype = None
 lib.llmq_debug_set_gemm_persist.argtypes = [_int]

@@ -115,11 +115,13 @@ __device__ __forceinline__ void sched_group() {
 }
 
 // SPLIT: blockIdx.y selects a K range of g.k_len elements and the raw accumulators go to g.partial.
+// B_FMT: fp8 format of the b operand (0 = e4m3, 1 = e5m2, the reference's gradient dtype option); b rows are
+// the first operand of the matrix instruction, whose format field takes this value directly.
 // PERSIST: the grid has one workgroup per compute unit and every workgroup walks a list of tiles.  The
 // operand stream then runs across tile boundaries: the copies of the next tile's first two K-steps are
 // issued during the last two K-steps of the current tile, so the epilogue of a tile overlaps with the
 // fetch of the next one and no pipeline fill or workgroup launch sits between tiles.  Needs K >= 256.
-template <int BLK_N, int BLK_M, int WV_N, int WV_M, typename OutT, bool SPLIT, bool PERSIST>
+template <int BLK_N, int BLK_M, int WV_N, int WV_M, typename OutT, bool SPLIT, bool PERSIST, int B_FMT>
 __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(GemmArgs g) {
     constexpr int T = WV_N * WV_M * 64;
     constexpr int WT_N = BLK_N / WV_N, WT_M = BLK_M / WV_M;
@@ -260,7 +262,7 @@ __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(Gemm
         for (int i = 0; i < NI; ++i) {
 #pragma unroll
             for (int j = 0; j < NJ; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[H][j], acc[i][j], 0, 0, 0, 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[H][j], acc[i][j], B_FMT, 0, 0, 0, 0, 0);
             if (i == 0) {
                 if constexpr (SYNC) {
                     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -509,21 +511,21 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs g, int spli
 }
 
 // ---- host side ------------------------------------------------------------------------------------
-template <int BLK_N, int BLK_M, int WV_N, int WV_M, typename OutT>
+template <int BLK_N, int BLK_M, int WV_N, int WV_M, typename OutT, int B_FMT>
 static int launch_pipe(const GemmArgs& g, int splits, int persistent_grid, hipStream_t stream) {
     const int tiles = (g.N / BLK_N) * (g.M / BLK_M);
     if (splits > 1) {
-        hipLaunchKernelGGL((gemm_tn_e4m3_pipe_kernel<BLK_N, BLK_M, WV_N, WV_M, OutT, true, false>),
+        hipLaunchKernelGGL((gemm_tn_e4m3_pipe_kernel<BLK_N, BLK_M, WV_N, WV_M, OutT, true, false, B_FMT>),
                            dim3((unsigned)tiles, (unsigned)splits), dim3(WV_N * WV_M * 64), 0, stream, g);
         LLMQ_HIP_TRY(hipGetLastError());
         const int64_t pairs = (int64_t)g.N * g.M / 2;
         hipLaunchKernelGGL((splitk_reduce_kernel<OutT>), dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, stream,
                            g, splits);
     } else if (persistent_grid > 0) {
-        hipLaunchKernelGGL((gemm_tn_e4m3_pipe_kernel<BLK_N, BLK_M, WV_N, WV_M, OutT, false, true>),
+        hipLaunchKernelGGL((gemm_tn_e4m3_pipe_kernel<BLK_N, BLK_M, WV_N, WV_M, OutT, false, true, B_FMT>),
                            dim3((unsigned)persistent_grid), dim3(WV_N * WV_M * 64), 0, stream, g);
     } else {
-        hipLaunchKernelGGL((gemm_tn_e4m3_pipe_kernel<BLK_N, BLK_M, WV_N, WV_M, OutT, false, false>),
+        hipLaunchKernelGGL((gemm_tn_e4m3_pipe_kernel<BLK_N, BLK_M, WV_N, WV_M, OutT, false, false, B_FMT>),
                            dim3((unsigned)tiles), dim3(WV_N * WV_M * 64), 0, stream, g);
     }
     LLMQ_HIP_TRY(hipGetLastError());
@@ -536,7 +538,7 @@ int g_gemm_tile = 0;
 int g_gemm_splits = 0;
 int g_gemm_persist = -1;  // -1 = automatic, 0 = never, 1 = whenever possible
 
-template <typename OutT>
+template <typename OutT, int B_FMT>
 static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     LLMQ_REQUIRE(g.M > 0 && g.N > 0 && g.K > 0, "matmul: M, N, K must be positive (got %d, %d, %d)", g.M, g.N, g.K);
     LLMQ_REQUIRE(g.M % 128 == 0 && g.N % 128 == 0 && g.K % 128 == 0,
@@ -591,8 +593,8 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
     int persistent_grid = 0;
     const bool can_persist = tile == 1 && splits == 1 && g.K >= 2 * kBK && cus % 8 == 0;
     if (can_persist && (g_gemm_persist == 1 || (g_gemm_persist < 0 && tiles > cus))) persistent_grid = cus;
-    if (tile == 1) return launch_pipe<256, 256, 2, 4, OutT>(g, splits, persistent_grid, stream);
-    return launch_pipe<128, 128, 2, 2, OutT>(g, splits, 0, stream);
+    if (tile == 1) return launch_pipe<256, 256, 2, 4, OutT, B_FMT>(g, splits, persistent_grid, stream);
+    return launch_pipe<128, 128, 2, 2, OutT, B_FMT>(g, splits, 0, stream);
 }
 
 }  // namespace llmq
@@ -601,7 +603,7 @@ extern "C" int llmq_gemm_tn_e4m3_bf16(uint16_t* c, const uint8_t* a, const uint8
                                       const float* sa_or_null, const float* sb_or_null, void* workspace_or_null,
                                       size_t workspace_bytes, int M, int N, int K, int accumulate, void* stream) {
     llmq::GemmArgs g{c, a, b, bias_or_null, sa_or_null, sb_or_null, M, N, K, 1, accumulate, 8, nullptr, 0};
-    return llmq::gemm_dispatch<uint16_t>(g, workspace_or_null, workspace_bytes, static_cast<hipStream_t>(stream));
+    return llmq::gemm_dispatch<uint16_t, 0>(g, workspace_or_null, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int llmq_gemm_tn_e4m3_f32(float* c, const uint8_t* a, const uint8_t* b, const void* bias_or_null,
@@ -609,7 +611,23 @@ extern "C" int llmq_gemm_tn_e4m3_f32(float* c, const uint8_t* a, const uint8_t* 
                                      void* workspace_or_null, size_t workspace_bytes, int M, int N, int K,
                                      int accumulate, void* stream) {
     llmq::GemmArgs g{c, a, b, bias_or_null, sa_or_null, sb_or_null, M, N, K, bias_is_bf16, accumulate, 8, nullptr, 0};
-    return llmq::gemm_dispatch<float>(g, workspace_or_null, workspace_bytes, static_cast<hipStream_t>(stream));
+    return llmq::gemm_dispatch<float, 0>(g, workspace_or_null, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int llmq_gemm_tn_e4m3_e5m2_bf16(uint16_t* c, const uint8_t* a, const uint8_t* b_e5m2,
+                                           const uint16_t* bias_or_null, const float* sa_or_null, const float* sb_or_null,
+                                           void* workspace_or_null, size_t workspace_bytes, int M, int N, int K,
+                                           int accumulate, void* stream) {
+    llmq::GemmArgs g{c, a, b_e5m2, bias_or_null, sa_or_null, sb_or_null, M, N, K, 1, accumulate, 8, nullptr, 0};
+    return llmq::gemm_dispatch<uint16_t, 1>(g, workspace_or_null, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int llmq_gemm_tn_e4m3_e5m2_f32(float* c, const uint8_t* a, const uint8_t* b_e5m2, const void* bias_or_null,
+                                          int bias_is_bf16, const float* sa_or_null, const float* sb_or_null,
+                                          void* workspace_or_null, size_t workspace_bytes, int M, int N, int K,
+                                          int accumulate, void* stream) {
+    llmq::GemmArgs g{c, a, b_e5m2, bias_or_null, sa_or_null, sb_or_null, M, N, K, bias_is_bf16, accumulate, 8, nullptr, 0};
+    return llmq::gemm_dispatch<float, 1>(g, workspace_or_null, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
 // Tuning / test hooks (not part of the drop-in surface).

@@ -78,17 +78,19 @@ def transpose(dst, src, stream=0):
     capi.check(capi.lib.llmq_transpose_u8(d, s, src.shape[0], src.shape[1], _stream(stream)))
 
 
-def matmul(c, a, b, bias, scale_a, scale_b, M, N, K, accumulate=False, stream=0, workspace=None):
+def matmul(c, a, b, bias, scale_a, scale_b, M, N, K, accumulate=False, stream=0, workspace=None, b_e5m2=False):
     """TN matmul in the convention of the reference's kernels.h: row-major a[M,K], b[N,K] (e4m3) give
     row-major c[N,M] = (b @ a.T) * scale_a * scale_b (+ bias[M]) (+ c).  c: bf16 or fp32.
     workspace: optional device byte tensor (the reference passes a 32 MiB one); it enables the
-    split-K path for outputs with too few tiles to fill the chip."""
+    split-K path for outputs with too few tiles to fill the chip.  b may hold e5m2 codes (the gradient
+    dtype option): a float8_e5m2 tensor, or uint8 with b_e5m2=True."""
     pws, ws_bytes = None, 0
     if workspace is not None:
         pws = _dev(workspace, "workspace", (torch.uint8, torch.int8, torch.float32))
         ws_bytes = workspace.numel() * workspace.element_size()
     pa = _dev(a, "a", (torch.float8_e4m3fn, torch.uint8))
-    pb = _dev(b, "b", (torch.float8_e4m3fn, torch.uint8))
+    pb = _dev(b, "b", (torch.float8_e4m3fn, torch.float8_e5m2, torch.uint8))
+    b_e5m2 = bool(b_e5m2) or b.dtype == torch.float8_e5m2
     pc = _dev(c, "c", (torch.bfloat16, torch.float32))
     if a.numel() != M * K or b.numel() != N * K or c.numel() != N * M:
         raise ValueError("operand sizes do not match M, N, K")
@@ -98,12 +100,12 @@ def matmul(c, a, b, bias, scale_a, scale_b, M, N, K, accumulate=False, stream=0,
         pbias = _dev(bias, "bias", (torch.bfloat16,), optional=True)
         if bias is not None and bias.numel() != M:
             raise ValueError("bias must have M elements")
-        capi.check(capi.lib.llmq_gemm_tn_e4m3_bf16(pc, pa, pb, pbias, sa, sb, pws, ws_bytes, M, N, K, int(accumulate),
-                                                   _stream(stream)))
+        fn = capi.lib.llmq_gemm_tn_e4m3_e5m2_bf16 if b_e5m2 else capi.lib.llmq_gemm_tn_e4m3_bf16
+        capi.check(fn(pc, pa, pb, pbias, sa, sb, pws, ws_bytes, M, N, K, int(accumulate), _stream(stream)))
     else:
         pbias = _dev(bias, "bias", (torch.bfloat16, torch.float32), optional=True)
         if bias is not None and bias.numel() != M:
             raise ValueError("bias must have M elements")
         is_bf16 = int(bias is not None and bias.dtype == torch.bfloat16)
-        capi.check(capi.lib.llmq_gemm_tn_e4m3_f32(pc, pa, pb, pbias, is_bf16, sa, sb, pws, ws_bytes, M, N, K,
-                                                  int(accumulate), _stream(stream)))
+        fn = capi.lib.llmq_gemm_tn_e4m3_e5m2_f32 if b_e5m2 else capi.lib.llmq_gemm_tn_e4m3_f32
+        capi.check(fn(pc, pa, pb, pbias, is_bf16, sa, sb, pws, ws_bytes, M, N, K, int(accumulate), _stream(stream)))

@@ -19,6 +19,7 @@
 
 uint8_t orc_e4m3_encode(float y);
 float orc_e4m3_decode(uint8_t c);
+float orc_e5m2_decode(uint8_t c);
 float orc_bf16_to_f32(uint16_t h);
 uint16_t orc_f32_to_bf16(float f);
 void orc_quant_scale(float absmax, float* scale, float* dequant);
@@ -134,13 +135,16 @@ static void micro_4x64(float* restrict acc, const float* restrict at, const floa
  * Restricted to c rows n in [n0,n1) so the benchmark can time a bounded slice of a large shape.
  * Requires M % 64 == 0 and (n1-n0) % 4 == 0.  Returns 0, or -1 on unsupported shape.
  */
-int mt_gemm_tn_e4m3(void* c, int c_is_f32, const uint8_t* a, const uint8_t* b,
-                    const uint16_t* bias_bf16, const float* sa, const float* sb,
-                    int M, int N, int K, int accumulate, int n0, int n1) {
+int mt_gemm_tn_fp8(void* c, int c_is_f32, const uint8_t* a, const uint8_t* b, int b_is_e5m2,
+                   const uint16_t* bias_bf16, const float* sa, const float* sb,
+                   int M, int N, int K, int accumulate, int n0, int n1) {
     (void)N;
     if (M % MB != 0 || (n1 - n0) % NB != 0) return -1;
-    float lut[256];
-    for (int i = 0; i < 256; ++i) lut[i] = orc_e4m3_decode((uint8_t)i);
+    float lut[256], lut_b[256];
+    for (int i = 0; i < 256; ++i) {
+        lut[i] = orc_e4m3_decode((uint8_t)i);
+        lut_b[i] = b_is_e5m2 ? orc_e5m2_decode((uint8_t)i) : lut[i];
+    }
     float scale = sa ? *sa : 1.f;
     if (sb) scale = scale * *sb;
 #pragma omp parallel
@@ -157,7 +161,7 @@ int mt_gemm_tn_e4m3(void* c, int c_is_f32, const uint8_t* a, const uint8_t* b,
             for (int n = n0; n < n1; n += NB) {
                 for (int j = 0; j < NB; ++j) {
                     const uint8_t* bn = b + (size_t)(n + j) * K;
-                    for (int k = 0; k < K; ++k) bq[(size_t)j * K + k] = lut[bn[k]];
+                    for (int k = 0; k < K; ++k) bq[(size_t)j * K + k] = lut_b[bn[k]];
                 }
                 micro_4x64(acc, at, bq, K);
                 for (int j = 0; j < NB; ++j)
@@ -176,4 +180,10 @@ int mt_gemm_tn_e4m3(void* c, int c_is_f32, const uint8_t* a, const uint8_t* b,
         free(bq);
     }
     return 0;
+}
+
+int mt_gemm_tn_e4m3(void* c, int c_is_f32, const uint8_t* a, const uint8_t* b,
+                    const uint16_t* bias_bf16, const float* sa, const float* sb,
+                    int M, int N, int K, int accumulate, int n0, int n1) {
+    return mt_gemm_tn_fp8(c, c_is_f32, a, b, 0, bias_bf16, sa, sb, M, N, K, accumulate, n0, n1);
 }

@@ -204,14 +204,23 @@ void orc_transpose_u8(uint8_t* dst, const uint8_t* src, int rows, int cols) {
  *   sumabs[n*M + m] = sum_k |dec(b[n,k]) * dec(a[m,k])|      (for the error bound; may be NULL)
  * Only rows n in [n0, n1) are produced (written at their absolute position).
  */
-void orc_gemm_tn_e4m3_exact(double* exact, double* sumabs, const uint8_t* a, const uint8_t* b,
-                            int M, int N, int K, int n0, int n1) {
-    double lut[256];
-    for (int i = 0; i < 256; ++i) lut[i] = (double)orc_e4m3_decode((uint8_t)i);
+/* decode tables: a is always e4m3; b is e4m3, or e5m2 for the gradient dtype of
+ * src/kernels/kernels.h:92-94 (matmul with __nv_fp8_e5m2 b) */
+static void fp8_luts(double* lut_a, double* lut_b, int b_is_e5m2) {
+    for (int i = 0; i < 256; ++i) {
+        lut_a[i] = (double)orc_e4m3_decode((uint8_t)i);
+        lut_b[i] = b_is_e5m2 ? (double)orc_e5m2_decode((uint8_t)i) : lut_a[i];
+    }
+}
+
+void orc_gemm_tn_fp8_exact(double* exact, double* sumabs, const uint8_t* a, const uint8_t* b, int b_is_e5m2,
+                           int M, int N, int K, int n0, int n1) {
+    double lut[256], lut_b[256];
+    fp8_luts(lut, lut_b, b_is_e5m2);
     (void)N;
     double* arow = (double*)malloc(sizeof(double) * (size_t)K);
     for (int64_t n = n0; n < n1; ++n) {
-        for (int k = 0; k < K; ++k) arow[k] = lut[b[n * K + k]];
+        for (int k = 0; k < K; ++k) arow[k] = lut_b[b[n * K + k]];
         for (int64_t m = 0; m < M; ++m) {
             const uint8_t* am = a + m * K;
             double s = 0.0, sa = 0.0;
@@ -227,25 +236,36 @@ void orc_gemm_tn_e4m3_exact(double* exact, double* sumabs, const uint8_t* a, con
     free(arow);
 }
 
+void orc_gemm_tn_e4m3_exact(double* exact, double* sumabs, const uint8_t* a, const uint8_t* b,
+                            int M, int N, int K, int n0, int n1) {
+    orc_gemm_tn_fp8_exact(exact, sumabs, a, b, 0, M, N, K, n0, n1);
+}
+
 /* Same, for a list of sampled output coordinates (idx_n[i], idx_m[i]). */
-void orc_gemm_tn_e4m3_exact_sampled(double* exact, double* sumabs, const uint8_t* a, const uint8_t* b,
-                                    int M, int N, int K, const int32_t* idx_n, const int32_t* idx_m,
-                                    int64_t count) {
-    double lut[256];
-    for (int i = 0; i < 256; ++i) lut[i] = (double)orc_e4m3_decode((uint8_t)i);
+void orc_gemm_tn_fp8_exact_sampled(double* exact, double* sumabs, const uint8_t* a, const uint8_t* b, int b_is_e5m2,
+                                   int M, int N, int K, const int32_t* idx_n, const int32_t* idx_m,
+                                   int64_t count) {
+    double lut[256], lut_b[256];
+    fp8_luts(lut, lut_b, b_is_e5m2);
     (void)M; (void)N;
     for (int64_t i = 0; i < count; ++i) {
         const uint8_t* bn = b + (int64_t)idx_n[i] * K;
         const uint8_t* am = a + (int64_t)idx_m[i] * K;
         double s = 0.0, sa = 0.0;
         for (int k = 0; k < K; ++k) {
-            double p = lut[bn[k]] * lut[am[k]];
+            double p = lut_b[bn[k]] * lut[am[k]];
             s += p;
             sa += fabs(p);
         }
         exact[i] = s;
         if (sumabs) sumabs[i] = sa;
     }
+}
+
+void orc_gemm_tn_e4m3_exact_sampled(double* exact, double* sumabs, const uint8_t* a, const uint8_t* b,
+                                    int M, int N, int K, const int32_t* idx_n, const int32_t* idx_m,
+                                    int64_t count) {
+    orc_gemm_tn_fp8_exact_sampled(exact, sumabs, a, b, 0, M, N, K, idx_n, idx_m, count);
 }
 
 /*
@@ -264,11 +284,11 @@ float orc_gemm_epilogue_f32(double exact, float scale, const float* bias_m, cons
 }
 
 /* Full TN GEMM with the epilogue, bf16 or fp32 output; used for sizes the oracle finishes quickly. */
-void orc_gemm_tn_e4m3(void* c, int c_is_f32, const uint8_t* a, const uint8_t* b,
-                      const uint16_t* bias_bf16, const float* bias_f32,
-                      const float* sa, const float* sb, int M, int N, int K, int accumulate) {
+void orc_gemm_tn_fp8(void* c, int c_is_f32, const uint8_t* a, const uint8_t* b, int b_is_e5m2,
+                     const uint16_t* bias_bf16, const float* bias_f32,
+                     const float* sa, const float* sb, int M, int N, int K, int accumulate) {
     double* ex = (double*)malloc(sizeof(double) * (size_t)M * (size_t)N);
-    orc_gemm_tn_e4m3_exact(ex, NULL, a, b, M, N, K, 0, N);
+    orc_gemm_tn_fp8_exact(ex, NULL, a, b, b_is_e5m2, M, N, K, 0, N);
     volatile float scale = (sa ? *sa : 1.f);
     if (sb) scale = scale * *sb;
     for (int64_t n = 0; n < N; ++n)
@@ -286,6 +306,12 @@ void orc_gemm_tn_e4m3(void* c, int c_is_f32, const uint8_t* a, const uint8_t* b,
             else ((uint16_t*)c)[n * M + m] = orc_f32_to_bf16(t);
         }
     free(ex);
+}
+
+void orc_gemm_tn_e4m3(void* c, int c_is_f32, const uint8_t* a, const uint8_t* b,
+                      const uint16_t* bias_bf16, const float* bias_f32,
+                      const float* sa, const float* sb, int M, int N, int K, int accumulate) {
+    orc_gemm_tn_fp8(c, c_is_f32, a, b, 0, bias_bf16, bias_f32, sa, sb, M, N, K, accumulate);
 }
 
 /* ------------------------------------------------------------------------------------------------

@@ -84,6 +84,17 @@ def lib():
     L.mt_gemm_tn_e4m3.restype = C.c_int
     L.mt_gemm_tn_e4m3.argtypes = [C.c_void_p, C.c_int, u8p, u8p, u16p, f32p, f32p,
                                   C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
+    L.orc_gemm_tn_fp8_exact.restype = None
+    L.orc_gemm_tn_fp8_exact.argtypes = [f64p, f64p, u8p, u8p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
+    L.orc_gemm_tn_fp8_exact_sampled.restype = None
+    L.orc_gemm_tn_fp8_exact_sampled.argtypes = [f64p, f64p, u8p, u8p, C.c_int, C.c_int, C.c_int, C.c_int, i32p, i32p,
+                                                C.c_int64]
+    L.orc_gemm_tn_fp8.restype = None
+    L.orc_gemm_tn_fp8.argtypes = [C.c_void_p, C.c_int, u8p, u8p, C.c_int, u16p, f32p, f32p, f32p,
+                                  C.c_int, C.c_int, C.c_int, C.c_int]
+    L.mt_gemm_tn_fp8.restype = C.c_int
+    L.mt_gemm_tn_fp8.argtypes = [C.c_void_p, C.c_int, u8p, u8p, C.c_int, u16p, f32p, f32p,
+                                 C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
     _lib = L
     return L
 
@@ -115,6 +126,12 @@ def e4m3_table():
         L = lib()
         _E4M3_TABLE = np.array([L.orc_e4m3_decode(i) for i in range(256)], dtype=np.float32)
     return _E4M3_TABLE
+
+
+def e5m2_table():
+    """float32[256]: value of every e5m2 code (NaN / Inf codes included)."""
+    L = lib()
+    return np.array([L.orc_e5m2_decode(i) for i in range(256)], dtype=np.float32)
 
 
 def e4m3_decode(codes):
@@ -161,9 +178,9 @@ def transpose_u8(x, mt=False):
     return out
 
 
-def gemm_exact(a, b, rows=None):
-    """a[M,K], b[N,K] e4m3 codes -> (exact float64 [N,M], sum|terms| float64 [N,M]); rows=(n0,n1)
-    restricts the computed rows (others are left zero)."""
+def gemm_exact(a, b, rows=None, b_e5m2=False):
+    """a[M,K] e4m3 codes, b[N,K] e4m3 (or e5m2) codes -> (exact float64 [N,M], sum|terms| float64 [N,M]);
+    rows=(n0,n1) restricts the computed rows (others are left zero)."""
     a = np.ascontiguousarray(a, dtype=np.uint8)
     b = np.ascontiguousarray(b, dtype=np.uint8)
     M, K = a.shape
@@ -172,12 +189,12 @@ def gemm_exact(a, b, rows=None):
     n0, n1 = rows if rows is not None else (0, N)
     ex = np.zeros((N, M), dtype=np.float64)
     sa = np.zeros((N, M), dtype=np.float64)
-    lib().orc_gemm_tn_e4m3_exact(_p(ex, C.c_double), _p(sa, C.c_double), _p(a, C.c_uint8), _p(b, C.c_uint8),
-                                 M, N, K, n0, n1)
+    lib().orc_gemm_tn_fp8_exact(_p(ex, C.c_double), _p(sa, C.c_double), _p(a, C.c_uint8), _p(b, C.c_uint8),
+                                int(b_e5m2), M, N, K, n0, n1)
     return ex, sa
 
 
-def gemm_exact_sampled(a, b, idx_n, idx_m):
+def gemm_exact_sampled(a, b, idx_n, idx_m, b_e5m2=False):
     a = np.ascontiguousarray(a, dtype=np.uint8)
     b = np.ascontiguousarray(b, dtype=np.uint8)
     M, K = a.shape
@@ -186,13 +203,13 @@ def gemm_exact_sampled(a, b, idx_n, idx_m):
     idx_m = np.ascontiguousarray(idx_m, dtype=np.int32)
     ex = np.zeros(idx_n.size, dtype=np.float64)
     sa = np.zeros(idx_n.size, dtype=np.float64)
-    lib().orc_gemm_tn_e4m3_exact_sampled(_p(ex, C.c_double), _p(sa, C.c_double), _p(a, C.c_uint8),
-                                         _p(b, C.c_uint8), M, N, K, _p(idx_n, C.c_int32),
-                                         _p(idx_m, C.c_int32), idx_n.size)
+    lib().orc_gemm_tn_fp8_exact_sampled(_p(ex, C.c_double), _p(sa, C.c_double), _p(a, C.c_uint8),
+                                        _p(b, C.c_uint8), int(b_e5m2), M, N, K, _p(idx_n, C.c_int32),
+                                        _p(idx_m, C.c_int32), idx_n.size)
     return ex, sa
 
 
-def gemm_tn(a, b, sa=None, sb=None, bias=None, c_old=None, out_f32=False, mt=False):
+def gemm_tn(a, b, sa=None, sb=None, bias=None, c_old=None, out_f32=False, mt=False, b_e5m2=False):
     """Full GEMM + epilogue.  bias: uint16 bf16 [M] or None.  c_old: previous c (accumulate) or None.
     Returns uint16 bf16 [N,M] or float32 [N,M]."""
     a = np.ascontiguousarray(a, dtype=np.uint8)
@@ -210,12 +227,12 @@ def gemm_tn(a, b, sa=None, sb=None, bias=None, c_old=None, out_f32=False, mt=Fal
         bias = np.ascontiguousarray(bias, dtype=np.uint16)
         bp = _p(bias, C.c_uint16)
     if mt:
-        rc = lib().mt_gemm_tn_e4m3(c.ctypes.data, int(out_f32), _p(a, C.c_uint8), _p(b, C.c_uint8), bp, fsa, fsb,
-                                   M, N, K, int(c_old is not None), 0, N)
+        rc = lib().mt_gemm_tn_fp8(c.ctypes.data, int(out_f32), _p(a, C.c_uint8), _p(b, C.c_uint8), int(b_e5m2), bp,
+                                  fsa, fsb, M, N, K, int(c_old is not None), 0, N)
         assert rc == 0
     else:
-        lib().orc_gemm_tn_e4m3(c.ctypes.data, int(out_f32), _p(a, C.c_uint8), _p(b, C.c_uint8), bp, None, fsa, fsb,
-                               M, N, K, int(c_old is not None))
+        lib().orc_gemm_tn_fp8(c.ctypes.data, int(out_f32), _p(a, C.c_uint8), _p(b, C.c_uint8), int(b_e5m2), bp, None,
+                              fsa, fsb, M, N, K, int(c_old is not None))
     return c
 
 

@@ -294,6 +294,41 @@ def test_gemm_automatic_split_k(K, O, mnk):
     gemm_check(c1.cpu().numpy(), exact, sumabs, np.float32(np.float32(0.01) * np.float32(0.02)), False)
 
 
+@pytest.mark.parametrize("variant", [(0, 0), (1, 1, 1), (2, 2)])
+def test_gemm_e5m2_b_operand(K, O, variant):
+    """a e4m3, b e5m2 (src/kernels/kernels.h:92-94): small integers are exact in both formats ->
+    bit-exact against the oracle; random codes within the stated tolerance of the exact product."""
+    M, N, Kd = 512, 768, 640
+    rng = np.random.default_rng(91)
+    ai, bi = rng.integers(-4, 5, (M, Kd)), rng.integers(-4, 5, (N, Kd))
+    enc4 = {v: O.lib().orc_e4m3_encode(float(v)) for v in range(-4, 5)}
+    enc5 = {v: O.lib().orc_e5m2_encode(float(v)) for v in range(-4, 5)}
+    a = np.vectorize(enc4.get)(ai).astype(np.uint8)
+    b = np.vectorize(enc5.get)(bi).astype(np.uint8)
+    s = float(np.sqrt(np.float32(4.0 / Kd)))
+    _, biasv = O.fill_int_e4m3(M, 91, 2)
+    bias = O.f32_to_bf16(biasv.astype(np.float32))
+    set_variant(variant)
+    try:
+        want = O.gemm_tn(a, b, sa=s, sb=s, bias=bias, mt=True, b_e5m2=True)
+        c = torch.full((N, M), float("nan"), dtype=torch.bfloat16, device="cuda")
+        K.matmul(c, dev_u8(a), dev_u8(b).view(torch.float8_e5m2), dev_bf16(bias), dev_scalar(s), dev_scalar(s), M, N, Kd,
+                 workspace=workspace())
+        assert np.array_equal(host_bits(c), want)
+        # same integers: the e5m2 result must equal the int64 product, i.e. differ from reading b as e4m3
+        ar = rng.integers(0, 256, (M, Kd)).astype(np.uint8)
+        br = rng.integers(0, 256, (N, Kd)).astype(np.uint8)
+        ar[(ar & 0x7F) == 0x7F] ^= 1
+        br[(br & 0x7C) == 0x7C] ^= 0x40                      # no Inf / NaN codes
+        br &= 0xBF                                           # magnitudes below 2: products stay modest
+        exact, sumabs = O.gemm_exact(ar, br, b_e5m2=True)
+        c32 = torch.empty((N, M), dtype=torch.float32, device="cuda")
+        K.matmul(c32, dev_u8(ar), dev_u8(br), None, dev_scalar(0.25), None, M, N, Kd, workspace=workspace(), b_e5m2=True)
+        gemm_check(c32.cpu().numpy(), exact, sumabs, 0.25, False)
+    finally:
+        set_variant((0, 0))
+
+
 def test_gemm_matches_swapped_operand_transpose(K, O):
     """c(a,b)^T == c(b,a): a size-independent identity that catches row/column mix-ups."""
     M, N, Kd = 384, 640, 256

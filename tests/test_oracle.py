@@ -221,6 +221,93 @@ def test_gemm_integer_known_answer(O, mnk, scale):
         assert np.array_equal(O.gemm_tn(a, b, sa=float(s), sb=float(s), bias=bias, c_old=old, mt=True), got)
 
 
+# ------------------------------------------------------------------ e5m2 (gradient dtype), same evidence
+def e5m2_value_of_code(c):
+    """IEEE-like binary8 E5M2 value of a 7-bit magnitude code below the Inf/NaN block (c < 0x7C)."""
+    e, m = c >> 2, c & 3
+    if e == 0:
+        return m * 2.0 ** -16
+    return (4 + m) * 2.0 ** (e - 17)
+
+
+def e5m2_encode_search(y):
+    y = np.asarray(y, dtype=np.float32)
+    vals = np.array([e5m2_value_of_code(c) for c in range(0x7C)], dtype=np.float64)   # 0 .. 57344
+    a = np.abs(y.astype(np.float64))
+    hi = np.clip(np.searchsorted(vals, a, side="left"), 0, 0x7B)
+    lo = np.clip(hi - 1, 0, 0x7B)
+    dlo, dhi = np.abs(a - vals[lo]), np.abs(vals[hi] - a)
+    code = np.where(dlo < dhi, lo, np.where(dhi < dlo, hi, np.where(lo % 2 == 0, lo, hi)))
+    code = np.where(a >= 57344.0, 0x7B, code)
+    sign = (y.view(np.uint32) >> 31).astype(np.uint8) << 7
+    out = (code.astype(np.uint8) | sign).astype(np.uint8)
+    out[np.isnan(y)] = 0x7F
+    return out
+
+
+def test_e5m2_decode_matches_definition_and_torch(O):
+    tab = O.e5m2_table()
+    for c in range(0x7C):
+        assert tab[c] == np.float32(e5m2_value_of_code(c)) and tab[c | 0x80] == -np.float32(e5m2_value_of_code(c))
+    assert np.isinf(tab[0x7C]) and np.isinf(tab[0xFC]) and np.all(np.isnan(tab[[0x7D, 0x7E, 0x7F, 0xFD, 0xFE, 0xFF]]))
+    t = torch.arange(256, dtype=torch.int32).to(torch.uint8).view(torch.float8_e5m2).float().numpy()
+    assert np.array_equal(np.nan_to_num(t, nan=12345.0), np.nan_to_num(tab, nan=12345.0))
+
+
+@pytest.mark.parametrize("absmax", [448.0, 1.0, 5.15625, 3.0e-5, 1e4, 0.0, 2.0 ** -7])
+def test_e5m2_encode_exhaustive_bf16_vs_search_and_torch(O, absmax):
+    """All 65536 bf16 inputs through the reference's 448-based scale (quant.cu:79 serves both fp8 output
+    types) into e5m2, against the nearest-code search and torch's float8_e5m2 cast."""
+    s, _ = O.quant_scale(absmax)
+    with np.errstate(over="ignore", invalid="ignore"):
+        y = (np.float32(s) * O.bf16_to_f32(ALL_BF16)).astype(np.float32)
+    got, _ = O.quantize_e4m3(ALL_BF16, absmax, fmt="e5m2")
+    assert np.array_equal(got, e5m2_encode_search(y))
+    finite = ~np.isnan(y)
+    t = torch.from_numpy(y[finite]).clamp(-57344.0, 57344.0).to(torch.float8_e5m2).view(torch.uint8).numpy()
+    assert np.array_equal(got[finite], t)
+    assert np.all(got[~finite] == 0x7F)
+
+
+def test_e5m2_encode_boundaries_closed_form(O):
+    enc = O.lib().orc_e5m2_encode
+    assert enc(0.0) == 0x00 and enc(-0.0) == 0x80 and enc(1.0) == 0x3C and enc(-1.0) == 0xBC
+    assert enc(2.0 ** -17) == 0x00 and enc(float(np.nextafter(np.float32(2.0 ** -17), np.float32(1)))) == 0x01
+    assert enc(1.125) == 0x3C and enc(1.375) == 0x3E                          # ties to even
+    assert enc(57344.0) == 0x7B and enc(61439.0) == 0x7B and enc(61440.0) == 0x7B and enc(1e30) == 0x7B
+    assert enc(float("inf")) == 0x7B and enc(float("-inf")) == 0xFB and enc(float("nan")) == 0x7F
+
+
+def test_gemm_e5m2_b_operand_vs_float64_matmul(O):
+    """a e4m3, b e5m2 (src/kernels/kernels.h:92-94): every product is exact in fp64 (4 x 3 significand
+    bits), so the oracle must equal numpy's float64 matmul of the decoded operands."""
+    rng = np.random.default_rng(8)
+    M, N, K = 64, 40, 384
+    a = rng.integers(0, 256, (M, K)).astype(np.uint8)
+    b = rng.integers(0, 256, (N, K)).astype(np.uint8)
+    a[(a & 0x7F) == 0x7F] = 0x7E
+    b[(b & 0x7C) == 0x7C] = 0x70                                                 # no Inf / NaN codes
+    ex, sabs = O.gemm_exact(a, b, b_e5m2=True)
+    ad = O.e4m3_decode(a).astype(np.float64)
+    bd = O.e5m2_table()[b].astype(np.float64)
+    ref, refabs = bd @ ad.T, np.abs(bd) @ np.abs(ad).T
+    assert np.allclose(ex, ref, rtol=0, atol=1e-9 * refabs) and np.allclose(sabs, refabs, rtol=1e-12)
+    idx_n = rng.integers(0, N, 64).astype(np.int32)
+    idx_m = rng.integers(0, M, 64).astype(np.int32)
+    exs, _ = O.gemm_exact_sampled(a, b, idx_n, idx_m, b_e5m2=True)
+    assert np.array_equal(exs, ex[idx_n, idx_m])
+    # small integers are exact in both formats -> int64 known answer through the full epilogue
+    ai = rng.integers(-4, 5, (M, K))
+    bi = rng.integers(-4, 5, (N, K))
+    lib = O.lib()
+    a8 = np.array([lib.orc_e4m3_encode(float(v)) for v in ai.ravel()], dtype=np.uint8).reshape(M, K)
+    b8 = np.array([lib.orc_e5m2_encode(float(v)) for v in bi.ravel()], dtype=np.uint8).reshape(N, K)
+    want = (bi.astype(np.int64) @ ai.astype(np.int64).T).astype(np.float32) * np.float32(0.25)
+    for mt in (False, True):
+        got = O.gemm_tn(a8, b8, sa=0.5, sb=0.5, out_f32=True, mt=mt, b_e5m2=True)
+        assert np.array_equal(got, want)
+
+
 def test_gemm_random_codes_vs_float64_matmul(O):
     rng = np.random.default_rng(3)
     M, N, K = 64, 48, 512
