@@ -128,6 +128,22 @@ int llmq_gemm_tn_e4m3_e5m2_f32(float* c, const uint8_t* a, const uint8_t* b_e5m2
                                void* workspace_or_null, size_t workspace_bytes, int M, int N, int K, int accumulate,
                                void* stream);
 
+/*
+ * Bias gradient from the (quantized) output gradient: with row-major dout[BT, OC],
+ *     dbias[oc] = round_bf16( (float)dbias[oc] + (sa*sb) * sum_bt value(dout[bt, oc]) )
+ * i.e. the result is ADDED to dbias.  dout_format: 0 = e4m3, 1 = e5m2, 2 = bf16.  sa / sb: device fp32
+ * scalars, both NULL (factor 1) or both non-NULL.  OC must be a multiple of 16 (fp8) or 8 (bf16).
+ * scratch: device buffer of at least llmq_backward_bias_scratch_bytes(BT, OC, dout_format) bytes,
+ * overwritten by every call (no need to clear it); fp32 sums in a fixed order -> deterministic.
+ * Replaces: backward_bias(nv_bfloat16* dbias, const __nv_fp8_e4m3* dout, const float* scale_a,
+ *           const float* scale_b, float* dbias_buffer, int B, int T, int OC, const cudaDeviceProp&, cudaStream_t)
+ *           src/kernels/kernels.h:104-106, src/kernels/bias.cu:151-195, and
+ *           get_bias_backward_scratch_size(ETensorDType, int OC, const cudaDeviceProp&) kernels.h:102, bias.cu:142-148.
+ */
+int64_t llmq_backward_bias_scratch_bytes(int BT, int OC, int dout_format);
+int llmq_backward_bias_bf16(uint16_t* dbias, const void* dout, int dout_format, const float* sa_or_null,
+                            const float* sb_or_null, float* scratch, size_t scratch_bytes, int BT, int OC, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

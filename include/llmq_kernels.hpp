@@ -287,4 +287,47 @@ inline void matmul(Tensor& c, const Tensor& a, const Tensor& b, const Tensor& bi
     }
 }
 
+// ---- backward_bias (reference: src/kernels/kernels.h:102-107, src/kernels/bias.cu:142-195) ---------------
+// dbias[OC] += (*scale_a * *scale_b) * column sums of dout[B*T, OC]; scales both null or both non-null.
+inline int get_bias_backward_scratch_size(ETensorDType dtype, int OC, const hipDeviceProp_t&) {
+    // sized for any B*T (the number of row bands saturates for large row counts)
+    return (int)llmq_backward_bias_scratch_bytes(1 << 30, OC, dtype == ETensorDType::BF16 ? 2 : 0);
+}
+inline void backward_bias(__hip_bfloat16* dbias, const __hip_fp8_e4m3* dout, const float* scale_a, const float* scale_b,
+                          float* dbias_buffer, int B, int T, int OC, const hipDeviceProp_t& dp, hipStream_t stream) {
+    llmq_detail::check(llmq_backward_bias_bf16(llmq_detail::u16(dbias), dout, 0, scale_a, scale_b, dbias_buffer,
+                                               (std::size_t)get_bias_backward_scratch_size(ETensorDType::FP8_E4M3, OC, dp),
+                                               B * T, OC, stream));
+}
+inline void backward_bias(__hip_bfloat16* dbias, const __hip_fp8_e5m2* dout, const float* scale_a, const float* scale_b,
+                          float* dbias_buffer, int B, int T, int OC, const hipDeviceProp_t& dp, hipStream_t stream) {
+    llmq_detail::check(llmq_backward_bias_bf16(llmq_detail::u16(dbias), dout, 1, scale_a, scale_b, dbias_buffer,
+                                               (std::size_t)get_bias_backward_scratch_size(ETensorDType::FP8_E5M2, OC, dp),
+                                               B * T, OC, stream));
+}
+inline void backward_bias(__hip_bfloat16* dbias, const __hip_bfloat16* dout, const float* scale_a, const float* scale_b,
+                          float* dbias_buffer, int B, int T, int OC, const hipDeviceProp_t& dp, hipStream_t stream) {
+    llmq_detail::check(llmq_backward_bias_bf16(llmq_detail::u16(dbias), dout, 2, scale_a, scale_b, dbias_buffer,
+                                               (std::size_t)get_bias_backward_scratch_size(ETensorDType::BF16, OC, dp),
+                                               B * T, OC, stream));
+}
+inline void backward_bias(Tensor& dbias, const Tensor& dout, const float* scale_a, const float* scale_b,
+                          Tensor& dbias_buffer, int B, int T, int OC, const hipDeviceProp_t& dp, hipStream_t stream) {
+    const std::size_t expected = (std::size_t)get_bias_backward_scratch_size(dout.DType, OC, dp);
+    if (dbias_buffer.bytes() < expected)
+        throw std::invalid_argument("scratch buffer too small: expected at least " + std::to_string(expected) +
+                                    " bytes, got " + std::to_string(dbias_buffer.bytes()));
+    if (dbias.DType != ETensorDType::BF16) llmq_detail::unsupported(__func__, dbias, dout, dbias_buffer);
+    if (dout.DType == ETensorDType::FP8_E4M3)
+        backward_bias(dbias.get<__hip_bfloat16>(), dout.get<__hip_fp8_e4m3>(), scale_a, scale_b,
+                      dbias_buffer.get<float>(), B, T, OC, dp, stream);
+    else if (dout.DType == ETensorDType::FP8_E5M2)
+        backward_bias(dbias.get<__hip_bfloat16>(), dout.get<__hip_fp8_e5m2>(), scale_a, scale_b,
+                      dbias_buffer.get<float>(), B, T, OC, dp, stream);
+    else if (dout.DType == ETensorDType::BF16)
+        backward_bias(dbias.get<__hip_bfloat16>(), dout.get<__hip_bfloat16>(), scale_a, scale_b,
+                      dbias_buffer.get<float>(), B, T, OC, dp, stream);
+    else llmq_detail::unsupported(__func__, dbias, dout, dbias_buffer);
+}
+
 #endif  // LLMQ_KERNELS_HPP

@@ -60,10 +60,12 @@ inline void forward_qmm(Tensor& out, QuantizableTensor& inp, Tensor& weight, con
            EMMTranspose::TN, false, stream, backend);
 }
 
-// dinp[B*T, C] = dout . weight ;  dweight[OC, C] (+)= dout^T . inp.
-inline void backward_qmm(Tensor& dinp, Tensor& dweight, QuantizableTensor& dout, QuantizableTensor& inp,
-                         Tensor& weight, bool accumulate_gradient, QmmRunState& rs, int B, int T, int C, int OC,
-                         bool reuse_inp, hipStream_t stream) {
+// dinp[B*T, C] = dout . weight ;  dweight[OC, C] (+)= dout^T . inp ;  dbias[OC] += column sums of dout when
+// dbias is non-empty (bias_buffer: scratch of get_bias_backward_scratch_size bytes).  Argument order as in the
+// reference (src/models/llama_model.cpp:280-285).
+inline void backward_qmm(Tensor& dinp, Tensor& dweight, Tensor dbias, QuantizableTensor& dout, QuantizableTensor& inp,
+                         Tensor& weight, Tensor bias_buffer, bool accumulate_gradient, QmmRunState& rs, int B, int T,
+                         int C, int OC, bool reuse_inp, hipStream_t stream) {
     if (weight.DType != ETensorDType::FP8_E4M3)
         throw std::invalid_argument("backward_qmm: this build implements the FP8 (e4m3 weight) branch only");
     quantize_with_abs_max(dout.Quant, dout.Quant.scale(), dout.Value, dout.Quant.abs_max(), (long)B * T * OC,
@@ -89,6 +91,9 @@ inline void backward_qmm(Tensor& dinp, Tensor& dweight, QuantizableTensor& dout,
     transpose(grad_tp, dout.Quant, B * T, OC, stream);
     matmul(dweight, activation_tp, grad_tp, no_bias, inp_q.scale(), dout.Quant.scale(), rs.BlasHandle, rs.Workspace, C,
            OC, B * T, EMMTranspose::TN, accumulate_gradient, stream, rs.MatmulBackend);
+    if (!dbias.empty()) {
+        backward_bias(dbias, dout.Quant, inp_q.scale(), dout.Quant.scale(), bias_buffer, B, T, OC, rs.DeviceProp, stream);
+    }
     rs.temp_free(grad_tp);
     rs.temp_free(activation_tp);
 }

@@ -19,6 +19,7 @@ EXPORTS = [
     "llmq_abs_max_bf16", "llmq_abs_max_f32",
     "llmq_quantize_e4m3_bf16", "llmq_quantize_e5m2_bf16", "llmq_quantize_transpose_e4m3_bf16",
     "llmq_transpose_u8", "llmq_gemm_tn_e4m3_bf16", "llmq_gemm_tn_e4m3_f32", "llmq_gemm_tn_e4m3_e5m2_bf16", "llmq_gemm_tn_e4m3_e5m2_f32",
+    "llmq_backward_bias_bf16", "llmq_backward_bias_scratch_bytes",
 ]
 
 if not os.path.exists(LIB_PATH):
@@ -40,6 +41,8 @@ lib.llmq_gemm_tn_e4m3_bf16.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, C.c_si
 lib.llmq_gemm_tn_e4m3_f32.argtypes = [_vp, _vp, _vp, _vp, _int, _vp, _vp, _vp, C.c_size_t, _int, _int, _int, _int, _vp]
 lib.llmq_gemm_tn_e4m3_e5m2_bf16.argtypes = lib.llmq_gemm_tn_e4m3_bf16.argtypes
 lib.llmq_gemm_tn_e4m3_e5m2_f32.argtypes = lib.llmq_gemm_tn_e4m3_f32.argtypes
+lib.llmq_backward_bias_bf16.argtypes = [_vp, _vp, _int, _vp, _vp, _vp, C.c_size_t, _int, _int, _vp]
+lib.llmq_backward_bias_scratch_bytes.argtypes = [_int, _int, _int]
 lib.llmq_debug_set_gemm_variant.argtypes = [_int, _int]
 lib.llmq_debug_set_gemm_variant.restype = None
 lib.llmq_debug_set_gemm_persist.argtypes = [_int]
@@ -50,6 +53,7 @@ lib.llmq_debug_mfma_ceiling.argtypes = [_vp, _int, _int, _int, _vp]
 lib.llmq_debug_mfma_ceiling.restype = _int
 for _name in EXPORTS[3:]:
     getattr(lib, _name).restype = _int
+lib.llmq_backward_bias_scratch_bytes.restype = _i64
 
 LLMQ_OK, LLMQ_ERR_INVALID_ARGUMENT, LLMQ_ERR_RUNTIME = 0, 1, 2
 

@@ -9,6 +9,8 @@ Names, argument order and in-place "out first" convention are the reference's:
     quantize_and_transpose_with_abs_max(out, scale, x, abs_max, stream=0)
     transpose(dst, src, stream=0)
     matmul(c, a, b, bias, scale_a, scale_b, M, N, K, accumulate=False, stream=0)   [kernels.h convention]
+    backward_bias(dbias, dout, scale_a, scale_b, dbias_buffer, stream=0)
+    get_bias_backward_scratch_size(dtype, OC, BT=...)
 `stream` is a raw hipStream_t handle (0 = torch's current stream).
 """
 import torch
@@ -109,3 +111,33 @@ def matmul(c, a, b, bias, scale_a, scale_b, M, N, K, accumulate=False, stream=0,
         is_bf16 = int(bias is not None and bias.dtype == torch.bfloat16)
         fn = capi.lib.llmq_gemm_tn_e4m3_e5m2_f32 if b_e5m2 else capi.lib.llmq_gemm_tn_e4m3_f32
         capi.check(fn(pc, pa, pb, pbias, is_bf16, sa, sb, pws, ws_bytes, M, N, K, int(accumulate), _stream(stream)))
+
+
+_BIAS_FMT = {torch.float8_e4m3fn: 0, torch.float8_e5m2: 1, torch.bfloat16: 2}
+
+
+def get_bias_backward_scratch_size(dtype, OC, BT=1 << 20):
+    """Bytes of scratch backward_bias needs for gradients of `dtype` with OC columns (reference:
+    get_bias_backward_scratch_size, src/kernels/bias.cu:142-148).  The reference sizes it from OC alone;
+    here the number of row bands also depends on the row count, so the default assumes a large one
+    (the value for a given B*T is never larger than for a larger B*T)."""
+    return int(capi.lib.llmq_backward_bias_scratch_bytes(int(BT), int(OC), _BIAS_FMT[dtype]))
+
+
+def backward_bias(dbias, dout, scale_a, scale_b, dbias_buffer, stream=0):
+    """dbias[OC] (bf16) += scale_a * scale_b * dout.sum over all leading dims.  dout: [..., OC] in
+    float8_e4m3fn, float8_e5m2 or bfloat16; scales both None or both fp32 device scalars
+    (reference: src/kernels/bias.cu:151-195, src/binding/kernel_binding.cpp:445-459)."""
+    if dout.dtype not in _BIAS_FMT:
+        raise ValueError("dout: unsupported dtype %s" % dout.dtype)
+    pd = _dev(dbias, "dbias", (torch.bfloat16,))
+    po = _dev(dout, "dout")
+    OC = dout.shape[-1]
+    if dbias.numel() != OC:
+        raise ValueError("dbias must have OC elements")
+    BT = dout.numel() // OC if OC else 0
+    sa = _dev(scale_a, "scale_a", (torch.float32,), optional=True)
+    sb = _dev(scale_b, "scale_b", (torch.float32,), optional=True)
+    pbuf = _dev(dbias_buffer, "dbias_buffer", (torch.float32,))
+    capi.check(capi.lib.llmq_backward_bias_bf16(pd, po, _BIAS_FMT[dout.dtype], sa, sb, pbuf, dbias_buffer.numel() * 4,
+                                                BT, OC, _stream(stream)))

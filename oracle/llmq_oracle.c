@@ -314,6 +314,36 @@ void orc_gemm_tn_e4m3(void* c, int c_is_f32, const uint8_t* a, const uint8_t* b,
     orc_gemm_tn_fp8(c, c_is_f32, a, b, 0, bias_bf16, bias_f32, sa, sb, M, N, K, accumulate);
 }
 
+/*
+ * Bias gradient (src/kernels/bias.cu:40-112, 151-195): dbias[oc] = bf16((float)dbias[oc] + scale * S[oc]) with
+ * S[oc] = sum_bt value(dout[bt, oc]).  The reference forms S in fp32 in an unspecified order; here S is
+ * the exact sum (fp64; exact for fp8 and bf16 inputs of these sizes) rounded once to fp32, so any fp32
+ * summation order lies within accumulation error of it.  fmt: 0 = e4m3, 1 = e5m2, 2 = bf16 (uint16).
+ * colsum / colabs (optional, may be NULL) receive S and sum |value| for error bounds.
+ */
+void orc_backward_bias_bf16(uint16_t* dbias, const void* dout, int fmt, const float* sa, const float* sb,
+                            int64_t BT, int OC, double* colsum, double* colabs) {
+    volatile float scale = 1.f;
+    if (sa && sb) scale = *sa * *sb;
+    for (int oc = 0; oc < OC; ++oc) {
+        double s = 0.0, sabs = 0.0;
+        for (int64_t r = 0; r < BT; ++r) {
+            double v;
+            if (fmt == 0) v = (double)orc_e4m3_decode(((const uint8_t*)dout)[r * OC + oc]);
+            else if (fmt == 1) v = (double)orc_e5m2_decode(((const uint8_t*)dout)[r * OC + oc]);
+            else v = (double)orc_bf16_to_f32(((const uint16_t*)dout)[r * OC + oc]);
+            s += v;
+            sabs += fabs(v);
+        }
+        if (colsum) colsum[oc] = s;
+        if (colabs) colabs[oc] = sabs;
+        volatile float t = (float)s;
+        t = t * scale;
+        t = t + orc_bf16_to_f32(dbias[oc]);
+        dbias[oc] = orc_f32_to_bf16(t);
+    }
+}
+
 /* ------------------------------------------------------------------------------------------------
  * Deterministic synthetic tensors: a counter-based generator (one 64-bit mix per element index),
  * so any slice can be produced independently and the same bytes feed the CPU and the GPU side.

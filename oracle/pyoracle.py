@@ -95,6 +95,8 @@ def lib():
     L.mt_gemm_tn_fp8.restype = C.c_int
     L.mt_gemm_tn_fp8.argtypes = [C.c_void_p, C.c_int, u8p, u8p, C.c_int, u16p, f32p, f32p,
                                  C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
+    L.orc_backward_bias_bf16.restype = None
+    L.orc_backward_bias_bf16.argtypes = [u16p, C.c_void_p, C.c_int, f32p, f32p, C.c_int64, C.c_int, f64p, f64p]
     _lib = L
     return L
 
@@ -253,3 +255,18 @@ def fill_int_e4m3(n, seed, stream, lo=-15, hi=15):
     vals = np.empty(int(n), dtype=np.int32)
     lib().orc_fill_int_e4m3(_p(out, C.c_uint8), _p(vals, C.c_int32), out.size, seed, stream, lo, hi)
     return out, vals
+
+
+def backward_bias(dbias, dout, fmt, sa=None, sb=None):
+    """dbias: uint16 bf16 [OC] (old value); dout: [BT, OC] uint8 codes (fmt "e4m3" / "e5m2") or uint16
+    bf16 (fmt "bf16").  Returns (new dbias uint16 [OC], exact column sums float64, sum |values| float64)."""
+    code = {"e4m3": 0, "e5m2": 1, "bf16": 2}[fmt]
+    dout = np.ascontiguousarray(dout, dtype=np.uint16 if code == 2 else np.uint8)
+    BT, OC = dout.shape
+    out = np.array(dbias, dtype=np.uint16, copy=True)
+    cs, ca = np.zeros(OC, dtype=np.float64), np.zeros(OC, dtype=np.float64)
+    ka = C.c_float(sa) if sa is not None else None
+    kb = C.c_float(sb) if sb is not None else None
+    lib().orc_backward_bias_bf16(_p(out, C.c_uint16), dout.ctypes.data, code, C.pointer(ka) if ka is not None else None,
+                                 C.pointer(kb) if kb is not None else None, BT, OC, _p(cs, C.c_double), _p(ca, C.c_double))
+    return out, cs, ca

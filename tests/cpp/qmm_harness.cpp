@@ -20,6 +20,7 @@ void orc_transpose_u8(uint8_t* dst, const uint8_t* src, int rows, int cols);
 void orc_gemm_tn_e4m3_exact_sampled(double* exact, double* sumabs, const uint8_t* a, const uint8_t* b, int M, int N, int K,
                                     const int32_t* idx_n, const int32_t* idx_m, int64_t count);
 void orc_fill_normal_bf16(uint16_t* out, int64_t n, uint64_t seed, uint64_t stream, float mean, float std);
+void orc_backward_bias_bf16(uint16_t* dbias, const void* dout, int fmt, const float* sa, const float* sb, int64_t BT, int OC, double* colsum, double* colabs);
 }
 
 #define HIP_OK(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) { std::printf("HIP error %s at line %d\n", hipGetErrorString(e_), __LINE__); return 2; } } while (0)
@@ -97,7 +98,14 @@ int main(int argc, char** argv) {
     abs_max(dout.Quant.abs_max(), dout.Value, (long)BT * OC, rs.DeviceProp, stream);
     quantize_with_abs_max(weight, weight.scale(), w_master, weight.abs_max(), (long)OC * C, rs.DeviceProp, stream);
     forward_qmm(out, inp, weight, no_bias, nullptr, workspace, B, T, C, OC, rs.DeviceProp, false, stream, EMatmulBackend::Custom);
-    backward_qmm(dinp, dweight, dout, inp, weight, false, rs, B, T, C, OC, reuse_inp, stream);
+    // bias gradient of the layer (the QKV projection has one): starts from a non-zero value, as an accumulated gradient
+    std::vector<uint16_t> hdb0(OC);
+    orc_fill_normal_bf16(hdb0.data(), hdb0.size(), 7, 4, 0.f, 1e-2f);
+    Tensor dbias = make(ETensorDType::BF16, dalloc<uint16_t>(OC), {OC});
+    HIP_OK(hipMemcpy(dbias.Data, hdb0.data(), (std::size_t)OC * 2, hipMemcpyHostToDevice));
+    const int bias_scratch = get_bias_backward_scratch_size(ETensorDType::BF16, OC, rs.DeviceProp);
+    Tensor bias_buffer = make(ETensorDType::FP32, dalloc<float>((std::size_t)bias_scratch / 4), {bias_scratch / 4});
+    backward_qmm(dinp, dweight, dbias, dout, inp, weight, bias_buffer, false, rs, B, T, C, OC, reuse_inp, stream);
     HIP_OK(hipStreamSynchronize(stream));
     EXPECT(rs.Top == 0 && rs.Live.empty(), "temporary stack not unwound");
     EXPECT(rs.HighWater == rs.Capacity, "backward_temp_bytes (%zu) != high-water mark (%zu)", rs.Capacity, rs.HighWater);
@@ -131,6 +139,21 @@ int main(int argc, char** argv) {
     check_gemm("forward", hy, {}, BT, OC, wq.data(), xq.data(), C, sw * sx);
     check_gemm("dgrad", hdx, {}, BT, C, wqt.data(), gq.data(), OC, sw * sg);
     check_gemm("wgrad", {}, hdw, OC, C, xqt.data(), gqt.data(), BT, sx * sg);
+
+    {   // dbias += sx*sg * column sums of the quantized gradient (llama_model.cpp:334-336)
+        std::vector<uint16_t> hdb(OC), want(hdb0);
+        std::vector<double> cs(OC), ca(OC);
+        HIP_OK(hipMemcpy(hdb.data(), dbias.Data, (std::size_t)OC * 2, hipMemcpyDeviceToHost));
+        orc_backward_bias_bf16(want.data(), gq.data(), 0, &sx, &sg, BT, OC, cs.data(), ca.data());
+        double worst = 0;
+        for (int oc = 0; oc < OC; ++oc) {
+            const double ref = cs[oc] * (double)(sx * sg) + (double)orc_bf16_to_f32(hdb0[oc]);
+            const double bound = std::ldexp(std::fabs(ref), -8) + std::ldexp((double)(sx * sg) * ca[oc], -18) + 1e-30;
+            worst = std::max(worst, std::fabs((double)orc_bf16_to_f32(hdb[oc]) - ref) / bound);
+        }
+        std::printf("%-8s worst error / bound %.3f\n", "dbias", worst);
+        EXPECT(worst <= 1.0, "dbias exceeds the element bound");
+    }
 
     // ---- error behaviour of the shim (reference: gemm_mma.cu:261-263, kernels.cpp:18-24) ----
     bool threw = false;

@@ -60,6 +60,13 @@ def test_invalid_arguments_are_rejected_without_a_gpu(capi):
     assert L.llmq_gemm_tn_e4m3_bf16(p, p, p, None, None, None, None, 4096, 128, 128, 128, 0, None) == INV
     assert b"workspace" in L.llmq_last_error()
     assert L.llmq_gemm_tn_e4m3_bf16(p, p, p, None, None, None, p + 4, 4096, 128, 128, 128, 0, None) == INV
+    # backward_bias: both-or-neither scales, vector-size rule, scratch size (bias.cu:163-168, kernels.cpp:378-380)
+    assert L.llmq_backward_bias_bf16(p, p, 0, p, None, p, 1 << 20, 8, 64, None) == INV
+    assert L.llmq_backward_bias_bf16(p, p, 0, None, None, p, 1 << 20, 8, 24, None) == INV
+    assert L.llmq_backward_bias_bf16(p, p, 0, None, None, p, 4, 8, 64, None) == INV
+    assert b"scratch buffer too small" in L.llmq_last_error()
+    assert L.llmq_backward_bias_bf16(p, p, 7, None, None, p, 1 << 20, 8, 64, None) == INV
+    assert L.llmq_backward_bias_scratch_bytes(8192, 1152, 0) >= 1152 * 4
     with pytest.raises(ValueError):
         capi.check(INV)
     with pytest.raises(RuntimeError):

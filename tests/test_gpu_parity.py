@@ -340,6 +340,72 @@ def test_gemm_matches_swapped_operand_transpose(K, O):
     assert torch.allclose(c1, c2.T, rtol=1e-5, atol=1e-4)
 
 
+# ------------------------------------------------------------------------------------ backward_bias
+BIAS_SHAPES = [(10, 64), (3, 256), (32, 128), (128, 512), (8192, 1152), (8192, 4608), (5000, 16), (16384, 2560)]
+
+
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2", "bf16"])
+@pytest.mark.parametrize("shape", BIAS_SHAPES)
+def test_backward_bias(K, O, fmt, shape):
+    """dbias += sa*sb * column sums of the (quantized) gradient, reference src/kernels/bias.cu:151-195 and
+    its tests scripts/test_kernels.py:834-890 (plain, scaled, accumulating).  Integer-valued gradients
+    make every fp32 partial sum exact -> bit-exact against the oracle; random gradients are checked
+    against the exact column sums within fp32 accumulation + bf16 rounding error."""
+    BT, OC = shape
+    rng = np.random.default_rng(BT * 7 + OC)
+    tdt = {"e4m3": torch.float8_e4m3fn, "e5m2": torch.float8_e5m2, "bf16": torch.bfloat16}[fmt]
+    buf = torch.empty(K.get_bias_backward_scratch_size(tdt, OC, BT) // 4 + 4, dtype=torch.float32, device="cuda")
+
+    def dev(x):
+        return dev_bf16(x) if fmt == "bf16" else dev_u8(x).view(tdt)
+
+    ints = rng.integers(-3, 4, (BT, OC))
+    if fmt == "bf16":
+        di = O.f32_to_bf16(ints.astype(np.float32))
+    else:
+        enc = O.lib().orc_e4m3_encode if fmt == "e4m3" else O.lib().orc_e5m2_encode
+        lut = np.array([enc(float(v)) for v in range(-3, 4)], dtype=np.uint8)
+        di = lut[ints + 3]
+    old = O.f32_to_bf16(rng.integers(-8, 9, OC).astype(np.float32))
+    for sa, sb, use_old in [(None, None, False), (0.25, 2.0, False), (0.5, 4.0, True)]:
+        start = old if use_old else np.zeros(OC, dtype=np.uint16)
+        want, _, _ = O.backward_bias(start, di, fmt, sa, sb)
+        dbias = dev_bf16(start).clone()
+        buf.fill_(float("nan"))                       # the scratch never needs clearing
+        K.backward_bias(dbias, dev(di), dev_scalar(sa) if sa is not None else None,
+                        dev_scalar(sb) if sb is not None else None, buf)
+        assert np.array_equal(host_bits(dbias), want), (sa, sb, use_old)
+    # random values
+    if fmt == "bf16":
+        dr = O.fill_normal_bf16(BT * OC, 77, BT + OC, 0.0, 1.0).reshape(BT, OC)
+    else:
+        dr = rng.integers(0, 256, (BT, OC)).astype(np.uint8)
+        dr[(dr & 0x7C) == 0x7C] ^= 0x40
+    startf = rng.standard_normal(OC).astype(np.float32)
+    start = O.f32_to_bf16(startf)
+    _, cs, ca = O.backward_bias(start, dr, fmt, 0.125, 0.5)
+    dbias = dev_bf16(start).clone()
+    K.backward_bias(dbias, dev(dr), dev_scalar(0.125), dev_scalar(0.5), buf)
+    got = O.bf16_to_f32(host_bits(dbias)).astype(np.float64)
+    ref = cs * 0.0625 + O.bf16_to_f32(start).astype(np.float64)
+    bound = 2.0 ** -8 * np.abs(ref) + 2.0 ** -18 * 0.0625 * ca + 1e-30
+    assert np.all(np.abs(got - ref) <= bound), float(np.max(np.abs(got - ref) / bound))
+
+
+def test_backward_bias_rejects_bad_arguments(K):
+    g = torch.zeros((8, 64), dtype=torch.float8_e4m3fn, device="cuda")
+    d = torch.zeros(64, dtype=torch.bfloat16, device="cuda")
+    s = torch.ones(1, device="cuda")
+    buf = torch.empty(K.get_bias_backward_scratch_size(torch.float8_e4m3fn, 64, 8) // 4, dtype=torch.float32, device="cuda")
+    with pytest.raises(ValueError):
+        K.backward_bias(d, g, s, None, buf)                                   # one scale only (bias.cu:163-165)
+    with pytest.raises(ValueError):
+        K.backward_bias(d, g, None, None, buf[:1])                            # scratch too small (kernels.cpp:378-380)
+    g2 = torch.zeros((8, 24), dtype=torch.float8_e4m3fn, device="cuda")
+    with pytest.raises(ValueError):
+        K.backward_bias(d[:24].contiguous(), g2, None, None, buf)             # OC % vector size (bias.cu:167-168)
+
+
 # ----------------------------------------------------------------------- configuration 1, end to end
 def test_config1_forward_pipeline(K, O):
     """X[4096x896]~N(0,1), W[4864x896]~N(0,0.02), seed 0: abs-max, quantize both, Y = X W^T (bf16)."""

@@ -347,3 +347,43 @@ def test_generators_are_deterministic_and_sane(O):
     assert np.array_equal(O.fill_normal_bf16(100, 4, 9, 0.0, 0.02), x1[:100])
     t = O.bf16_to_f32(O.fill_student_t3_bf16(1 << 16, 5, 1))
     assert np.isfinite(t).all() and np.abs(t).max() > 8.0 and abs(np.median(t)) < 0.02
+
+
+# ----------------------------------------------------------------------------------- backward_bias
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2", "bf16"])
+def test_backward_bias_vs_numpy(O, fmt):
+    """Column sums against numpy float64 / int64 (the constructions of scripts/test_kernels.py:834-890
+    in the reference: plain sum, with scales, accumulating into an existing dbias)."""
+    rng = np.random.default_rng(12)
+    BT, OC = 80, 64
+    if fmt == "bf16":
+        vals = rng.standard_normal((BT, OC)).astype(np.float32)
+        dout = O.f32_to_bf16(vals)
+        dec = O.bf16_to_f32(dout).astype(np.float64)
+    else:
+        dout = rng.integers(0, 256, (BT, OC)).astype(np.uint8)
+        if fmt == "e4m3":
+            dout[(dout & 0x7F) == 0x7F] = 0x7E
+            dec = O.e4m3_table()[dout].astype(np.float64)
+        else:
+            dout[(dout & 0x7C) == 0x7C] = 0x70
+            dec = O.e5m2_table()[dout].astype(np.float64)
+    zero = np.zeros(OC, dtype=np.uint16)
+    got, cs, ca = O.backward_bias(zero, dout, fmt)
+    assert np.allclose(cs, dec.sum(0), rtol=1e-12, atol=1e-12) and np.allclose(ca, np.abs(dec).sum(0), rtol=1e-12)
+    assert np.array_equal(got, O.f32_to_bf16(dec.sum(0).astype(np.float32)))
+    # scales and accumulation: dbias_new = bf16(old + 0.5 * sum), evaluated in fp32
+    old = O.f32_to_bf16(rng.standard_normal(OC).astype(np.float32))
+    got2, _, _ = O.backward_bias(old, dout, fmt, sa=0.25, sb=2.0)
+    want2 = O.f32_to_bf16((dec.sum(0).astype(np.float32) * np.float32(0.5) + O.bf16_to_f32(old)).astype(np.float32))
+    assert np.array_equal(got2, want2)
+    # integer-valued gradients: exact known answer
+    ints = rng.integers(-3, 4, (BT, OC))
+    if fmt == "bf16":
+        di = O.f32_to_bf16(ints.astype(np.float32))
+    else:
+        enc = O.lib().orc_e4m3_encode if fmt == "e4m3" else O.lib().orc_e5m2_encode
+        lut = {v: enc(float(v)) for v in range(-3, 4)}
+        di = np.vectorize(lut.get)(ints).astype(np.uint8)
+    got3, _, _ = O.backward_bias(zero, di, fmt)
+    assert np.array_equal(O.bf16_to_f32(got3), ints.sum(0).astype(np.float32))
