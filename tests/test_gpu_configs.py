@@ -259,3 +259,57 @@ def test_hip_graph_replay_matches_eager(K, O):
         for a, b in zip(want, got):
             assert torch.equal(a.view(torch.uint8) if a.dtype != torch.uint8 else a,
                                b.view(torch.uint8) if b.dtype != torch.uint8 else b), "replay for seed %d differs" % seed
+
+
+def test_backward_with_e5m2_gradients(K, O):
+    """The e5m2 gradient dtype (`--gradient-dtype=e5m2` in the reference): dY is quantized to e5m2 with the
+    same 448-based scale (src/kernels/quant.cu:79, 130-132), transposed as bytes, and multiplied as the b
+    operand of e4m3 x e5m2 matmuls (src/kernels/kernels.h:92-94); the bias gradient reads the same bytes
+    (src/kernels/bias.cu:193-195)."""
+    BT, C, OC = 4096, 896, 1152
+    F5 = torch.float8_e5m2
+    x = dev_bf16(O.fill_normal_bf16(BT * C, 6, 1).reshape(BT, C))
+    w = dev_bf16(O.fill_normal_bf16(OC * C, 6, 2, 0.0, 0.02).reshape(OC, C))
+    dy = dev_bf16(O.fill_normal_bf16(BT * OC, 6, 3, 0.0, 1e-3).reshape(BT, OC))
+    inp, wq, dout = QT(x), QT(w), QT(dy)
+    dout.quant = torch.empty(dy.shape, dtype=F5, device="cuda")
+    for t in (inp, wq, dout):
+        K.abs_max(t.abs_max, t.value)
+    K.quantize_with_abs_max(wq.quant, wq.scale, wq.value, wq.abs_max)
+    K.quantize_with_abs_max(inp.quant, inp.scale, inp.value, inp.abs_max)
+    # backward_qmm with an e5m2 gradient
+    K.quantize_with_abs_max(dout.quant, dout.scale, dout.value, dout.abs_max)
+    w_tp = torch.empty((C, OC), dtype=F8, device="cuda")
+    K.transpose(w_tp, wq.quant)
+    dinp = torch.empty((BT, C), dtype=torch.bfloat16, device="cuda")
+    K.matmul(dinp, w_tp, dout.quant, None, wq.scale, dout.scale, C, BT, OC, workspace=workspace())
+    a_tp = torch.empty((C, BT), dtype=F8, device="cuda")
+    g_tp = torch.empty((OC, BT), dtype=F5, device="cuda")
+    K.quantize_and_transpose_with_abs_max(a_tp, None, inp.value, inp.abs_max)
+    K.transpose(g_tp, dout.quant)
+    dweight = torch.empty((OC, C), dtype=torch.bfloat16, device="cuda")
+    K.matmul(dweight, a_tp, g_tp, None, inp.scale, dout.scale, C, OC, BT, workspace=workspace())
+    dbias = torch.zeros(OC, dtype=torch.bfloat16, device="cuda")
+    buf = torch.empty(K.get_bias_backward_scratch_size(F5, OC, BT) // 4, dtype=torch.float32, device="cuda")
+    K.backward_bias(dbias, dout.quant, inp.scale, dout.scale, buf)
+    torch.cuda.synchronize()
+
+    gbits = host_bits(dy)
+    ag = O.abs_max_bf16(gbits)
+    gc, dg_s = O.quantize_e4m3(gbits, ag, mt=False, fmt="e5m2")
+    assert np.array_equal(host_bits(dout.quant), gc) and dout.stats.cpu().numpy()[1] == dg_s
+    assert np.array_equal(host_bits(g_tp), gc.T)
+    xc, dx_s = check_quant(O, inp, "x")
+    wc, dw_s = check_quant(O, wq, "w")
+    for name, c, a_codes, b_codes, sa in (("dgrad e5m2", dinp, np.ascontiguousarray(wc.T), gc, dw_s),
+                                          ("wgrad e5m2", dweight, np.ascontiguousarray(xc.T), np.ascontiguousarray(gc.T), dx_s)):
+        N, M = c.shape
+        idx_n, idx_m = sample_idx(N, M, 61)
+        ex, sabs = O.gemm_exact_sampled(a_codes, b_codes, idx_n, idx_m, b_e5m2=True)
+        got = c.float().cpu().numpy()[idx_n, idx_m]
+        mx, fro = gemm_check(got, ex, sabs, np.float32(np.float32(sa) * np.float32(dg_s)), True)
+        print("%-12s max-abs err %.3e  rel-Frobenius %.3e" % (name, mx, fro))
+    want, cs, ca = O.backward_bias(np.zeros(OC, dtype=np.uint16), gc, "e5m2", float(dx_s), float(dg_s))
+    got = O.bf16_to_f32(host_bits(dbias)).astype(np.float64)
+    ref = cs * float(np.float32(dx_s) * np.float32(dg_s))
+    assert np.all(np.abs(got - ref) <= 2.0 ** -8 * np.abs(ref) + 2.0 ** -18 * float(dx_s * dg_s) * ca + 1e-30)
