@@ -74,6 +74,15 @@ int llmq_quantize_transpose_e4m3_bf16(uint8_t* out, float* scale_or_null, const 
                                       const float* absmax, int rows, int cols, void* stream);
 
 /*
+ * Extension with no counterpart in the reference (it reads the tensor twice instead: quantize_with_abs_max
+ * followed by transpose of the codes, src/models/llama_model.cpp:310-331): one read of in[rows, cols] produces
+ * both out[r*cols + c] and out_transposed[c*rows + r], the same bytes the two reference calls give.
+ * format: 0 = e4m3, 1 = e5m2 (448-based scale for both, as src/kernels/quant.cu:79).  rows, cols multiples of 8.
+ */
+int llmq_quantize_both_bf16(uint8_t* out, uint8_t* out_transposed, float* scale_or_null, const uint16_t* in,
+                            const float* absmax, int rows, int cols, int format, void* stream);
+
+/*
  * Byte transpose: dst[c*rows + r] = src[r*cols + c]  (e4m3 / e5m2 codes).  Any rows, cols >= 0.
  * Replaces: transpose(__nv_fp8_e4m3*, const __nv_fp8_e4m3*, int rows, int cols, cudaStream_t)
  *           src/kernels/kernels.h:267 (and the e5m2 overload :268), src/kernels/transpose.cu:38-43.

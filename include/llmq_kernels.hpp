@@ -207,6 +207,19 @@ inline void transpose(Tensor& dst, const Tensor& src, int rows, int cols, hipStr
     else llmq_detail::unsupported(__func__, dst, src);
 }
 
+// Extension (no counterpart in the reference): quantize_with_abs_max and the transpose of its result from
+// one read of the input.  out[rows, cols] and out_tp[cols, rows] must have the same fp8 dtype.
+inline void quantize_with_abs_max_and_transpose(Tensor& out, Tensor& out_tp, float* scale_ptr, const Tensor& in,
+                                                const float* abs_max, int rows, int cols, const hipDeviceProp_t&,
+                                                hipStream_t stream) {
+    if (in.DType != ETensorDType::BF16 || out.DType != out_tp.DType ||
+        (out.DType != ETensorDType::FP8_E4M3 && out.DType != ETensorDType::FP8_E5M2))
+        llmq_detail::unsupported(__func__, out, out_tp, in);
+    llmq_detail::check(llmq_quantize_both_bf16(reinterpret_cast<uint8_t*>(out.Data), reinterpret_cast<uint8_t*>(out_tp.Data),
+                                               scale_ptr, llmq_detail::u16(in.get<__hip_bfloat16>()), abs_max, rows, cols,
+                                               out.DType == ETensorDType::FP8_E5M2 ? 1 : 0, stream));
+}
+
 // ---- matmul (reference: src/kernels/kernels.h:72-78, 88-90, 96-98) --------------------------------------
 // Row-major a[M,K], b[N,K] -> row-major c[N,M] = (b . a^T) * (*scale_a * *scale_b) (+ bias[M]) (+ c).
 inline void matmul(__hip_bfloat16* c, const __hip_fp8_e4m3* a, const __hip_fp8_e4m3* b, const __hip_bfloat16* bias,

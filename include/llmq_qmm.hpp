@@ -21,6 +21,9 @@ struct QmmRunState {
     llmqBlasHandle_t BlasHandle = nullptr;
     Tensor Workspace{};
     EMatmulBackend MatmulBackend = EMatmulBackend::Custom;
+    // Extension: quantize the output gradient and produce its transpose from one read of dout.Value (saves one
+    // read and one launch per layer; the transposed gradient then lives on the stack during the dgrad as well).
+    bool FuseGradTranspose = false;
     std::vector<std::byte*> Live;
 
     Tensor temp_alloc(ETensorDType dtype, const std::vector<long>& shape) {
@@ -40,9 +43,10 @@ struct QmmRunState {
         t.Data = nullptr;
     }
     // Bytes of stack backward_qmm needs for one layer (the dry run of llama_run_state.cpp:362-390).
-    static std::size_t backward_temp_bytes(int B, int T, int C, int OC) {
+    static std::size_t backward_temp_bytes(int B, int T, int C, int OC, bool fuse_grad_transpose = false) {
         auto up = [](std::size_t b) { return (b + 4095) / 4096 * 4096; };
         const std::size_t wt = up((std::size_t)C * OC), at = up((std::size_t)C * B * T), gt = up((std::size_t)OC * B * T);
+        if (fuse_grad_transpose) return gt + (wt > at ? wt : at);
         return wt > at + gt ? wt : at + gt;
     }
 };
@@ -68,8 +72,15 @@ inline void backward_qmm(Tensor& dinp, Tensor& dweight, Tensor dbias, Quantizabl
                          int C, int OC, bool reuse_inp, hipStream_t stream) {
     if (weight.DType != ETensorDType::FP8_E4M3)
         throw std::invalid_argument("backward_qmm: this build implements the FP8 (e4m3 weight) branch only");
-    quantize_with_abs_max(dout.Quant, dout.Quant.scale(), dout.Value, dout.Quant.abs_max(), (long)B * T * OC,
-                          rs.DeviceProp, stream);
+    Tensor grad_tp{};
+    if (rs.FuseGradTranspose) {
+        grad_tp = rs.temp_alloc(dout.Quant.DType, {OC, (long)B * T});
+        quantize_with_abs_max_and_transpose(dout.Quant, grad_tp, dout.Quant.scale(), dout.Value, dout.Quant.abs_max(),
+                                            B * T, OC, rs.DeviceProp, stream);
+    } else {
+        quantize_with_abs_max(dout.Quant, dout.Quant.scale(), dout.Value, dout.Quant.abs_max(), (long)B * T * OC,
+                              rs.DeviceProp, stream);
+    }
 
     auto& inp_q = inp.Quant;
     Tensor weight_tp = rs.temp_alloc(inp_q.DType, {C, OC});
@@ -80,7 +91,7 @@ inline void backward_qmm(Tensor& dinp, Tensor& dweight, Tensor dbias, Quantizabl
     rs.temp_free(weight_tp);
 
     Tensor activation_tp = rs.temp_alloc(inp_q.DType, {C, (long)B * T});
-    Tensor grad_tp = rs.temp_alloc(rs.GradDType, {OC, (long)B * T});
+    if (!rs.FuseGradTranspose) grad_tp = rs.temp_alloc(dout.Quant.DType, {OC, (long)B * T});
     if (reuse_inp) {
         transpose(activation_tp, inp_q, B * T, C, stream);
     } else {
@@ -88,14 +99,19 @@ inline void backward_qmm(Tensor& dinp, Tensor& dweight, Tensor dbias, Quantizabl
         quantize_and_transpose_with_abs_max(activation_tp, activation_tp.scale(), inp.Value, inp.Quant.abs_max(),
                                             B * T, C, rs.DeviceProp, stream);
     }
-    transpose(grad_tp, dout.Quant, B * T, OC, stream);
+    if (!rs.FuseGradTranspose) transpose(grad_tp, dout.Quant, B * T, OC, stream);
     matmul(dweight, activation_tp, grad_tp, no_bias, inp_q.scale(), dout.Quant.scale(), rs.BlasHandle, rs.Workspace, C,
            OC, B * T, EMMTranspose::TN, accumulate_gradient, stream, rs.MatmulBackend);
     if (!dbias.empty()) {
         backward_bias(dbias, dout.Quant, inp_q.scale(), dout.Quant.scale(), bias_buffer, B, T, OC, rs.DeviceProp, stream);
     }
-    rs.temp_free(grad_tp);
-    rs.temp_free(activation_tp);
+    if (rs.FuseGradTranspose) {
+        rs.temp_free(activation_tp);
+        rs.temp_free(grad_tp);
+    } else {
+        rs.temp_free(grad_tp);
+        rs.temp_free(activation_tp);
+    }
 }
 
 #endif  // LLMQ_QMM_HPP

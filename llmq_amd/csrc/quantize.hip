@@ -95,8 +95,11 @@ constexpr int kQtRows = 256;       // tile extent along the input rows (= contig
 constexpr int kQtStride = 65;      // LDS row stride in dwords (64 dwords of payload + 1 pad)
 
 // NCH = number of 8-column chunks per tile: the tile is [kQtRows rows] x [8*NCH cols].
-template <int NCH, bool ROW_MAJOR_GRID>
+// BOTH: the untransposed codes are written as well (out_plain[r*cols + c]), from the same single read of
+// the input: 8 bytes per lane and row, 8*NCH contiguous bytes per row segment.
+template <int FMT, int NCH, bool ROW_MAJOR_GRID, bool BOTH>
 __global__ __launch_bounds__(256) void quantize_transpose_kernel(uint8_t* __restrict__ out,
+                                                                 uint8_t* __restrict__ out_plain,
                                                                  float* __restrict__ scale_ptr,
                                                                  const uint16_t* __restrict__ in,
                                                                  const float* __restrict__ absmax, int rows,
@@ -139,12 +142,20 @@ __global__ __launch_bounds__(256) void quantize_transpose_kernel(uint8_t* __rest
                                   {v[p][3].x, v[p][3].y, v[p][3].z, v[p][3].w}};
 #pragma unroll
         for (int k = 0; k < 4; ++k) {  // word k holds columns 2k (low half) and 2k+1 (high half)
-            const uint32_t even = encode4<kE4M3>(s * bf16_lo(w[0][k]), s * bf16_lo(w[1][k]),
-                                                 s * bf16_lo(w[2][k]), s * bf16_lo(w[3][k]));
-            const uint32_t odd = encode4<kE4M3>(s * bf16_hi(w[0][k]), s * bf16_hi(w[1][k]),
-                                                s * bf16_hi(w[2][k]), s * bf16_hi(w[3][k]));
+            const uint32_t even = encode4<FMT>(s * bf16_lo(w[0][k]), s * bf16_lo(w[1][k]),
+                                               s * bf16_lo(w[2][k]), s * bf16_lo(w[3][k]));
+            const uint32_t odd = encode4<FMT>(s * bf16_hi(w[0][k]), s * bf16_hi(w[1][k]),
+                                              s * bf16_hi(w[2][k]), s * bf16_hi(w[3][k]));
             tile[(8 * chunk + 2 * k) * kQtStride + rq] = even;
             tile[(8 * chunk + 2 * k + 1) * kQtStride + rq] = odd;
+        }
+        if constexpr (BOTH) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int row = r0 + 4 * rq + j;
+                if (row < rows && col < cols)
+                    *reinterpret_cast<uint2*>(out_plain + (int64_t)row * cols + col) = encode8<FMT>(v[p][j], s);
+            }
         }
     }
     __syncthreads();
@@ -206,39 +217,62 @@ extern "C" int llmq_quantize_e5m2_bf16(uint8_t* out, float* scale_or_null, const
 
 extern "C" void llmq_debug_set_qt_order(int v) { llmq::g_qt_row_major_grid = v; }
 
-extern "C" int llmq_quantize_transpose_e4m3_bf16(uint8_t* out, float* scale_or_null, const uint16_t* in,
-                                                 const float* absmax, int rows, int cols, void* stream) {
-    using namespace llmq;
+namespace llmq {
+
+template <int FMT, bool BOTH>
+static int launch_quantize_transpose(uint8_t* out, uint8_t* out_plain, float* scale_or_null, const uint16_t* in,
+                                     const float* absmax, int rows, int cols, hipStream_t st) {
     LLMQ_REQUIRE(rows >= 0 && cols >= 0, "quantize_and_transpose_with_abs_max: negative shape %d x %d", rows, cols);
     LLMQ_REQUIRE(rows % 8 == 0 && cols % 8 == 0,
                  "quantize_and_transpose_with_abs_max: rows (%d) and cols (%d) must be multiples of 8", rows, cols);
     LLMQ_REQUIRE(absmax != nullptr, "quantize_and_transpose_with_abs_max: abs_max pointer is null");
     const bool empty = rows == 0 || cols == 0;
-    LLMQ_REQUIRE(empty || (out != nullptr && in != nullptr), "quantize_and_transpose_with_abs_max: null tensor pointer");
-    LLMQ_REQUIRE(aligned16(in) && aligned16(out), "quantize_and_transpose_with_abs_max: tensors must be 16-byte aligned");
-    hipStream_t st = static_cast<hipStream_t>(stream);
+    LLMQ_REQUIRE(empty || (out != nullptr && in != nullptr && (!BOTH || out_plain != nullptr)),
+                 "quantize_and_transpose_with_abs_max: null tensor pointer");
+    LLMQ_REQUIRE(aligned16(in) && aligned16(out) && aligned16(out_plain),
+                 "quantize_and_transpose_with_abs_max: tensors must be 16-byte aligned");
     const int rows_mult16 = rows % 16 == 0;
     const unsigned gy = empty ? 1u : (unsigned)((rows + kQtRows - 1) / kQtRows);
     // Wide tiles (256-byte row segments on the read side) once there are enough of them to fill the chip.
     const int64_t wide_tiles = (int64_t)((cols + 127) / 128) * gy;
     const bool rm = g_qt_row_major_grid != 0;
+    const int r = empty ? 0 : rows, c = empty ? 0 : cols;
     if (!empty && cols >= 128 && wide_tiles >= 2LL * cu_count()) {
         const unsigned gx = (unsigned)((cols + 127) / 128);
         if (rm && gx <= 65535u)
-            hipLaunchKernelGGL((quantize_transpose_kernel<16, true>), dim3(gy, gx), dim3(256), 0, st, out, scale_or_null,
-                               in, absmax, rows, cols, rows_mult16);
+            hipLaunchKernelGGL((quantize_transpose_kernel<FMT, 16, true, BOTH>), dim3(gy, gx), dim3(256), 0, st, out,
+                               out_plain, scale_or_null, in, absmax, r, c, rows_mult16);
         else
-            hipLaunchKernelGGL((quantize_transpose_kernel<16, false>), dim3(gx, gy), dim3(256), 0, st, out, scale_or_null,
-                               in, absmax, rows, cols, rows_mult16);
+            hipLaunchKernelGGL((quantize_transpose_kernel<FMT, 16, false, BOTH>), dim3(gx, gy), dim3(256), 0, st, out,
+                               out_plain, scale_or_null, in, absmax, r, c, rows_mult16);
     } else {
         const unsigned gx = empty ? 1u : (unsigned)((cols + 63) / 64);
         if (rm && gx <= 65535u)
-            hipLaunchKernelGGL((quantize_transpose_kernel<8, true>), dim3(gy, gx), dim3(256), 0, st, out, scale_or_null, in,
-                               absmax, empty ? 0 : rows, empty ? 0 : cols, rows_mult16);
+            hipLaunchKernelGGL((quantize_transpose_kernel<FMT, 8, true, BOTH>), dim3(gy, gx), dim3(256), 0, st, out,
+                               out_plain, scale_or_null, in, absmax, r, c, rows_mult16);
         else
-            hipLaunchKernelGGL((quantize_transpose_kernel<8, false>), dim3(gx, gy), dim3(256), 0, st, out, scale_or_null, in,
-                               absmax, empty ? 0 : rows, empty ? 0 : cols, rows_mult16);
+            hipLaunchKernelGGL((quantize_transpose_kernel<FMT, 8, false, BOTH>), dim3(gx, gy), dim3(256), 0, st, out,
+                               out_plain, scale_or_null, in, absmax, r, c, rows_mult16);
     }
     LLMQ_HIP_TRY(hipGetLastError());
     return LLMQ_OK;
+}
+
+}  // namespace llmq
+
+extern "C" int llmq_quantize_transpose_e4m3_bf16(uint8_t* out, float* scale_or_null, const uint16_t* in,
+                                                 const float* absmax, int rows, int cols, void* stream) {
+    return llmq::launch_quantize_transpose<llmq::kE4M3, false>(out, nullptr, scale_or_null, in, absmax, rows, cols,
+                                                               static_cast<hipStream_t>(stream));
+}
+
+extern "C" int llmq_quantize_both_bf16(uint8_t* out, uint8_t* out_transposed, float* scale_or_null, const uint16_t* in,
+                                       const float* absmax, int rows, int cols, int format, void* stream) {
+    using namespace llmq;
+    LLMQ_REQUIRE(format == kE4M3 || format == kE5M2, "quantize (plain + transposed): unknown fp8 format %d", format);
+    LLMQ_REQUIRE(out != out_transposed || out == nullptr, "quantize (plain + transposed): outputs must be distinct");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (format == kE4M3)
+        return launch_quantize_transpose<kE4M3, true>(out_transposed, out, scale_or_null, in, absmax, rows, cols, st);
+    return launch_quantize_transpose<kE5M2, true>(out_transposed, out, scale_or_null, in, absmax, rows, cols, st);
 }

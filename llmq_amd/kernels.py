@@ -69,6 +69,22 @@ def quantize_and_transpose_with_abs_max(out, scale, x, abs_max, stream=0):
     capi.check(capi.lib.llmq_quantize_transpose_e4m3_bf16(o, s, i, a, x.shape[0], x.shape[1], _stream(stream)))
 
 
+def quantize_with_abs_max_and_transpose(out, out_t, scale, x, abs_max, stream=0):
+    """One read of x [rows, cols] (bf16) gives out [rows, cols] and out_t [cols, rows] in the fp8 dtype of
+    `out` -- the bytes of quantize_with_abs_max followed by transpose.  No counterpart in the reference."""
+    if x.dim() != 2 or out.shape != x.shape or out_t.dim() != 2 or out_t.shape[0] != x.shape[1] or out_t.shape[1] != x.shape[0]:
+        raise ValueError("x and out must be [rows, cols], out_t [cols, rows]")
+    if out.dtype != out_t.dtype:
+        raise ValueError("out and out_t must have the same dtype")
+    o = _dev(out, "out", _FP8)
+    ot = _dev(out_t, "out_t", _FP8)
+    s = _dev(scale, "scale", (torch.float32,), optional=True)
+    i = _dev(x, "x", (torch.bfloat16,))
+    a = _dev(abs_max, "abs_max", (torch.float32,))
+    fmt = 1 if out.dtype == torch.float8_e5m2 else 0
+    capi.check(capi.lib.llmq_quantize_both_bf16(o, ot, s, i, a, x.shape[0], x.shape[1], fmt, _stream(stream)))
+
+
 def transpose(dst, src, stream=0):
     """src: [rows, cols] fp8 codes -> dst: [cols, rows]."""
     if src.dim() != 2 or dst.dim() != 2 or dst.shape[0] != src.shape[1] or dst.shape[1] != src.shape[0]:

@@ -62,11 +62,13 @@ static void check_gemm(const char* name, const std::vector<uint16_t>& got_bf16, 
 int main(int argc, char** argv) {
     const int BT = argc > 1 ? std::atoi(argv[1]) : 1024, C = argc > 2 ? std::atoi(argv[2]) : 896, OC = argc > 3 ? std::atoi(argv[3]) : 1152;
     const bool reuse_inp = argc > 4 && std::atoi(argv[4]) != 0;
+    const bool fuse = argc > 5 && std::atoi(argv[5]) != 0;   // gradient quantize + transpose from one read
     const int B = 1, T = BT;
-    std::printf("qmm_harness BT=%d C=%d OC=%d reuse_inp=%d\n", BT, C, OC, (int)reuse_inp);
+    std::printf("qmm_harness BT=%d C=%d OC=%d reuse_inp=%d fuse=%d\n", BT, C, OC, (int)reuse_inp, (int)fuse);
     hipStream_t stream; HIP_OK(hipStreamCreate(&stream));
     QmmRunState rs; HIP_OK(hipGetDeviceProperties(&rs.DeviceProp, 0));
-    rs.Capacity = QmmRunState::backward_temp_bytes(B, T, C, OC);
+    rs.FuseGradTranspose = fuse;
+    rs.Capacity = QmmRunState::backward_temp_bytes(B, T, C, OC, fuse);
     rs.Arena = dalloc<std::byte>(rs.Capacity);
 
     std::vector<uint16_t> hx((std::size_t)BT * C), hw((std::size_t)OC * C), hdy((std::size_t)BT * OC);

@@ -11,7 +11,8 @@ BIN = os.path.join(HERE, "cpp", "build", "qmm_harness")
 
 
 @pytest.mark.parametrize("args", [("1024", "896", "1152", "0"), ("2048", "896", "896", "1"), ("512", "4864", "896", "0"),
-                                  ("4096", "1536", "1792", "0")])
+                                  ("4096", "1536", "1792", "0"), ("1024", "896", "1152", "0", "1"),
+                                  ("2048", "1152", "896", "1", "1")])
 def test_qmm_harness(args):
     assert os.path.exists(BIN), "build it with `make -C tests/cpp` (done by __graft_entry__.build())"
     r = subprocess.run([BIN, *args], capture_output=True, text=True, timeout=150)

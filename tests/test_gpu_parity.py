@@ -129,6 +129,28 @@ def test_quantize_transpose_bit_exact(K, O, shape):
     assert np.array_equal(host_bits(out2), want.T)
 
 
+@pytest.mark.parametrize("fmt", [torch.float8_e4m3fn, torch.float8_e5m2])
+@pytest.mark.parametrize("shape", QT_SHAPES)
+def test_quantize_plain_and_transposed_in_one_read(K, O, shape, fmt):
+    """The fused kernel must give exactly the bytes of quantize_with_abs_max followed by transpose (the
+    two-route byte identity idea of src/testing/test-swiglu.cu:243-315), for both fp8 formats."""
+    rows, cols = shape
+    x = O.fill_student_t3_bf16(rows * cols, 9, rows + cols, 0.5).reshape(rows, cols)
+    x[0, 0] = 0x7FC0                                   # a NaN
+    x[rows - 1, cols - 1] = 0xFF80                     # -Inf
+    am = O.abs_max_bf16(x[np.isfinite(O.bf16_to_f32(x))])
+    e5 = fmt == torch.float8_e5m2
+    want, d = O.quantize_e4m3(x, am, mt=not e5, fmt="e5m2" if e5 else "e4m3")
+    xd = dev_bf16(x)
+    out = torch.zeros((rows, cols), dtype=fmt, device="cuda")
+    out_t = torch.zeros((cols, rows), dtype=fmt, device="cuda")
+    sc = torch.zeros(1, device="cuda")
+    K.quantize_with_abs_max_and_transpose(out, out_t, sc, xd, dev_scalar(am))
+    assert np.array_equal(host_bits(out), want.reshape(rows, cols))
+    assert np.array_equal(host_bits(out_t), want.reshape(rows, cols).T)
+    assert sc.cpu().numpy()[0] == d
+
+
 @pytest.mark.parametrize("shape", QT_SHAPES + [(1, 1), (3, 5), (17, 33), (100, 7), (64, 65), (4864, 896), (16, 4096)])
 def test_transpose_bit_exact(K, shape):
     rows, cols = shape
