@@ -106,7 +106,7 @@ def matmul(c, a, b, bias, scale_a, scale_b, M, N, K, accumulate=False, stream=0,
     if workspace is not None:
         pws = _dev(workspace, "workspace", (torch.uint8, torch.int8, torch.float32))
         ws_bytes = workspace.numel() * workspace.element_size()
-    pa = _dev(a, "a", (torch.float8_e4m3fn, torch.uint8))
+    pa = _dev(a, "a", (torch.float8_e4m3fn, torch.uint8))   # e5m2 is supported for b only (kernels.h:92-94)
     pb = _dev(b, "b", (torch.float8_e4m3fn, torch.float8_e5m2, torch.uint8))
     b_e5m2 = bool(b_e5m2) or b.dtype == torch.float8_e5m2
     pc = _dev(c, "c", (torch.bfloat16, torch.float32))

@@ -71,3 +71,15 @@ def test_invalid_arguments_are_rejected_without_a_gpu(capi):
         capi.check(INV)
     with pytest.raises(RuntimeError):
         capi.check(capi.LLMQ_ERR_RUNTIME)
+
+
+def test_reference_python_ops_register_without_a_gpu():
+    """llmq_amd.ops registers the reference's operator names (src/binding/python/kernels.py:118-165) at import."""
+    import torch
+    from llmq_amd import ops
+    for name in ("abs_max", "quantize_with_abs_max", "quantize_and_transpose_with_abs_max", "transpose", "matmul",
+                 "backward_bias"):
+        assert hasattr(torch.ops.llmq, name)
+    assert ops.MODE_NT == 2 and ops.create_cublas_handle() == 0
+    with pytest.raises(ValueError):                      # host tensors are rejected before any launch
+        ops.abs_max(torch.zeros(1), torch.zeros(8, dtype=torch.bfloat16))

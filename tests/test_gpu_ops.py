@@ -1,0 +1,82 @@
+"""The reference's Python-visible contract for the path (src/binding/python/kernels.py:118-165): the same
+operator names and signatures, called through torch.ops.llmq.* and through the module functions, on the
+constructions of the reference's scripts/test_kernels.py (abs-max :40-65, quantize :641-652, 1168-1185,
+matmul :937-1040 restricted to what FP8 supports, backward_bias :834-890)."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import gemm_check
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def P():
+    from llmq_amd import ops
+    return ops
+
+
+def test_ops_are_registered_with_reference_names(P):
+    for name in ("abs_max", "quantize_with_abs_max", "quantize_and_transpose_with_abs_max", "transpose", "matmul",
+                 "backward_bias"):
+        assert hasattr(torch.ops.llmq, name)
+
+
+def test_abs_max_and_quantize_through_ops(P, O):
+    torch.manual_seed(0)
+    x = torch.randn(1000 * 64, device="cuda", dtype=torch.bfloat16) * 3
+    scale = torch.zeros(1, device="cuda")
+    torch.ops.llmq.abs_max(scale, x)
+    assert scale.item() == x.float().abs().max().item()                      # exact, as test_kernels.py:56-65
+    q = torch.empty(x.shape, dtype=torch.float8_e4m3fn, device="cuda")
+    dq = torch.zeros(1, device="cuda")
+    P.quantize_with_abs_max(q, dq, x, scale)
+    assert dq.item() == pytest.approx(scale.item() / 448.0, rel=1e-6)        # test_kernels.py:223-241
+    back = q.float() * dq
+    assert torch.allclose(back, x.float(), rtol=0.1, atol=0.1 * scale.item() / 448 * 8)   # loose dequant check :641-652
+    x2 = x.view(1000, 64)
+    qt = torch.empty((64, 1000), dtype=torch.float8_e4m3fn, device="cuda")
+    P.quantize_and_transpose_with_abs_max(qt, dq, x2, scale)
+    assert torch.equal(qt.view(torch.uint8), q.view(1000, 64).view(torch.uint8).T)
+    t2 = torch.empty((1000, 64), dtype=torch.float8_e4m3fn, device="cuda")
+    P.transpose(t2, qt)
+    assert torch.equal(t2.view(torch.uint8), q.view(1000, 64).view(torch.uint8))
+
+
+def test_matmul_torch_convention(P, O):
+    """c[M,N] = (a[M,K] @ b[N,K]^T) * scale_a * scale_b + bias[N] (+ c), mode NT."""
+    M, N, Kd = 384, 256, 512
+    rng = np.random.default_rng(4)
+    a = rng.integers(0, 0x7E, (M, Kd)).astype(np.uint8)
+    b = (rng.integers(0, 0x7E, (N, Kd)).astype(np.uint8) | 0x80)
+    ad = torch.from_numpy(a).cuda().view(torch.float8_e4m3fn)
+    bd = torch.from_numpy(b).cuda().view(torch.float8_e4m3fn)
+    sa, sb = torch.tensor([0.03], device="cuda"), torch.tensor([0.5], device="cuda")
+    bias = torch.randn(N, device="cuda", dtype=torch.bfloat16)
+    ws = torch.empty(32 << 20, dtype=torch.uint8, device="cuda")
+    handle = P.create_cublas_handle()
+    c = torch.randn(M, N, device="cuda", dtype=torch.bfloat16)
+    old = c.clone()
+    P.matmul(c, ad, bd, bias, sa, sb, handle, ws, P.MODE_NT, True)
+    P.destroy_cublas_handle(handle)
+    exact, sumabs = O.gemm_exact(b, a)            # oracle convention: rows of the first operand index the columns of c
+    scale = np.float32(np.float32(0.03) * np.float32(0.5))
+    extra = bias.float().cpu().numpy().astype(np.float64)[None, :] + old.float().cpu().numpy().astype(np.float64)
+    gemm_check(c.float().cpu().numpy(), exact, sumabs, scale, True, extra=extra)
+    with pytest.raises(ValueError):
+        P.matmul(c, ad, bd, None, None, None, 0, ws, P.MODE_NN, False)       # FP8 is TN-only in the kernel layer
+    with pytest.raises(ValueError):
+        P.matmul(c, ad, bd[:, :256].contiguous(), None, None, None, 0, ws, P.MODE_NT, False)
+
+
+def test_backward_bias_through_ops(P):
+    torch.manual_seed(0)
+    B, T, OC = 8, 16, 512                                                    # test_kernels.py:837-853
+    dout = torch.randn((B, T, OC), device="cuda", dtype=torch.bfloat16)
+    initial = torch.randn((OC,), device="cuda", dtype=torch.bfloat16)
+    dbias = initial.clone()
+    buf = torch.empty(P.get_bias_backward_scratch_size(torch.bfloat16, OC) // 4, device="cuda", dtype=torch.float32)
+    torch.ops.llmq.backward_bias(dbias, dout, None, None, buf)
+    ref = (initial.float() + dout.float().sum(dim=(0, 1))).to(torch.bfloat16)
+    assert torch.allclose(dbias.float(), ref.float(), rtol=1e-2, atol=1e-2)
