@@ -64,6 +64,16 @@ int llmq_quantize_e5m2_bf16(uint8_t* out, float* scale_or_null, const uint16_t* 
                             int64_t n, void* stream);
 
 /*
+ * fp32-input variants (fp32 master weights / fp32 model dtype); same arithmetic, any n >= 0.
+ * Replaces: quantize_with_abs_max(__nv_fp8_e4m3* out, float* scale_ptr, const float* in, ...) src/kernels/kernels.h:251
+ *           and the __nv_fp8_e5m2 overload :252, src/kernels/quant.cu:121-126.
+ */
+int llmq_quantize_e4m3_f32(uint8_t* out, float* scale_or_null, const float* in, const float* absmax, int64_t n,
+                           void* stream);
+int llmq_quantize_e5m2_f32(uint8_t* out, float* scale_or_null, const float* in, const float* absmax, int64_t n,
+                           void* stream);
+
+/*
  * As llmq_quantize_e4m3_bf16 on a row-major [rows, cols] input, written transposed:
  * out[c*rows + r] = q(in[r*cols + c]).  rows % 8 == 0 and cols % 8 == 0 required.
  * Replaces: quantize_and_transpose_with_abs_max(__nv_fp8_e4m3*, float*, const nv_bfloat16*,

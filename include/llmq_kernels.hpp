@@ -168,9 +168,21 @@ inline void quantize_with_abs_max(__hip_fp8_e5m2* out, float* scale_ptr, const _
                                   long N, const hipDeviceProp_t&, hipStream_t stream) {
     llmq_detail::check(llmq_quantize_e5m2_bf16(llmq_detail::u8(out), scale_ptr, llmq_detail::u16(in), abs_max, N, stream));
 }
+inline void quantize_with_abs_max(__hip_fp8_e4m3* out, float* scale_ptr, const float* in, const float* abs_max, long N,
+                                  const hipDeviceProp_t&, hipStream_t stream) {
+    llmq_detail::check(llmq_quantize_e4m3_f32(llmq_detail::u8(out), scale_ptr, in, abs_max, N, stream));
+}
+inline void quantize_with_abs_max(__hip_fp8_e5m2* out, float* scale_ptr, const float* in, const float* abs_max, long N,
+                                  const hipDeviceProp_t&, hipStream_t stream) {
+    llmq_detail::check(llmq_quantize_e5m2_f32(llmq_detail::u8(out), scale_ptr, in, abs_max, N, stream));
+}
 inline void quantize_with_abs_max(Tensor& out, float* scale_ptr, const Tensor& in, const float* abs_max, long N,
                                   const hipDeviceProp_t& dp, hipStream_t stream) {
-    if (in.DType == ETensorDType::BF16 && out.DType == ETensorDType::FP8_E4M3)
+    if (in.DType == ETensorDType::FP32 && out.DType == ETensorDType::FP8_E4M3)
+        quantize_with_abs_max(out.get<__hip_fp8_e4m3>(), scale_ptr, in.get<float>(), abs_max, N, dp, stream);
+    else if (in.DType == ETensorDType::FP32 && out.DType == ETensorDType::FP8_E5M2)
+        quantize_with_abs_max(out.get<__hip_fp8_e5m2>(), scale_ptr, in.get<float>(), abs_max, N, dp, stream);
+    else if (in.DType == ETensorDType::BF16 && out.DType == ETensorDType::FP8_E4M3)
         quantize_with_abs_max(out.get<__hip_fp8_e4m3>(), scale_ptr, in.get<__hip_bfloat16>(), abs_max, N, dp, stream);
     else if (in.DType == ETensorDType::BF16 && out.DType == ETensorDType::FP8_E5M2)
         quantize_with_abs_max(out.get<__hip_fp8_e5m2>(), scale_ptr, in.get<__hip_bfloat16>(), abs_max, N, dp, stream);

@@ -19,7 +19,7 @@ EXPORTS = [
     "llmq_abs_max_bf16", "llmq_abs_max_f32",
     "llmq_quantize_e4m3_bf16", "llmq_quantize_e5m2_bf16", "llmq_quantize_transpose_e4m3_bf16",
     "llmq_transpose_u8", "llmq_gemm_tn_e4m3_bf16", "llmq_gemm_tn_e4m3_f32", "llmq_gemm_tn_e4m3_e5m2_bf16", "llmq_gemm_tn_e4m3_e5m2_f32",
-    "llmq_backward_bias_bf16", "llmq_backward_bias_scratch_bytes", "llmq_quantize_both_bf16",
+    "llmq_backward_bias_bf16", "llmq_backward_bias_scratch_bytes", "llmq_quantize_both_bf16", "llmq_quantize_e4m3_f32", "llmq_quantize_e5m2_f32",
 ]
 
 if not os.path.exists(LIB_PATH):
@@ -36,6 +36,8 @@ lib.llmq_abs_max_f32.argtypes = [_vp, _vp, _i64, _vp]
 lib.llmq_quantize_e4m3_bf16.argtypes = [_vp, _vp, _vp, _vp, _i64, _vp]
 lib.llmq_quantize_e5m2_bf16.argtypes = [_vp, _vp, _vp, _vp, _i64, _vp]
 lib.llmq_quantize_transpose_e4m3_bf16.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _vp]
+lib.llmq_quantize_e4m3_f32.argtypes = [_vp, _vp, _vp, _vp, _i64, _vp]
+lib.llmq_quantize_e5m2_f32.argtypes = [_vp, _vp, _vp, _vp, _i64, _vp]
 lib.llmq_quantize_both_bf16.argtypes = [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp]
 lib.llmq_transpose_u8.argtypes = [_vp, _vp, _int, _int, _vp]
 lib.llmq_gemm_tn_e4m3_bf16.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, C.c_size_t, _int, _int, _int, _int, _vp]

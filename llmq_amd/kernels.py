@@ -50,11 +50,15 @@ def quantize_with_abs_max(out, scale, x, abs_max, stream=0):
     """out = fp8(448/abs_max * x); scale[0] = abs_max/448 (as 1/(448/abs_max)).  scale may be None."""
     o = _dev(out, "out", _FP8)
     s = _dev(scale, "scale", (torch.float32,), optional=True)
-    i = _dev(x, "x", (torch.bfloat16,))
+    i = _dev(x, "x", (torch.bfloat16, torch.float32))
     a = _dev(abs_max, "abs_max", (torch.float32,))
     if out.numel() != x.numel():
         raise ValueError("out and x must have the same number of elements")
-    f = capi.lib.llmq_quantize_e5m2_bf16 if out.dtype == torch.float8_e5m2 else capi.lib.llmq_quantize_e4m3_bf16
+    e5 = out.dtype == torch.float8_e5m2
+    if x.dtype == torch.float32:
+        f = capi.lib.llmq_quantize_e5m2_f32 if e5 else capi.lib.llmq_quantize_e4m3_f32
+    else:
+        f = capi.lib.llmq_quantize_e5m2_bf16 if e5 else capi.lib.llmq_quantize_e4m3_bf16
     capi.check(f(o, s, i, a, x.numel(), _stream(stream)))
 
 

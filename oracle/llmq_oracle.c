@@ -177,6 +177,18 @@ void orc_quantize_e5m2_bf16(uint8_t* out, float* scale_out, const uint16_t* in, 
     }
 }
 
+/* fp32 input (src/kernels/kernels.h:251-252): the same multiply and conversion without the bf16 widening.
+ * fmt: 0 = e4m3, 1 = e5m2. */
+void orc_quantize_fp8_f32(uint8_t* out, float* scale_out, const float* in, float absmax, int64_t n, int fmt) {
+    float s, d;
+    orc_quant_scale(absmax, &s, &d);
+    if (scale_out) *scale_out = d;
+    for (int64_t i = 0; i < n; ++i) {
+        volatile float y = s * in[i];
+        out[i] = fmt ? orc_e5m2_encode(y) : orc_e4m3_encode(y);
+    }
+}
+
 /* out[c*rows + r] = e4m3(scale * in[r*cols + c]) (quant.cu:151-164, transpose_template.cuh:21-33). */
 void orc_quantize_transpose_e4m3_bf16(uint8_t* out, float* scale_out, const uint16_t* in, float absmax,
                                       int rows, int cols) {

@@ -95,6 +95,8 @@ def lib():
     L.mt_gemm_tn_fp8.restype = C.c_int
     L.mt_gemm_tn_fp8.argtypes = [C.c_void_p, C.c_int, u8p, u8p, C.c_int, u16p, f32p, f32p,
                                  C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
+    L.orc_quantize_fp8_f32.restype = None
+    L.orc_quantize_fp8_f32.argtypes = [u8p, f32p, f32p, C.c_float, C.c_int64, C.c_int]
     L.orc_backward_bias_bf16.restype = None
     L.orc_backward_bias_bf16.argtypes = [u16p, C.c_void_p, C.c_int, f32p, f32p, C.c_int64, C.c_int, f64p, f64p]
     _lib = L
@@ -270,3 +272,13 @@ def backward_bias(dbias, dout, fmt, sa=None, sb=None):
     lib().orc_backward_bias_bf16(_p(out, C.c_uint16), dout.ctypes.data, code, C.pointer(ka) if ka is not None else None,
                                  C.pointer(kb) if kb is not None else None, BT, OC, _p(cs, C.c_double), _p(ca, C.c_double))
     return out, cs, ca
+
+
+def quantize_f32(x, absmax, fmt="e4m3"):
+    """x: float32 array -> (fp8 codes uint8, dequant scale float32), fp32-input overloads of quantize_with_abs_max."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty(x.shape, dtype=np.uint8)
+    sc = np.zeros(1, dtype=np.float32)
+    lib().orc_quantize_fp8_f32(_p(out, C.c_uint8), _p(sc, C.c_float), _p(x, C.c_float), C.c_float(absmax), x.size,
+                               1 if fmt == "e5m2" else 0)
+    return out, sc[0]

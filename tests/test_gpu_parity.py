@@ -161,6 +161,23 @@ def test_transpose_bit_exact(K, shape):
     assert np.array_equal(d.cpu().numpy(), src.T)
 
 
+@pytest.mark.parametrize("fmt", [torch.float8_e4m3fn, torch.float8_e5m2])
+@pytest.mark.parametrize("n", [0, 1, 3, 4, 1000, 4099, 1 << 20])
+def test_quantize_fp32_input_bit_exact(K, O, fmt, n):
+    """fp32-input overloads of quantize_with_abs_max (src/kernels/kernels.h:251-252), incl. ragged tails."""
+    rng = np.random.default_rng(n + 5)
+    x = (rng.standard_normal(n) * 10.0 ** rng.uniform(-6, 2, n)).astype(np.float32)
+    if n >= 1000:
+        x[:6] = [0.0, -0.0, np.inf, -np.inf, np.nan, 1e-30]
+    fin = x[np.isfinite(x)]
+    am = float(np.abs(fin).max()) if fin.size else 0.0
+    want, d = O.quantize_f32(x, am, "e5m2" if fmt == torch.float8_e5m2 else "e4m3")
+    out = torch.zeros(n, dtype=fmt, device="cuda")
+    sc = torch.zeros(1, device="cuda")
+    K.quantize_with_abs_max(out, sc, torch.from_numpy(x).cuda(), dev_scalar(am))
+    assert np.array_equal(host_bits(out), want) and sc.cpu().numpy()[0] == d
+
+
 # --------------------------------------------------------------------------------------------- GEMM
 def set_variant(v):
     """v = (tile, splits[, persistent]): tile 0 = automatic, 1 = 256 x 256, 2 = 128 x 128; splits 0 =

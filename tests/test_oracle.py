@@ -387,3 +387,19 @@ def test_backward_bias_vs_numpy(O, fmt):
         di = np.vectorize(lut.get)(ints).astype(np.uint8)
     got3, _, _ = O.backward_bias(zero, di, fmt)
     assert np.array_equal(O.bf16_to_f32(got3), ints.sum(0).astype(np.float32))
+
+
+def test_quantize_fp32_input_vs_search(O):
+    """fp32-input overloads (src/kernels/kernels.h:251-252): scale*x in fp32, then the same encoders; checked against
+    the nearest-code searches on a wide random sample plus the special values."""
+    rng = np.random.default_rng(21)
+    x = (rng.standard_normal(50000) * 10.0 ** rng.uniform(-6, 2, 50000)).astype(np.float32)
+    x[:6] = [0.0, -0.0, np.inf, -np.inf, np.nan, 1e-30]
+    am = float(np.abs(x[np.isfinite(x)]).max())
+    s, d = O.quant_scale(am)
+    with np.errstate(over="ignore", invalid="ignore"):
+        y = (np.float32(s) * x).astype(np.float32)
+    q4, d4 = O.quantize_f32(x, am, "e4m3")
+    q5, d5 = O.quantize_f32(x, am, "e5m2")
+    assert np.array_equal(q4, e4m3_encode_search(y)) and np.array_equal(q5, e5m2_encode_search(y))
+    assert d4 == np.float32(d) and d5 == np.float32(d)
