@@ -510,6 +510,273 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs g, int spli
     PairIo<OutT>::store((LLMQ_GLOBAL OutT*)dst, v0, v1);
 }
 
+// ---- four-wave variant ----------------------------------------------------------------------------
+// Same 256 x 256 x 128 workgroup tile, LDS layout, copies and tile order as above, with a different
+// division of labour: 4 waves (one per SIMD, up to 512 registers each) of 128 x 128 outputs and the
+// K = 128 matrix instruction v_mfma_f32_16x16x128_f8f6f4.  Against the 8-wave kernel this
+//   * reads a third fewer fragment bytes from LDS (16 fragments of 16 rows per wave and K-step, 128 KiB
+//     per workgroup instead of 192 KiB),
+//   * moves half the accumulator registers per flop through the matrix pipe (4 per 65536 flop instead of
+//     16 per 131072), which the chip turns into clock under its power limit: a register-only loop of this
+//     instruction sustains about 8 % more than the 32x32x64 one on random operands,
+//   * needs no LDS staging in the epilogue: the a-tile row permutation gives each lane 8 adjacent
+//     columns, i.e. one 16-byte bf16 store, 16 lanes covering 256 contiguous bytes.
+// With a single wave per SIMD nothing hides a stall, so the K loop is a software pipeline written out
+// instruction by instruction: the 8 fragments of the second operand for step s+1 are read during rows
+// 4..7 of step s into the other half of fb, the first operand's fragments rotate through 4 slots with a
+// distance of 4 rows; the workgroup barrier sits after row 4, where every read of the current stage has
+// been issued (and awaited) and the copies for step s+2 may overwrite it.
+// The workgroup is persistent (one per compute unit, walking its XCD's tile list) and the stream of
+// K-steps and copies runs across tile boundaries.  Needs K to be a multiple of 256: the LDS stage and the
+// fb half of a step are then compile-time functions of the step's parity.
+template <typename OutT, int B_FMT>
+__global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
+    constexpr int BLK = 256, T = 256, WT = 128, NF = 8;
+    constexpr int P_BYTES = BLK * kBK, STAGE = 2 * P_BYTES;
+    constexpr int ITERS = BLK * 8 / T;  // 16-byte copies per lane, operand and K-step
+    typedef float v4f __attribute__((ext_vector_type(4)));
+
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * STAGE];
+
+    const int tid = threadIdx.x;
+    const int lane = tid % 64;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
+    const int wn = wave / 2, wm = wave % 2;
+    const int l16 = lane % 16, kg = lane / 16;
+
+    // tile list of this workgroup: XCD x owns a contiguous range of the logical tile sequence
+    const int tiles_n = g.N / BLK, tiles_m = g.M / BLK;
+    const int total = tiles_n * tiles_m;
+    const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
+    const int xq = total / 8, xr = total % 8;
+    const int xcd_first = xcd * xq + (xcd < xr ? xcd : xr);
+    const int xcd_count = xq + (xcd < xr ? 1 : 0);
+    const int tile_stride = gridDim.x / 8;
+    const int my_tiles = slot < xcd_count ? (xcd_count - slot + tile_stride - 1) / tile_stride : 0;
+    if (my_tiles == 0) return;  // uniform for the whole workgroup, before any barrier
+    auto decode = [&](int logical, int& n_blk, int& m_blk) {
+        const int per_group = g.group * tiles_m;
+        const int gid = logical / per_group;
+        const int first_n = gid * g.group;
+        const int gsz = (tiles_n - first_n) < g.group ? (tiles_n - first_n) : g.group;
+        const int in_group = logical % per_group;
+        n_blk = (first_n + in_group % gsz) * BLK;
+        m_blk = (in_group / gsz) * BLK;
+    };
+
+    // copies: lane -> (row tid/8 of a 32-row slab, physical 16-byte chunk tid%8); every address is a
+    // wave-uniform base plus a 32-bit lane offset
+    const int ld_row = tid / 8;
+    const int ld_chunk = (tid & 7) ^ ((ld_row >> 1) & 7);
+    const uint32_t p_lane = (uint32_t)ld_row * (uint32_t)g.K + (uint32_t)ld_chunk * 16u;
+    // LDS row rho of the a-tile holds global row (rho/128)*128 + 8*(rho%16) + (rho%128)/16
+    const uint32_t q_lane = (uint32_t)(8 * (ld_row % 16) + ld_row / 16) * (uint32_t)g.K + (uint32_t)ld_chunk * 16u;
+    // The copy stream runs two K-steps ahead of the matrix instructions and has its own position: tile
+    // number, K offset and the operand bases of that tile already advanced to the K offset.
+    int copy_k0 = 0, copy_tile = 0;
+    const uint8_t *p_cur, *q_cur;
+    auto tile_bases = [&](int logical, const uint8_t*& pb, const uint8_t*& qb) {
+        int nb, mb;
+        decode(logical, nb, mb);
+        pb = g.b + (int64_t)nb * g.K;
+        qb = g.a + (int64_t)mb * g.K;
+    };
+    tile_bases(xcd_first + slot, p_cur, q_cur);
+    // after the copies of one K-step; past the last tile the stream re-reads that tile's first K-steps
+    // (harmless, and no step needs a special case)
+    auto advance_copy = [&]() {
+        copy_k0 += kBK;
+        p_cur += kBK;
+        q_cur += kBK;
+        if (copy_k0 == g.K) {
+            copy_k0 = 0;
+            if (copy_tile + 1 < my_tiles) ++copy_tile;
+            tile_bases(xcd_first + slot + copy_tile * tile_stride, p_cur, q_cur);
+        }
+    };
+    // Copy number c of a K-step, c = 0 .. 2*ITERS-1: first the b-rows slabs, then the a-rows slabs.  Written
+    // as an asm statement to get the addressing form "scalar base + 32-bit lane offset" (no vector address
+    // arithmetic between the matrix instructions); M0 carries the LDS destination of the wave.
+    const uint32_t lds_wave = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds + wave * 1024;
+    const int64_t slab_p = (int64_t)32 * g.K;
+    auto issue_load = [&](int c, int stage_ofs) {
+        const uint8_t* src;
+        uint32_t dst, lane_ofs;
+        if (c < ITERS) {
+            src = p_cur + c * slab_p;
+            dst = lds_wave + stage_ofs + c * T * 16;
+            lane_ofs = p_lane;
+        } else {
+            // slab `it` covers LDS rows 32 it .. 32 it + 31 = global rows (it/4)*128 + 2*(it%4) + (those of slab 0)
+            const int it = c - ITERS;
+            src = q_cur + (int64_t)((it / 4) * 128 + 2 * (it % 4)) * g.K;
+            dst = lds_wave + stage_ofs + P_BYTES + it * T * 16;
+            lane_ofs = q_lane;
+        }
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                     :
+                     : "v"(lane_ofs), "s"(src), "s"(dst)
+                     : "memory", "m0");
+    };
+
+    const int sw = (l16 >> 1) & 7;
+    const int c0 = ((2 * kg) ^ sw) * 16, c1 = ((2 * kg + 1) ^ sw) * 16;
+    const int p_frag = (wn * WT + l16) * kBK;
+    const int q_frag = P_BYTES + (wm * WT + l16) * kBK;
+    auto read_frag = [&](const uint8_t* row) -> v8i {
+        const v4i lo = *reinterpret_cast<const v4i*>(row + c0);
+        const v4i hi = *reinterpret_cast<const v4i*>(row + c1);
+        return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    };
+
+    // The matrix instruction as an asm statement with the accumulator tied in place in the accumulation
+    // registers: with all 256 of them holding the wave tile there is no spare for the register allocator's
+    // untied form.  The memory clobber keeps every LDS read and copy in its source position relative to
+    // the matrix instructions, so a K-step is issued exactly as written below.
+    auto mfma = [&](v4f& c, const v8i& a, const v8i& b) {
+        if constexpr (B_FMT == 0)
+            asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b) : "memory");
+        else
+            asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:1" : "+a"(c) : "v"(a), "v"(b) : "memory");
+    };
+    // first K-step of a tile: the accumulator input is the constant 0, so no register is initialised by an
+    // instruction whose distance to the matrix instruction the compiler could not police
+    auto mfma_first = [&](v4f& c, const v8i& a, const v8i& b) {
+        if constexpr (B_FMT == 0)
+            asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0" : "=a"(c) : "v"(a), "v"(b) : "memory");
+        else
+            asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0 cbsz:1" : "=a"(c) : "v"(a), "v"(b) : "memory");
+    };
+
+    v4f acc[NF][NF];  // written by the first K-step of every tile
+    v8i fa[4], fb[2][NF];
+
+    // prologue of the stream: the first two K-steps of the first tile
+#pragma unroll
+    for (int c = 0; c < 2 * ITERS; ++c) issue_load(c, 0);
+    advance_copy();
+#pragma unroll
+    for (int c = 0; c < 2 * ITERS; ++c) issue_load(c, STAGE);
+    advance_copy();
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * ITERS) : "memory");
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) fa[i] = read_frag(lds + p_frag + i * 16 * kBK);
+#pragma unroll
+    for (int j = 0; j < NF; ++j) fb[0][j] = read_frag(lds + q_frag + j * 16 * kBK);
+
+    // One K-step of parity PAR (LDS stage PAR, fb half PAR): rows i = 0..7 of first-operand fragments
+    // against all 8 second-operand fragments.  fa rotates through 4 slots (fragment i+4 is read once row i
+    // has been issued; rows 4..7 fetch the next step's first four from the other stage); the next step's
+    // second-operand fragments go into the other half of fb, two per row in rows 4..7 (after the barrier).  The 16 copies of
+    // the step after next go into the stage this step releases: 4 right after the barrier, then one after
+    // each of the six middle matrix instructions of rows 5 and 6.
+    auto k_step = [&](auto par_tag, auto first_tag) {
+        constexpr int PAR = decltype(par_tag)::value;
+        constexpr bool FIRST = decltype(first_tag)::value;
+        const uint8_t* cur = lds + PAR * STAGE;
+        const uint8_t* nxt = lds + (1 - PAR) * STAGE;
+#pragma unroll
+        for (int i = 0; i < NF; ++i) {
+#pragma unroll
+            for (int j = 0; j < NF; ++j) {
+                if constexpr (FIRST) mfma_first(acc[i][j], fa[i % 4], fb[PAR][j]);
+                else mfma(acc[i][j], fa[i % 4], fb[PAR][j]);
+                if ((i == 5 || i == 6) && j >= 1 && j <= 6) issue_load(4 + 6 * (i - 5) + (j - 1), PAR * STAGE);
+                if (i >= 5 && (j == 2 || j == 5)) {  // rows 5..7: fragments 2..7 of the next step
+                    const int f = 2 * (i - 4) + (j == 5 ? 1 : 0);
+                    fb[1 - PAR][f] = read_frag(nxt + q_frag + f * 16 * kBK);
+                }
+            }
+            if (i == 4) {
+                // every read of the current stage has been issued (the last one after row 3); once they
+                // have returned and all waves are here the stage may be overwritten, and the next stage
+                // (copied one step ago) is complete
+                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                __syncthreads();
+#pragma unroll
+                for (int c = 0; c < 4; ++c) issue_load(c, PAR * STAGE);
+                fb[1 - PAR][0] = read_frag(nxt + q_frag);
+                fb[1 - PAR][1] = read_frag(nxt + q_frag + 16 * kBK);
+            }
+            if (i < 4) fa[i % 4] = read_frag(cur + p_frag + (i + 4) * 16 * kBK);
+            else fa[i % 4] = read_frag(nxt + p_frag + (i - 4) * 16 * kBK);
+        }
+        advance_copy();
+    };
+
+    using std::integral_constant;
+    constexpr integral_constant<int, 0> P0{};
+    constexpr integral_constant<int, 1> P1{};
+    constexpr integral_constant<bool, true> Y{};
+    constexpr integral_constant<bool, false> NO{};
+    const int KT = g.K / kBK;  // even
+    int logical = xcd_first + slot;
+    for (int t = 0; t < my_tiles; ++t) {
+        k_step(P0, Y);
+        k_step(P1, NO);
+        for (int kt = 2; kt < KT; kt += 2) {
+            k_step(P0, NO);
+            k_step(P1, NO);
+        }
+        // the compiler does not know the statements above are matrix instructions: give the last ones time
+        // to retire before their results are read (generously: four times the instruction's 32 cycles)
+        asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+
+        // Epilogue.  acc[i][j][r] is c row 16 i + 4 kg + r of the wave tile and, thanks to the a-tile row
+        // permutation, column 8 l16 + j: a lane owns 8 adjacent columns of each of its 32 rows.
+        int n_blk, m_blk;
+        decode(logical, n_blk, m_blk);
+        logical += tile_stride;
+        float scale = g.sa ? *g.sa : 1.f;
+        if (g.sb) scale = scale * *g.sb;
+        const int e_lane = opaque(threadIdx.x) % 64;
+        const int el16 = e_lane % 16, ekg = e_lane / 16;
+        const int m_lane = m_blk + wm * WT + 8 * el16;
+        float bias_v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) bias_v[j] = g.bias ? load_bias(g.bias, g.bias_is_bf16, m_lane + j) : 0.f;
+        OutT* c = reinterpret_cast<OutT*>(g.c);
+        const uint32_t lane_bytes = ((uint32_t)(4 * ekg) * (uint32_t)g.M + (uint32_t)m_lane) * (uint32_t)sizeof(OutT);
+        const int row0 = n_blk + wn * WT;
+        const bool accumulate = g.accumulate != 0;
+#pragma unroll
+        for (int i = 0; i < NF; ++i) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                LLMQ_GLOBAL char* row = scalar_ptr((LLMQ_GLOBAL char*)(c + (int64_t)(row0 + 16 * i + r) * g.M)) + lane_bytes;
+                float v[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) v[j] = acc[i][j][r] * scale + bias_v[j];
+                if (accumulate) {
+#pragma unroll
+                    for (int j = 0; j < 8; j += 2) {
+                        float o0, o1;
+                        PairIo<OutT>::load(row + j * sizeof(OutT), o0, o1);
+                        v[j] = v[j] + o0;
+                        v[j + 1] = v[j + 1] + o1;
+                    }
+                }
+                if constexpr (std::is_same_v<OutT, uint16_t>) {
+                    v4i packed;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const f32x2_t pr = {v[2 * j], v[2 * j + 1]};
+                        packed[j] = __builtin_bit_cast(int, __builtin_convertvector(pr, bf16x2_t));
+                    }
+                    *(LLMQ_GLOBAL v4i*)row = packed;
+                } else {
+                    typedef float v4fl __attribute__((ext_vector_type(4)));
+                    const v4fl lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
+                    *(LLMQ_GLOBAL v4fl*)row = lo;
+                    *(LLMQ_GLOBAL v4fl*)(row + 16) = hi;
+                }
+            }
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the surplus copies issued during the last tile
+}
+
 // ---- host side ------------------------------------------------------------------------------------
 template <int BLK_N, int BLK_M, int WV_N, int WV_M, typename OutT, int B_FMT>
 static int launch_pipe(const GemmArgs& g, int splits, int persistent_grid, hipStream_t stream) {
@@ -550,9 +817,13 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
     g.group = 8;
     const int cus = cu_count();
     int tile = g_gemm_tile;
-    LLMQ_REQUIRE(tile >= 0 && tile <= 2, "matmul: unknown tile selector %d", tile);
+    LLMQ_REQUIRE(tile >= 0 && tile <= 3, "matmul: unknown tile selector %d", tile);
     const bool fits256 = g.N % 256 == 0 && g.M % 256 == 0;
-    LLMQ_REQUIRE(tile != 1 || fits256, "matmul: the 256 x 256 tile needs M and N divisible by 256");
+    LLMQ_REQUIRE((tile != 1 && tile != 3) || fits256, "matmul: the 256 x 256 tile needs M and N divisible by 256");
+    const bool w4_ok = fits256 && g.K % (2 * kBK) == 0 && cus % 8 == 0;
+    if (tile == 3) {
+        LLMQ_REQUIRE(w4_ok && g_gemm_splits <= 1, "matmul: the four-wave kernel needs K divisible by 256 and no K split");
+    }
     if (tile == 0) {
         // Rounds of workgroups the chip needs: one 256 x 256 tile per compute unit and round (four units
         // of work), or two co-resident 128 x 128 tiles (two units, at about 0.8 of the rate per unit).
@@ -564,7 +835,7 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
 
     // Split K when the tiles alone leave most of the chip idle: aim at about one workgroup per compute
     // unit, keep at least 512 elements of K per split, and stay inside the caller's workspace.
-    const int64_t tiles = tile == 1 ? (int64_t)(g.N / 256) * (g.M / 256) : (int64_t)(g.N / 128) * (g.M / 128);
+    const int64_t tiles = tile != 2 ? (int64_t)(g.N / 256) * (g.M / 256) : (int64_t)(g.N / 128) * (g.M / 128);
     const int64_t slice_bytes = (int64_t)g.N * g.M * 4;
     const int64_t ws_splits = (int64_t)(workspace_bytes / (size_t)slice_bytes);
     int splits = g_gemm_splits;
@@ -582,6 +853,7 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
         LLMQ_REQUIRE(ws_splits >= splits, "matmul: workspace of %zu bytes is too small for %d splits", workspace_bytes,
                      splits);
     }
+    if (tile == 3) splits = 1;
     if (splits > 1) {
         const int steps = g.K / kBK;
         g.k_len = ((steps + splits - 1) / splits) * kBK;
@@ -593,6 +865,14 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
     int persistent_grid = 0;
     const bool can_persist = tile == 1 && splits == 1 && g.K >= 2 * kBK && cus % 8 == 0;
     if (can_persist && (g_gemm_persist == 1 || (g_gemm_persist < 0 && tiles > cus))) persistent_grid = cus;
+    // The four-wave kernel takes every large-tile launch it can (K a multiple of 256, no K split).
+    if ((tile == 3 || (tile == 1 && g_gemm_tile == 0 && w4_ok)) && splits == 1) {
+        const int tiles256 = (g.N / 256) * (g.M / 256);
+        const int grid = tiles256 < cus ? (tiles256 + 7) / 8 * 8 : cus;
+        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<OutT, B_FMT>), dim3((unsigned)grid), dim3(256), 0, stream, g);
+        LLMQ_HIP_TRY(hipGetLastError());
+        return LLMQ_OK;
+    }
     if (tile == 1) return launch_pipe<256, 256, 2, 4, OutT, B_FMT>(g, splits, persistent_grid, stream);
     return launch_pipe<128, 128, 2, 2, OutT, B_FMT>(g, splits, 0, stream);
 }

@@ -180,14 +180,15 @@ def test_quantize_fp32_input_bit_exact(K, O, fmt, n):
 
 # --------------------------------------------------------------------------------------------- GEMM
 def set_variant(v):
-    """v = (tile, splits[, persistent]): tile 0 = automatic, 1 = 256 x 256, 2 = 128 x 128; splits 0 =
+    """v = (tile, splits[, persistent]): tile 0 = automatic, 1 = 256 x 256 (8 waves), 2 = 128 x 128, 3 = 256 x 256
+    (4 waves, 16x16x128 matrix instruction); splits 0 =
     automatic; persistent -1 = automatic, 0 = one workgroup per tile, 1 = persistent tile walk."""
     from llmq_amd import capi
     capi.lib.llmq_debug_set_gemm_variant(v[0], v[1])
     capi.lib.llmq_debug_set_gemm_persist(v[2] if len(v) > 2 else -1)
 
 
-VARIANTS = [(0, 0), (1, 0, 0), (1, 1, 1), (2, 0), (1, 2), (2, 2), (2, 3)]
+VARIANTS = [(0, 0), (1, 0, 0), (1, 1, 1), (2, 0), (1, 2), (2, 2), (2, 3), (3, 1)]
 _WORKSPACE = {}
 
 
@@ -198,8 +199,10 @@ def workspace():
 
 
 def skip_unsupported(variant, M, N, Kd):
-    if variant[0] == 1 and (M % 256 or N % 256):
+    if variant[0] in (1, 3) and (M % 256 or N % 256):
         pytest.skip("the 256 x 256 tile needs multiples of 256")
+    if variant[0] == 3 and Kd % 256:
+        pytest.skip("the four-wave kernel needs K divisible by 256")
     if variant[1] > Kd // 128:
         pytest.skip("more splits than K-steps")
     if len(variant) > 2 and variant[2] == 1 and Kd < 256:
@@ -220,7 +223,7 @@ def run_gemm(K, a, b, M, N, Kd, sa, sb, bias_bits=None, old=None, out_f32=False)
 
 
 @pytest.mark.parametrize("variant", VARIANTS)
-@pytest.mark.parametrize("mnk", [(128, 128, 128), (256, 256, 256), (512, 768, 384), (256, 512, 1024)])
+@pytest.mark.parametrize("mnk", [(128, 128, 128), (256, 256, 256), (512, 768, 384), (256, 512, 1024), (768, 512, 512)])
 def test_gemm_integer_known_answer_exact(K, O, variant, mnk):
     """Construction of src/testing/test-gemm.cpp:54-85: integer operands, exact fp32 sums -> the bf16
     output must equal the oracle bit for bit (set / bias / accumulate)."""
@@ -250,7 +253,7 @@ def test_gemm_integer_known_answer_exact(K, O, variant, mnk):
 @pytest.mark.parametrize("variant", VARIANTS)
 @pytest.mark.parametrize("out_f32", [False, True])
 def test_gemm_random_codes_within_tolerance(K, O, variant, out_f32):
-    M, N, Kd = 512, 256, 896
+    M, N, Kd = (512, 256, 896) if variant[0] != 3 else (512, 256, 1024)
     skip_unsupported(variant, M, N, Kd)
     rng = np.random.default_rng(17)
     a = rng.integers(0, 256, (M, Kd)).astype(np.uint8)
@@ -279,12 +282,14 @@ def test_gemm_random_codes_within_tolerance(K, O, variant, out_f32):
         set_variant((0, 0))
 
 
-@pytest.mark.parametrize("mnk", [(4352, 4352, 384), (4608, 4096, 256), (8192, 4864, 512)])
-def test_gemm_persistent_tile_walk(K, O, mnk):
+@pytest.mark.parametrize("variant", [(1, 1, 1), (3, 1)])
+@pytest.mark.parametrize("mnk", [(4352, 4352, 384), (4608, 4096, 256), (8192, 4864, 512), (4352, 4352, 1024)])
+def test_gemm_persistent_tile_walk(K, O, mnk, variant):
     """More tiles than compute units: workgroups walk several tiles each and the operand stream crosses
     tile boundaries (odd and even numbers of K-steps flip the LDS stage parity differently).  Integer
     operands -> bit-exact against the oracle, with bias and accumulation, bf16 and fp32 outputs."""
     M, N, Kd = mnk
+    skip_unsupported(variant, M, N, Kd)
     a, _ = O.fill_int_e4m3(M * Kd, 4242, 0)
     b, _ = O.fill_int_e4m3(N * Kd, 4242, 1)
     a, b = a.reshape(M, Kd), b.reshape(N, Kd)
@@ -293,7 +298,7 @@ def test_gemm_persistent_tile_walk(K, O, mnk):
     _, oldv = O.fill_int_e4m3(N * M, 4242, 3)
     bias = O.f32_to_bf16(biasv.astype(np.float32))
     old = O.f32_to_bf16(oldv.astype(np.float32)).reshape(N, M)
-    set_variant((1, 1, 1))
+    set_variant(variant)
     try:
         want = O.gemm_tn(a, b, sa=s, sb=s, mt=True)
         got = run_gemm(K, a, b, M, N, Kd, s, s)
@@ -333,11 +338,11 @@ def test_gemm_automatic_split_k(K, O, mnk):
     gemm_check(c1.cpu().numpy(), exact, sumabs, np.float32(np.float32(0.01) * np.float32(0.02)), False)
 
 
-@pytest.mark.parametrize("variant", [(0, 0), (1, 1, 1), (2, 2)])
+@pytest.mark.parametrize("variant", [(0, 0), (1, 1, 1), (2, 2), (3, 1)])
 def test_gemm_e5m2_b_operand(K, O, variant):
     """a e4m3, b e5m2 (src/kernels/kernels.h:92-94): small integers are exact in both formats ->
     bit-exact against the oracle; random codes within the stated tolerance of the exact product."""
-    M, N, Kd = 512, 768, 640
+    M, N, Kd = 512, 768, 768
     rng = np.random.default_rng(91)
     ai, bi = rng.integers(-4, 5, (M, Kd)), rng.integers(-4, 5, (N, Kd))
     enc4 = {v: O.lib().orc_e4m3_encode(float(v)) for v in range(-4, 5)}
