@@ -2,11 +2,12 @@
 //
 //  * llmq_debug_copy_u8: a plain streaming copy whose HBM bytes are known exactly (n read + n
 //    written); hardware traffic counters of the real kernels are scaled by what they read for it.
-//  * llmq_debug_mfma_ceiling: a loop of v_mfma_f32_32x32x64_f8f6f4 on register operands with no
-//    memory traffic at all, 8 waves per compute unit.  With constant operands it runs at the nominal
-//    clock; with random fp8 operands that change every iteration (what a real K loop feeds the matrix
-//    cores) the chip lowers its clock under power, and the rate it sustains is the practical ceiling
-//    any fp8 GEMM on this part is measured against.
+//  * llmq_debug_mfma_ceiling: a loop of fp8 matrix instructions on register operands with no memory
+//    traffic at all, 8 waves per compute unit.  With constant operands it runs at the nominal clock;
+//    with random fp8 operands that change every iteration (what a real K loop feeds the matrix cores)
+//    the chip lowers its clock under power, and the rate it sustains is the practical ceiling any fp8
+//    GEMM on this part is measured against.  The 16x16x128 instruction moves half the accumulator
+//    registers per flop of the 32x32x64 one and sustains a higher rate under that limit.
 #include "common.hpp"
 
 namespace llmq {
@@ -30,12 +31,16 @@ __device__ __forceinline__ uint32_t mix32(uint32_t x) {
     return x;
 }
 
-template <bool RANDOM>
+// MODE 0: 32x32x64 instruction, constant operands; 1: 32x32x64, random operands that change every
+// iteration; 2: 16x16x128, random operands.  All use 128 accumulator registers per lane like a GEMM
+// wave tile, 8 waves per workgroup.
+template <int MODE>
 __global__ __launch_bounds__(512) void mfma_ceiling_kernel(float* out, int iters) {
+    typedef float v4f __attribute__((ext_vector_type(4)));
     v8i a[2], b[2];
     for (int s = 0; s < 2; ++s)
         for (int i = 0; i < 8; ++i) {
-            if (!RANDOM) {
+            if (MODE == 0) {
                 a[s][i] = 0x38383838;  // 1.0 in every byte
                 b[s][i] = 0x38383838;
             } else {
@@ -44,24 +49,42 @@ __global__ __launch_bounds__(512) void mfma_ceiling_kernel(float* out, int iters
                 b[s][i] = rb & 0xBFBFBFBFu;
             }
         }
-    v16f acc[4];
-    for (int n = 0; n < 4; ++n)
-        for (int i = 0; i < 16; ++i) acc[n][i] = 0.f;
-    for (int it = 0; it < iters; ++it) {
+    float s = 0;
+    if constexpr (MODE != 2) {
+        v16f acc[8];
+        for (int n = 0; n < 8; ++n)
+            for (int i = 0; i < 16; ++i) acc[n][i] = 0.f;
+        for (int it = 0; it < iters; ++it) {
 #pragma unroll
-        for (int n = 0; n < 4; ++n)
-            acc[n] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[n & 1], b[(n >> 1) & 1], acc[n], 0, 0, 0, 0, 0, 0);
-        if (RANDOM) {
+            for (int n = 0; n < 8; ++n)
+                acc[n] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[n & 1], b[(n >> 1) & 1], acc[n], 0, 0, 0, 0, 0, 0);
+            if (MODE == 1) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    a[0][i] ^= 0x15150a0a;
+                    b[1][i] ^= 0x0a0a1515;
+                }
+            }
+        }
+        for (int n = 0; n < 8; ++n)
+            for (int i = 0; i < 16; ++i) s += acc[n][i];
+    } else {
+        v4f acc[32];
+        for (int n = 0; n < 32; ++n)
+            for (int i = 0; i < 4; ++i) acc[n][i] = 0.f;
+        for (int it = 0; it < iters; it += 2) {  // two iterations' worth of flop per trip: 32 x 65536
+#pragma unroll
+            for (int n = 0; n < 32; ++n)
+                acc[n] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a[n & 1], b[(n >> 1) & 1], acc[n], 0, 0, 0, 0, 0, 0);
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 a[0][i] ^= 0x15150a0a;
                 b[1][i] ^= 0x0a0a1515;
             }
         }
+        for (int n = 0; n < 32; ++n)
+            for (int i = 0; i < 4; ++i) s += acc[n][i];
     }
-    float s = 0;
-    for (int n = 0; n < 4; ++n)
-        for (int i = 0; i < 16; ++i) s += acc[n][i];
     out[blockIdx.x * blockDim.x + threadIdx.x] = s;
 }
 
@@ -80,14 +103,18 @@ extern "C" int llmq_debug_copy_u8(uint8_t* dst, const uint8_t* src, int64_t n, v
     return LLMQ_OK;
 }
 
-// Launches one ceiling kernel: `blocks` workgroups of 512 lanes, `iters` iterations of 4 matrix
-// instructions per wave (= blocks * 8 * iters * 4 * 131072 flop).  scratch: blocks * 512 floats.
-extern "C" int llmq_debug_mfma_ceiling(float* scratch, int blocks, int iters, int random_operands, void* stream) {
+// Launches one ceiling kernel: `blocks` workgroups of 512 lanes, `iters` (even) iterations of
+// 8 * 131072 flop per wave (= blocks * 8 * iters * 1048576 flop).  mode: 0 = 32x32x64 instruction with
+// constant operands, 1 = 32x32x64 with random operands, 2 = 16x16x128 with random operands.
+// scratch: blocks * 512 floats.
+extern "C" int llmq_debug_mfma_ceiling(float* scratch, int blocks, int iters, int mode, void* stream) {
     using namespace llmq;
-    LLMQ_REQUIRE(scratch != nullptr && blocks > 0 && iters > 0, "mfma_ceiling: bad arguments");
+    LLMQ_REQUIRE(scratch != nullptr && blocks > 0 && iters > 0 && iters % 2 == 0 && mode >= 0 && mode <= 2,
+                 "mfma_ceiling: bad arguments");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (random_operands) hipLaunchKernelGGL(mfma_ceiling_kernel<true>, dim3((unsigned)blocks), dim3(512), 0, st, scratch, iters);
-    else hipLaunchKernelGGL(mfma_ceiling_kernel<false>, dim3((unsigned)blocks), dim3(512), 0, st, scratch, iters);
+    if (mode == 0) hipLaunchKernelGGL(mfma_ceiling_kernel<0>, dim3((unsigned)blocks), dim3(512), 0, st, scratch, iters);
+    else if (mode == 1) hipLaunchKernelGGL(mfma_ceiling_kernel<1>, dim3((unsigned)blocks), dim3(512), 0, st, scratch, iters);
+    else hipLaunchKernelGGL(mfma_ceiling_kernel<2>, dim3((unsigned)blocks), dim3(512), 0, st, scratch, iters);
     LLMQ_HIP_TRY(hipGetLastError());
     return LLMQ_OK;
 }

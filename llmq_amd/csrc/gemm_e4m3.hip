@@ -671,6 +671,7 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     // second-operand fragments go into the other half of fb, two per row in rows 4..7 (after the barrier).  The 16 copies of
     // the step after next go into the stage this step releases: 4 right after the barrier, then one after
     // each of the six middle matrix instructions of rows 5 and 6.
+    bool pending_stores = false;  // an epilogue without accumulation has just issued its stores
     auto k_step = [&](auto par_tag, auto first_tag) {
         constexpr int PAR = decltype(par_tag)::value;
         constexpr bool FIRST = decltype(first_tag)::value;
@@ -692,7 +693,19 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
                 // every read of the current stage has been issued (the last one after row 3); once they
                 // have returned and all waves are here the stage may be overwritten, and the next stage
                 // (copied one step ago) is complete
-                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                if constexpr (FIRST) {
+                    // Behind the copies this barrier is about (the tile's second K-step, issued before the
+                    // previous tile's epilogue) sit that epilogue's stores; the counter retires in issue
+                    // order, so allowing as many outstanding operations as there were stores is enough.
+                    if (pending_stores) {
+                        if constexpr (sizeof(OutT) == 2) asm volatile("s_waitcnt vmcnt(32) lgkmcnt(0)" ::: "memory");
+                        else asm volatile("s_waitcnt vmcnt(63) lgkmcnt(0)" ::: "memory");
+                    } else {
+                        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                    }
+                } else {
+                    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                }
                 __syncthreads();
 #pragma unroll
                 for (int c = 0; c < 4; ++c) issue_load(c, PAR * STAGE);
@@ -733,45 +746,83 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         const int e_lane = opaque(threadIdx.x) % 64;
         const int el16 = e_lane % 16, ekg = e_lane / 16;
         const int m_lane = m_blk + wm * WT + 8 * el16;
-        float bias_v[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) bias_v[j] = g.bias ? load_bias(g.bias, g.bias_is_bf16, m_lane + j) : 0.f;
         OutT* c = reinterpret_cast<OutT*>(g.c);
         const uint32_t lane_bytes = ((uint32_t)(4 * ekg) * (uint32_t)g.M + (uint32_t)m_lane) * (uint32_t)sizeof(OutT);
         const int row0 = n_blk + wn * WT;
-        const bool accumulate = g.accumulate != 0;
+        auto rows = [&](auto bias_tag, auto acc_tag) {
+            constexpr bool BIAS = decltype(bias_tag)::value;
+            constexpr bool ACC = decltype(acc_tag)::value;
+            typedef float v4fl __attribute__((ext_vector_type(4)));
+            float bias_v[8];
+            if constexpr (BIAS) {
 #pragma unroll
-        for (int i = 0; i < NF; ++i) {
+                for (int j = 0; j < 8; ++j) bias_v[j] = load_bias(g.bias, g.bias_is_bf16, m_lane + j);
+            }
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                LLMQ_GLOBAL char* row = scalar_ptr((LLMQ_GLOBAL char*)(c + (int64_t)(row0 + 16 * i + r) * g.M)) + lane_bytes;
-                float v[8];
+            for (int i = 0; i < NF; ++i) {
+                LLMQ_GLOBAL char* row[4];
 #pragma unroll
-                for (int j = 0; j < 8; ++j) v[j] = acc[i][j][r] * scale + bias_v[j];
-                if (accumulate) {
+                for (int r = 0; r < 4; ++r)
+                    row[r] = scalar_ptr((LLMQ_GLOBAL char*)(c + (int64_t)(row0 + 16 * i + r) * g.M)) + lane_bytes;
+                // the old values of the fragment row's four c rows are requested together
+                float old[4][8];
+                if constexpr (ACC) {
 #pragma unroll
-                    for (int j = 0; j < 8; j += 2) {
-                        float o0, o1;
-                        PairIo<OutT>::load(row + j * sizeof(OutT), o0, o1);
-                        v[j] = v[j] + o0;
-                        v[j + 1] = v[j + 1] + o1;
+                    for (int r = 0; r < 4; ++r) {
+                        if constexpr (std::is_same_v<OutT, uint16_t>) {
+                            const v4i w = *(const LLMQ_GLOBAL v4i*)row[r];
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) {
+                                old[r][2 * j] = __uint_as_float((uint32_t)w[j] << 16);
+                                old[r][2 * j + 1] = __uint_as_float((uint32_t)w[j] & 0xFFFF0000u);
+                            }
+                        } else {
+                            const v4fl lo = *(const LLMQ_GLOBAL v4fl*)row[r], hi = *(const LLMQ_GLOBAL v4fl*)(row[r] + 16);
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) {
+                                old[r][j] = lo[j];
+                                old[r][4 + j] = hi[j];
+                            }
+                        }
                     }
                 }
-                if constexpr (std::is_same_v<OutT, uint16_t>) {
-                    v4i packed;
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const f32x2_t pr = {v[2 * j], v[2 * j + 1]};
-                        packed[j] = __builtin_bit_cast(int, __builtin_convertvector(pr, bf16x2_t));
+                for (int r = 0; r < 4; ++r) {
+                    float v[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        v[j] = acc[i][j][r] * scale;
+                        if constexpr (BIAS) v[j] = v[j] + bias_v[j];
+                        if constexpr (ACC) v[j] = v[j] + old[r][j];
                     }
-                    *(LLMQ_GLOBAL v4i*)row = packed;
-                } else {
-                    typedef float v4fl __attribute__((ext_vector_type(4)));
-                    const v4fl lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
-                    *(LLMQ_GLOBAL v4fl*)row = lo;
-                    *(LLMQ_GLOBAL v4fl*)(row + 16) = hi;
+                    if constexpr (std::is_same_v<OutT, uint16_t>) {
+                        v4i packed;
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const f32x2_t pr = {v[2 * j], v[2 * j + 1]};
+                            packed[j] = __builtin_bit_cast(int, __builtin_convertvector(pr, bf16x2_t));
+                        }
+                        *(LLMQ_GLOBAL v4i*)row[r] = packed;
+                    } else {
+                        const v4fl lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
+                        *(LLMQ_GLOBAL v4fl*)row[r] = lo;
+                        *(LLMQ_GLOBAL v4fl*)(row[r] + 16) = hi;
+                    }
                 }
             }
+        };
+        constexpr std::true_type yes{};
+        constexpr std::false_type no{};
+        if (g.accumulate) {
+            if (g.bias) rows(yes, yes);
+            else rows(no, yes);
+            // the loads of old values have been consumed; make the next tile's first barrier wait for
+            // everything (its relaxed form counts stores only)
+            pending_stores = false;
+        } else {
+            if (g.bias) rows(yes, no);
+            else rows(no, no);
+            pending_stores = true;
         }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the surplus copies issued during the last tile
