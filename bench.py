@@ -271,7 +271,7 @@ def main():
 def measured_traffic():
     """HBM-side bytes per GEMM launch (L2 fetch + write-back) from the hardware-counter summary kept
     under profiles/ for this same workload; None when that file is absent."""
-    path = os.path.join(ROOT, "profiles", "gemm_tn_e4m3_pipe_kernel__bench_qwen7b_mlp__traffic.txt")
+    path = os.path.join(ROOT, "profiles", "gemm_tn_e4m3_w4_kernel__bench_qwen7b_mlp__traffic.txt")
     try:
         for line in open(path):
             if line.startswith("traffic_bytes_per_launch"):

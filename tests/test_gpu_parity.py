@@ -313,6 +313,35 @@ def test_gemm_persistent_tile_walk(K, O, mnk, variant):
         set_variant((0, 0))
 
 
+def test_gemm_four_wave_large_repeatable(K, O):
+    """The four-wave kernel issues its matrix instructions from asm statements (the compiler does not see
+    them as such), so beyond the exact small cases: a chip-filling shape with random codes, repeated, must
+    give bit-identical results every time and agree with the exact product on sampled outputs."""
+    M, N, Kd = 4096, 8192, 2048
+    rng = np.random.default_rng(33)
+    a = rng.integers(0, 0x7E, (M, Kd)).astype(np.uint8) | (rng.integers(0, 2, (M, Kd)).astype(np.uint8) << 7)
+    b = rng.integers(0, 0x7E, (N, Kd)).astype(np.uint8) | (rng.integers(0, 2, (N, Kd)).astype(np.uint8) << 7)
+    ad, bd = dev_u8(a), dev_u8(b)
+    sa = dev_scalar(2.0 ** -6)
+    set_variant((3, 1))
+    try:
+        first = None
+        for rep in range(8):
+            c = torch.full((N, M), float("nan"), dtype=torch.float32, device="cuda")
+            K.matmul(c, ad, bd, None, sa, None, M, N, Kd, workspace=workspace())
+            torch.cuda.synchronize()
+            if first is None:
+                first = c
+            else:
+                assert torch.equal(first.view(torch.int32), c.view(torch.int32)), "run %d differs" % rep
+    finally:
+        set_variant((0, 0))
+    idx_n = rng.integers(0, N, 40000).astype(np.int32)
+    idx_m = rng.integers(0, M, 40000).astype(np.int32)
+    ex, sabs = O.gemm_exact_sampled(a, b, idx_n, idx_m)
+    gemm_check(first.cpu().numpy()[idx_n, idx_m], ex, sabs, np.float32(2.0 ** -6), False)
+
+
 @pytest.mark.parametrize("mnk", [(128, 128, 4096), (256, 384, 2048), (896, 896, 8192)])
 def test_gemm_automatic_split_k(K, O, mnk):
     """Few-tile shapes with a workspace take the split-K path on their own; integer operands keep
