@@ -16,6 +16,11 @@ One JSON line is printed:
   quantize        abs-max + quantize (+transpose) launches: algorithmic bytes / event-timed duration
                   against 8 TB/s
   cpu_baseline    the multithreaded CPU port of the same path on a bounded sample (host cores of this box)
+Extra fields: roofline.mfma_only_ceiling_TFLOPs (register-only matrix-instruction loops: what the chip sustains
+under its power limit), roofline.traffic (hardware-counter bytes per GEMM launch, from profiles/), hip_graph_replay
+(the same step replayed from a HIP graph), fused_quantize_transpose_step (the step with the single-read
+quantize + transposed-copy extension), vendor_gemm (torch._scaled_mm, i.e. hipBLASLt, on the six GEMM shapes,
+alternating with this library's GEMM: context for the roofline fraction, not part of the path).
 """
 import argparse
 import json
@@ -197,6 +202,44 @@ def main():
             step_fused()
         torch.cuda.synchronize()
         fused_ms = (time.perf_counter() - f0) * 1e3 / args.steps
+    vendor = None
+    if not args.no_graph and hasattr(torch, "_scaled_mm"):
+        one = torch.ones(1, device=dev)
+        shapes = [("gate_up fwd", q["w_up"], q["x"], out["y_up"]), ("down fwd", q["w_down"], q["h"], out["y_down"]),
+                  ("down dgrad", q["w_down_t"], q["dy_down"], out["dh"]), ("down wgrad", q["h_t"], q["dy_down_t"], out["dw_down"]),
+                  ("gate_up dgrad", q["w_up_t"], q["dy_up"], out["dx"]), ("gate_up wgrad", q["x_t"], q["dy_up_t"], out["dw_up"])]
+
+        def us_of(fn, iters=5):
+            fn()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(iters):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / iters * 1e3
+
+        try:
+            per_shape, ours_total, theirs_total = {}, 0.0, 0.0
+            for name, a_op, b_op, c_out in shapes:
+                M_, Kd_ = a_op.shape
+                N_ = b_op.shape[0]
+                mine = lambda: K.matmul(c_out, a_op, b_op, None, one, one, M_, N_, Kd_, workspace=ws)
+                theirs = lambda: torch._scaled_mm(b_op, a_op.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16)
+                t_mine = min(us_of(mine), us_of(mine))
+                t_theirs = min(us_of(theirs), us_of(theirs))
+                t_mine = min(t_mine, us_of(mine))
+                t_theirs = min(t_theirs, us_of(theirs))
+                flop = 2.0 * M_ * N_ * Kd_
+                per_shape[name] = {"this_library_TFLOPs": flop / t_mine / 1e6, "vendor_TFLOPs": flop / t_theirs / 1e6}
+                ours_total += t_mine
+                theirs_total += t_theirs
+            vendor = {"what": "torch._scaled_mm (hipBLASLt) on the same e4m3 operands, bf16 output, best of 3 x 5 launches, "
+                              "alternating with this library", "per_shape": per_shape,
+                      "six_gemms_us": {"this_library": ours_total, "vendor": theirs_total},
+                      "speed_vs_vendor": theirs_total / ours_total}
+        except Exception as ex:   # the comparison is context only; a torch build without fp8 support skips it
+            vendor = {"skipped": str(ex)[:200]}
     if args.calibrate_copy:
         src = torch.randint(0, 255, (1 << 30,), dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
@@ -260,6 +303,7 @@ def main():
         "fused_quantize_transpose_step": None if fused_ms is None else {
             "ms_per_step": fused_ms, "value": gemm_flop / (fused_ms * 1e-3) / 1e12,
             "note": "extension: single-read quantize + transposed copy for weights and output gradients"},
+        "vendor_gemm": vendor,
         "library": capi.version(),
     }
 

@@ -5,35 +5,40 @@
 // contiguous) produce row-major c[N,M],
 //     c[n,m] = round( (sum_k b[n,k] a[m,k]) * (sa*sb) + bias[m] + (accumulate ? c[n,m] : 0) ).
 //
-// Kernel design (nothing here is derived from the reference's mma.sync kernel):
-//   * one workgroup computes a BLK_N x BLK_M tile of c, K is walked in steps of 128 bytes;
+// Kernel design (nothing here is derived from the reference's mma.sync kernel).  Two kernels share the
+// tiling, the LDS layout and the copy scheme; each has its own description further down:
+//   * gemm_tn_e4m3_w4_kernel: 256 x 256 tile, 4 waves of 128 x 128, v_mfma_f32_16x16x128_f8f6f4,
+//     persistent; the default whenever M, N are multiples of 256 and K is a multiple of 256;
+//   * gemm_tn_e4m3_pipe_kernel: 256 x 256 tile with 8 waves of 128 x 64 or 128 x 128 tile with 4 waves
+//     of 64 x 64, v_mfma_f32_32x32x64_f8f6f4; every other shape, and the split-K path.
+// Common to both:
+//   * one workgroup computes a tile of c, K is walked in steps of 128 bytes;
 //   * both operand tiles are staged in LDS, double buffered, by 16-byte-per-lane direct-to-LDS loads
-//     (no VGPR staging) issued one K-step ahead;
+//     (no VGPR staging);
 //   * LDS rows are 128 bytes (one K-step) and the eight 16-byte chunks of a row are XOR-swizzled
 //     with (row >> 1) & 7, which makes the 128-bit fragment reads of 16 consecutive rows hit all 64
 //     banks exactly once; the swizzle is applied on the global side (each lane picks its source chunk)
 //     because direct-to-LDS loads land linearly (lane i -> base + 16 i);
-//   * the matrix instruction is v_mfma_f32_32x32x64_f8f6f4 (fp8 x fp8, K = 64 per instruction, two per
-//     K-step); both operands use the same lane->K mapping, so any consistent mapping is correct;
-//   * rows of the a-tile (the m / column index of c) are permuted on their way into LDS so that the two
+//   * both operands of the matrix instruction use the same lane->K mapping, so any consistent mapping
+//     is correct;
+//   * rows of the a-tile (the m / column index of c) are permuted on their way into LDS so that the
 //     accumulators a lane holds for one c row are consecutive columns: the epilogue stores packed
-//     pairs and 32 lanes cover a contiguous row segment;
-//   * the K loop is an explicit software pipeline over half-steps (K = 64, one matrix instruction
-//     deep).  Within a half-step the matrix instructions run row by row (b-rows fragment i against all
-//     a-rows fragments); as soon as row i has been issued its fragment registers are refilled from LDS
-//     for the next half-step, and the other operand's fragments of the next half-step go into a second
-//     small buffer.  LDS reads therefore stream under the matrix instructions with (NI + 2 NJ)
-//     fragment registers instead of a full double buffer.  The single workgroup barrier per K-step sits
-//     in the second half-step right after its first row has been queued: at that point every wave has
-//     finished reading the stage the next direct-to-LDS copies overwrite, and the stage fetched one
-//     step earlier has landed;
+//     groups and neighbouring lanes cover a contiguous row segment;
 //   * the linear workgroup id is remapped so that each of the 8 XCDs (workgroups are dealt to XCDs
 //     round-robin) works on a contiguous range of tiles, walked in column-major groups of `group`
-//     tile-rows for L2 reuse of both operands;
-//   * shapes with too few output tiles to fill the chip (weight gradients of small layers) split K
-//     over gridDim.y: every split writes its raw fp32 accumulators to a slice of the caller's
-//     workspace, and a second kernel adds the slices in a fixed order and applies the epilogue, so the
-//     result does not depend on scheduling.
+//     tile-rows for L2 reuse of both operands.
+// The 8-wave kernel's K loop is an explicit software pipeline over half-steps (K = 64, one matrix
+// instruction deep).  Within a half-step the matrix instructions run row by row (b-rows fragment i
+// against all a-rows fragments); as soon as row i has been issued its fragment registers are refilled
+// from LDS for the next half-step, and the other operand's fragments of the next half-step go into a
+// second small buffer.  LDS reads therefore stream under the matrix instructions with (NI + 2 NJ)
+// fragment registers instead of a full double buffer.  The single workgroup barrier per K-step sits in
+// the second half-step right after its first row has been queued: at that point every wave has
+// finished reading the stage the next direct-to-LDS copies overwrite, and the stage fetched one step
+// earlier has landed.  Shapes with too few output tiles to fill the chip (weight gradients of small
+// layers) split K over gridDim.y: every split writes its raw fp32 accumulators to a slice of the
+// caller's workspace, and a second kernel adds the slices in a fixed order and applies the epilogue, so
+// the result does not depend on scheduling.
 #include <type_traits>
 
 #include "common.hpp"
