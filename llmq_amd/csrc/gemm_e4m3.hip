@@ -64,9 +64,30 @@ struct GemmArgs {
     int bias_is_bf16;
     int accumulate;
     int group;       // tile-rows per rasterisation group
-    float* partial;  // split-K only: [splits][N][M] raw accumulators
-    int k_len;       // split-K only: K elements per split (multiple of 128)
+    float* partial;  // split-K only: [splits][N][M] raw accumulators (four-wave kernel: 256 x 256 tiles)
+    int k_len;       // split-K only: K elements per split (multiple of 128; four-wave kernel: of 256)
+    int rem_split;   // four-wave kernel: K segments per tile of an XCD's last, partial round (1 = none)
+    int part_per_xcd;  // four-wave kernel: partial tiles reserved per XCD in `partial`
 };
+
+// XCD x owns a contiguous range of the logical tile sequence (the first total % 8 XCDs one tile more).
+__device__ __forceinline__ void xcd_tile_range(int total, int xcd, int& first, int& count) {
+    const int xq = total / 8, xr = total % 8;
+    first = xcd * xq + (xcd < xr ? xcd : xr);
+    count = xq + (xcd < xr ? 1 : 0);
+}
+
+// Logical tile number -> tile origin: groups of `group` tile-rows, column-major inside a group.
+__device__ __forceinline__ void decode_tile256(const GemmArgs& g, int logical, int& n_blk, int& m_blk) {
+    const int tiles_n = g.N / 256, tiles_m = g.M / 256;
+    const int per_group = g.group * tiles_m;
+    const int gid = logical / per_group;
+    const int first_n = gid * g.group;
+    const int gsz = (tiles_n - first_n) < g.group ? (tiles_n - first_n) : g.group;
+    const int in_group = logical % per_group;
+    n_blk = (first_n + in_group % gsz) * 256;
+    m_blk = (in_group / gsz) * 256;
+}
 
 #define LLMQ_GLOBAL __attribute__((address_space(1)))
 
@@ -534,7 +555,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs g, int spli
 // The workgroup is persistent (one per compute unit, walking its XCD's tile list) and the stream of
 // K-steps and copies runs across tile boundaries.  Needs K to be a multiple of 256: the LDS stage and the
 // fb half of a step are then compile-time functions of the step's parity.
-template <typename OutT, int B_FMT>
+template <typename OutT, int B_FMT, bool SEG>
 __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     constexpr int BLK = 256, T = 256, WT = 128, NF = 8;
     constexpr int P_BYTES = BLK * kBK, STAGE = 2 * P_BYTES;
@@ -549,25 +570,29 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     const int wn = wave / 2, wm = wave % 2;
     const int l16 = lane % 16, kg = lane / 16;
 
-    // tile list of this workgroup: XCD x owns a contiguous range of the logical tile sequence
-    const int tiles_n = g.N / BLK, tiles_m = g.M / BLK;
-    const int total = tiles_n * tiles_m;
+    // Work list of this workgroup.  XCD x owns a contiguous range of the logical tile sequence and its
+    // workgroups (slots) take every tile_stride-th tile of it.  With g.rem_split = S > 1 the tiles of the
+    // XCD's last, partial round are left to a second launch of this kernel (SEG) that cuts each of them
+    // into S segments of K (slot s: tile s / S, segment s % S) and writes raw accumulators as a 256 x 256
+    // fp32 tile to g.partial for the reduction kernel below: the round then costs 1 / S of a tile.
+    const int total = (g.N / BLK) * (g.M / BLK);
     const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
-    const int xq = total / 8, xr = total % 8;
-    const int xcd_first = xcd * xq + (xcd < xr ? xcd : xr);
-    const int xcd_count = xq + (xcd < xr ? 1 : 0);
+    int xcd_first, xcd_count;
+    xcd_tile_range(total, xcd, xcd_first, xcd_count);
     const int tile_stride = gridDim.x / 8;
-    const int my_tiles = slot < xcd_count ? (xcd_count - slot + tile_stride - 1) / tile_stride : 0;
-    if (my_tiles == 0) return;  // uniform for the whole workgroup, before any barrier
-    auto decode = [&](int logical, int& n_blk, int& m_blk) {
-        const int per_group = g.group * tiles_m;
-        const int gid = logical / per_group;
-        const int first_n = gid * g.group;
-        const int gsz = (tiles_n - first_n) < g.group ? (tiles_n - first_n) : g.group;
-        const int in_group = logical % per_group;
-        n_blk = (first_n + in_group % gsz) * BLK;
-        m_blk = (in_group / gsz) * BLK;
-    };
+    int my_tiles, k_first = 0, k_total = g.K;
+    if constexpr (SEG) {
+        const int rem = xcd_count % tile_stride;
+        my_tiles = slot < rem * g.rem_split ? 1 : 0;
+        xcd_first += xcd_count - rem + slot / g.rem_split - slot;  // so that tile "slot" below is the segment's tile
+        k_first = (slot % g.rem_split) * g.k_len;
+        k_total = k_first + g.k_len < g.K ? g.k_len : g.K - k_first;
+    } else {
+        my_tiles = slot < xcd_count ? (xcd_count - slot + tile_stride - 1) / tile_stride : 0;
+        if (g.rem_split > 1) my_tiles = xcd_count / tile_stride;
+    }
+    if (my_tiles <= 0) return;  // uniform for the whole workgroup, before any barrier
+    auto decode = [&](int logical, int& n_blk, int& m_blk) { decode_tile256(g, logical, n_blk, m_blk); };
 
     // copies: lane -> (row tid/8 of a 32-row slab, physical 16-byte chunk tid%8); every address is a
     // wave-uniform base plus a 32-bit lane offset
@@ -583,8 +608,8 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     auto tile_bases = [&](int logical, const uint8_t*& pb, const uint8_t*& qb) {
         int nb, mb;
         decode(logical, nb, mb);
-        pb = g.b + (int64_t)nb * g.K;
-        qb = g.a + (int64_t)mb * g.K;
+        pb = g.b + (int64_t)nb * g.K + k_first;
+        qb = g.a + (int64_t)mb * g.K + k_first;
     };
     tile_bases(xcd_first + slot, p_cur, q_cur);
     // after the copies of one K-step; past the last tile the stream re-reads that tile's first K-steps
@@ -593,7 +618,7 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         copy_k0 += kBK;
         p_cur += kBK;
         q_cur += kBK;
-        if (copy_k0 == g.K) {
+        if (copy_k0 == k_total) {
             copy_k0 = 0;
             if (copy_tile + 1 < my_tiles) ++copy_tile;
             tile_bases(xcd_first + slot + copy_tile * tile_stride, p_cur, q_cur);
@@ -728,7 +753,7 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     constexpr integral_constant<int, 1> P1{};
     constexpr integral_constant<bool, true> Y{};
     constexpr integral_constant<bool, false> NO{};
-    const int KT = g.K / kBK;  // even
+    const int KT = k_total / kBK;  // even
     int logical = xcd_first + slot;
     for (int t = 0; t < my_tiles; ++t) {
         k_step(P0, Y);
@@ -746,13 +771,21 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         int n_blk, m_blk;
         decode(logical, n_blk, m_blk);
         logical += tile_stride;
-        float scale = g.sa ? *g.sa : 1.f;
-        if (g.sb) scale = scale * *g.sb;
+        float scale = 1.f;
+        int ldc = BLK;
+        OutT* c = reinterpret_cast<OutT*>(g.partial + ((int64_t)xcd * g.part_per_xcd + slot) * (BLK * BLK));
+        if constexpr (SEG) {
+            n_blk = m_blk = 0;  // tile-local coordinates in this slot's partial tile
+        } else {
+            if (g.sa) scale = *g.sa;
+            if (g.sb) scale = scale * *g.sb;
+            ldc = g.M;
+            c = reinterpret_cast<OutT*>(g.c);
+        }
         const int e_lane = opaque(threadIdx.x) % 64;
         const int el16 = e_lane % 16, ekg = e_lane / 16;
         const int m_lane = m_blk + wm * WT + 8 * el16;
-        OutT* c = reinterpret_cast<OutT*>(g.c);
-        const uint32_t lane_bytes = ((uint32_t)(4 * ekg) * (uint32_t)g.M + (uint32_t)m_lane) * (uint32_t)sizeof(OutT);
+        const uint32_t lane_bytes = ((uint32_t)(4 * ekg) * (uint32_t)ldc + (uint32_t)m_lane) * (uint32_t)sizeof(OutT);
         const int row0 = n_blk + wn * WT;
         auto rows = [&](auto bias_tag, auto acc_tag) {
             constexpr bool BIAS = decltype(bias_tag)::value;
@@ -768,7 +801,7 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
                 LLMQ_GLOBAL char* row[4];
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
-                    row[r] = scalar_ptr((LLMQ_GLOBAL char*)(c + (int64_t)(row0 + 16 * i + r) * g.M)) + lane_bytes;
+                    row[r] = scalar_ptr((LLMQ_GLOBAL char*)(c + (int64_t)(row0 + 16 * i + r) * ldc)) + lane_bytes;
                 // the old values of the fragment row's four c rows are requested together
                 float old[4][8];
                 if constexpr (ACC) {
@@ -818,7 +851,9 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         };
         constexpr std::true_type yes{};
         constexpr std::false_type no{};
-        if (g.accumulate) {
+        if constexpr (SEG) {
+            rows(no, no);
+        } else if (g.accumulate) {
             if (g.bias) rows(yes, yes);
             else rows(no, yes);
             // the loads of old values have been consumed; make the next tile's first barrier wait for
@@ -831,6 +866,49 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the surplus copies issued during the last tile
+}
+
+// Sums the K segments of the last-round tiles that the four-wave kernel's segment launch left in
+// g.partial (fixed order: the result does not depend on timing) and applies the epilogue.  One thread per
+// 8 adjacent outputs; block -> (XCD, last-round tile t, 8-row band of the tile).  Must be launched with the
+// same tile_stride, rem_split and part_per_xcd as the kernel that wrote the partial tiles.
+template <typename OutT>
+__global__ __launch_bounds__(256) void w4_segment_reduce_kernel(GemmArgs g, int tile_stride, int rem_max) {
+    typedef float v4fl __attribute__((ext_vector_type(4)));
+    const int band = blockIdx.x % 32, tr = blockIdx.x / 32;
+    const int t = tr % rem_max, xcd = tr / rem_max;
+    int xcd_first, xcd_count;
+    xcd_tile_range((g.N / 256) * (g.M / 256), xcd, xcd_first, xcd_count);
+    const int rem = xcd_count % tile_stride;
+    if (t >= rem) return;
+    int n_blk, m_blk;
+    decode_tile256(g, xcd_first + xcd_count - rem + t, n_blk, m_blk);
+    const int row = band * 8 + threadIdx.x / 32, col = (threadIdx.x % 32) * 8;
+    const float* part = g.partial + ((int64_t)xcd * g.part_per_xcd + (int64_t)t * g.rem_split) * 65536 + row * 256 + col;
+    v4fl lo = *reinterpret_cast<const v4fl*>(part), hi = *reinterpret_cast<const v4fl*>(part + 4);
+    for (int q = 1; q < g.rem_split; ++q) {
+        lo = lo + *reinterpret_cast<const v4fl*>(part + (int64_t)q * 65536);
+        hi = hi + *reinterpret_cast<const v4fl*>(part + (int64_t)q * 65536 + 4);
+    }
+    float scale = g.sa ? *g.sa : 1.f;
+    if (g.sb) scale = scale * *g.sb;
+    const int m = m_blk + col;
+    OutT* dst = reinterpret_cast<OutT*>(g.c) + (int64_t)(n_blk + row) * g.M + m;
+#pragma unroll
+    for (int h = 0; h < 4; ++h) {
+        float v0 = (h < 2 ? lo[2 * h] : hi[2 * h - 4]) * scale, v1 = (h < 2 ? lo[2 * h + 1] : hi[2 * h - 3]) * scale;
+        if (g.bias) {
+            v0 = v0 + load_bias(g.bias, g.bias_is_bf16, m + 2 * h);
+            v1 = v1 + load_bias(g.bias, g.bias_is_bf16, m + 2 * h + 1);
+        }
+        if (g.accumulate) {
+            float o0, o1;
+            PairIo<OutT>::load((const LLMQ_GLOBAL OutT*)(dst + 2 * h), o0, o1);
+            v0 = v0 + o0;
+            v1 = v1 + o1;
+        }
+        PairIo<OutT>::store((LLMQ_GLOBAL OutT*)(dst + 2 * h), v0, v1);
+    }
 }
 
 // ---- host side ------------------------------------------------------------------------------------
@@ -861,6 +939,59 @@ int g_gemm_tile = 0;
 int g_gemm_splits = 0;
 int g_gemm_persist = -1;  // -1 = automatic, 0 = never, 1 = whenever possible
 
+// Launch plan of the four-wave kernel.  A persistent grid of `grid` workgroups (grid / 8 per XCD) walks
+// tiles256 tiles.  When the last round of an XCD holds only a few tiles, those can be cut into rem_split K
+// segments each, computed by a second launch into partial tiles in the workspace and summed by
+// w4_segment_reduce_kernel: the round then takes 1 / rem_split of a tile's time, at the price of two more
+// launches.  The decision uses measured figures (microseconds): a tile of depth K on an otherwise idle
+// chip takes about K / 164 (twice as fast as in a full round); the operand bytes of the round stream at
+// about 3.5 TB/s from memory (10 TB/s when both operands fit the 256 MB last-level cache) whichever way
+// the round is organised; the extra launches cost about 14, a partial tile 0.03 in the reduction.
+struct W4Plan {
+    int grid, rem_split, k_len, part_per_xcd, rem_max;
+};
+static W4Plan plan_w4(int tiles256, int cus, int M, int N, int K, int forced_split, size_t workspace_bytes) {
+    W4Plan p{tiles256 < cus ? (tiles256 + 7) / 8 * 8 : cus, 1, K, 0, 0};
+    if (forced_split == 1) return p;
+    const int stride = cus / 8;
+    const int xq = tiles256 / 8, xr = tiles256 % 8;
+    // tiles in the last round of the XCDs (those with one tile more and the others)
+    const int rem_hi = xr ? (xq + 1) % stride : 0, rem_lo = xq % stride;
+    const int rem_max = rem_hi > rem_lo ? rem_hi : rem_lo;
+    if (rem_max == 0) return p;
+    const int pairs = K / (2 * kBK);  // segments are whole pairs of K-steps
+    const int64_t ws_tiles = (int64_t)(workspace_bytes / (size_t)(256 * 256 * 4));
+    const int rem_total = xr * rem_hi + (8 - xr) * rem_lo;
+    const double stream_us = (double)rem_total * 512.0 * K / (((double)M + N) * K <= 192e6 ? 10e6 : 3.5e6);
+    const double tile_us = (double)K / 164.0;
+    const double whole_us = tile_us > stream_us ? tile_us : stream_us;
+    int best = 1;
+    double best_gain = 5.0;  // what a cut must win to be worth it
+    for (int s = 2; s <= stride / rem_max && s <= pairs; ++s) {
+        const int seg_pairs = (pairs + s - 1) / s;
+        if ((s - 1) * seg_pairs >= pairs) continue;  // would leave the last segment empty
+        if ((int64_t)8 * rem_max * s > ws_tiles) break;
+        if (forced_split > 1) {
+            if (s == forced_split) best = s;
+            continue;
+        }
+        const double seg_us = tile_us * seg_pairs / pairs;
+        const double cut_us = (seg_us > stream_us ? seg_us : stream_us) + 14.0 + 0.03 * rem_total * s;
+        if (whole_us - cut_us > best_gain) {
+            best_gain = whole_us - cut_us;
+            best = s;
+        }
+    }
+    if (best > 1) {
+        p.grid = cus;
+        p.rem_split = best;
+        p.k_len = (pairs + best - 1) / best * 2 * kBK;
+        p.part_per_xcd = rem_max * best;
+        p.rem_max = rem_max;
+    }
+    return p;
+}
+
 template <typename OutT, int B_FMT>
 static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     LLMQ_REQUIRE(g.M > 0 && g.N > 0 && g.K > 0, "matmul: M, N, K must be positive (got %d, %d, %d)", g.M, g.N, g.K);
@@ -878,7 +1009,7 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
     LLMQ_REQUIRE((tile != 1 && tile != 3) || fits256, "matmul: the 256 x 256 tile needs M and N divisible by 256");
     const bool w4_ok = fits256 && g.K % (2 * kBK) == 0 && cus % 8 == 0;
     if (tile == 3) {
-        LLMQ_REQUIRE(w4_ok && g_gemm_splits <= 1, "matmul: the four-wave kernel needs K divisible by 256 and no K split");
+        LLMQ_REQUIRE(w4_ok, "matmul: the four-wave kernel needs K divisible by 256");
     }
     if (tile == 0) {
         // Rounds of workgroups the chip needs: one 256 x 256 tile per compute unit and round (four units
@@ -894,7 +1025,7 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
     const int64_t tiles = tile != 2 ? (int64_t)(g.N / 256) * (g.M / 256) : (int64_t)(g.N / 128) * (g.M / 128);
     const int64_t slice_bytes = (int64_t)g.N * g.M * 4;
     const int64_t ws_splits = (int64_t)(workspace_bytes / (size_t)slice_bytes);
-    int splits = g_gemm_splits;
+    int splits = tile == 3 ? 1 : g_gemm_splits;  // for the four-wave kernel the knob cuts the last round instead
     LLMQ_REQUIRE(splits >= 0, "matmul: negative split count %d", splits);
     if (splits == 0) {
         splits = 1;
@@ -909,7 +1040,6 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
         LLMQ_REQUIRE(ws_splits >= splits, "matmul: workspace of %zu bytes is too small for %d splits", workspace_bytes,
                      splits);
     }
-    if (tile == 3) splits = 1;
     if (splits > 1) {
         const int steps = g.K / kBK;
         g.k_len = ((steps + splits - 1) / splits) * kBK;
@@ -924,9 +1054,25 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
     // The four-wave kernel takes every large-tile launch it can (K a multiple of 256, no K split).
     if ((tile == 3 || (tile == 1 && g_gemm_tile == 0 && w4_ok)) && splits == 1) {
         const int tiles256 = (g.N / 256) * (g.M / 256);
-        const int grid = tiles256 < cus ? (tiles256 + 7) / 8 * 8 : cus;
-        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<OutT, B_FMT>), dim3((unsigned)grid), dim3(256), 0, stream, g);
+        W4Plan plan = plan_w4(tiles256, cus, g.M, g.N, g.K, tile == 3 ? g_gemm_splits : 0, workspace ? workspace_bytes : 0);
+        LLMQ_REQUIRE(tile != 3 || g_gemm_splits <= 1 || plan.rem_split == g_gemm_splits,
+                     "matmul: cannot cut the last round into %d segments (K = %d, workspace %zu bytes)", g_gemm_splits,
+                     g.K, workspace_bytes);
+        g.rem_split = plan.rem_split;
+        g.k_len = plan.k_len;
+        g.part_per_xcd = plan.part_per_xcd;
+        g.partial = reinterpret_cast<float*>(workspace);
+        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<OutT, B_FMT, false>), dim3((unsigned)plan.grid), dim3(256), 0, stream,
+                           g);
         LLMQ_HIP_TRY(hipGetLastError());
+        if (plan.rem_split > 1) {
+            hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<float, B_FMT, true>), dim3((unsigned)plan.grid), dim3(256), 0,
+                               stream, g);
+            LLMQ_HIP_TRY(hipGetLastError());
+            hipLaunchKernelGGL((w4_segment_reduce_kernel<OutT>), dim3((unsigned)(8 * plan.rem_max * 32)), dim3(256), 0,
+                               stream, g, plan.grid / 8, plan.rem_max);
+            LLMQ_HIP_TRY(hipGetLastError());
+        }
         return LLMQ_OK;
     }
     if (tile == 1) return launch_pipe<256, 256, 2, 4, OutT, B_FMT>(g, splits, persistent_grid, stream);
@@ -938,7 +1084,7 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
 extern "C" int llmq_gemm_tn_e4m3_bf16(uint16_t* c, const uint8_t* a, const uint8_t* b, const uint16_t* bias_or_null,
                                       const float* sa_or_null, const float* sb_or_null, void* workspace_or_null,
                                       size_t workspace_bytes, int M, int N, int K, int accumulate, void* stream) {
-    llmq::GemmArgs g{c, a, b, bias_or_null, sa_or_null, sb_or_null, M, N, K, 1, accumulate, 8, nullptr, 0};
+    llmq::GemmArgs g{c, a, b, bias_or_null, sa_or_null, sb_or_null, M, N, K, 1, accumulate, 8, nullptr, 0, 1, 0};
     return llmq::gemm_dispatch<uint16_t, 0>(g, workspace_or_null, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
@@ -946,7 +1092,7 @@ extern "C" int llmq_gemm_tn_e4m3_f32(float* c, const uint8_t* a, const uint8_t* 
                                      int bias_is_bf16, const float* sa_or_null, const float* sb_or_null,
                                      void* workspace_or_null, size_t workspace_bytes, int M, int N, int K,
                                      int accumulate, void* stream) {
-    llmq::GemmArgs g{c, a, b, bias_or_null, sa_or_null, sb_or_null, M, N, K, bias_is_bf16, accumulate, 8, nullptr, 0};
+    llmq::GemmArgs g{c, a, b, bias_or_null, sa_or_null, sb_or_null, M, N, K, bias_is_bf16, accumulate, 8, nullptr, 0, 1, 0};
     return llmq::gemm_dispatch<float, 0>(g, workspace_or_null, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
@@ -954,7 +1100,7 @@ extern "C" int llmq_gemm_tn_e4m3_e5m2_bf16(uint16_t* c, const uint8_t* a, const 
                                            const uint16_t* bias_or_null, const float* sa_or_null, const float* sb_or_null,
                                            void* workspace_or_null, size_t workspace_bytes, int M, int N, int K,
                                            int accumulate, void* stream) {
-    llmq::GemmArgs g{c, a, b_e5m2, bias_or_null, sa_or_null, sb_or_null, M, N, K, 1, accumulate, 8, nullptr, 0};
+    llmq::GemmArgs g{c, a, b_e5m2, bias_or_null, sa_or_null, sb_or_null, M, N, K, 1, accumulate, 8, nullptr, 0, 1, 0};
     return llmq::gemm_dispatch<uint16_t, 1>(g, workspace_or_null, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
@@ -962,7 +1108,7 @@ extern "C" int llmq_gemm_tn_e4m3_e5m2_f32(float* c, const uint8_t* a, const uint
                                           int bias_is_bf16, const float* sa_or_null, const float* sb_or_null,
                                           void* workspace_or_null, size_t workspace_bytes, int M, int N, int K,
                                           int accumulate, void* stream) {
-    llmq::GemmArgs g{c, a, b_e5m2, bias_or_null, sa_or_null, sb_or_null, M, N, K, bias_is_bf16, accumulate, 8, nullptr, 0};
+    llmq::GemmArgs g{c, a, b_e5m2, bias_or_null, sa_or_null, sb_or_null, M, N, K, bias_is_bf16, accumulate, 8, nullptr, 0, 1, 0};
     return llmq::gemm_dispatch<float, 1>(g, workspace_or_null, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 

@@ -188,7 +188,9 @@ def set_variant(v):
     capi.lib.llmq_debug_set_gemm_persist(v[2] if len(v) > 2 else -1)
 
 
-VARIANTS = [(0, 0), (1, 0, 0), (1, 1, 1), (2, 0), (1, 2), (2, 2), (2, 3), (3, 1)]
+# (tile selector, K splits[, persistent walk]); for the four-wave kernel (tile 3) the second number cuts the
+# tiles of each XCD's last round into that many K segments
+VARIANTS = [(0, 0), (1, 0, 0), (1, 1, 1), (2, 0), (1, 2), (2, 2), (2, 3), (3, 1), (3, 2), (3, 4)]
 _WORKSPACE = {}
 
 
@@ -203,6 +205,16 @@ def skip_unsupported(variant, M, N, Kd):
         pytest.skip("the 256 x 256 tile needs multiples of 256")
     if variant[0] == 3 and Kd % 256:
         pytest.skip("the four-wave kernel needs K divisible by 256")
+    if variant[0] == 3 and variant[1] > 1:
+        # mirrors the launch plan: 32 workgroups per XCD, segments of whole pairs of K-steps, none empty,
+        # and one 256 KiB partial tile per segment in the 32 MiB workspace
+        S, pairs, tiles = variant[1], Kd // 256, (M // 256) * (N // 256)
+        xq, xr = divmod(tiles, 8)
+        rem_max = max((xq + 1) % 32 if xr else 0, xq % 32)
+        seg = -(-pairs // S)
+        if rem_max == 0 or rem_max * S > 32 or 8 * rem_max * S > 128 or (S - 1) * seg >= pairs:
+            pytest.skip("the last round cannot be cut this way")
+        return
     if variant[1] > Kd // 128:
         pytest.skip("more splits than K-steps")
     if len(variant) > 2 and variant[2] == 1 and Kd < 256:
@@ -282,11 +294,14 @@ def test_gemm_random_codes_within_tolerance(K, O, variant, out_f32):
         set_variant((0, 0))
 
 
-@pytest.mark.parametrize("variant", [(1, 1, 1), (3, 1)])
-@pytest.mark.parametrize("mnk", [(4352, 4352, 384), (4608, 4096, 256), (8192, 4864, 512), (4352, 4352, 1024)])
+@pytest.mark.parametrize("variant", [(1, 1, 1), (3, 1), (3, 2), (3, 3), (3, 4)])
+@pytest.mark.parametrize("mnk", [(4352, 4352, 384), (4608, 4096, 256), (8192, 4864, 512), (4352, 4352, 1024),
+                                 (4352, 4096, 1024), (4352, 4352, 1536)])
 def test_gemm_persistent_tile_walk(K, O, mnk, variant):
     """More tiles than compute units: workgroups walk several tiles each and the operand stream crosses
-    tile boundaries (odd and even numbers of K-steps flip the LDS stage parity differently).  Integer
+    tile boundaries (odd and even numbers of K-steps flip the LDS stage parity differently); the (3, S)
+    variants cut the tiles left over after the full rounds into S segments of K (XCDs with 5 and 4, or
+    2 such tiles; segments of equal and unequal length).  Integer
     operands -> bit-exact against the oracle, with bias and accumulation, bf16 and fp32 outputs."""
     M, N, Kd = mnk
     skip_unsupported(variant, M, N, Kd)
@@ -313,17 +328,20 @@ def test_gemm_persistent_tile_walk(K, O, mnk, variant):
         set_variant((0, 0))
 
 
-def test_gemm_four_wave_large_repeatable(K, O):
+@pytest.mark.parametrize("variant,mnk", [((3, 1), (4096, 8192, 2048)), ((0, 0), (18944, 3584, 8192))])
+def test_gemm_four_wave_large_repeatable(K, O, variant, mnk):
     """The four-wave kernel issues its matrix instructions from asm statements (the compiler does not see
     them as such), so beyond the exact small cases: a chip-filling shape with random codes, repeated, must
-    give bit-identical results every time and agree with the exact product on sampled outputs."""
-    M, N, Kd = 4096, 8192, 2048
+    give bit-identical results every time and agree with the exact product on sampled outputs.  The
+    second case is a weight-gradient shape on which the automatic plan cuts the last round's one or two
+    tiles per XCD into K segments summed by a separate kernel."""
+    M, N, Kd = mnk
     rng = np.random.default_rng(33)
     a = rng.integers(0, 0x7E, (M, Kd)).astype(np.uint8) | (rng.integers(0, 2, (M, Kd)).astype(np.uint8) << 7)
     b = rng.integers(0, 0x7E, (N, Kd)).astype(np.uint8) | (rng.integers(0, 2, (N, Kd)).astype(np.uint8) << 7)
     ad, bd = dev_u8(a), dev_u8(b)
     sa = dev_scalar(2.0 ** -6)
-    set_variant((3, 1))
+    set_variant(variant)
     try:
         first = None
         for rep in range(8):
