@@ -240,6 +240,32 @@ def main():
                       "speed_vs_vendor": theirs_total / ours_total}
         except Exception as ex:   # the comparison is context only; a torch build without fp8 support skips it
             vendor = {"skipped": str(ex)[:200]}
+    # The activation between the two projections and its gradient (the producers of `h` and `dy_up`), with
+    # the abs-max of their outputs computed on the way: not part of the step above, which starts from given
+    # tensors as BASELINE.json's configuration does; reported for the next stage of the path.
+    swiglu = None
+    if not args.no_graph:
+        def gbs(fn, nbytes, iters=5):
+            fn()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(iters):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) / iters * 1e3
+            return {"GBps": nbytes / us / 1e3, "frac_hbm": nbytes / us / 1e3 / HBM_PEAK_GBS, "mean_us": us}
+
+        y3, h3, dh3, dy3 = (v.view(1, BT, -1) for v in (out["y_up"], t["h"], out["dh"], t["dy_up"]))
+        hq3 = q["h"].view(1, BT, -1)
+        n_act = BT * FFN
+        sw_am, sw_sc = torch.zeros(1, device=dev), torch.zeros(1, device=dev)
+        swiglu = {
+            "what": "h = swiglu(y_up) [8192 x 18944] with the abs-max epilogue; the same as e4m3 codes; its backward",
+            "swiglu_forward+abs_max (6 B/el)": gbs(lambda: K.swiglu_forward(h3, y3, sw_am), 6 * n_act),
+            "swiglu_forward_quant (5 B/el)": gbs(lambda: K.swiglu_forward_quant(hq3, sw_sc, y3, sw_am), 5 * n_act),
+            "swiglu_backward+abs_max (10 B/el)": gbs(lambda: K.swiglu_backward(dy3, dh3, y3, sw_am), 10 * n_act),
+        }
     if args.calibrate_copy:
         src = torch.randint(0, 255, (1 << 30,), dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
@@ -304,6 +330,7 @@ def main():
             "ms_per_step": fused_ms, "value": gemm_flop / (fused_ms * 1e-3) / 1e12,
             "note": "extension: single-read quantize + transposed copy for weights and output gradients"},
         "vendor_gemm": vendor,
+        "swiglu": swiglu,
         "library": capi.version(),
     }
 

@@ -163,6 +163,42 @@ int64_t llmq_backward_bias_scratch_bytes(int BT, int OC, int dout_format);
 int llmq_backward_bias_bf16(uint16_t* dbias, const void* dout, int dout_format, const float* sa_or_null,
                             const float* sb_or_null, float* scratch, size_t scratch_bytes, int BT, int OC, void* stream);
 
+/*
+ * SwiGLU producers adjacent to the quantized matmuls.  inp: row-major [B*T, 2*C] bf16, each row [up(C) | gate(C)].
+ *     s = 1 / (1 + exp(-gate));   out[bt, c] = bf16((up * gate) * s)
+ * abs_max_or_null: if non-NULL, reset and then set to max |out| over the rounded bf16 outputs (NaNs ignored),
+ * bit-identical to llmq_abs_max_bf16(out).  C must be a multiple of 8 and 2*B*T*C < 2^31 (as in the reference;
+ * B*T*C need not be a multiple of the launch's block share).  exp and the reciprocal are the hardware's
+ * (about 1 ulp each): results lie within one bf16 ulp of the correctly rounded value; the reference's own are
+ * not bit-specified either (CUDA expf + approximate reciprocal).
+ * Replaces: swiglu_forward(nv_bfloat16* out, const nv_bfloat16* inp, float* abs_max_ptr, int B, int T, int C,
+ *           cudaStream_t)  src/kernels/kernels.h:156, src/kernels/swiglu.cu:25-65,104-179,304-346.
+ */
+int llmq_swiglu_forward_bf16(uint16_t* out, const uint16_t* inp, float* abs_max_or_null, int B, int T, int C,
+                             void* stream);
+
+/*
+ * SwiGLU written directly as e4m3 codes with a known abs-max: byte-identical to llmq_swiglu_forward_bf16
+ * followed by llmq_quantize_e4m3_bf16 with the same abs_max (the invariant the reference tests,
+ * src/testing/test-swiglu.cu:243-315), without the bf16 tensor ever reaching memory.
+ * scale = 448 / max(*abs_max, 1e-10); *scale_or_null = 1 / scale.
+ * Replaces: swiglu_forward_quant(__nv_fp8_e4m3* out, float* scale_ptr, const nv_bfloat16* inp,
+ *           const float* abs_max_ptr, int B, int T, int C, cudaStream_t)
+ *           src/kernels/kernels.h:160, src/kernels/swiglu.cu:67-98,181-242,348-372.
+ */
+int llmq_swiglu_forward_quant_bf16(uint8_t* out, float* scale_or_null, const uint16_t* inp, const float* abs_max,
+                                   int B, int T, int C, void* stream);
+
+/*
+ * SwiGLU backward: dinp [B*T, 2*C] = [dup | dgate] from dout [B*T, C] and the forward input,
+ *     dup = bf16(dout * gate * s),   dgate = bf16(dout * up * s * (1 + gate * (1 - s)))
+ * (products left to right in fp32).  abs_max_or_null as above, over both halves of dinp.
+ * Replaces: swiglu_backward(nv_bfloat16* dinp, const nv_bfloat16* dout, const nv_bfloat16* inp, float* abs_max,
+ *           int B, int T, int C, cudaStream_t)  src/kernels/kernels.h:163, src/kernels/swiglu.cu:244-300,374-401.
+ */
+int llmq_swiglu_backward_bf16(uint16_t* dinp, const uint16_t* dout, const uint16_t* inp, float* abs_max_or_null,
+                              int B, int T, int C, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -355,4 +355,37 @@ inline void backward_bias(Tensor& dbias, const Tensor& dout, const float* scale_
     else llmq_detail::unsupported(__func__, dbias, dout, dbias_buffer);
 }
 
+// ---- swiglu (reference: src/kernels/kernels.h:155-165, src/kernels/swiglu.cu) --------------------------------
+// inp[B, T, 2C] rows are [up | gate]; bf16 only (the fp32 overloads of the reference belong to its fp32 models).
+inline void swiglu_forward(__hip_bfloat16* out, const __hip_bfloat16* inp, float* abs_max_ptr, int B, int T, int C,
+                           hipStream_t stream) {
+    llmq_detail::check(llmq_swiglu_forward_bf16(llmq_detail::u16(out), llmq_detail::u16(inp), abs_max_ptr, B, T, C, stream));
+}
+inline void swiglu_forward(Tensor& out, const Tensor& inp, float* abs_max_ptr, int B, int T, int C, hipStream_t stream) {
+    if (out.DType != ETensorDType::BF16 || inp.DType != ETensorDType::BF16) llmq_detail::unsupported(__func__, out, inp);
+    swiglu_forward(out.get<__hip_bfloat16>(), inp.get<__hip_bfloat16>(), abs_max_ptr, B, T, C, stream);
+}
+inline void swiglu_forward_quant(__hip_fp8_e4m3* out, float* scale_ptr, const __hip_bfloat16* inp, const float* abs_max_ptr,
+                                 int B, int T, int C, hipStream_t stream) {
+    llmq_detail::check(llmq_swiglu_forward_quant_bf16(llmq_detail::u8(out), scale_ptr, llmq_detail::u16(inp),
+                                                      abs_max_ptr, B, T, C, stream));
+}
+inline void swiglu_forward_quant(Tensor& out, float* scale_ptr, const Tensor& inp, const float* abs_max_ptr, int B, int T,
+                                 int C, hipStream_t stream) {
+    if (out.DType != ETensorDType::FP8_E4M3 || inp.DType != ETensorDType::BF16) llmq_detail::unsupported(__func__, out, inp);
+    swiglu_forward_quant(out.get<__hip_fp8_e4m3>(), scale_ptr, inp.get<__hip_bfloat16>(), abs_max_ptr, B, T, C, stream);
+}
+inline void swiglu_backward(__hip_bfloat16* dinp, const __hip_bfloat16* dout, const __hip_bfloat16* inp, float* abs_max,
+                            int B, int T, int C, hipStream_t stream) {
+    llmq_detail::check(llmq_swiglu_backward_bf16(llmq_detail::u16(dinp), llmq_detail::u16(dout), llmq_detail::u16(inp),
+                                                 abs_max, B, T, C, stream));
+}
+inline void swiglu_backward(Tensor& dinp, const Tensor& dout, const Tensor& inp, float* abs_max, int B, int T, int C,
+                            hipStream_t stream) {
+    if (dinp.DType != ETensorDType::BF16 || dout.DType != ETensorDType::BF16 || inp.DType != ETensorDType::BF16)
+        llmq_detail::unsupported(__func__, dinp, dout, inp);
+    swiglu_backward(dinp.get<__hip_bfloat16>(), dout.get<__hip_bfloat16>(), inp.get<__hip_bfloat16>(), abs_max, B, T, C,
+                    stream);
+}
+
 #endif  // LLMQ_KERNELS_HPP

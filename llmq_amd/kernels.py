@@ -11,6 +11,9 @@ Names, argument order and in-place "out first" convention are the reference's:
     matmul(c, a, b, bias, scale_a, scale_b, M, N, K, accumulate=False, stream=0)   [kernels.h convention]
     backward_bias(dbias, dout, scale_a, scale_b, dbias_buffer, stream=0)
     get_bias_backward_scratch_size(dtype, OC, BT=...)
+    swiglu_forward(out, inp, abs_max, stream=0)
+    swiglu_forward_quant(out, scale, inp, abs_max, stream=0)
+    swiglu_backward(dinp, dout, inp, abs_max, stream=0)
 `stream` is a raw hipStream_t handle (0 = torch's current stream).
 """
 import torch
@@ -161,3 +164,45 @@ def backward_bias(dbias, dout, scale_a, scale_b, dbias_buffer, stream=0):
     pbuf = _dev(dbias_buffer, "dbias_buffer", (torch.float32,))
     capi.check(capi.lib.llmq_backward_bias_bf16(pd, po, _BIAS_FMT[dout.dtype], sa, sb, pbuf, dbias_buffer.numel() * 4,
                                                 BT, OC, _stream(stream)))
+
+
+def _swiglu_dims(inp, other, name):
+    """inp: [B, T, 2C]; other: [B, T, C] (reference: src/binding/kernel_binding.cpp:289-322)."""
+    if inp.dim() != 3 or other.dim() != 3:
+        raise ValueError("inp and %s must have 3 dimensions" % name)
+    if inp.shape[2] % 2 or inp.shape[0] != other.shape[0] or inp.shape[1] != other.shape[1] or inp.shape[2] != 2 * other.shape[2]:
+        raise ValueError("inp must be [B, T, 2C] and %s [B, T, C]" % name)
+    return int(inp.shape[0]), int(inp.shape[1]), int(other.shape[2])
+
+
+def swiglu_forward(out, inp, abs_max, stream=0):
+    """out[B,T,C] = up * gate * sigmoid(gate) for inp[B,T,2C] = [up | gate] (bf16); abs_max (fp32 device scalar
+    or None) receives max |out|."""
+    B, T, Cc = _swiglu_dims(inp, out, "out")
+    o = _dev(out, "out", (torch.bfloat16,))
+    i = _dev(inp, "inp", (torch.bfloat16,))
+    a = _dev(abs_max, "abs_max", (torch.float32,), optional=True)
+    capi.check(capi.lib.llmq_swiglu_forward_bf16(o, i, a, B, T, Cc, _stream(stream)))
+
+
+def swiglu_forward_quant(out, scale, inp, abs_max, stream=0):
+    """e4m3 codes of swiglu_forward(inp) for a known abs_max, the bytes of swiglu_forward followed by
+    quantize_with_abs_max; scale[0] = abs_max / 448."""
+    B, T, Cc = _swiglu_dims(inp, out, "out")
+    o = _dev(out, "out", (torch.float8_e4m3fn, torch.uint8))
+    s = _dev(scale, "scale", (torch.float32,), optional=True)
+    i = _dev(inp, "inp", (torch.bfloat16,))
+    a = _dev(abs_max, "abs_max", (torch.float32,))
+    capi.check(capi.lib.llmq_swiglu_forward_quant_bf16(o, s, i, a, B, T, Cc, _stream(stream)))
+
+
+def swiglu_backward(dinp, dout, inp, abs_max, stream=0):
+    """dinp[B,T,2C] = [dup | dgate] from dout[B,T,C] and the forward input; abs_max receives max |dinp|."""
+    B, T, Cc = _swiglu_dims(inp, dout, "dout")
+    if dinp.shape != inp.shape:
+        raise ValueError("dinp must have the shape of inp")
+    d = _dev(dinp, "dinp", (torch.bfloat16,))
+    g = _dev(dout, "dout", (torch.bfloat16,))
+    i = _dev(inp, "inp", (torch.bfloat16,))
+    a = _dev(abs_max, "abs_max", (torch.float32,), optional=True)
+    capi.check(capi.lib.llmq_swiglu_backward_bf16(d, g, i, a, B, T, Cc, _stream(stream)))

@@ -29,6 +29,9 @@
  *   transpose          numpy .T
  *   GEMM               numpy int64 matmul on integer-valued operands (the reference's own
  *                      test-gemm.cpp construction), numpy float64 matmul on decoded operands
+ *   swiglu             torch's CPU silu and autograd in float64 (the construction of the reference's
+ *                      scripts/test_kernels.py:197-207), scipy.special.expit, closed forms (gate = 0, large
+ *                      |gate|, silu(g) - silu(-g) = g), central differences for the gradient
  * The bit-level results of the CUDA conversion instruction and of cuBLASLt themselves cannot be
  * observed here (no CUDA device or toolkit): for NaN sign/payload and for the accumulation order
  * of the closed-source GEMM the parity is unpinned by anything the reference ships; the oracle
@@ -353,6 +356,48 @@ void orc_backward_bias_bf16(uint16_t* dbias, const void* dout, int fmt, const fl
         t = t * scale;
         t = t + orc_bf16_to_f32(dbias[oc]);
         dbias[oc] = orc_f32_to_bf16(t);
+    }
+}
+
+/*
+ * SwiGLU forward / backward on bf16 tensors (kernel: src/kernels/swiglu.cu:20-23,25-65,244-300; CPU
+ * baselines of the reference's own tests: src/testing/test-swiglu.cu:28-72).  inp rows are [up(C) | gate(C)]:
+ *     s = 1 / (1 + exp(-gate));  out = up * gate * s;  dup = dout * gate * s;
+ *     dgate = dout * up * s * (1 + gate * (1 - s)).
+ * The reference's device code uses expf and an approximate reciprocal whose bits are not specified, and its
+ * tests accept 3e-2 absolute error; the oracle therefore evaluates the formulas in double and rounds once
+ * (double -> float -> bf16), i.e. it gives the correctly rounded result a device implementation is measured
+ * against.  exact_* (optional, may be NULL) receive the double values.
+ */
+void orc_swiglu_forward_bf16(uint16_t* out, double* exact_out, const uint16_t* inp, int64_t BT, int C) {
+    for (int64_t r = 0; r < BT; ++r) {
+        for (int c = 0; c < C; ++c) {
+            const double up = (double)orc_bf16_to_f32(inp[r * 2 * C + c]);
+            const double gate = (double)orc_bf16_to_f32(inp[r * 2 * C + C + c]);
+            const double v = up * gate * (1.0 / (1.0 + exp(-gate)));
+            if (exact_out) exact_out[r * C + c] = v;
+            out[r * C + c] = orc_f32_to_bf16((float)v);
+        }
+    }
+}
+
+void orc_swiglu_backward_bf16(uint16_t* dinp, double* exact_dinp, const uint16_t* dout, const uint16_t* inp,
+                              int64_t BT, int C) {
+    for (int64_t r = 0; r < BT; ++r) {
+        for (int c = 0; c < C; ++c) {
+            const double up = (double)orc_bf16_to_f32(inp[r * 2 * C + c]);
+            const double gate = (double)orc_bf16_to_f32(inp[r * 2 * C + C + c]);
+            const double d = (double)orc_bf16_to_f32(dout[r * C + c]);
+            const double s = 1.0 / (1.0 + exp(-gate));
+            const double d1 = d * gate * s;
+            const double d2 = d * up * s * (1.0 + gate * (1.0 - s));
+            if (exact_dinp) {
+                exact_dinp[r * 2 * C + c] = d1;
+                exact_dinp[r * 2 * C + C + c] = d2;
+            }
+            dinp[r * 2 * C + c] = orc_f32_to_bf16((float)d1);
+            dinp[r * 2 * C + C + c] = orc_f32_to_bf16((float)d2);
+        }
     }
 }
 

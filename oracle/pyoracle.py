@@ -16,7 +16,9 @@ _lib = None
 
 def build(force=False):
     """Compile the oracle with gcc (a second or two)."""
-    if force or not os.path.exists(_LIB_PATH):
+    sources = [os.path.join(_HERE, f) for f in ("llmq_oracle.c", "llmq_cpu_mt.c", "Makefile")]
+    stale = not os.path.exists(_LIB_PATH) or any(os.path.getmtime(f) > os.path.getmtime(_LIB_PATH) for f in sources)
+    if force or stale:
         subprocess.check_call(["make", "-C", _HERE] + (["-B"] if force else []), stdout=subprocess.DEVNULL)
     return _LIB_PATH
 
@@ -99,6 +101,10 @@ def lib():
     L.orc_quantize_fp8_f32.argtypes = [u8p, f32p, f32p, C.c_float, C.c_int64, C.c_int]
     L.orc_backward_bias_bf16.restype = None
     L.orc_backward_bias_bf16.argtypes = [u16p, C.c_void_p, C.c_int, f32p, f32p, C.c_int64, C.c_int, f64p, f64p]
+    L.orc_swiglu_forward_bf16.restype = None
+    L.orc_swiglu_forward_bf16.argtypes = [u16p, f64p, u16p, C.c_int64, C.c_int]
+    L.orc_swiglu_backward_bf16.restype = None
+    L.orc_swiglu_backward_bf16.argtypes = [u16p, f64p, u16p, u16p, C.c_int64, C.c_int]
     _lib = L
     return L
 
@@ -282,3 +288,25 @@ def quantize_f32(x, absmax, fmt="e4m3"):
     lib().orc_quantize_fp8_f32(_p(out, C.c_uint8), _p(sc, C.c_float), _p(x, C.c_float), C.c_float(absmax), x.size,
                                1 if fmt == "e5m2" else 0)
     return out, sc[0]
+
+
+def swiglu_forward(inp):
+    """inp: uint16 bf16 bits [BT, 2C] (rows [up | gate]) -> (out bits uint16 [BT, C], exact float64 [BT, C])."""
+    inp = np.ascontiguousarray(inp, dtype=np.uint16)
+    BT, C2 = inp.shape
+    out = np.empty((BT, C2 // 2), dtype=np.uint16)
+    exact = np.empty((BT, C2 // 2), dtype=np.float64)
+    lib().orc_swiglu_forward_bf16(_p(out, C.c_uint16), _p(exact, C.c_double), _p(inp, C.c_uint16), BT, C2 // 2)
+    return out, exact
+
+
+def swiglu_backward(dout, inp):
+    """dout: bf16 bits [BT, C], inp: [BT, 2C] -> (dinp bits uint16 [BT, 2C] = [dup | dgate], exact float64)."""
+    inp = np.ascontiguousarray(inp, dtype=np.uint16)
+    dout = np.ascontiguousarray(dout, dtype=np.uint16)
+    BT, C2 = inp.shape
+    dinp = np.empty((BT, C2), dtype=np.uint16)
+    exact = np.empty((BT, C2), dtype=np.float64)
+    lib().orc_swiglu_backward_bf16(_p(dinp, C.c_uint16), _p(exact, C.c_double), _p(dout, C.c_uint16),
+                                   _p(inp, C.c_uint16), BT, C2 // 2)
+    return dinp, exact

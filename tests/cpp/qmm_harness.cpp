@@ -1,5 +1,5 @@
 // C++ harness: replays forward_qmm / backward_qmm (include/llmq_qmm.hpp) for one linear layer on the
-// GPU through the C++ shim and compares every result with the CPU oracle (oracle/llmq_oracle.c, linked
+// GPU through the C++ shim (plus the SwiGLU activation on the projection output) and compares every result with the CPU oracle (oracle/llmq_oracle.c, linked
 // into this test binary only).  Also exercises the shim's exception behaviour.
 //   usage: qmm_harness BT C OC [reuse_inp]
 #include <hip/hip_runtime.h>
@@ -20,6 +20,7 @@ void orc_transpose_u8(uint8_t* dst, const uint8_t* src, int rows, int cols);
 void orc_gemm_tn_e4m3_exact_sampled(double* exact, double* sumabs, const uint8_t* a, const uint8_t* b, int M, int N, int K,
                                     const int32_t* idx_n, const int32_t* idx_m, int64_t count);
 void orc_fill_normal_bf16(uint16_t* out, int64_t n, uint64_t seed, uint64_t stream, float mean, float std);
+void orc_swiglu_forward_bf16(uint16_t* out, double* exact_out, const uint16_t* inp, int64_t BT, int C);
 void orc_backward_bias_bf16(uint16_t* dbias, const void* dout, int fmt, const float* sa, const float* sb, int64_t BT, int OC, double* colsum, double* colabs);
 }
 
@@ -155,6 +156,48 @@ int main(int argc, char** argv) {
         }
         std::printf("%-8s worst error / bound %.3f\n", "dbias", worst);
         EXPECT(worst <= 1.0, "dbias exceeds the element bound");
+    }
+
+    if (OC % 16 == 0) {
+        // The projection's output as the [up | gate] input of the activation in front of the next matmul
+        // (llama_model.cpp:216 and :613-617): swiglu_forward with its abs-max, then the e4m3 codes either by
+        // quantize_with_abs_max or directly by swiglu_forward_quant -- the same bytes.
+        const int D = OC / 2;
+        const std::size_t n = (std::size_t)BT * D;
+        float* hstat = dalloc<float>(4);
+        Tensor act = make(ETensorDType::BF16, dalloc<uint16_t>(n), {BT, D});
+        Tensor act_q = make(ETensorDType::FP8_E4M3, dalloc<uint8_t>(n), {BT, D}, hstat);
+        Tensor act_q2 = make(ETensorDType::FP8_E4M3, dalloc<uint8_t>(n), {BT, D}, hstat + 2);
+        swiglu_forward(act, out, act_q.abs_max(), B, T, D, stream);
+        quantize_with_abs_max(act_q, act_q.scale(), act, act_q.abs_max(), (long)n, rs.DeviceProp, stream);
+        swiglu_forward_quant(act_q2, act_q2.scale(), out, act_q.abs_max(), B, T, D, stream);
+        HIP_OK(hipStreamSynchronize(stream));
+        std::vector<uint16_t> hact(n), want(n);
+        std::vector<double> exact(n);
+        std::vector<uint8_t> q1(n), q2(n), qo(n);
+        float st[4];
+        HIP_OK(hipMemcpy(hact.data(), act.Data, n * 2, hipMemcpyDeviceToHost));
+        HIP_OK(hipMemcpy(q1.data(), act_q.Data, n, hipMemcpyDeviceToHost));
+        HIP_OK(hipMemcpy(q2.data(), act_q2.Data, n, hipMemcpyDeviceToHost));
+        HIP_OK(hipMemcpy(st, hstat, 16, hipMemcpyDeviceToHost));
+        orc_swiglu_forward_bf16(want.data(), exact.data(), hy.data(), BT, D);
+        double worst = 0;
+        for (std::size_t i = 0; i < n; ++i)
+            worst = std::fmax(worst, std::fabs((double)orc_bf16_to_f32(hact[i]) - (double)orc_bf16_to_f32(want[i])) /
+                                         (std::ldexp(std::fabs(exact[i]), -7) + 1e-38));
+        std::printf("%-10s [%d x %d]: worst error / (one bf16 ulp) %.3f\n", "swiglu", BT, D, worst);
+        EXPECT(worst <= 1.0, "swiglu_forward is more than one bf16 ulp from the oracle");
+        const float aa = orc_abs_max_bf16(hact.data(), n);
+        float sq;
+        orc_quantize_e4m3_bf16(qo.data(), &sq, hact.data(), aa, n);
+        EXPECT(std::memcmp(&st[0], &aa, 4) == 0, "swiglu abs-max differs from the abs-max of its output");
+        EXPECT(std::memcmp(&st[1], &sq, 4) == 0 && std::memcmp(&st[3], &sq, 4) == 0, "swiglu quantization scales differ");
+        EXPECT(std::memcmp(q1.data(), qo.data(), n) == 0, "quantized activation differs from the oracle");
+        EXPECT(std::memcmp(q1.data(), q2.data(), n) == 0, "swiglu_forward_quant differs from swiglu_forward + quantize");
+        bool sw_threw = false;
+        try { swiglu_forward(act, out, nullptr, B, T, D + 4, stream); }
+        catch (const std::invalid_argument&) { sw_threw = true; }
+        EXPECT(sw_threw, "swiglu_forward with C %% 8 != 0 must throw std::invalid_argument");
     }
 
     // ---- error behaviour of the shim (reference: gemm_mma.cu:261-263, kernels.cpp:18-24) ----

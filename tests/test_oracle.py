@@ -403,3 +403,70 @@ def test_quantize_fp32_input_vs_search(O):
     q5, d5 = O.quantize_f32(x, am, "e5m2")
     assert np.array_equal(q4, e4m3_encode_search(y)) and np.array_equal(q5, e5m2_encode_search(y))
     assert d4 == np.float32(d) and d5 == np.float32(d)
+
+
+# ------------------------------------------------------------------------------------------ swiglu
+def _swiglu_inputs(O, BT, C, seed, spread=2.0):
+    inp = O.fill_normal_bf16(BT * 2 * C, seed, 0, 0.0, spread).reshape(BT, 2 * C)
+    dout = O.fill_normal_bf16(BT * C, seed, 1, 0.0, 1.0).reshape(BT, C)
+    return inp, dout
+
+
+def test_swiglu_forward_vs_torch_silu_and_expit(O):
+    """The construction of the reference's scripts/test_kernels.py:197-199 (silu(second half) * first half)
+    in float64 on torch's CPU kernels, and scipy's expit: the oracle's double values must agree to
+    double precision and its bf16 bits must be the rounding of those values."""
+    from scipy.special import expit
+    BT, C = 37, 48
+    inp, _ = _swiglu_inputs(O, BT, C, 101)
+    bits, exact = O.swiglu_forward(inp)
+    x = torch.from_numpy(O.bf16_to_f32(inp).astype(np.float64))
+    a, b = torch.tensor_split(x, 2, dim=-1)
+    ref = (torch.nn.functional.silu(b) * a).numpy()
+    assert np.allclose(exact, ref, rtol=1e-13, atol=1e-300)
+    up, gate = O.bf16_to_f32(inp[:, :C]).astype(np.float64), O.bf16_to_f32(inp[:, C:]).astype(np.float64)
+    assert np.allclose(exact, up * gate * expit(gate), rtol=1e-13, atol=1e-300)
+    # rounding: bits are the nearest bf16 of the double value (ties are measure-zero here)
+    want = O.f32_to_bf16(ref.astype(np.float32))
+    assert np.array_equal(bits, want)
+
+
+def test_swiglu_forward_closed_forms(O):
+    """gate = 0 gives 0; large gate gives up * gate; very negative gate gives (signed) zero;
+    silu(g) - silu(-g) = g."""
+    C = 8
+    f = lambda v: O.f32_to_bf16(np.asarray(v, dtype=np.float32))
+    up = f([1.5, -2.0, 3.0, 0.5, 1.0, -1.0, 7.0, 0.25])
+    for gate_val, expect in ((0.0, lambda u: 0.0 * u), (64.0, lambda u: u * 64.0), (-200.0, lambda u: 0.0 * u)):
+        inp = np.concatenate([up, f([gate_val] * C)]).reshape(1, 2 * C)
+        bits, _ = O.swiglu_forward(inp)
+        assert np.array_equal(O.bf16_to_f32(bits)[0], expect(O.bf16_to_f32(up)).astype(np.float32))
+    g = f(np.linspace(-6, 6, C))
+    ones = f([1.0] * C)
+    _, pos = O.swiglu_forward(np.concatenate([ones, g]).reshape(1, 2 * C))
+    neg_g = f(-O.bf16_to_f32(g))
+    _, neg = O.swiglu_forward(np.concatenate([ones, neg_g]).reshape(1, 2 * C))
+    assert np.allclose(pos - neg, O.bf16_to_f32(g).astype(np.float64), rtol=1e-12, atol=1e-12)
+
+
+def test_swiglu_backward_vs_torch_autograd_and_differences(O):
+    """Gradient against torch autograd in float64 (scripts/test_kernels.py:202-207 in the reference) and
+    against central differences of the forward formula; the halves of dinp are [dup | dgate]."""
+    BT, C = 9, 24
+    inp, dout = _swiglu_inputs(O, BT, C, 202)
+    bits, exact = O.swiglu_backward(dout, inp)
+    x = torch.from_numpy(O.bf16_to_f32(inp).astype(np.float64)).requires_grad_(True)
+    a, b = torch.tensor_split(x, 2, dim=-1)
+    (torch.nn.functional.silu(b) * a).backward(torch.from_numpy(O.bf16_to_f32(dout).astype(np.float64)))
+    ref = x.grad.numpy()
+    assert np.allclose(exact, ref, rtol=1e-12, atol=1e-14)
+    assert np.array_equal(bits, O.f32_to_bf16(ref.astype(np.float32)))
+    xv = O.bf16_to_f32(inp).astype(np.float64)
+    fwd = lambda v: v[:, :C] * v[:, C:] / (1.0 + np.exp(-v[:, C:]))
+    h = 1e-6
+    d = O.bf16_to_f32(dout).astype(np.float64)
+    for half in (0, 1):
+        step = np.zeros_like(xv)
+        step[:, half * C:(half + 1) * C] = h
+        num = (fwd(xv + step) - fwd(xv - step)) / (2 * h) * d
+        assert np.allclose(exact[:, half * C:(half + 1) * C], num, rtol=1e-6, atol=1e-8)
