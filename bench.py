@@ -261,11 +261,19 @@ def main():
         n_act = BT * FFN
         sw_am, sw_sc = torch.zeros(1, device=dev), torch.zeros(1, device=dev)
         swiglu = {
-            "what": "h = swiglu(y_up) [8192 x 18944] with the abs-max epilogue; the same as e4m3 codes; its backward",
+            "what": "producers of the projections' inputs with the abs-max of their output computed on the way: "
+                    "h = swiglu(y_up) [8192 x 18944], the same as e4m3 codes, its backward, and the residual add + rmsnorm",
             "swiglu_forward+abs_max (6 B/el)": gbs(lambda: K.swiglu_forward(h3, y3, sw_am), 6 * n_act),
             "swiglu_forward_quant (5 B/el)": gbs(lambda: K.swiglu_forward_quant(hq3, sw_sc, y3, sw_am), 5 * n_act),
             "swiglu_backward+abs_max (10 B/el)": gbs(lambda: K.swiglu_backward(dy3, dh3, y3, sw_am), 10 * n_act),
         }
+        # x = rmsnorm(residual + attention output) [8192 x 3584], the producer of the gate+up projection's input
+        x3 = t["x"].view(1, BT, C)
+        r_in, r_att = torch.randn_like(x3), torch.randn_like(x3)
+        r_out, r_norm, r_rms = torch.empty_like(x3), torch.empty_like(x3), torch.empty((1, BT), device=dev)
+        r_w = torch.ones(C, dtype=torch.bfloat16, device=dev)
+        swiglu["fused_residual_rmsnorm_forward+abs_max (8 B/el)"] = gbs(
+            lambda: K.fused_residual_rmsnorm_forward(r_out, r_norm, r_rms, r_in, r_att, r_w, sw_am, 1e-6), 8 * BT * C, iters=10)
     if args.calibrate_copy:
         src = torch.randint(0, 255, (1 << 30,), dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
@@ -330,7 +338,7 @@ def main():
             "ms_per_step": fused_ms, "value": gemm_flop / (fused_ms * 1e-3) / 1e12,
             "note": "extension: single-read quantize + transposed copy for weights and output gradients"},
         "vendor_gemm": vendor,
-        "swiglu": swiglu,
+        "producers": swiglu,
         "library": capi.version(),
     }
 

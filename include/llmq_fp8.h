@@ -199,6 +199,32 @@ int llmq_swiglu_forward_quant_bf16(uint8_t* out, float* scale_or_null, const uin
 int llmq_swiglu_backward_bf16(uint16_t* dinp, const uint16_t* dout, const uint16_t* inp, float* abs_max_or_null,
                               int B, int T, int C, void* stream);
 
+/*
+ * RMSNorm forward, the producer of the projections' bf16 input.  Per row of C elements of inp [B*T, C]:
+ *     s = 1 / sqrt(mean(x^2) + epsilon);  out = bf16((float)bf16(s * x) * (float)weight[c]);  rms[row] = s
+ * (the normalised value is rounded to bf16 before the scale, as in the reference).  abs_max_or_null: reset, then
+ * max |out| over the rounded outputs, bit-identical to llmq_abs_max_bf16(out).  rms_or_null may be NULL.
+ * C must be a multiple of 8 and at most 16384.  The squares are summed in fp32 in a fixed order (deterministic);
+ * s is within a few fp32 ulp of the exact value, the reference's own s (approximate rsqrt, launch-dependent
+ * summation order) is not bit-specified.
+ * Replaces: rmsnorm_forward(nv_bfloat16* out, float* rms, const nv_bfloat16* inp, const nv_bfloat16* weight,
+ *           float* abs_max_ptr, float epsilon, int B, int T, int C, cudaStream_t)
+ *           src/kernels/kernels.h:46, src/kernels/rmsnorm.cu:17-86,168-178,183-217.
+ */
+int llmq_rmsnorm_forward_bf16(uint16_t* out, float* rms_or_null, const uint16_t* inp, const uint16_t* weight,
+                              float* abs_max_or_null, float epsilon, int B, int T, int C, void* stream);
+
+/*
+ * The same with the residual add in front: residual[row] = bf16((float)inp1 + (float)inp2) is stored and normalised;
+ * N rows.  residual may be the same buffer as inp1 or inp2.
+ * Replaces: fused_residual_rmsnorm_forward(nv_bfloat16* residual, nv_bfloat16* normed, float* rrms,
+ *           const nv_bfloat16* inp1, const nv_bfloat16* inp2, const nv_bfloat16* weight, float* abs_max_ptr,
+ *           float epsilon, int N, int C, cudaStream_t)  src/kernels/kernels.h:59-60, src/kernels/rmsnorm.cu:88-164,224-227.
+ */
+int llmq_fused_residual_rmsnorm_forward_bf16(uint16_t* residual, uint16_t* normed, float* rrms, const uint16_t* inp1,
+                                             const uint16_t* inp2, const uint16_t* weight, float* abs_max_or_null,
+                                             float epsilon, int N, int C, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -388,4 +388,37 @@ inline void swiglu_backward(Tensor& dinp, const Tensor& dout, const Tensor& inp,
                     stream);
 }
 
+// ---- rmsnorm forward (reference: src/kernels/kernels.h:45-47,57-62, src/kernels/rmsnorm.cu) ------------------------
+inline void rmsnorm_forward(__hip_bfloat16* out, float* rms, const __hip_bfloat16* inp, const __hip_bfloat16* weight,
+                            float* abs_max_ptr, float epsilon, int B, int T, int C, hipStream_t stream) {
+    llmq_detail::check(llmq_rmsnorm_forward_bf16(llmq_detail::u16(out), rms, llmq_detail::u16(inp), llmq_detail::u16(weight),
+                                                 abs_max_ptr, epsilon, B, T, C, stream));
+}
+inline void rmsnorm_forward(Tensor& out, Tensor& rms, const Tensor& inp, const Tensor& weight, float* abs_max_ptr,
+                            float epsilon, int B, int T, int C, hipStream_t stream) {
+    if (out.DType != ETensorDType::BF16 || inp.DType != ETensorDType::BF16 || weight.DType != ETensorDType::BF16 ||
+        rms.DType != ETensorDType::FP32)
+        llmq_detail::unsupported(__func__, out, rms, inp, weight);
+    rmsnorm_forward(out.get<__hip_bfloat16>(), rms.get<float>(), inp.get<__hip_bfloat16>(), weight.get<__hip_bfloat16>(),
+                    abs_max_ptr, epsilon, B, T, C, stream);
+}
+inline void fused_residual_rmsnorm_forward(__hip_bfloat16* residual, __hip_bfloat16* normed, float* rrms,
+                                           const __hip_bfloat16* inp1, const __hip_bfloat16* inp2,
+                                           const __hip_bfloat16* weight, float* abs_max_ptr, float epsilon, int N, int C,
+                                           hipStream_t stream) {
+    llmq_detail::check(llmq_fused_residual_rmsnorm_forward_bf16(llmq_detail::u16(residual), llmq_detail::u16(normed), rrms,
+                                                                llmq_detail::u16(inp1), llmq_detail::u16(inp2),
+                                                                llmq_detail::u16(weight), abs_max_ptr, epsilon, N, C, stream));
+}
+inline void fused_residual_rmsnorm_forward(Tensor& residual, Tensor& normed, Tensor& rrms, const Tensor& inp1,
+                                           const Tensor& inp2, const Tensor& weight, float* abs_max_ptr, float epsilon,
+                                           int N, int C, hipStream_t stream) {
+    if (residual.DType != ETensorDType::BF16 || normed.DType != ETensorDType::BF16 || inp1.DType != ETensorDType::BF16 ||
+        inp2.DType != ETensorDType::BF16 || weight.DType != ETensorDType::BF16 || rrms.DType != ETensorDType::FP32)
+        llmq_detail::unsupported(__func__, residual, normed, rrms, inp1, inp2, weight);
+    fused_residual_rmsnorm_forward(residual.get<__hip_bfloat16>(), normed.get<__hip_bfloat16>(), rrms.get<float>(),
+                                   inp1.get<__hip_bfloat16>(), inp2.get<__hip_bfloat16>(), weight.get<__hip_bfloat16>(),
+                                   abs_max_ptr, epsilon, N, C, stream);
+}
+
 #endif  // LLMQ_KERNELS_HPP

@@ -21,6 +21,7 @@ EXPORTS = [
     "llmq_transpose_u8", "llmq_gemm_tn_e4m3_bf16", "llmq_gemm_tn_e4m3_f32", "llmq_gemm_tn_e4m3_e5m2_bf16", "llmq_gemm_tn_e4m3_e5m2_f32",
     "llmq_backward_bias_bf16", "llmq_backward_bias_scratch_bytes", "llmq_quantize_both_bf16", "llmq_quantize_e4m3_f32", "llmq_quantize_e5m2_f32",
     "llmq_swiglu_forward_bf16", "llmq_swiglu_forward_quant_bf16", "llmq_swiglu_backward_bf16",
+    "llmq_rmsnorm_forward_bf16", "llmq_fused_residual_rmsnorm_forward_bf16",
 ]
 
 if not os.path.exists(LIB_PATH):
@@ -50,6 +51,8 @@ lib.llmq_backward_bias_scratch_bytes.argtypes = [_int, _int, _int]
 lib.llmq_swiglu_forward_bf16.argtypes = [_vp, _vp, _vp, _int, _int, _int, _vp]
 lib.llmq_swiglu_forward_quant_bf16.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _vp]
 lib.llmq_swiglu_backward_bf16.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _vp]
+lib.llmq_rmsnorm_forward_bf16.argtypes = [_vp, _vp, _vp, _vp, _vp, C.c_float, _int, _int, _int, _vp]
+lib.llmq_fused_residual_rmsnorm_forward_bf16.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, C.c_float, _int, _int, _vp]
 lib.llmq_debug_set_gemm_variant.argtypes = [_int, _int]
 lib.llmq_debug_set_gemm_variant.restype = None
 lib.llmq_debug_set_gemm_persist.argtypes = [_int]

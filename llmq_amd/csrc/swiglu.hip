@@ -55,13 +55,15 @@ __device__ __forceinline__ uint32_t input_chunk(uint32_t idx, uint32_t chunks_pe
 }
 
 // MODE 0: bf16 output; 1: bf16 output + abs-max; 2: e4m3 output with the scale from *absmax_in
-template <int MODE, int UNROLL>
-__global__ __launch_bounds__(256) void swiglu_forward_kernel(void* __restrict__ out, const uint4* __restrict__ inp,
+// THREADS: 256, or 1024 with the abs-max (fewer workgroups -> fewer atomics on the one slot when the
+// workgroups of the first resident round finish together and all find it empty).
+template <int MODE, int UNROLL, int THREADS>
+__global__ __launch_bounds__(THREADS) void swiglu_forward_kernel(void* __restrict__ out, const uint4* __restrict__ inp,
                                                              unsigned* __restrict__ absmax_out,
                                                              const float* __restrict__ absmax_in,
                                                              float* __restrict__ scale_ptr, uint32_t nchunks,
                                                              uint32_t chunks_per_row) {
-    const uint32_t base = blockIdx.x * (256u * UNROLL) + threadIdx.x;
+    const uint32_t base = blockIdx.x * ((uint32_t)THREADS * UNROLL) + threadIdx.x;
     float s = 0.f;
     if constexpr (MODE == 2) {
         s = quant_scale(*absmax_in);
@@ -70,7 +72,7 @@ __global__ __launch_bounds__(256) void swiglu_forward_kernel(void* __restrict__ 
     uint4 up[UNROLL], gate[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-        const uint32_t idx = base + u * 256u;
+        const uint32_t idx = base + u * (uint32_t)THREADS;
         up[u] = gate[u] = make_uint4(0, 0, 0, 0);
         if (idx < nchunks) {
             const uint32_t src = input_chunk(idx, chunks_per_row);
@@ -81,7 +83,7 @@ __global__ __launch_bounds__(256) void swiglu_forward_kernel(void* __restrict__ 
     uint32_t acc = 0x7F807F80u;
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-        const uint32_t idx = base + u * 256u;
+        const uint32_t idx = base + u * (uint32_t)THREADS;
         const uint4 r = swiglu_chunk(up[u], gate[u]);  // zeros for the predicated-off chunks
         if constexpr (MODE == 1) acc = fold_vec(acc, r);
         if (idx < nchunks) {
@@ -110,16 +112,16 @@ __device__ __forceinline__ void swiglu_grad_pair(uint32_t dout, uint32_t up, uin
     dgate = pack_bf16(d2[0], d2[1]);
 }
 
-template <bool ABSMAX, int UNROLL>
-__global__ __launch_bounds__(256) void swiglu_backward_kernel(uint4* __restrict__ dinp, const uint4* __restrict__ dout,
+template <bool ABSMAX, int UNROLL, int THREADS>
+__global__ __launch_bounds__(THREADS) void swiglu_backward_kernel(uint4* __restrict__ dinp, const uint4* __restrict__ dout,
                                                               const uint4* __restrict__ inp,
                                                               unsigned* __restrict__ absmax_out, uint32_t nchunks,
                                                               uint32_t chunks_per_row) {
-    const uint32_t base = blockIdx.x * (256u * UNROLL) + threadIdx.x;
+    const uint32_t base = blockIdx.x * ((uint32_t)THREADS * UNROLL) + threadIdx.x;
     uint4 d[UNROLL], up[UNROLL], gate[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-        const uint32_t idx = base + u * 256u;
+        const uint32_t idx = base + u * (uint32_t)THREADS;
         d[u] = up[u] = gate[u] = make_uint4(0, 0, 0, 0);
         if (idx < nchunks) {
             const uint32_t src = input_chunk(idx, chunks_per_row);
@@ -131,7 +133,7 @@ __global__ __launch_bounds__(256) void swiglu_backward_kernel(uint4* __restrict_
     uint32_t acc = 0x7F807F80u;
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-        const uint32_t idx = base + u * 256u;
+        const uint32_t idx = base + u * (uint32_t)THREADS;
         uint4 g1, g2;
         swiglu_grad_pair(d[u].x, up[u].x, gate[u].x, g1.x, g2.x);
         swiglu_grad_pair(d[u].y, up[u].y, gate[u].y, g1.y, g2.y);
@@ -162,7 +164,11 @@ static int check_shape(const char* what, int B, int T, int C, int64_t& nchunks) 
     return LLMQ_OK;
 }
 
-constexpr int kFwdUnroll = 4, kBwdUnroll = 2;
+constexpr int kFwdUnroll = 4, kBwdUnroll = 2, kAbsmaxThreads = 1024;
+
+static unsigned blocks_for(int64_t nchunks, int threads, int unroll) {
+    return (unsigned)((nchunks + (int64_t)threads * unroll - 1) / ((int64_t)threads * unroll));
+}
 
 }  // namespace llmq
 
@@ -180,13 +186,14 @@ extern "C" int llmq_swiglu_forward_bf16(uint16_t* out, const uint16_t* inp, floa
     if (nchunks == 0) return LLMQ_OK;
     LLMQ_REQUIRE(out && inp, "swiglu_forward: null tensor pointer");
     LLMQ_REQUIRE(aligned16(out) && aligned16(inp), "swiglu_forward: pointers must be 16-byte aligned");
-    const unsigned blocks = (unsigned)((nchunks + 256 * kFwdUnroll - 1) / (256 * kFwdUnroll));
     if (abs_max_or_null)
-        hipLaunchKernelGGL((swiglu_forward_kernel<1, kFwdUnroll>), dim3(blocks), dim3(256), 0, stream, out,
+        hipLaunchKernelGGL((swiglu_forward_kernel<1, kFwdUnroll, kAbsmaxThreads>),
+                           dim3(blocks_for(nchunks, kAbsmaxThreads, kFwdUnroll)), dim3(kAbsmaxThreads), 0, stream, out,
                            reinterpret_cast<const uint4*>(inp), reinterpret_cast<unsigned*>(abs_max_or_null), nullptr,
                            nullptr, (uint32_t)nchunks, (uint32_t)(C / 8));
     else
-        hipLaunchKernelGGL((swiglu_forward_kernel<0, kFwdUnroll>), dim3(blocks), dim3(256), 0, stream, out,
+        hipLaunchKernelGGL((swiglu_forward_kernel<0, kFwdUnroll, 256>), dim3(blocks_for(nchunks, 256, kFwdUnroll)),
+                           dim3(256), 0, stream, out,
                            reinterpret_cast<const uint4*>(inp), nullptr, nullptr, nullptr, (uint32_t)nchunks,
                            (uint32_t)(C / 8));
     LLMQ_HIP_TRY(hipGetLastError());
@@ -203,8 +210,8 @@ extern "C" int llmq_swiglu_forward_quant_bf16(uint8_t* out, float* scale_or_null
     LLMQ_REQUIRE(aligned16(inp) && (reinterpret_cast<uintptr_t>(out) & 7u) == 0,
                  "swiglu_forward_quant: inp must be 16-byte and out 8-byte aligned");
     // an empty tensor still gets its scale written, by the same kernel (grid of one workgroup)
-    const unsigned blocks = nchunks ? (unsigned)((nchunks + 256 * kFwdUnroll - 1) / (256 * kFwdUnroll)) : 1u;
-    hipLaunchKernelGGL((swiglu_forward_kernel<2, kFwdUnroll>), dim3(blocks), dim3(256), 0, stream, out,
+    const unsigned blocks = nchunks ? blocks_for(nchunks, 256, kFwdUnroll) : 1u;
+    hipLaunchKernelGGL((swiglu_forward_kernel<2, kFwdUnroll, 256>), dim3(blocks), dim3(256), 0, stream, out,
                        reinterpret_cast<const uint4*>(inp), nullptr, abs_max, scale_or_null, (uint32_t)nchunks,
                        (uint32_t)(C > 0 ? C / 8 : 1));
     LLMQ_HIP_TRY(hipGetLastError());
@@ -223,14 +230,15 @@ extern "C" int llmq_swiglu_backward_bf16(uint16_t* dinp, const uint16_t* dout, c
     if (nchunks == 0) return LLMQ_OK;
     LLMQ_REQUIRE(dinp && dout && inp, "swiglu_backward: null tensor pointer");
     LLMQ_REQUIRE(aligned16(dinp) && aligned16(dout) && aligned16(inp), "swiglu_backward: pointers must be 16-byte aligned");
-    const unsigned blocks = (unsigned)((nchunks + 256 * kBwdUnroll - 1) / (256 * kBwdUnroll));
     if (abs_max_or_null)
-        hipLaunchKernelGGL((swiglu_backward_kernel<true, kBwdUnroll>), dim3(blocks), dim3(256), 0, stream,
+        hipLaunchKernelGGL((swiglu_backward_kernel<true, kBwdUnroll, kAbsmaxThreads>),
+                           dim3(blocks_for(nchunks, kAbsmaxThreads, kBwdUnroll)), dim3(kAbsmaxThreads), 0, stream,
                            reinterpret_cast<uint4*>(dinp), reinterpret_cast<const uint4*>(dout),
                            reinterpret_cast<const uint4*>(inp), reinterpret_cast<unsigned*>(abs_max_or_null),
                            (uint32_t)nchunks, (uint32_t)(C / 8));
     else
-        hipLaunchKernelGGL((swiglu_backward_kernel<false, kBwdUnroll>), dim3(blocks), dim3(256), 0, stream,
+        hipLaunchKernelGGL((swiglu_backward_kernel<false, kBwdUnroll, 256>), dim3(blocks_for(nchunks, 256, kBwdUnroll)),
+                           dim3(256), 0, stream,
                            reinterpret_cast<uint4*>(dinp), reinterpret_cast<const uint4*>(dout),
                            reinterpret_cast<const uint4*>(inp), nullptr, (uint32_t)nchunks, (uint32_t)(C / 8));
     LLMQ_HIP_TRY(hipGetLastError());

@@ -14,6 +14,8 @@ Names, argument order and in-place "out first" convention are the reference's:
     swiglu_forward(out, inp, abs_max, stream=0)
     swiglu_forward_quant(out, scale, inp, abs_max, stream=0)
     swiglu_backward(dinp, dout, inp, abs_max, stream=0)
+    rmsnorm_forward(out, rms, inp, weight, abs_max, epsilon, stream=0)
+    fused_residual_rmsnorm_forward(residual, normed, rrms, inp1, inp2, weight, abs_max, epsilon, stream=0)
 `stream` is a raw hipStream_t handle (0 = torch's current stream).
 """
 import torch
@@ -206,3 +208,36 @@ def swiglu_backward(dinp, dout, inp, abs_max, stream=0):
     i = _dev(inp, "inp", (torch.bfloat16,))
     a = _dev(abs_max, "abs_max", (torch.float32,), optional=True)
     capi.check(capi.lib.llmq_swiglu_backward_bf16(d, g, i, a, B, T, Cc, _stream(stream)))
+
+
+def rmsnorm_forward(out, rms, inp, weight, abs_max, epsilon, stream=0):
+    """out[B,T,C] = bf16(bf16(inp / rms(inp)) * weight), rms[B,T] = 1/sqrt(mean(inp^2) + epsilon); abs_max (fp32
+    device scalar or None) receives max |out| (reference: src/binding/kernel_binding.cpp:130-143)."""
+    if inp.dim() != 3 or out.shape != inp.shape or weight.dim() != 1 or weight.shape[0] != inp.shape[2]:
+        raise ValueError("inp and out must be [B, T, C] and weight [C]")
+    if rms is not None and (rms.dim() != 2 or rms.shape[0] != inp.shape[0] or rms.shape[1] != inp.shape[1]):
+        raise ValueError("rms must be [B, T]")
+    o = _dev(out, "out", (torch.bfloat16,))
+    r = _dev(rms, "rms", (torch.float32,), optional=True)
+    i = _dev(inp, "inp", (torch.bfloat16,))
+    w = _dev(weight, "weight", (torch.bfloat16,))
+    a = _dev(abs_max, "abs_max", (torch.float32,), optional=True)
+    B, T, Cc = (int(v) for v in inp.shape)
+    capi.check(capi.lib.llmq_rmsnorm_forward_bf16(o, r, i, w, a, float(epsilon), B, T, Cc, _stream(stream)))
+
+
+def fused_residual_rmsnorm_forward(residual, normed, rrms, inp1, inp2, weight, abs_max, epsilon, stream=0):
+    """residual = bf16(inp1 + inp2); normed, rrms = rmsnorm(residual) as above
+    (reference: src/binding/kernel_binding.cpp:172-190)."""
+    if inp1.dim() != 3 or any(t.shape != inp1.shape for t in (inp2, residual, normed)) or weight.dim() != 1 \
+            or weight.shape[0] != inp1.shape[2]:
+        raise ValueError("inp1, inp2, residual and normed must be [B, T, C] and weight [C]")
+    if rrms.dim() != 2 or rrms.shape[0] != inp1.shape[0] or rrms.shape[1] != inp1.shape[1]:
+        raise ValueError("rrms must be [B, T]")
+    ptrs = [_dev(t, n, (torch.bfloat16,)) for t, n in ((residual, "residual"), (normed, "normed"))]
+    r = _dev(rrms, "rrms", (torch.float32,))
+    ins = [_dev(t, n, (torch.bfloat16,)) for t, n in ((inp1, "inp1"), (inp2, "inp2"), (weight, "weight"))]
+    a = _dev(abs_max, "abs_max", (torch.float32,), optional=True)
+    N, Cc = int(inp1.shape[0] * inp1.shape[1]), int(inp1.shape[2])
+    capi.check(capi.lib.llmq_fused_residual_rmsnorm_forward_bf16(ptrs[0], ptrs[1], r, ins[0], ins[1], ins[2], a,
+                                                                 float(epsilon), N, Cc, _stream(stream)))

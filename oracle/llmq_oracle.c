@@ -32,6 +32,9 @@
  *   swiglu             torch's CPU silu and autograd in float64 (the construction of the reference's
  *                      scripts/test_kernels.py:197-207), scipy.special.expit, closed forms (gate = 0, large
  *                      |gate|, silu(g) - silu(-g) = g), central differences for the gradient
+ *   rmsnorm            torch float64 mean / rsqrt on the construction of scripts/test_kernels.py:88-93 and
+ *                      :583-586 (values and 1/rms), torch's CPU bf16 multiply for the rounded-then-scaled
+ *                      output, constant rows (closed form), scaling invariance
  * The bit-level results of the CUDA conversion instruction and of cuBLASLt themselves cannot be
  * observed here (no CUDA device or toolkit): for NaN sign/payload and for the accumulation order
  * of the closed-source GEMM the parity is unpinned by anything the reference ships; the oracle
@@ -399,6 +402,47 @@ void orc_swiglu_backward_bf16(uint16_t* dinp, double* exact_dinp, const uint16_t
             dinp[r * 2 * C + C + c] = orc_f32_to_bf16((float)d2);
         }
     }
+}
+
+/*
+ * RMSNorm forward, plain (inp2 == NULL) or with the residual add in front (src/kernels/rmsnorm.cu:17-86,
+ * 88-164): res = inp1 or bf16((float)inp1 + (float)inp2) [stored to residual]; s = 1/sqrt(mean(res^2) + eps);
+ * out = bf16((float)bf16(s * res) * (float)weight) -- the reference rounds the normalised value to bf16 before
+ * the scale (rmsnorm.cu:68-71).  The reference's s comes from an fp32 sum in a launch-dependent order and
+ * the approximate rsqrt; the oracle takes the sum, mean and inverse root in double and rounds s once to
+ * fp32, the value any such implementation approximates.  exact_out (optional) receives s_double * res *
+ * weight without the intermediate rounding.
+ */
+void orc_rmsnorm_forward_bf16(uint16_t* residual, uint16_t* normed, float* rrms, double* exact_out,
+                              const uint16_t* inp1, const uint16_t* inp2, const uint16_t* weight, float eps,
+                              int64_t N, int C) {
+    uint16_t* row = (uint16_t*)malloc((size_t)(C > 0 ? C : 1) * sizeof(uint16_t));
+    for (int64_t r = 0; r < N; ++r) {
+        double acc = 0.0;
+        for (int c = 0; c < C; ++c) {
+            uint16_t v = inp1[r * C + c];
+            if (inp2) {
+                volatile float sum = orc_bf16_to_f32(v) + orc_bf16_to_f32(inp2[r * C + c]);
+                v = orc_f32_to_bf16(sum);
+                if (residual) residual[r * C + c] = v;
+            }
+            row[c] = v;
+            const double x = (double)orc_bf16_to_f32(v);
+            acc += x * x;
+        }
+        const double sd = 1.0 / sqrt(acc / (double)C + (double)eps);
+        const float s = (float)sd;
+        if (rrms) rrms[r] = s;
+        for (int c = 0; c < C; ++c) {
+            const float x = orc_bf16_to_f32(row[c]), w = orc_bf16_to_f32(weight[c]);
+            volatile float n = s * x;
+            const float nb = orc_bf16_to_f32(orc_f32_to_bf16(n));
+            volatile float prod = nb * w;
+            normed[r * C + c] = orc_f32_to_bf16(prod);
+            if (exact_out) exact_out[r * C + c] = sd * (double)x * (double)w;
+        }
+    }
+    free(row);
 }
 
 /* ------------------------------------------------------------------------------------------------

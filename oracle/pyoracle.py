@@ -105,6 +105,8 @@ def lib():
     L.orc_swiglu_forward_bf16.argtypes = [u16p, f64p, u16p, C.c_int64, C.c_int]
     L.orc_swiglu_backward_bf16.restype = None
     L.orc_swiglu_backward_bf16.argtypes = [u16p, f64p, u16p, u16p, C.c_int64, C.c_int]
+    L.orc_rmsnorm_forward_bf16.restype = None
+    L.orc_rmsnorm_forward_bf16.argtypes = [u16p, u16p, f32p, f64p, u16p, u16p, u16p, C.c_float, C.c_int64, C.c_int]
     _lib = L
     return L
 
@@ -310,3 +312,24 @@ def swiglu_backward(dout, inp):
     lib().orc_swiglu_backward_bf16(_p(dinp, C.c_uint16), _p(exact, C.c_double), _p(dout, C.c_uint16),
                                    _p(inp, C.c_uint16), BT, C2 // 2)
     return dinp, exact
+
+
+def rmsnorm_forward(inp1, weight, eps, inp2=None):
+    """inp1 (and inp2): bf16 bits [N, C]; weight: bf16 bits [C].  Returns (normed bits [N, C], rrms float32 [N],
+    exact float64 [N, C], residual bits [N, C] or None)."""
+    inp1 = np.ascontiguousarray(inp1, dtype=np.uint16)
+    weight = np.ascontiguousarray(weight, dtype=np.uint16)
+    N, Cc = inp1.shape
+    normed = np.empty((N, Cc), dtype=np.uint16)
+    rrms = np.empty(N, dtype=np.float32)
+    exact = np.empty((N, Cc), dtype=np.float64)
+    res = None
+    p2 = None
+    if inp2 is not None:
+        inp2 = np.ascontiguousarray(inp2, dtype=np.uint16)
+        res = np.empty((N, Cc), dtype=np.uint16)
+        p2 = _p(inp2, C.c_uint16)
+    lib().orc_rmsnorm_forward_bf16(_p(res, C.c_uint16) if res is not None else None, _p(normed, C.c_uint16),
+                                   _p(rrms, C.c_float), _p(exact, C.c_double), _p(inp1, C.c_uint16), p2,
+                                   _p(weight, C.c_uint16), C.c_float(eps), N, Cc)
+    return normed, rrms, exact, res

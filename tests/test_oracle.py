@@ -470,3 +470,47 @@ def test_swiglu_backward_vs_torch_autograd_and_differences(O):
         step[:, half * C:(half + 1) * C] = h
         num = (fwd(xv + step) - fwd(xv - step)) / (2 * h) * d
         assert np.allclose(exact[:, half * C:(half + 1) * C], num, rtol=1e-6, atol=1e-8)
+
+
+# ----------------------------------------------------------------------------------------- rmsnorm
+def test_rmsnorm_forward_vs_torch(O):
+    """Construction of the reference's scripts/test_kernels.py:88-93 and :583-586 in float64 on torch's CPU
+    kernels: 1/rms and the unrounded product agree to double precision; the bf16 bits are torch's bf16
+    rounding of s*x followed by torch's bf16 multiply with the weight (the reference's order of roundings,
+    src/kernels/rmsnorm.cu:68-71); the residual is torch's bf16 rounding of the fp32 sum."""
+    N, Cc, eps = 13, 96, 1e-6
+    x1 = O.fill_normal_bf16(N * Cc, 31, 0, 0.0, 1.5).reshape(N, Cc)
+    x2 = O.fill_normal_bf16(N * Cc, 31, 1, 0.0, 0.7).reshape(N, Cc)
+    w = O.fill_normal_bf16(Cc, 31, 2, 1.0, 0.3)
+    as_t = lambda bits: torch.from_numpy(np.ascontiguousarray(bits).view(np.int16)).view(torch.bfloat16)
+    for fused in (False, True):
+        normed, rrms, exact, res = O.rmsnorm_forward(x1, w, eps, x2 if fused else None)
+        r = as_t(x1)
+        if fused:
+            r = (as_t(x1).float() + as_t(x2).float()).to(torch.bfloat16)
+            assert np.array_equal(res, r.view(torch.int16).numpy().view(np.uint16))
+        rd = r.double()
+        r_rms = 1.0 / torch.sqrt((rd ** 2).mean(dim=-1, keepdim=True) + float(np.float32(eps)))
+        assert np.allclose(exact, (rd * r_rms * as_t(w).double()).numpy(), rtol=1e-13, atol=0)
+        assert np.array_equal(rrms, r_rms.squeeze(-1).float().numpy())
+        n_b = (r.float() * torch.from_numpy(rrms).unsqueeze(-1)).to(torch.bfloat16)
+        want = (n_b * as_t(w)).view(torch.int16).numpy().view(np.uint16)
+        assert np.array_equal(normed, want)
+
+
+def test_rmsnorm_forward_closed_forms(O):
+    """A constant row v gives s = 1/sqrt(v^2 + eps) and out = bf16(bf16(s v) w); scaling the input by a
+    power of two leaves the output unchanged when eps is 0."""
+    Cc = 64
+    f = lambda v: O.f32_to_bf16(np.asarray(v, dtype=np.float32))
+    w = f(np.linspace(0.5, 2.0, Cc))
+    row = f([3.0] * Cc).reshape(1, Cc)
+    normed, rrms, _, _ = O.rmsnorm_forward(row, w, 0.25)
+    s = np.float32(1.0 / np.sqrt(9.0 + 0.25))
+    assert rrms[0] == s
+    nb = O.bf16_to_f32(f([s * np.float32(3.0)]))[0]
+    assert np.array_equal(normed[0], f(nb * O.bf16_to_f32(w)))
+    x = O.fill_normal_bf16(4 * Cc, 77, 0).reshape(4, Cc)
+    a, ra, _, _ = O.rmsnorm_forward(x, w, 0.0)
+    b, rb, _, _ = O.rmsnorm_forward(f(O.bf16_to_f32(x) * 8.0), w, 0.0)
+    assert np.array_equal(a, b) and np.array_equal(ra, rb * np.float32(8.0))
