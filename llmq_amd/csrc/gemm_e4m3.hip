@@ -946,7 +946,7 @@ int g_gemm_persist = -1;  // -1 = automatic, 0 = never, 1 = whenever possible
 // launches.  The decision uses measured figures (microseconds): a tile of depth K on an otherwise idle
 // chip takes about K / 164 (twice as fast as in a full round); the operand bytes of the round stream at
 // about 3.5 TB/s from memory (10 TB/s when both operands fit the 256 MB last-level cache) whichever way
-// the round is organised; the extra launches cost about 14, a partial tile 0.03 in the reduction.
+// the round is organised; the extra launches cost about 20, a partial tile 0.03 in the reduction.
 struct W4Plan {
     int grid, rem_split, k_len, part_per_xcd, rem_max;
 };
@@ -976,7 +976,7 @@ static W4Plan plan_w4(int tiles256, int cus, int M, int N, int K, int forced_spl
             continue;
         }
         const double seg_us = tile_us * seg_pairs / pairs;
-        const double cut_us = (seg_us > stream_us ? seg_us : stream_us) + 14.0 + 0.03 * rem_total * s;
+        const double cut_us = (seg_us > stream_us ? seg_us : stream_us) + 20.0 + 0.03 * rem_total * s;
         if (whole_us - cut_us > best_gain) {
             best_gain = whole_us - cut_us;
             best = s;
