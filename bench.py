@@ -262,7 +262,8 @@ def main():
         sw_am, sw_sc = torch.zeros(1, device=dev), torch.zeros(1, device=dev)
         swiglu = {
             "what": "producers of the projections' inputs with the abs-max of their output computed on the way: "
-                    "h = swiglu(y_up) [8192 x 18944], the same as e4m3 codes, its backward, and the residual add + rmsnorm",
+                    "h = swiglu(y_up) [8192 x 18944], the same as e4m3 codes, its backward, the residual add + rmsnorm [8192 x 3584] "
+                    "and the rmsnorm backward",
             "swiglu_forward+abs_max (6 B/el)": gbs(lambda: K.swiglu_forward(h3, y3, sw_am), 6 * n_act),
             "swiglu_forward_quant (5 B/el)": gbs(lambda: K.swiglu_forward_quant(hq3, sw_sc, y3, sw_am), 5 * n_act),
             "swiglu_backward+abs_max (10 B/el)": gbs(lambda: K.swiglu_backward(dy3, dh3, y3, sw_am), 10 * n_act),
@@ -272,6 +273,13 @@ def main():
         r_in, r_att = torch.randn_like(x3), torch.randn_like(x3)
         r_out, r_norm, r_rms = torch.empty_like(x3), torch.empty_like(x3), torch.empty((1, BT), device=dev)
         r_w = torch.ones(C, dtype=torch.bfloat16, device=dev)
+        # dy_down = rmsnorm_backward(...) [8192 x 3584], the producer of the down projection's gradient input
+        r_scr = torch.empty(K.get_rmsnorm_backward_scratch_size(C), dtype=torch.float32, device=dev)
+        r_dw = torch.zeros(C, dtype=torch.bfloat16, device=dev)
+        r_rstd = torch.ones((1, BT), device=dev)
+        swiglu["rmsnorm_backward+abs_max (8 B/el)"] = gbs(
+            lambda: K.rmsnorm_backward(r_out, r_dw, r_scr, r_att, out["dx"].view(1, BT, C), r_in, r_w, r_rstd, sw_am),
+            8 * BT * C, iters=10)
         swiglu["fused_residual_rmsnorm_forward+abs_max (8 B/el)"] = gbs(
             lambda: K.fused_residual_rmsnorm_forward(r_out, r_norm, r_rms, r_in, r_att, r_w, sw_am, 1e-6), 8 * BT * C, iters=10)
     if args.calibrate_copy:

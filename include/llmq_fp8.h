@@ -225,6 +225,27 @@ int llmq_fused_residual_rmsnorm_forward_bf16(uint16_t* residual, uint16_t* norme
                                              const uint16_t* inp2, const uint16_t* weight, float* abs_max_or_null,
                                              float epsilon, int N, int C, void* stream);
 
+/*
+ * RMSNorm backward.  Per row bt of dout / inp [B*T, C], with r = rstd[bt] (the 1/rms the forward stored):
+ *     g_c = (float)weight[c] * (float)dout[bt, c];      k = (sum_c g_c * inp[bt, c]) / C * r
+ *     dinp[bt, c] = bf16( (float)dresidual[bt, c] + (g_c - inp[bt, c] * r * k) * r )
+ *     dweight[c]  = bf16( (float)dweight[c] + sum_bt inp[bt, c] * r * dout[bt, c] )          (ADDED to dweight)
+ * dresidual may be the same buffer as dinp (the reference copies it into dinp first when it is not).
+ * abs_max_or_null: reset, then max |dinp| over the rounded outputs, bit-identical to llmq_abs_max_bf16(dinp).
+ * scratch: device buffer of at least llmq_rmsnorm_backward_scratch_bytes(C) bytes, overwritten by every call (no
+ * need to clear it); all sums are fp32 in a fixed order -> deterministic.  C: multiple of 8, at most 8192.
+ * Replaces: rmsnorm_backward(nv_bfloat16* dinp, nv_bfloat16* dweight, std::byte* scratch, const nv_bfloat16* dresidual,
+ *           const nv_bfloat16* dout, const nv_bfloat16* inp, const nv_bfloat16* weight, const float* rstd,
+ *           float* abs_max_ptr, int B, int T, int C, const cudaDeviceProp&, cudaStream_t)
+ *           src/kernels/kernels.h:52-53, src/kernels/rmsnorm.cu:229-440,447-470, and
+ *           get_rmsnorm_backward_scratch_size(int C, const cudaDeviceProp&) kernels.h:49, rmsnorm.cu:442-445.
+ */
+int64_t llmq_rmsnorm_backward_scratch_bytes(int C);
+int llmq_rmsnorm_backward_bf16(uint16_t* dinp, uint16_t* dweight, void* scratch, size_t scratch_bytes,
+                               const uint16_t* dresidual, const uint16_t* dout, const uint16_t* inp,
+                               const uint16_t* weight, const float* rstd, float* abs_max_or_null, int B, int T, int C,
+                               void* stream);
+
 #ifdef __cplusplus
 }
 #endif

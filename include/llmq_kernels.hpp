@@ -421,4 +421,33 @@ inline void fused_residual_rmsnorm_forward(Tensor& residual, Tensor& normed, Ten
                                    abs_max_ptr, epsilon, N, C, stream);
 }
 
+// ---- rmsnorm backward (reference: src/kernels/kernels.h:49-55, src/kernels/rmsnorm.cu:229-470) ----------------------
+inline int get_rmsnorm_backward_scratch_size(int C, const hipDeviceProp_t&) { return (int)llmq_rmsnorm_backward_scratch_bytes(C); }
+inline void rmsnorm_backward(__hip_bfloat16* dinp, __hip_bfloat16* dweight, std::byte* scratch, const __hip_bfloat16* dresidual,
+                             const __hip_bfloat16* dout, const __hip_bfloat16* inp, const __hip_bfloat16* weight,
+                             const float* rstd, float* abs_max_ptr, int B, int T, int C, const hipDeviceProp_t& dp,
+                             hipStream_t stream) {
+    llmq_detail::check(llmq_rmsnorm_backward_bf16(llmq_detail::u16(dinp), llmq_detail::u16(dweight), scratch,
+                                                  (std::size_t)get_rmsnorm_backward_scratch_size(C, dp),
+                                                  llmq_detail::u16(dresidual), llmq_detail::u16(dout), llmq_detail::u16(inp),
+                                                  llmq_detail::u16(weight), rstd, abs_max_ptr, B, T, C, stream));
+}
+inline void rmsnorm_backward(Tensor& dinp, Tensor& dweight, Tensor& scratch, const Tensor& dresidual, const Tensor& dout,
+                             const Tensor& inp, const Tensor& weight, const Tensor& rstd, float* abs_max_ptr, int B, int T,
+                             int C, const hipDeviceProp_t& dp, hipStream_t stream) {
+    if (dinp.DType != ETensorDType::BF16 || dweight.DType != ETensorDType::BF16 || dresidual.DType != ETensorDType::BF16 ||
+        dout.DType != ETensorDType::BF16 || inp.DType != ETensorDType::BF16 || weight.DType != ETensorDType::BF16 ||
+        rstd.DType != ETensorDType::FP32)
+        llmq_detail::unsupported(__func__, dinp, dweight, dresidual, dout, inp, weight, rstd);
+    if (scratch.bytes() < (std::size_t)get_rmsnorm_backward_scratch_size(C, dp))
+        throw std::invalid_argument("rmsnorm_backward: scratch buffer too small");
+    llmq_detail::check(llmq_rmsnorm_backward_bf16(llmq_detail::u16(dinp.get<__hip_bfloat16>()),
+                                                  llmq_detail::u16(dweight.get<__hip_bfloat16>()), scratch.Data, scratch.bytes(),
+                                                  llmq_detail::u16(dresidual.get<__hip_bfloat16>()),
+                                                  llmq_detail::u16(dout.get<__hip_bfloat16>()),
+                                                  llmq_detail::u16(inp.get<__hip_bfloat16>()),
+                                                  llmq_detail::u16(weight.get<__hip_bfloat16>()), rstd.get<float>(),
+                                                  abs_max_ptr, B, T, C, stream));
+}
+
 #endif  // LLMQ_KERNELS_HPP

@@ -22,6 +22,7 @@ EXPORTS = [
     "llmq_backward_bias_bf16", "llmq_backward_bias_scratch_bytes", "llmq_quantize_both_bf16", "llmq_quantize_e4m3_f32", "llmq_quantize_e5m2_f32",
     "llmq_swiglu_forward_bf16", "llmq_swiglu_forward_quant_bf16", "llmq_swiglu_backward_bf16",
     "llmq_rmsnorm_forward_bf16", "llmq_fused_residual_rmsnorm_forward_bf16",
+    "llmq_rmsnorm_backward_bf16", "llmq_rmsnorm_backward_scratch_bytes",
 ]
 
 if not os.path.exists(LIB_PATH):
@@ -53,6 +54,8 @@ lib.llmq_swiglu_forward_quant_bf16.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _
 lib.llmq_swiglu_backward_bf16.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _vp]
 lib.llmq_rmsnorm_forward_bf16.argtypes = [_vp, _vp, _vp, _vp, _vp, C.c_float, _int, _int, _int, _vp]
 lib.llmq_fused_residual_rmsnorm_forward_bf16.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, C.c_float, _int, _int, _vp]
+lib.llmq_rmsnorm_backward_bf16.argtypes = [_vp, _vp, _vp, C.c_size_t, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp]
+lib.llmq_rmsnorm_backward_scratch_bytes.argtypes = [_int]
 lib.llmq_debug_set_gemm_variant.argtypes = [_int, _int]
 lib.llmq_debug_set_gemm_variant.restype = None
 lib.llmq_debug_set_gemm_persist.argtypes = [_int]
@@ -64,6 +67,7 @@ lib.llmq_debug_mfma_ceiling.restype = _int
 for _name in EXPORTS[3:]:
     getattr(lib, _name).restype = _int
 lib.llmq_backward_bias_scratch_bytes.restype = _i64
+lib.llmq_rmsnorm_backward_scratch_bytes.restype = _i64
 
 LLMQ_OK, LLMQ_ERR_INVALID_ARGUMENT, LLMQ_ERR_RUNTIME = 0, 1, 2
 

@@ -16,6 +16,8 @@ Names, argument order and in-place "out first" convention are the reference's:
     swiglu_backward(dinp, dout, inp, abs_max, stream=0)
     rmsnorm_forward(out, rms, inp, weight, abs_max, epsilon, stream=0)
     fused_residual_rmsnorm_forward(residual, normed, rrms, inp1, inp2, weight, abs_max, epsilon, stream=0)
+    rmsnorm_backward(dinp, dweight, scratch, dresidual, dout, inp, weight, rstd, abs_max, stream=0)
+    get_rmsnorm_backward_scratch_size(C)
 `stream` is a raw hipStream_t handle (0 = torch's current stream).
 """
 import torch
@@ -241,3 +243,29 @@ def fused_residual_rmsnorm_forward(residual, normed, rrms, inp1, inp2, weight, a
     N, Cc = int(inp1.shape[0] * inp1.shape[1]), int(inp1.shape[2])
     capi.check(capi.lib.llmq_fused_residual_rmsnorm_forward_bf16(ptrs[0], ptrs[1], r, ins[0], ins[1], ins[2], a,
                                                                  float(epsilon), N, Cc, _stream(stream)))
+
+
+def get_rmsnorm_backward_scratch_size(C):
+    """Number of fp32 elements of the scratch tensor rmsnorm_backward needs for rows of C elements (the reference's
+    binding sizes it in fp32 elements too: scripts/test_kernels.py:149)."""
+    return int(capi.lib.llmq_rmsnorm_backward_scratch_bytes(int(C))) // 4
+
+
+def rmsnorm_backward(dinp, dweight, scratch, dresidual, dout, inp, weight, rstd, abs_max, stream=0):
+    """dinp = dresidual + d(rmsnorm)/d(inp) . dout; dweight += d/d(weight); abs_max receives max |dinp|
+    (reference: src/binding/kernel_binding.cpp:145-169).  scratch: fp32 device tensor of
+    get_rmsnorm_backward_scratch_size(C) elements."""
+    if inp.dim() != 3 or any(t.shape != inp.shape for t in (dinp, dresidual, dout)) or weight.dim() != 1 \
+            or weight.shape[0] != inp.shape[2] or dweight.shape != weight.shape:
+        raise ValueError("dinp, dresidual, dout and inp must be [B, T, C], weight and dweight [C]")
+    if rstd.dim() != 2 or rstd.shape[0] != inp.shape[0] or rstd.shape[1] != inp.shape[1]:
+        raise ValueError("rstd must be [B, T]")
+    bf = (torch.bfloat16,)
+    p = [_dev(t, n, bf) for t, n in ((dinp, "dinp"), (dweight, "dweight"))]
+    sc = _dev(scratch, "scratch")
+    q = [_dev(t, n, bf) for t, n in ((dresidual, "dresidual"), (dout, "dout"), (inp, "inp"), (weight, "weight"))]
+    r = _dev(rstd, "rstd", (torch.float32,))
+    a = _dev(abs_max, "abs_max", (torch.float32,), optional=True)
+    B, T, Cc = (int(v) for v in inp.shape)
+    capi.check(capi.lib.llmq_rmsnorm_backward_bf16(p[0], p[1], sc, scratch.numel() * scratch.element_size(), q[0], q[1],
+                                                   q[2], q[3], r, a, B, T, Cc, _stream(stream)))

@@ -34,7 +34,9 @@
  *                      |gate|, silu(g) - silu(-g) = g), central differences for the gradient
  *   rmsnorm            torch float64 mean / rsqrt on the construction of scripts/test_kernels.py:88-93 and
  *                      :583-586 (values and 1/rms), torch's CPU bf16 multiply for the rounded-then-scaled
- *                      output, constant rows (closed form), scaling invariance
+ *                      output, constant rows (closed form), scaling invariance; backward: torch autograd in
+ *                      float64 through the same forward, the reference's own formula construction
+ *                      (scripts/test_kernels.py:96-113), accumulation into dresidual / dweight
  * The bit-level results of the CUDA conversion instruction and of cuBLASLt themselves cannot be
  * observed here (no CUDA device or toolkit): for NaN sign/payload and for the accumulation order
  * of the closed-source GEMM the parity is unpinned by anything the reference ships; the oracle
@@ -443,6 +445,48 @@ void orc_rmsnorm_forward_bf16(uint16_t* residual, uint16_t* normed, float* rrms,
         }
     }
     free(row);
+}
+
+/*
+ * RMSNorm backward (src/kernels/rmsnorm.cu:229-440): with r = rstd[bt], g_c = weight[c] * dout[bt,c],
+ * k = (sum_c g_c * inp[bt,c]) / C * r:
+ *     dinp[bt,c] = bf16(dresidual[bt,c] + (g_c - inp[bt,c] * r * k) * r)
+ *     dweight[c] = bf16(dweight[c] + sum_bt inp[bt,c] * r * dout[bt,c])
+ * evaluated in double and rounded once (double -> float -> bf16); the reference's fp32 sums have a launch-
+ * dependent order.  exact_* receive the double values, mag_* the sums of the absolute values of the terms
+ * (the scale of the fp32 evaluation error, for tolerances); all four are optional.
+ */
+void orc_rmsnorm_backward_bf16(uint16_t* dinp, uint16_t* dweight, double* exact_dinp, double* mag_dinp,
+                               double* exact_dw, double* mag_dw, const uint16_t* dresidual, const uint16_t* dout,
+                               const uint16_t* inp, const uint16_t* weight, const float* rstd, int64_t N, int C) {
+    double* dw = (double*)calloc((size_t)(C > 0 ? C : 1), sizeof(double));
+    double* dwa = (double*)calloc((size_t)(C > 0 ? C : 1), sizeof(double));
+    for (int64_t bt = 0; bt < N; ++bt) {
+        const double r = (double)rstd[bt];
+        double dot = 0.0;
+        for (int c = 0; c < C; ++c)
+            dot += (double)orc_bf16_to_f32(weight[c]) * (double)orc_bf16_to_f32(dout[bt * C + c]) *
+                   (double)orc_bf16_to_f32(inp[bt * C + c]);
+        const double k = dot / (double)C * r;
+        for (int c = 0; c < C; ++c) {
+            const double x = (double)orc_bf16_to_f32(inp[bt * C + c]), d = (double)orc_bf16_to_f32(dout[bt * C + c]);
+            const double g = (double)orc_bf16_to_f32(weight[c]) * d, old = (double)orc_bf16_to_f32(dresidual[bt * C + c]);
+            const double v = old + (g - x * r * k) * r;
+            dw[c] += x * r * d;
+            dwa[c] += fabs(x * r * d);
+            if (exact_dinp) exact_dinp[bt * C + c] = v;
+            if (mag_dinp) mag_dinp[bt * C + c] = fabs(old) + (fabs(g) + fabs(x * r * k)) * fabs(r);
+            dinp[bt * C + c] = orc_f32_to_bf16((float)v);
+        }
+    }
+    for (int c = 0; c < C; ++c) {
+        const double old = (double)orc_bf16_to_f32(dweight[c]);
+        if (exact_dw) exact_dw[c] = old + dw[c];
+        if (mag_dw) mag_dw[c] = fabs(old) + dwa[c];
+        dweight[c] = orc_f32_to_bf16((float)(old + dw[c]));
+    }
+    free(dw);
+    free(dwa);
 }
 
 /* ------------------------------------------------------------------------------------------------

@@ -107,6 +107,8 @@ def lib():
     L.orc_swiglu_backward_bf16.argtypes = [u16p, f64p, u16p, u16p, C.c_int64, C.c_int]
     L.orc_rmsnorm_forward_bf16.restype = None
     L.orc_rmsnorm_forward_bf16.argtypes = [u16p, u16p, f32p, f64p, u16p, u16p, u16p, C.c_float, C.c_int64, C.c_int]
+    L.orc_rmsnorm_backward_bf16.restype = None
+    L.orc_rmsnorm_backward_bf16.argtypes = [u16p, u16p, f64p, f64p, f64p, f64p, u16p, u16p, u16p, u16p, f32p, C.c_int64, C.c_int]
     _lib = L
     return L
 
@@ -333,3 +335,22 @@ def rmsnorm_forward(inp1, weight, eps, inp2=None):
                                    _p(rrms, C.c_float), _p(exact, C.c_double), _p(inp1, C.c_uint16), p2,
                                    _p(weight, C.c_uint16), C.c_float(eps), N, Cc)
     return normed, rrms, exact, res
+
+
+def rmsnorm_backward(dresidual, dweight, dout, inp, weight, rstd):
+    """bf16 bits: dresidual, dout, inp [N, C]; dweight (old value), weight [C]; rstd float32 [N].
+    Returns dict(dinp, dweight (bits), exact_dinp, mag_dinp, exact_dw, mag_dw (float64))."""
+    inp = np.ascontiguousarray(inp, dtype=np.uint16)
+    N, Cc = inp.shape
+    dres = np.ascontiguousarray(dresidual, dtype=np.uint16)
+    dout = np.ascontiguousarray(dout, dtype=np.uint16)
+    weight = np.ascontiguousarray(weight, dtype=np.uint16)
+    rstd = np.ascontiguousarray(rstd, dtype=np.float32)
+    dinp = np.empty((N, Cc), dtype=np.uint16)
+    dw = np.array(dweight, dtype=np.uint16, copy=True)
+    ed, md = np.empty((N, Cc)), np.empty((N, Cc))
+    ew, mw = np.empty(Cc), np.empty(Cc)
+    lib().orc_rmsnorm_backward_bf16(_p(dinp, C.c_uint16), _p(dw, C.c_uint16), _p(ed, C.c_double), _p(md, C.c_double),
+                                    _p(ew, C.c_double), _p(mw, C.c_double), _p(dres, C.c_uint16), _p(dout, C.c_uint16),
+                                    _p(inp, C.c_uint16), _p(weight, C.c_uint16), _p(rstd, C.c_float), N, Cc)
+    return dict(dinp=dinp, dweight=dw, exact_dinp=ed, mag_dinp=md, exact_dw=ew, mag_dw=mw)

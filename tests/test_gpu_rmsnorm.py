@@ -156,3 +156,114 @@ def test_rmsnorm_full_size_properties(K, O):
     K.quantize_with_abs_max(q, stats[1:2], normed, stats[0:1])
     codes, dq = O.quantize_e4m3(host_bits(normed.reshape(-1, C)[rows]), stats[0].item())
     assert np.array_equal(host_bits(q[rows]), codes) and np.float32(dq) == stats[1].item()
+
+
+# ---------------------------------------------------------------------------------------- backward
+# Bars for rmsnorm_backward against the oracle (double evaluation, one rounding):
+#   dinp:    |err| <= one bf16 ulp of the value + 2^-18 of the sum of the magnitudes of its terms (the scale of
+#            the fp32 evaluation error where the terms cancel);
+#   dweight: the same with the sum over all rows of |inp * rstd * dout| as the magnitude;
+#   bit exact: abs-max against abs_max(dinp); repeated launches (fixed summation order).
+# The reference's own tolerances (rtol 1e-2 / atol 5e-3, scripts/test_kernels.py:153-157) are asserted on its
+# construction as well.
+BWD_SHAPES = [(2, 3, 16), (1, 4, 64), (4, 8, 256), (1, 37, 3584), (1, 9, 896), (1, 5, 8192), (2, 600, 128), (1, 1, 8)]
+
+
+def run_backward(K, dres, dw0, dout, x, w, rstd, B, T, C, with_absmax=True, in_place=False):
+    d_dres = dev_bf16(dres).reshape(B, T, C)
+    dinp = d_dres if in_place else torch.full((B, T, C), float("nan"), dtype=torch.bfloat16, device="cuda")
+    dweight = dev_bf16(dw0).clone()
+    scratch = torch.full((K.get_rmsnorm_backward_scratch_size(C),), float("nan"), dtype=torch.float32, device="cuda")
+    am = torch.full((1,), 9.0, dtype=torch.float32, device="cuda") if with_absmax else None
+    K.rmsnorm_backward(dinp, dweight, scratch, d_dres, dev_bf16(dout).reshape(B, T, C), dev_bf16(x).reshape(B, T, C),
+                       dev_bf16(w), torch.from_numpy(rstd).cuda().reshape(B, T), am)
+    return dinp, dweight, am
+
+
+@pytest.mark.parametrize("btc", BWD_SHAPES)
+def test_rmsnorm_backward_matches_oracle(K, O, btc):
+    B, T, C = btc
+    N = B * T
+    x, _, w = make_inputs(O, N, C, 800 + C)
+    dout = O.fill_normal_bf16(N * C, 800 + C, 3, 0.0, 0.8).reshape(N, C)
+    dres = O.fill_normal_bf16(N * C, 800 + C, 4, 0.0, 0.5).reshape(N, C)
+    dw0 = O.fill_normal_bf16(C, 800 + C, 5, 0.0, 2.0)
+    _, rstd, _, _ = O.rmsnorm_forward(x, w, 1e-6)
+    want = O.rmsnorm_backward(dres, dw0, dout, x, w, rstd)
+    dinp, dweight, am = run_backward(K, dres, dw0, dout, x, w, rstd, B, T, C)
+    got = O.bf16_to_f32(host_bits(dinp)).reshape(N, C).astype(np.float64)
+    tol = np.abs(want["exact_dinp"]) * 2.0 ** -7 + want["mag_dinp"] * 2.0 ** -18 + 1e-38
+    assert np.all(np.abs(got - O.bf16_to_f32(want["dinp"])) <= tol)
+    gw = O.bf16_to_f32(host_bits(dweight)).astype(np.float64)
+    tolw = np.abs(want["exact_dw"]) * 2.0 ** -7 + want["mag_dw"] * 2.0 ** -18 + 1e-38
+    assert np.all(np.abs(gw - O.bf16_to_f32(want["dweight"])) <= tolw)
+    ref_am = torch.zeros(1, dtype=torch.float32, device="cuda")
+    K.abs_max(ref_am, dinp)
+    assert am.cpu().numpy().view(np.uint32)[0] == ref_am.cpu().numpy().view(np.uint32)[0]
+    # in place on dresidual, without the abs-max: the same bits, twice
+    dinp2, dweight2, _ = run_backward(K, dres, dw0, dout, x, w, rstd, B, T, C, with_absmax=False, in_place=True)
+    assert torch.equal(dinp.view(torch.int16), dinp2.view(torch.int16))
+    assert torch.equal(dweight.view(torch.int16), dweight2.view(torch.int16))
+
+
+def test_rmsnorm_backward_reference_test_construction(K, O):
+    """scripts/test_kernels.py:136-190: randn tensors, zero and non-zero dresidual, torch float reference."""
+    B, T, C, eps = 4, 8, 256, 1e-6
+    g = torch.Generator(device="cuda").manual_seed(1)
+    rn = lambda *s: torch.randn(s, device="cuda", dtype=torch.float32, generator=g).to(torch.bfloat16)
+    inp, weight, dout, dres = rn(B, T, C), rn(C), rn(B, T, C), rn(B, T, C)
+    r = 1.0 / torch.sqrt((inp.float() ** 2).mean(dim=-1, keepdim=True) + eps)
+    normed, dy_w = inp.float() * r, dout.float() * weight.float()
+    ref_dinp = r * (dy_w - normed * (dy_w * normed).sum(dim=-1, keepdim=True) / C)
+    ref_dw = (dout.float() * inp.float() * r).sum(dim=(0, 1))
+    scratch = torch.zeros(K.get_rmsnorm_backward_scratch_size(C), device="cuda", dtype=torch.float32)
+    for start in (torch.zeros_like(dres), dres):
+        dinp, dweight = torch.empty_like(inp), torch.zeros(C, device="cuda", dtype=torch.bfloat16)
+        K.rmsnorm_backward(dinp, dweight, scratch, start, dout, inp, weight, r.squeeze(-1).contiguous(), None)
+        assert torch.allclose(dinp.float(), (start.float() + ref_dinp).to(torch.bfloat16).float(), rtol=1e-2, atol=5e-3)
+        assert torch.allclose(dweight.float(), ref_dw.to(torch.bfloat16).float(), rtol=1e-2, atol=5e-3)
+
+
+def test_rmsnorm_backward_argument_errors(K):
+    B, T, C = 1, 4, 64
+    z = lambda *s: torch.zeros(s, dtype=torch.bfloat16, device="cuda")
+    rstd = torch.ones((B, T), dtype=torch.float32, device="cuda")
+    small = torch.zeros(8, dtype=torch.float32, device="cuda")
+    with pytest.raises(ValueError, match="scratch"):
+        K.rmsnorm_backward(z(B, T, C), z(C), small, z(B, T, C), z(B, T, C), z(B, T, C), z(C), rstd, None)
+    scratch = torch.zeros(K.get_rmsnorm_backward_scratch_size(8200), dtype=torch.float32, device="cuda")
+    with pytest.raises(ValueError, match="8192"):
+        K.rmsnorm_backward(z(B, T, 8200), z(8200), scratch, z(B, T, 8200), z(B, T, 8200), z(B, T, 8200), z(8200), rstd, None)
+    with pytest.raises(ValueError):
+        K.rmsnorm_backward(z(B, T, C), z(C), scratch, z(B, T, C), z(B, T, C), z(B, T, C), z(C // 2), rstd, None)
+
+
+def test_rmsnorm_backward_full_size_properties(K, O):
+    """Configuration-4 size (8192 x 3584): sampled rows of dinp and all of dweight against the oracle run on a
+    row subset is not possible for dweight (it sums every row), so dweight is checked against a float64 torch
+    reduction on the device; abs-max invariant on the whole tensor."""
+    B, T, C, eps = 8, 1024, 3584, 1e-6
+    g = torch.Generator(device="cuda").manual_seed(3)
+    rn = lambda s, std: (std * torch.randn(s, device="cuda", dtype=torch.float32, generator=g)).to(torch.bfloat16)
+    inp, dout, dres = rn((B, T, C), 1.0), rn((B, T, C), 0.01), rn((B, T, C), 0.01)
+    w = (1.0 + 0.2 * torch.randn((C,), device="cuda", dtype=torch.float32, generator=g)).to(torch.bfloat16)
+    out, rstd = torch.empty_like(inp), torch.empty((B, T), dtype=torch.float32, device="cuda")
+    K.rmsnorm_forward(out, rstd, inp, w, None, eps)
+    dinp, dweight = torch.empty_like(inp), torch.zeros(C, dtype=torch.bfloat16, device="cuda")
+    scratch = torch.empty(K.get_rmsnorm_backward_scratch_size(C), dtype=torch.float32, device="cuda")
+    am = torch.zeros(1, dtype=torch.float32, device="cuda")
+    K.rmsnorm_backward(dinp, dweight, scratch, dres, dout, inp, w, rstd, am)
+    ref_am = torch.zeros(1, dtype=torch.float32, device="cuda")
+    K.abs_max(ref_am, dinp)
+    assert am.item() == ref_am.item() and am.item() > 0
+    rows = torch.tensor([0, 5, 4099, 8191], device="cuda")
+    sub = lambda t: host_bits(t.reshape(-1, C)[rows])
+    want = O.rmsnorm_backward(sub(dres), np.zeros(C, np.uint16), sub(dout), sub(inp), host_bits(w),
+                              rstd.reshape(-1)[rows].cpu().numpy())
+    got = O.bf16_to_f32(sub(dinp)).astype(np.float64)
+    tol = np.abs(want["exact_dinp"]) * 2.0 ** -7 + want["mag_dinp"] * 2.0 ** -18 + 1e-38
+    assert np.all(np.abs(got - O.bf16_to_f32(want["dinp"])) <= tol)
+    terms = inp.double().reshape(-1, C) * rstd.double().reshape(-1, 1) * dout.double().reshape(-1, C)
+    exact_dw, mag_dw = terms.sum(dim=0).cpu().numpy(), terms.abs().sum(dim=0).cpu().numpy()
+    gw = dweight.float().cpu().numpy().astype(np.float64)
+    assert np.all(np.abs(gw - exact_dw) <= np.abs(exact_dw) * 2.0 ** -7 + mag_dw * 2.0 ** -18)

@@ -514,3 +514,35 @@ def test_rmsnorm_forward_closed_forms(O):
     a, ra, _, _ = O.rmsnorm_forward(x, w, 0.0)
     b, rb, _, _ = O.rmsnorm_forward(f(O.bf16_to_f32(x) * 8.0), w, 0.0)
     assert np.array_equal(a, b) and np.array_equal(ra, rb * np.float32(8.0))
+
+
+def test_rmsnorm_backward_vs_torch_autograd(O):
+    """The gradient of out = x * rsqrt(mean(x^2) + eps) * w by torch autograd in float64 (eps = 0 so that the
+    stored 1/rms determines the forward exactly), plus the reference's explicit formulas
+    (scripts/test_kernels.py:96-113), with accumulation into a non-zero dresidual and dweight."""
+    N, Cc = 11, 40
+    x = O.fill_normal_bf16(N * Cc, 41, 0, 0.0, 1.3).reshape(N, Cc)
+    d = O.fill_normal_bf16(N * Cc, 41, 1, 0.0, 0.8).reshape(N, Cc)
+    w = O.fill_normal_bf16(Cc, 41, 2, 1.0, 0.4)
+    dres = O.fill_normal_bf16(N * Cc, 41, 3, 0.0, 0.5).reshape(N, Cc)
+    dw0 = O.fill_normal_bf16(Cc, 41, 4, 0.0, 2.0)
+    t64 = lambda bits: torch.from_numpy(O.bf16_to_f32(bits).astype(np.float64))
+    xt = t64(x).requires_grad_(True)
+    wt = t64(w).requires_grad_(True)
+    r = torch.rsqrt((xt ** 2).mean(dim=-1, keepdim=True))
+    (xt * r * wt).backward(t64(d))
+    rstd = r.detach().squeeze(-1).numpy()
+    # the oracle takes rstd as fp32 (what the forward stored): feed the double value's rounding and allow for it
+    res = O.rmsnorm_backward(dres, dw0, d, x, w, rstd.astype(np.float32))
+    assert np.allclose(res["exact_dinp"], t64(dres).numpy() + xt.grad.numpy(), rtol=2e-6, atol=1e-7)
+    assert np.allclose(res["exact_dw"], t64(dw0).numpy() + wt.grad.numpy(), rtol=2e-6, atol=1e-6)
+    # explicit formulas with the same fp32 rstd: agreement to double precision
+    rr = torch.from_numpy(rstd.astype(np.float32).astype(np.float64)).unsqueeze(-1)
+    xd, dd, wd = t64(x), t64(d), t64(w)
+    normed = xd * rr
+    dy_w = dd * wd
+    dinp = rr * (dy_w - normed * (dy_w * normed).sum(dim=-1, keepdim=True) / Cc)
+    assert np.allclose(res["exact_dinp"], (t64(dres) + dinp).numpy(), rtol=1e-12, atol=1e-14)
+    assert np.allclose(res["exact_dw"], (t64(dw0) + (dd * xd * rr).sum(dim=0)).numpy(), rtol=1e-12, atol=1e-14)
+    assert np.array_equal(res["dinp"], O.f32_to_bf16((t64(dres) + dinp).numpy().astype(np.float32)))
+    assert np.array_equal(res["dweight"], O.f32_to_bf16((t64(dw0) + (dd * xd * rr).sum(dim=0)).numpy().astype(np.float32)))
