@@ -246,6 +246,27 @@ int llmq_rmsnorm_backward_bf16(uint16_t* dinp, uint16_t* dweight, void* scratch,
                                const uint16_t* weight, const float* rstd, float* abs_max_or_null, int B, int T, int C,
                                void* stream);
 
+/*
+ * Rotary position embedding on the fused QKV tensor [B, T, Nq + 2*Nkv, head_dim] (bf16); freqs_cis_f16 is [T, head_dim]
+ * fp16 with (cos, sin) pairs for d = 0 .. head_dim/2 - 1.  Query and key heads, with real = x[d], imag = x[d + head_dim/2]:
+ *     out[d] = bf16(real*cos - imag*sin),  out[d + head_dim/2] = bf16(real*sin + imag*cos)      (backward: sin -> -sin)
+ * in fp32; value heads are copied (left alone when out == inp).  abs_max_or_null: reset, then max |out| over all heads
+ * including the value heads, bit-identical to llmq_abs_max_bf16(out).  head_dim must be a multiple of 8.
+ * Replaces: rope_forward / rope_backward(nv_bfloat16* out, const nv_bfloat16* in, const half* freqs_cis, float* abs_max_ptr,
+ *           int B, int T, int Nq, int Nkv, int head_dim, cudaStream_t)  src/kernels/kernels.h:113,116,
+ *           src/kernels/rope.cu:42-163.
+ */
+int llmq_rope_forward_bf16(uint16_t* out, const uint16_t* inp, const uint16_t* freqs_cis_f16, float* abs_max_or_null, int B,
+                           int T, int Nq, int Nkv, int head_dim, void* stream);
+int llmq_rope_backward_bf16(uint16_t* dinp, const uint16_t* dout, const uint16_t* freqs_cis_f16, float* abs_max_or_null,
+                            int B, int T, int Nq, int Nkv, int head_dim, void* stream);
+/*
+ * Host-side table for the two above: freqs_cis_host[t*dim + 2i] = fp16(cos(t / theta^(2i/dim))), [.. + 2i + 1] = fp16(sin(..)),
+ * t < end, i < dim/2, evaluated in fp32 with the C library as the reference does.
+ * Replaces: precompute_freqs_cis(half* freqs_cis, int dim, int end, float theta)  src/kernels/kernels.h:111, rope.cu:15-40.
+ */
+int llmq_precompute_freqs_cis_f16(uint16_t* freqs_cis_host, int dim, int end, float theta);
+
 #ifdef __cplusplus
 }
 #endif

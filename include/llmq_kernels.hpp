@@ -13,6 +13,7 @@
 #define LLMQ_KERNELS_HPP
 
 #include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
 #include <hip/hip_fp8.h>
 #include <hip/hip_runtime_api.h>
 
@@ -448,6 +449,23 @@ inline void rmsnorm_backward(Tensor& dinp, Tensor& dweight, Tensor& scratch, con
                                                   llmq_detail::u16(inp.get<__hip_bfloat16>()),
                                                   llmq_detail::u16(weight.get<__hip_bfloat16>()), rstd.get<float>(),
                                                   abs_max_ptr, B, T, C, stream));
+}
+
+// ---- rope (reference: src/kernels/kernels.h:110-117, src/kernels/rope.cu) ------------------------------------------
+inline void precompute_freqs_cis(__half* freqs_cis, int dim, int end, float theta) {
+    llmq_detail::check(llmq_precompute_freqs_cis_f16(reinterpret_cast<std::uint16_t*>(freqs_cis), dim, end, theta));
+}
+inline void rope_forward(__hip_bfloat16* out, const __hip_bfloat16* in, const __half* freqs_cis, float* abs_max_ptr, int B,
+                         int T, int Nq, int Nkv, int head_dim, hipStream_t stream) {
+    llmq_detail::check(llmq_rope_forward_bf16(llmq_detail::u16(out), llmq_detail::u16(in),
+                                              reinterpret_cast<const std::uint16_t*>(freqs_cis), abs_max_ptr, B, T, Nq, Nkv,
+                                              head_dim, stream));
+}
+inline void rope_backward(__hip_bfloat16* dinp, const __hip_bfloat16* dout, const __half* freqs_cis, float* abs_max_ptr, int B,
+                          int T, int Nq, int Nkv, int head_dim, hipStream_t stream) {
+    llmq_detail::check(llmq_rope_backward_bf16(llmq_detail::u16(dinp), llmq_detail::u16(dout),
+                                               reinterpret_cast<const std::uint16_t*>(freqs_cis), abs_max_ptr, B, T, Nq, Nkv,
+                                               head_dim, stream));
 }
 
 #endif  // LLMQ_KERNELS_HPP

@@ -23,6 +23,7 @@ EXPORTS = [
     "llmq_swiglu_forward_bf16", "llmq_swiglu_forward_quant_bf16", "llmq_swiglu_backward_bf16",
     "llmq_rmsnorm_forward_bf16", "llmq_fused_residual_rmsnorm_forward_bf16",
     "llmq_rmsnorm_backward_bf16", "llmq_rmsnorm_backward_scratch_bytes",
+    "llmq_rope_forward_bf16", "llmq_rope_backward_bf16", "llmq_precompute_freqs_cis_f16",
 ]
 
 if not os.path.exists(LIB_PATH):
@@ -56,6 +57,9 @@ lib.llmq_rmsnorm_forward_bf16.argtypes = [_vp, _vp, _vp, _vp, _vp, C.c_float, _i
 lib.llmq_fused_residual_rmsnorm_forward_bf16.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, C.c_float, _int, _int, _vp]
 lib.llmq_rmsnorm_backward_bf16.argtypes = [_vp, _vp, _vp, C.c_size_t, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp]
 lib.llmq_rmsnorm_backward_scratch_bytes.argtypes = [_int]
+lib.llmq_rope_forward_bf16.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _vp]
+lib.llmq_rope_backward_bf16.argtypes = lib.llmq_rope_forward_bf16.argtypes
+lib.llmq_precompute_freqs_cis_f16.argtypes = [_vp, _int, _int, C.c_float]
 lib.llmq_debug_set_gemm_variant.argtypes = [_int, _int]
 lib.llmq_debug_set_gemm_variant.restype = None
 lib.llmq_debug_set_gemm_persist.argtypes = [_int]

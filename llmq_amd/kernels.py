@@ -18,6 +18,8 @@ Names, argument order and in-place "out first" convention are the reference's:
     fused_residual_rmsnorm_forward(residual, normed, rrms, inp1, inp2, weight, abs_max, epsilon, stream=0)
     rmsnorm_backward(dinp, dweight, scratch, dresidual, dout, inp, weight, rstd, abs_max, stream=0)
     get_rmsnorm_backward_scratch_size(C)
+    rope_forward(out, inp, freqs_cis, abs_max, Nq, Nkv, stream=0);  rope_backward(dinp, dout, freqs_cis, abs_max, Nq, Nkv, stream=0)
+    precompute_freqs_cis(dim, end, theta)
 `stream` is a raw hipStream_t handle (0 = torch's current stream).
 """
 import torch
@@ -269,3 +271,34 @@ def rmsnorm_backward(dinp, dweight, scratch, dresidual, dout, inp, weight, rstd,
     B, T, Cc = (int(v) for v in inp.shape)
     capi.check(capi.lib.llmq_rmsnorm_backward_bf16(p[0], p[1], sc, scratch.numel() * scratch.element_size(), q[0], q[1],
                                                    q[2], q[3], r, a, B, T, Cc, _stream(stream)))
+
+
+def _rope(fn, out, inp, freqs_cis, abs_max, Nq, Nkv, stream):
+    """Tensors [B, T, (Nq + 2 Nkv) * HD] bf16 (reference: src/binding/kernel_binding.cpp:193-223); freqs_cis [T, HD] fp16."""
+    if inp.dim() != 3 or out.shape != inp.shape or freqs_cis.dim() != 2 or freqs_cis.shape[0] < inp.shape[1]:
+        raise ValueError("inp and out must be [B, T, C] and freqs_cis [>= T, HD]")
+    HD = int(freqs_cis.shape[1])
+    if HD == 0 or inp.shape[2] != (Nq + 2 * Nkv) * HD:
+        raise ValueError("C must equal (Nq + 2 Nkv) * head_dim")
+    o = _dev(out, "out", (torch.bfloat16,))
+    i = _dev(inp, "inp", (torch.bfloat16,))
+    f = _dev(freqs_cis, "freqs_cis", (torch.float16,))
+    a = _dev(abs_max, "abs_max", (torch.float32,), optional=True)
+    capi.check(fn(o, i, f, a, int(inp.shape[0]), int(inp.shape[1]), int(Nq), int(Nkv), HD, _stream(stream)))
+
+
+def rope_forward(out, inp, freqs_cis, abs_max, Nq, Nkv, stream=0):
+    """Rotary embedding of the query and key heads of the fused QKV tensor (out may be inp); abs_max receives max |out|."""
+    _rope(capi.lib.llmq_rope_forward_bf16, out, inp, freqs_cis, abs_max, Nq, Nkv, stream)
+
+
+def rope_backward(dinp, dout, freqs_cis, abs_max, Nq, Nkv, stream=0):
+    """Gradient of rope_forward: the rotation by the negative angle."""
+    _rope(capi.lib.llmq_rope_backward_bf16, dinp, dout, freqs_cis, abs_max, Nq, Nkv, stream)
+
+
+def precompute_freqs_cis(dim, end, theta):
+    """Host tensor [end, dim] fp16 of (cos, sin) pairs (reference: precompute_freqs_cis, src/kernels/rope.cu:15-40)."""
+    tab = torch.empty((end, dim), dtype=torch.float16)
+    capi.check(capi.lib.llmq_precompute_freqs_cis_f16(tab.data_ptr(), int(dim), int(end), float(theta)))
+    return tab

@@ -37,6 +37,9 @@
  *                      output, constant rows (closed form), scaling invariance; backward: torch autograd in
  *                      float64 through the same forward, the reference's own formula construction
  *                      (scripts/test_kernels.py:96-113), accumulation into dresidual / dweight
+ *   rope               numpy complex128 multiplication by (cos + i sin) of numpy's fp16 decoding, norm
+ *                      preservation, backward(forward(x)) = x (cos^2 + sin^2), value heads untouched; the
+ *                      host table against numpy float64 cos / sin within fp16 rounding
  * The bit-level results of the CUDA conversion instruction and of cuBLASLt themselves cannot be
  * observed here (no CUDA device or toolkit): for NaN sign/payload and for the accumulation order
  * of the closed-source GEMM the parity is unpinned by anything the reference ships; the oracle
@@ -487,6 +490,50 @@ void orc_rmsnorm_backward_bf16(uint16_t* dinp, uint16_t* dweight, double* exact_
     }
     free(dw);
     free(dwa);
+}
+
+/*
+ * Rotary embedding on [BT][N = Nq + 2 Nkv][HD] bf16 with an fp16 table [T][HD] of (cos, sin) pairs
+ * (src/kernels/rope.cu:42-127): query and key heads rotate (x[d], x[d + HD/2]) by the angle of (t, d), the
+ * backward by the negative angle; value heads pass through.  Evaluated in double (products of bf16 and fp16
+ * values are exact there) and rounded once.  t = bt % T.  exact / mag (optional): the double value and
+ * |real*cos| + |imag*sin| (resp. |real*sin| + |imag*cos|), the scale of an fp32 evaluation's error.
+ */
+static double f16_to_double(uint16_t h) {
+    const int sign = h >> 15, e = (h >> 10) & 31, m = h & 1023;
+    double v;
+    if (e == 0) v = ldexp((double)m, -24);
+    else if (e == 31) v = m ? NAN : INFINITY;
+    else v = ldexp((double)(m | 1024), e - 25);
+    return sign ? -v : v;
+}
+
+void orc_rope_bf16(uint16_t* out, double* exact, double* mag, const uint16_t* inp, const uint16_t* freqs_f16,
+                   int64_t BT, int T, int Nq, int Nkv, int HD, int backward) {
+    const int N = Nq + 2 * Nkv, half = HD / 2;
+    for (int64_t bt = 0; bt < BT; ++bt) {
+        const int t = (int)(bt % T);
+        for (int h = 0; h < N; ++h) {
+            const int64_t base = (bt * N + h) * HD;
+            for (int d = 0; d < half; ++d) {
+                const double re = (double)orc_bf16_to_f32(inp[base + d]), im = (double)orc_bf16_to_f32(inp[base + half + d]);
+                double o_re = re, o_im = im, m_re = fabs(re), m_im = fabs(im);
+                if (h < Nq + Nkv) {
+                    const double c = f16_to_double(freqs_f16[(int64_t)t * HD + 2 * d]);
+                    double sn = f16_to_double(freqs_f16[(int64_t)t * HD + 2 * d + 1]);
+                    if (backward) sn = -sn;
+                    o_re = re * c - im * sn;
+                    o_im = re * sn + im * c;
+                    m_re = fabs(re * c) + fabs(im * sn);
+                    m_im = fabs(re * sn) + fabs(im * c);
+                }
+                out[base + d] = h < Nq + Nkv ? orc_f32_to_bf16((float)o_re) : inp[base + d];
+                out[base + half + d] = h < Nq + Nkv ? orc_f32_to_bf16((float)o_im) : inp[base + half + d];
+                if (exact) { exact[base + d] = o_re; exact[base + half + d] = o_im; }
+                if (mag) { mag[base + d] = m_re; mag[base + half + d] = m_im; }
+            }
+        }
+    }
 }
 
 /* ------------------------------------------------------------------------------------------------

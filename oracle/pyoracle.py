@@ -109,6 +109,8 @@ def lib():
     L.orc_rmsnorm_forward_bf16.argtypes = [u16p, u16p, f32p, f64p, u16p, u16p, u16p, C.c_float, C.c_int64, C.c_int]
     L.orc_rmsnorm_backward_bf16.restype = None
     L.orc_rmsnorm_backward_bf16.argtypes = [u16p, u16p, f64p, f64p, f64p, f64p, u16p, u16p, u16p, u16p, f32p, C.c_int64, C.c_int]
+    L.orc_rope_bf16.restype = None
+    L.orc_rope_bf16.argtypes = [u16p, f64p, f64p, u16p, u16p, C.c_int64, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
     _lib = L
     return L
 
@@ -354,3 +356,16 @@ def rmsnorm_backward(dresidual, dweight, dout, inp, weight, rstd):
                                     _p(ew, C.c_double), _p(mw, C.c_double), _p(dres, C.c_uint16), _p(dout, C.c_uint16),
                                     _p(inp, C.c_uint16), _p(weight, C.c_uint16), _p(rstd, C.c_float), N, Cc)
     return dict(dinp=dinp, dweight=dw, exact_dinp=ed, mag_dinp=md, exact_dw=ew, mag_dw=mw)
+
+
+def rope(inp, freqs_f16, T, Nq, Nkv, backward=False):
+    """inp: bf16 bits [BT, Nq + 2 Nkv, HD]; freqs_f16: fp16 bits [T, HD] of (cos, sin) pairs.
+    Returns (out bits, exact float64, magnitude float64), all shaped like inp."""
+    inp = np.ascontiguousarray(inp, dtype=np.uint16)
+    freqs = np.ascontiguousarray(freqs_f16, dtype=np.uint16)
+    BT, N, HD = inp.shape
+    out = np.empty_like(inp)
+    exact, mag = np.empty(inp.shape), np.empty(inp.shape)
+    lib().orc_rope_bf16(_p(out, C.c_uint16), _p(exact, C.c_double), _p(mag, C.c_double), _p(inp, C.c_uint16),
+                        _p(freqs, C.c_uint16), BT, T, Nq, Nkv, HD, 1 if backward else 0)
+    return out, exact, mag

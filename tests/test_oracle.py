@@ -546,3 +546,43 @@ def test_rmsnorm_backward_vs_torch_autograd(O):
     assert np.allclose(res["exact_dw"], (t64(dw0) + (dd * xd * rr).sum(dim=0)).numpy(), rtol=1e-12, atol=1e-14)
     assert np.array_equal(res["dinp"], O.f32_to_bf16((t64(dres) + dinp).numpy().astype(np.float32)))
     assert np.array_equal(res["dweight"], O.f32_to_bf16((t64(dw0) + (dd * xd * rr).sum(dim=0)).numpy().astype(np.float32)))
+
+
+# -------------------------------------------------------------------------------------------- rope
+def _rope_table(T, HD, theta=10000.0):
+    i = np.arange(HD // 2, dtype=np.float64)
+    ang = np.arange(T, dtype=np.float64)[:, None] / theta ** (2 * i / HD)[None, :]
+    tab = np.empty((T, HD), dtype=np.float16)
+    tab[:, 0::2], tab[:, 1::2] = np.cos(ang), np.sin(ang)
+    return tab
+
+
+def test_rope_vs_complex_multiplication(O):
+    """Rotation = multiplication of (real + i imag) by (cos + i sin) in numpy complex128 with numpy's own
+    fp16 decoding of the table; value heads untouched; norm preserved up to cos^2 + sin^2 of the rounded
+    table; the backward undoes the forward up to that factor."""
+    B, T, Nq, Nkv, HD = 2, 5, 3, 2, 16
+    N, half = Nq + 2 * Nkv, HD // 2
+    x = O.fill_normal_bf16(B * T * N * HD, 51, 0).reshape(B * T, N, HD)
+    tab = _rope_table(T, HD)
+    out, exact, _ = O.rope(x, tab.view(np.uint16), T, Nq, Nkv)
+    xf = O.bf16_to_f32(x).astype(np.float64)
+    z = xf[..., :half] + 1j * xf[..., half:]
+    rot = (tab[:, 0::2].astype(np.float64) + 1j * tab[:, 1::2].astype(np.float64))
+    rot_bt = np.tile(rot, (B, 1))[:, None, :]                      # t = bt % T
+    want = z * rot_bt
+    qk = slice(0, Nq + Nkv)
+    assert np.allclose(exact[:, qk, :half], want[:, qk].real, rtol=1e-14, atol=1e-300)
+    assert np.allclose(exact[:, qk, half:], want[:, qk].imag, rtol=1e-14, atol=1e-300)
+    assert np.array_equal(out[:, Nq + Nkv:], x[:, Nq + Nkv:]) and np.array_equal(exact[:, Nq + Nkv:], xf[:, Nq + Nkv:])
+    assert np.array_equal(out[:, qk], O.f32_to_bf16(np.concatenate([want[:, qk].real, want[:, qk].imag], -1).astype(np.float32)))
+    gain = np.abs(rot_bt) ** 2
+    n_in, n_out = np.abs(z[:, qk]) ** 2, exact[:, qk, :half] ** 2 + exact[:, qk, half:] ** 2
+    assert np.allclose(n_out, n_in * gain, rtol=1e-12)
+    # backward of the exact forward values = x * (cos^2 + sin^2)
+    fwd_bits = O.f32_to_bf16(exact.astype(np.float32))
+    _, back, _ = O.rope(fwd_bits, tab.view(np.uint16), T, Nq, Nkv, backward=True)
+    zf = O.bf16_to_f32(fwd_bits).astype(np.float64)
+    zz = (zf[..., :half] + 1j * zf[..., half:]) * np.conj(rot_bt)
+    assert np.allclose(back[:, qk, :half], zz[:, qk].real, rtol=1e-14, atol=1e-300)
+    assert np.allclose(back[:, qk, half:], zz[:, qk].imag, rtol=1e-14, atol=1e-300)
