@@ -263,7 +263,7 @@ def main():
         swiglu = {
             "what": "producers of the projections' inputs with the abs-max of their output computed on the way: "
                     "h = swiglu(y_up) [8192 x 18944], the same as e4m3 codes, its backward, the residual add + rmsnorm [8192 x 3584] "
-                    "and the rmsnorm backward",
+                    "and the rmsnorm backward, the AdamW step of a weight",
             "swiglu_forward+abs_max (6 B/el)": gbs(lambda: K.swiglu_forward(h3, y3, sw_am), 6 * n_act),
             "swiglu_forward_quant (5 B/el)": gbs(lambda: K.swiglu_forward_quant(hq3, sw_sc, y3, sw_am), 5 * n_act),
             "swiglu_backward+abs_max (10 B/el)": gbs(lambda: K.swiglu_backward(dy3, dh3, y3, sw_am), 10 * n_act),
@@ -280,6 +280,13 @@ def main():
         swiglu["rmsnorm_backward+abs_max (8 B/el)"] = gbs(
             lambda: K.rmsnorm_backward(r_out, r_dw, r_scr, r_att, out["dx"].view(1, BT, C), r_in, r_w, r_rstd, sw_am),
             8 * BT * C, iters=10)
+        # the optimizer step on W_up [37888 x 3584] with bf16 moments: its epilogue is the weight abs-max of the next step
+        a_m, a_v = torch.zeros_like(t["w_up"]), torch.zeros_like(t["w_up"])
+        a_p, a_g = t["w_up"].clone(), (1e-3 * torch.randn_like(t["w_up"]))
+        a_gs = torch.ones(1, device=dev)
+        swiglu["adamw_update+abs_max, bf16 moments (14 B/param)"] = gbs(
+            lambda: K.adamw_update(a_p, a_g, a_m, a_v, 1e-4, 0.9, 0.95, 2, 1e-8, 0.1, a_gs, None, sw_am, 7), 14 * UP * C)
+        del a_m, a_v, a_p, a_g
         swiglu["fused_residual_rmsnorm_forward+abs_max (8 B/el)"] = gbs(
             lambda: K.fused_residual_rmsnorm_forward(r_out, r_norm, r_rms, r_in, r_att, r_w, sw_am, 1e-6), 8 * BT * C, iters=10)
     if args.calibrate_copy:

@@ -267,6 +267,26 @@ int llmq_rope_backward_bf16(uint16_t* dinp, const uint16_t* dout, const uint16_t
  */
 int llmq_precompute_freqs_cis_f16(uint16_t* freqs_cis_host, int dim, int end, float theta);
 
+/*
+ * AdamW update of bf16 parameters from bf16 gradients, moments in fp32 or bf16 (m_dtype / v_dtype: 0 = fp32, 1 = bf16;
+ * supported pairs (m, v): (0, 0), (1, 0), (1, 1)), per element:
+ *     grad = *grad_scale * g;  m = fma(beta1, m, fma(-beta1, grad, grad));  v = fma(beta2, v, fma(-beta2, grad^2, grad^2))
+ *     p = fma(-lr, fma(wd, p, (m*c1) / (sqrt(v*c2) + eps)), p),   c1 = 1/(1 - beta1^t), c2 = 1/(1 - beta2^t)
+ * Values narrower than fp32 are written with the reference's stochastic rounding (SquirrelNoise5 hash of the element
+ * index and `seed`; see llmq_amd/csrc/adamw.hip for the threshold of each tensor): reproducible bit for bit.
+ * abs_max_or_null: max |new p| is merged into the slot with an atomic max; the slot is NOT reset by this call
+ * (as in the reference: the caller clears it, one slot may cover several calls).  num_parameters % 8 == 0.
+ * Replaces: adamw_update(nv_bfloat16* params, const nv_bfloat16* grads, {float|nv_bfloat16}* m, {float|nv_bfloat16}* v,
+ *           size_t num_parameters, float learning_rate, float beta1, float beta2, int t, float eps, float weight_decay,
+ *           const float* grad_scale, float* abs_max, unsigned int seed, cudaStream_t)
+ *           src/kernels/kernels.h:225-235, src/kernels/adamw.cu:18-195.  Not provided: fp32 parameters and the
+ *           fp8 first moment with block scales (kernels.h:221,237).
+ */
+int llmq_adamw_update_bf16(uint16_t* params, const uint16_t* grads, void* m, int m_dtype, void* v, int v_dtype,
+                           int64_t num_parameters, float learning_rate, float beta1, float beta2, int t, float eps,
+                           float weight_decay, const float* grad_scale, float* abs_max_or_null, unsigned int seed,
+                           void* stream);
+
 #ifdef __cplusplus
 }
 #endif

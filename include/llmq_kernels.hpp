@@ -468,4 +468,28 @@ inline void rope_backward(__hip_bfloat16* dinp, const __hip_bfloat16* dout, cons
                                                head_dim, stream));
 }
 
+// ---- adamw (reference: src/kernels/kernels.h:225-235, src/kernels/adamw.cu) ----------------------------------------
+// bf16 parameters and gradients; moments fp32/fp32, bf16/fp32 or bf16/bf16.  abs_max is merged, not reset.
+inline void adamw_update(__hip_bfloat16* params, const __hip_bfloat16* grads, float* m, float* v, std::size_t num_parameters,
+                         float learning_rate, float beta1, float beta2, int t, float eps, float weight_decay,
+                         const float* grad_scale, float* abs_max, unsigned int seed, hipStream_t stream) {
+    llmq_detail::check(llmq_adamw_update_bf16(llmq_detail::u16(params), llmq_detail::u16(grads), m, 0, v, 0,
+                                              (std::int64_t)num_parameters, learning_rate, beta1, beta2, t, eps, weight_decay,
+                                              grad_scale, abs_max, seed, stream));
+}
+inline void adamw_update(__hip_bfloat16* params, const __hip_bfloat16* grads, __hip_bfloat16* m, float* v,
+                         std::size_t num_parameters, float learning_rate, float beta1, float beta2, int t, float eps,
+                         float weight_decay, const float* grad_scale, float* abs_max, unsigned int seed, hipStream_t stream) {
+    llmq_detail::check(llmq_adamw_update_bf16(llmq_detail::u16(params), llmq_detail::u16(grads), m, 1, v, 0,
+                                              (std::int64_t)num_parameters, learning_rate, beta1, beta2, t, eps, weight_decay,
+                                              grad_scale, abs_max, seed, stream));
+}
+inline void adamw_update(__hip_bfloat16* params, const __hip_bfloat16* grads, __hip_bfloat16* m, __hip_bfloat16* v,
+                         std::size_t num_parameters, float learning_rate, float beta1, float beta2, int t, float eps,
+                         float weight_decay, const float* grad_scale, float* abs_max, unsigned int seed, hipStream_t stream) {
+    llmq_detail::check(llmq_adamw_update_bf16(llmq_detail::u16(params), llmq_detail::u16(grads), m, 1, v, 1,
+                                              (std::int64_t)num_parameters, learning_rate, beta1, beta2, t, eps, weight_decay,
+                                              grad_scale, abs_max, seed, stream));
+}
+
 #endif  // LLMQ_KERNELS_HPP

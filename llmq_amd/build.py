@@ -13,7 +13,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "csrc", "build")
 LIB = os.path.join(HERE, "lib", "libllmq_fp8.so")
 
-SOURCES = ["runtime.hip", "absmax.hip", "quantize.hip", "transpose.hip", "gemm_e4m3.hip", "bias.hip", "swiglu.hip", "rmsnorm.hip", "rope.hip", "calibrate.hip"]
+SOURCES = ["runtime.hip", "absmax.hip", "quantize.hip", "transpose.hip", "gemm_e4m3.hip", "bias.hip", "swiglu.hip", "rmsnorm.hip", "rope.hip", "adamw.hip", "calibrate.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

@@ -24,6 +24,7 @@ EXPORTS = [
     "llmq_rmsnorm_forward_bf16", "llmq_fused_residual_rmsnorm_forward_bf16",
     "llmq_rmsnorm_backward_bf16", "llmq_rmsnorm_backward_scratch_bytes",
     "llmq_rope_forward_bf16", "llmq_rope_backward_bf16", "llmq_precompute_freqs_cis_f16",
+    "llmq_adamw_update_bf16",
 ]
 
 if not os.path.exists(LIB_PATH):
@@ -60,6 +61,8 @@ lib.llmq_rmsnorm_backward_scratch_bytes.argtypes = [_int]
 lib.llmq_rope_forward_bf16.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _vp]
 lib.llmq_rope_backward_bf16.argtypes = lib.llmq_rope_forward_bf16.argtypes
 lib.llmq_precompute_freqs_cis_f16.argtypes = [_vp, _int, _int, C.c_float]
+lib.llmq_adamw_update_bf16.argtypes = [_vp, _vp, _vp, _int, _vp, _int, _i64, C.c_float, C.c_float, C.c_float, _int, C.c_float,
+                                       C.c_float, _vp, _vp, C.c_uint, _vp]
 lib.llmq_debug_set_gemm_variant.argtypes = [_int, _int]
 lib.llmq_debug_set_gemm_variant.restype = None
 lib.llmq_debug_set_gemm_persist.argtypes = [_int]

@@ -1,0 +1,184 @@
+// AdamW update of bf16 parameters for gfx950 with the abs-max of the updated parameters computed on the
+// way: the producer of the weight tensors' abs-max, which the per-step weight quantization consumes (no
+// separate pass over the weights).
+//
+// Semantics follow the reference (src/kernels/adamw.cu:18-170, src/kernels/squirrel_noise.cuh), per element i:
+//     grad  = *grad_scale * (float)g[i]
+//     m     = fma(beta1, m, fma(-beta1, grad, grad))                  (the reference's two-operation lerp)
+//     v     = fma(beta2, v, fma(-beta2, grad*grad, grad*grad))
+//     param = p - lr * ( (m * c1) / (sqrt(v * c2) + eps) + wd * p ),   c1 = 1/(1 - beta1^t), c2 = 1/(1 - beta2^t)
+// with m, v kept in fp32 or bf16.  Everything narrower than fp32 is written with stochastic rounding: the low
+// 16 bits of the fp32 value are compared with a 16-bit threshold from the SquirrelNoise5 hash; above it the
+// value rounds away from zero, otherwise towards zero.  Thresholds: parameters hash(i, seed); v the same hash
+// rotated left by 20; m hash(first index of i's vector, 51245) rotated left by 7 per position in the vector,
+// where the reference's vector has 4 elements unless m and v are both bf16 (then 8).  The hash is integer
+// arithmetic and every floating-point operation is correctly rounded, so results are reproducible bit for bit;
+// the parameter line is evaluated as fma(-lr, fma(wd, p, quotient), p), the contraction the reference's
+// compiler applies by default.  The abs-max slot is NOT reset here (the reference does not either: one slot
+// may cover several calls; the caller clears it).
+//
+// HBM bound: 14 bytes per parameter with bf16 moments (read p, g, m, v; write p, m, v), 22 with fp32 moments.
+// A lane takes 8 consecutive parameters: 16-byte accesses throughout.
+#include <cmath>
+
+#include "common.hpp"
+#include "absmax_reduce.hpp"
+
+namespace llmq {
+
+typedef float f32x2_aw __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_aw __attribute__((ext_vector_type(2)));
+
+__host__ __device__ constexpr uint32_t squirrel_noise_5(uint32_t position, uint32_t seed) {
+    uint32_t b = position;
+    b *= 0xd2a80a3fu;
+    b += seed;
+    b ^= b >> 9;
+    b += 0xa884f197u;
+    b ^= b >> 11;
+    b *= 0x6C736F4Bu;
+    b ^= b >> 13;
+    b += 0xB79F3ABBu;
+    b ^= b >> 15;
+    b *= 0x1b56c4f5u;
+    b ^= b >> 17;
+    return b;
+}
+
+__device__ __forceinline__ uint32_t rotl32(uint32_t x, int k) { return (x << k) | (x >> (32 - k)); }
+
+// fp32 -> bf16 with the reference's stochastic rounding (squirrel_noise.cuh:47-56): returns the 16-bit pattern
+__device__ __forceinline__ uint32_t sr_bf16(float x, uint32_t random) {
+    uint32_t bits = __float_as_uint(x);
+    bits = (bits & 0xFFFFu) > (random & 0xFFFFu) ? (bits | 0xFFFFu) : (bits & ~0xFFFFu);
+    const f32x2_aw p = {__uint_as_float(bits), 0.f};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(p, bf16x2_aw)) & 0xFFFFu;
+}
+
+struct AdamArgs {
+    float lr, beta1, beta2, c1, c2, eps, wd;
+    unsigned seed;
+};
+
+// M_BF16 / V_BF16: storage type of the moments.  THREADS: 1024 with the abs-max (fewer atomics on the slot).
+template <bool M_BF16, bool V_BF16, bool ABSMAX, int THREADS>
+__global__ __launch_bounds__(THREADS) void adamw_kernel(uint4* __restrict__ params, const uint4* __restrict__ grads,
+                                                        void* __restrict__ m_mem, void* __restrict__ v_mem, int64_t nvec,
+                                                        AdamArgs a, const float* __restrict__ grad_scale,
+                                                        unsigned* __restrict__ absmax_out) {
+    constexpr int REF_VEC = (M_BF16 && V_BF16) ? 8 : 4;  // elements per lane in the reference's launch
+    const int64_t vec = (int64_t)blockIdx.x * THREADS + threadIdx.x;
+    uint32_t fold = 0x7F807F80u;
+    if (vec < nvec) {
+        const float gs = *grad_scale;
+        const uint4 pw = params[vec], gw = grads[vec];
+        float m[8], v[8];
+        if constexpr (M_BF16) {
+            const uint4 w = reinterpret_cast<const uint4*>(m_mem)[vec];
+            const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) { m[2 * k] = bf16_lo(ww[k]); m[2 * k + 1] = bf16_hi(ww[k]); }
+        } else {
+            const float4 lo = reinterpret_cast<const float4*>(m_mem)[2 * vec], hi = reinterpret_cast<const float4*>(m_mem)[2 * vec + 1];
+            m[0] = lo.x; m[1] = lo.y; m[2] = lo.z; m[3] = lo.w; m[4] = hi.x; m[5] = hi.y; m[6] = hi.z; m[7] = hi.w;
+        }
+        if constexpr (V_BF16) {
+            const uint4 w = reinterpret_cast<const uint4*>(v_mem)[vec];
+            const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) { v[2 * k] = bf16_lo(ww[k]); v[2 * k + 1] = bf16_hi(ww[k]); }
+        } else {
+            const float4 lo = reinterpret_cast<const float4*>(v_mem)[2 * vec], hi = reinterpret_cast<const float4*>(v_mem)[2 * vec + 1];
+            v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w; v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+        }
+        const uint32_t pws[4] = {pw.x, pw.y, pw.z, pw.w}, gws[4] = {gw.x, gw.y, gw.z, gw.w};
+        uint32_t p_out[8], m_out[8], v_out[8];
+        const uint32_t first = (uint32_t)(vec * 8);  // the reference hashes the 32-bit truncation of the index
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const uint32_t pword = pws[e / 2], gword = gws[e / 2];
+            const float p_old = (e & 1) ? bf16_hi(pword) : bf16_lo(pword);
+            const float grad = gs * ((e & 1) ? bf16_hi(gword) : bf16_lo(gword));
+            const float m_new = __builtin_fmaf(a.beta1, m[e], __builtin_fmaf(-a.beta1, grad, grad));
+            const float g2 = grad * grad;
+            const float v_new = __builtin_fmaf(a.beta2, v[e], __builtin_fmaf(-a.beta2, g2, g2));
+            const uint32_t random = squirrel_noise_5(first + e, a.seed);
+            const float m_hat = m_new * a.c1, v_hat = v_new * a.c2;
+            const float quot = __fdiv_rn(m_hat, __fsqrt_rn(v_hat) + a.eps);
+            const float p_new = __builtin_fmaf(-a.lr, __builtin_fmaf(a.wd, p_old, quot), p_old);
+            p_out[e] = sr_bf16(p_new, random);
+            m[e] = m_new;
+            v[e] = v_new;
+            if constexpr (V_BF16) v_out[e] = sr_bf16(v_new, rotl32(random, 20));
+            if constexpr (M_BF16) {
+                const uint32_t base = squirrel_noise_5(first + (e / REF_VEC) * REF_VEC, 51245u);
+                const int pos = e % REF_VEC;
+                m_out[e] = sr_bf16(m_new, pos == 0 ? base : rotl32(base, (7 * pos) % 32));
+            }
+        }
+        const uint4 pnew = make_uint4(p_out[0] | (p_out[1] << 16), p_out[2] | (p_out[3] << 16), p_out[4] | (p_out[5] << 16),
+                                      p_out[6] | (p_out[7] << 16));
+        params[vec] = pnew;
+        if constexpr (ABSMAX) fold = fold_vec(fold, pnew);
+        if constexpr (M_BF16) {
+            reinterpret_cast<uint4*>(m_mem)[vec] = make_uint4(m_out[0] | (m_out[1] << 16), m_out[2] | (m_out[3] << 16),
+                                                              m_out[4] | (m_out[5] << 16), m_out[6] | (m_out[7] << 16));
+        } else {
+            reinterpret_cast<float4*>(m_mem)[2 * vec] = make_float4(m[0], m[1], m[2], m[3]);
+            reinterpret_cast<float4*>(m_mem)[2 * vec + 1] = make_float4(m[4], m[5], m[6], m[7]);
+        }
+        if constexpr (V_BF16) {
+            reinterpret_cast<uint4*>(v_mem)[vec] = make_uint4(v_out[0] | (v_out[1] << 16), v_out[2] | (v_out[3] << 16),
+                                                              v_out[4] | (v_out[5] << 16), v_out[6] | (v_out[7] << 16));
+        } else {
+            reinterpret_cast<float4*>(v_mem)[2 * vec] = make_float4(v[0], v[1], v[2], v[3]);
+            reinterpret_cast<float4*>(v_mem)[2 * vec + 1] = make_float4(v[4], v[5], v[6], v[7]);
+        }
+    }
+    if constexpr (ABSMAX) {
+        const uint32_t lo = fold & 0xFFFFu, hi = fold >> 16;
+        block_min_to_atomic_max(absmax_out, lo < hi ? lo : hi, 0x7F80u, 16);
+    }
+}
+
+}  // namespace llmq
+
+// m_dtype / v_dtype: 0 = fp32, 1 = bf16; supported pairs (m, v): (0, 0), (1, 0), (1, 1), as in the reference.
+extern "C" int llmq_adamw_update_bf16(uint16_t* params, const uint16_t* grads, void* m, int m_dtype, void* v, int v_dtype,
+                                      int64_t num_parameters, float learning_rate, float beta1, float beta2, int t,
+                                      float eps, float weight_decay, const float* grad_scale, float* abs_max_or_null,
+                                      unsigned int seed, void* stream_) {
+    using namespace llmq;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    LLMQ_REQUIRE(num_parameters >= 0, "adamw_update: negative parameter count %lld", (long long)num_parameters);
+    LLMQ_REQUIRE(num_parameters % 8 == 0, "adamw_update: num_parameters must be divisible by 8 (got %lld)",
+                 (long long)num_parameters);
+    LLMQ_REQUIRE((m_dtype == 0 || m_dtype == 1) && (v_dtype == 0 || v_dtype == 1) && !(m_dtype == 0 && v_dtype == 1),
+                 "adamw_update: unsupported moment types (m %d, v %d): fp32/fp32, bf16/fp32 or bf16/bf16", m_dtype, v_dtype);
+    LLMQ_REQUIRE(grad_scale != nullptr, "adamw_update: grad_scale pointer is null");
+    if (num_parameters == 0) return LLMQ_OK;
+    LLMQ_REQUIRE(params && grads && m && v, "adamw_update: null tensor pointer");
+    LLMQ_REQUIRE(aligned16(params) && aligned16(grads) && aligned16(m) && aligned16(v),
+                 "adamw_update: tensors must be 16-byte aligned");
+    // bias corrections on the host in fp32, as the reference computes them (adamw.cu:153-158)
+    const float c1 = 1.0f / (1.0f - powf(beta1, (float)t)), c2 = 1.0f / (1.0f - powf(beta2, (float)t));
+    const AdamArgs a{learning_rate, beta1, beta2, c1, c2, eps, weight_decay, seed};
+    const int64_t nvec = num_parameters / 8;
+    auto launch = [&](auto kernel, int threads) {
+        hipLaunchKernelGGL(kernel, dim3((unsigned)((nvec + threads - 1) / threads)), dim3(threads), 0, stream,
+                           reinterpret_cast<uint4*>(params), reinterpret_cast<const uint4*>(grads), m, v, nvec, a, grad_scale,
+                           reinterpret_cast<unsigned*>(abs_max_or_null));
+    };
+    LLMQ_REQUIRE((nvec + 255) / 256 <= 0x7FFFFFFF, "adamw_update: tensor too large");
+#define LLMQ_ADAM(MB, VB)                                                     \
+    do {                                                                      \
+        if (abs_max_or_null) launch(adamw_kernel<MB, VB, true, 1024>, 1024);  \
+        else launch(adamw_kernel<MB, VB, false, 256>, 256);                   \
+    } while (0)
+    if (m_dtype == 0) LLMQ_ADAM(false, false);
+    else if (v_dtype == 0) LLMQ_ADAM(true, false);
+    else LLMQ_ADAM(true, true);
+#undef LLMQ_ADAM
+    LLMQ_HIP_TRY(hipGetLastError());
+    return LLMQ_OK;
+}

@@ -20,6 +20,8 @@ Names, argument order and in-place "out first" convention are the reference's:
     get_rmsnorm_backward_scratch_size(C)
     rope_forward(out, inp, freqs_cis, abs_max, Nq, Nkv, stream=0);  rope_backward(dinp, dout, freqs_cis, abs_max, Nq, Nkv, stream=0)
     precompute_freqs_cis(dim, end, theta)
+    adamw_update(params, grads, m, v, learning_rate, beta1, beta2, t, eps, weight_decay, grad_scale, m_scales=None,
+                 abs_max=None, seed=0, stream=0)
 `stream` is a raw hipStream_t handle (0 = torch's current stream).
 """
 import torch
@@ -302,3 +304,24 @@ def precompute_freqs_cis(dim, end, theta):
     tab = torch.empty((end, dim), dtype=torch.float16)
     capi.check(capi.lib.llmq_precompute_freqs_cis_f16(tab.data_ptr(), int(dim), int(end), float(theta)))
     return tab
+
+
+def adamw_update(params, grads, m, v, learning_rate, beta1, beta2, t, eps, weight_decay, grad_scale, m_scales=None,
+                 abs_max=None, seed=0, stream=0):
+    """In-place AdamW step on bf16 params with fp32 or bf16 moments and stochastic rounding (reference:
+    src/binding/kernel_binding.cpp:536-551).  grad_scale: fp32 device scalar.  abs_max, if given, is merged
+    with max |new params| (not reset).  m_scales (the fp8 first moment's block scales) is not supported."""
+    if m_scales is not None:
+        raise ValueError("adamw_update: the fp8 first moment with block scales is not supported")
+    n = params.numel()
+    if any(x.numel() != n for x in (grads, m, v)):
+        raise ValueError("adamw_update: shape mismatch")
+    p = _dev(params, "params", (torch.bfloat16,))
+    g = _dev(grads, "grads", (torch.bfloat16,))
+    pm = _dev(m, "m", (torch.float32, torch.bfloat16))
+    pv = _dev(v, "v", (torch.float32, torch.bfloat16))
+    gs = _dev(grad_scale, "grad_scale", (torch.float32,))
+    a = _dev(abs_max, "abs_max", (torch.float32,), optional=True)
+    capi.check(capi.lib.llmq_adamw_update_bf16(p, g, pm, int(m.dtype == torch.bfloat16), pv, int(v.dtype == torch.bfloat16), n,
+                                               float(learning_rate), float(beta1), float(beta2), int(t), float(eps),
+                                               float(weight_decay), gs, a, int(seed) & 0xFFFFFFFF, _stream(stream)))

@@ -40,6 +40,14 @@
  *   rope               numpy complex128 multiplication by (cos + i sin) of numpy's fp16 decoding, norm
  *                      preservation, backward(forward(x)) = x (cos^2 + sin^2), value heads untouched; the
  *                      host table against numpy float64 cos / sin within fp16 rounding
+ *   adamw              torch float64 evaluation of the reference's own test formulas
+ *                      (scripts/test_kernels.py:695-727) for fp32 moments (exact fp32 outputs) and within the
+ *                      stochastic rounding's one-ulp spread for bf16 ones; stochastic rounding: both
+ *                      neighbours only, exact values unchanged, unbiased over the hash (mean over 2^16
+ *                      positions); the hash: a bijection of the position (no collisions over 2^20 positions),
+ *                      balanced bits.  The hash's individual output bits have no known-answer vector in the
+ *                      reference tree: PARITY UNPINNED for them beyond these properties, and for the last bit
+ *                      of the parameter update (compiler contraction, see orc_adamw_update_bf16).
  * The bit-level results of the CUDA conversion instruction and of cuBLASLt themselves cannot be
  * observed here (no CUDA device or toolkit): for NaN sign/payload and for the accumulation order
  * of the closed-source GEMM the parity is unpinned by anything the reference ships; the oracle
@@ -534,6 +542,65 @@ void orc_rope_bf16(uint16_t* out, double* exact, double* mag, const uint16_t* in
             }
         }
     }
+}
+
+/*
+ * AdamW on bf16 parameters with stochastic rounding (src/kernels/adamw.cu:18-170, squirrel_noise.cuh:15-56).
+ * Integer hash + correctly rounded fp32 operations: reproducible bit for bit.  The parameter update is
+ * evaluated as fma(-lr, fma(wd, p, q), p): the reference's source writes p - lr * (q + wd * p) and leaves the
+ * contraction to its compiler, so that last bit is not specified by the source.  m_dtype / v_dtype: 0 = fp32,
+ * 1 = bf16.  Returns max |new parameter| (the abs-max epilogue; the caller combines it with the slot's old value).
+ */
+uint32_t orc_squirrel_noise_5(uint32_t position, uint32_t seed) {
+    uint32_t b = position;
+    b *= 0xd2a80a3fu; b += seed; b ^= b >> 9;
+    b += 0xa884f197u; b ^= b >> 11;
+    b *= 0x6C736F4Bu; b ^= b >> 13;
+    b += 0xB79F3ABBu; b ^= b >> 15;
+    b *= 0x1b56c4f5u; b ^= b >> 17;
+    return b;
+}
+
+uint16_t orc_stochastic_round_bf16(float x, uint32_t random) {
+    uint32_t bits = f32_bits(x);
+    bits = (bits & 0xFFFFu) > (random & 0xFFFFu) ? (bits | 0xFFFFu) : (bits & ~0xFFFFu);
+    return orc_f32_to_bf16(bits_f32(bits));
+}
+
+static inline uint32_t rotl32(uint32_t x, int k) { k &= 31; return k ? (x << k) | (x >> (32 - k)) : x; }
+
+float orc_adamw_update_bf16(uint16_t* params, const uint16_t* grads, void* m_mem, int m_dtype, void* v_mem, int v_dtype,
+                            int64_t n, float lr, float beta1, float beta2, int t, float eps, float wd, float grad_scale,
+                            uint32_t seed) {
+    const float c1 = 1.0f / (1.0f - powf(beta1, (float)t)), c2 = 1.0f / (1.0f - powf(beta2, (float)t));
+    const int ref_vec = (m_dtype == 1 && v_dtype == 1) ? 8 : 4;
+    float amax = 0.f;
+    for (int64_t i = 0; i < n; ++i) {
+        const float m_old = m_dtype ? orc_bf16_to_f32(((uint16_t*)m_mem)[i]) : ((float*)m_mem)[i];
+        const float v_old = v_dtype ? orc_bf16_to_f32(((uint16_t*)v_mem)[i]) : ((float*)v_mem)[i];
+        const float p_old = orc_bf16_to_f32(params[i]);
+        volatile float grad = grad_scale * orc_bf16_to_f32(grads[i]);
+        const float m_new = fmaf(beta1, m_old, fmaf(-beta1, grad, grad));
+        volatile float g2 = grad * grad;
+        const float v_new = fmaf(beta2, v_old, fmaf(-beta2, g2, g2));
+        const uint32_t random = orc_squirrel_noise_5((uint32_t)i, seed);
+        volatile float m_hat = m_new * c1, v_hat = v_new * c2;
+        volatile float den = sqrtf(v_hat) + eps;
+        volatile float quot = m_hat / den;
+        const float p_new = fmaf(-lr, fmaf(wd, p_old, quot), p_old);
+        params[i] = orc_stochastic_round_bf16(p_new, random);
+        const float pa = fabsf(orc_bf16_to_f32(params[i]));
+        if (pa > amax) amax = pa;   /* NaNs are skipped, as in the abs-max reduction */
+        if (v_dtype) ((uint16_t*)v_mem)[i] = orc_stochastic_round_bf16(v_new, rotl32(random, 20));
+        else ((float*)v_mem)[i] = v_new;
+        if (m_dtype) {
+            const uint32_t base = orc_squirrel_noise_5((uint32_t)(i - i % ref_vec), 51245u);
+            ((uint16_t*)m_mem)[i] = orc_stochastic_round_bf16(m_new, rotl32(base, 7 * (int)(i % ref_vec)));
+        } else {
+            ((float*)m_mem)[i] = m_new;
+        }
+    }
+    return amax;
 }
 
 /* ------------------------------------------------------------------------------------------------

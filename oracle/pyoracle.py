@@ -111,6 +111,13 @@ def lib():
     L.orc_rmsnorm_backward_bf16.argtypes = [u16p, u16p, f64p, f64p, f64p, f64p, u16p, u16p, u16p, u16p, f32p, C.c_int64, C.c_int]
     L.orc_rope_bf16.restype = None
     L.orc_rope_bf16.argtypes = [u16p, f64p, f64p, u16p, u16p, C.c_int64, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
+    L.orc_squirrel_noise_5.restype = C.c_uint32
+    L.orc_squirrel_noise_5.argtypes = [C.c_uint32, C.c_uint32]
+    L.orc_stochastic_round_bf16.restype = C.c_uint16
+    L.orc_stochastic_round_bf16.argtypes = [C.c_float, C.c_uint32]
+    L.orc_adamw_update_bf16.restype = C.c_float
+    L.orc_adamw_update_bf16.argtypes = [u16p, u16p, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int64, C.c_float, C.c_float,
+                                        C.c_float, C.c_int, C.c_float, C.c_float, C.c_float, C.c_uint32]
     _lib = L
     return L
 
@@ -369,3 +376,15 @@ def rope(inp, freqs_f16, T, Nq, Nkv, backward=False):
     lib().orc_rope_bf16(_p(out, C.c_uint16), _p(exact, C.c_double), _p(mag, C.c_double), _p(inp, C.c_uint16),
                         _p(freqs, C.c_uint16), BT, T, Nq, Nkv, HD, 1 if backward else 0)
     return out, exact, mag
+
+
+def adamw_update(params, grads, m, v, lr, beta1, beta2, t, eps, wd, grad_scale, seed):
+    """params, grads: bf16 bits; m, v: float32 arrays (fp32 moments) or uint16 bf16 bits.  Returns new
+    (params, m, v, abs-max of the new params); inputs are not modified."""
+    p = np.array(params, dtype=np.uint16, copy=True)
+    g = np.ascontiguousarray(grads, dtype=np.uint16)
+    mm, vv = np.array(m, copy=True), np.array(v, copy=True)
+    md, vd = int(mm.dtype == np.uint16), int(vv.dtype == np.uint16)
+    am = lib().orc_adamw_update_bf16(_p(p, C.c_uint16), _p(g, C.c_uint16), mm.ctypes.data, md, vv.ctypes.data, vd, p.size,
+                                     lr, beta1, beta2, t, eps, wd, grad_scale, seed)
+    return p, mm, vv, np.float32(am)

@@ -586,3 +586,79 @@ def test_rope_vs_complex_multiplication(O):
     zz = (zf[..., :half] + 1j * zf[..., half:]) * np.conj(rot_bt)
     assert np.allclose(back[:, qk, :half], zz[:, qk].real, rtol=1e-14, atol=1e-300)
     assert np.allclose(back[:, qk, half:], zz[:, qk].imag, rtol=1e-14, atol=1e-300)
+
+
+# ------------------------------------------------------------------------------------------- adamw
+def test_squirrel_noise_properties(O):
+    """No known-answer vectors exist in the reference tree; what the construction guarantees is checked: for a
+    fixed seed the hash is a bijection of the position (no collisions), its bits are balanced, and different
+    seeds give unrelated streams."""
+    L = O.lib()
+    n = 1 << 20
+    vals = np.fromiter((L.orc_squirrel_noise_5(i, 1234) for i in range(0, n, 1)), dtype=np.uint32, count=n)
+    assert np.unique(vals).size == n
+    bits = np.unpackbits(vals[: 1 << 16].view(np.uint8))
+    assert abs(bits.mean() - 0.5) < 0.004
+    other = np.fromiter((L.orc_squirrel_noise_5(i, 1235) for i in range(1 << 16)), dtype=np.uint32, count=1 << 16)
+    assert np.mean(other == vals[: 1 << 16]) < 1e-3
+    low = vals[: 1 << 18] & 0xFFFF                   # the 16-bit thresholds: uniform
+    hist = np.bincount(low >> 8, minlength=256)
+    assert hist.min() > 0.85 * (1 << 18) / 256 and hist.max() < 1.15 * (1 << 18) / 256
+
+
+def test_stochastic_rounding_properties(O):
+    """Values exactly representable in bf16 are unchanged; any other value goes to one of its two bf16
+    neighbours (away from zero iff its low 16 bits exceed the threshold); the mean over the hash's thresholds
+    is the value itself (the reference's own unbiasedness test, scripts/test_kernels.py:812-828)."""
+    L = O.lib()
+    for x in (1.0, -2.5, 0.0, 3.0e5, -7.0e-9):
+        xb = np.asarray(O.bf16_to_f32(O.f32_to_bf16(np.array([x], np.float32)))).reshape(-1)[0]
+        for rnd in (0, 0x1234, 0xFFFF, 0xFFFFFFFF):
+            assert O.bf16_to_f32(np.array([L.orc_stochastic_round_bf16(float(xb), rnd)], np.uint16))[0] == xb
+    x = np.float32(1.0 + 2.0 ** -9 + 2.0 ** -13)           # between 1 and 1 + 2^-7
+    lo, hi = np.float32(1.0), np.float32(1.0 + 2.0 ** -7)
+    low_bits = int(np.float32(x).view(np.uint32)) & 0xFFFF
+    outs = []
+    for i in range(1 << 16):
+        rnd = L.orc_squirrel_noise_5(i, 99)
+        r = O.bf16_to_f32(np.array([L.orc_stochastic_round_bf16(float(x), rnd)], np.uint16))[0]
+        assert r == (hi if low_bits > (rnd & 0xFFFF) else lo)
+        outs.append(r)
+    assert abs(np.mean(outs, dtype=np.float64) - float(x)) < 2.0 ** -7 * 0.01
+    neg = [O.bf16_to_f32(np.array([L.orc_stochastic_round_bf16(float(-x), L.orc_squirrel_noise_5(i, 7))], np.uint16))[0] for i in range(4096)]
+    assert set(neg) == {-lo, -hi}
+
+
+@pytest.mark.parametrize("moments", ["f32f32", "bf16f32", "bf16bf16"])
+def test_adamw_vs_torch_formulas(O, moments):
+    """The reference's test construction (scripts/test_kernels.py:695-727) in float64."""
+    n = 4096
+    rng = np.random.default_rng(0)
+    f = lambda a: O.f32_to_bf16(a.astype(np.float32))
+    params, grads = f(rng.standard_normal(n)), f(rng.standard_normal(n))
+    m0 = (rng.standard_normal(n) * 0.1).astype(np.float32)
+    v0 = (rng.random(n) * 0.01 + 1e-8).astype(np.float32)
+    m_in = f(m0) if moments.startswith("bf16") else m0
+    v_in = f(v0) if moments.endswith("bf16") else v0
+    lr, b1, b2, t, eps, wd, gs = 1e-3, 0.9, 0.999, 1, 1e-8, 0.1, 0.75
+    p1, m1, v1, am = O.adamw_update(params, grads, m_in, v_in, lr, b1, b2, t, eps, wd, gs, 42)
+    dec = lambda a: O.bf16_to_f32(a).astype(np.float64) if a.dtype == np.uint16 else a.astype(np.float64)
+    g, p, m, v = dec(grads) * np.float64(np.float32(gs)), dec(params), dec(m_in), dec(v_in)
+    b1d, b2d = np.float64(np.float32(b1)), np.float64(np.float32(b2))
+    m_new = b1d * m + (1 - b1d) * g
+    v_new = b2d * v + (1 - b2d) * g ** 2
+    p_new = p * (1 - np.float64(np.float32(lr)) * np.float64(np.float32(wd))) - np.float64(np.float32(lr)) * (m_new / (1 - b1d ** t)) / (
+        np.sqrt(v_new / (1 - b2d ** t)) + np.float64(np.float32(eps)))
+    ulp = lambda x: np.maximum(np.abs(x), 1e-30) * 2.0 ** -7
+    assert np.all(np.abs(dec(p1) - p_new) <= ulp(p_new))                      # one of the two bf16 neighbours
+    if m1.dtype == np.uint16:
+        assert np.all(np.abs(dec(m1) - m_new) <= ulp(m_new) + 2.0 ** -22 * (np.abs(m) + np.abs(g)))
+    else:
+        assert np.all(np.abs(m1 - m_new) <= 2.0 ** -22 * (np.abs(m) + np.abs(g)))     # fp32 evaluation of the lerp
+    if v1.dtype == np.uint16:
+        assert np.all(np.abs(dec(v1) - v_new) <= ulp(v_new))
+    else:
+        assert np.all(np.abs(v1 - v_new) <= 2.0 ** -22 * (np.abs(v) + g ** 2))
+    assert am == np.abs(O.bf16_to_f32(p1)).max()
+    # stochastic rounding is unbiased: the mean error of the parameters is far below half an ulp
+    assert abs(np.mean((dec(p1) - p_new) / ulp(p_new))) < 0.05
