@@ -114,4 +114,53 @@ inline void backward_qmm(Tensor& dinp, Tensor& dweight, Tensor dbias, Quantizabl
     }
 }
 
+// ---- weight side: quantize on gather, cached per optimizer version ------------------------------------------
+// The reference keeps bf16 master weights and hands the matmuls an e4m3 copy that it rebuilds only when the
+// optimizer has changed the weights (src/models/llama_weights.cpp:207-223 convert_dtype_for_gather, :434-504 the
+// LayerIdx / Version cache of LLamaWeightsManager).  On one GPU the gather itself is the identity; what remains is
+// this cache: a small number of e4m3 slots (the reference double-buffers two layers), each remembering which layer
+// and which weight version it holds.  The master tensor's Stats carry [abs_max, scale]: abs_max comes from the
+// optimizer's epilogue (adamw_update) or from abs_max() at initialisation; the scale is written by the quantizer.
+class QuantizedWeightCache {
+public:
+    struct Slot {
+        Tensor Quant{};
+        int LayerIdx = -1;
+        int Version = -1;
+    };
+
+    // storage: one e4m3 tensor per slot, all of the weight's shape
+    explicit QuantizedWeightCache(std::vector<Tensor> storage) {
+        for (auto& t : storage) {
+            if (t.DType != ETensorDType::FP8_E4M3) throw std::invalid_argument("QuantizedWeightCache: slots must be e4m3 tensors");
+            Slots.push_back(Slot{t, -1, -1});
+        }
+        if (Slots.empty()) throw std::invalid_argument("QuantizedWeightCache: at least one slot");
+    }
+
+    // the optimizer has written new master weights: every cached copy is stale from now on
+    void invalidate() { ++mVersion; }
+    int version() const { return mVersion; }
+    long quantize_calls() const { return mQuantizeCalls; }
+
+    // e4m3 copy of layer `layer_idx`'s weight; requantized only if its slot holds another layer or an older version
+    Tensor& get(int layer_idx, const Tensor& master, const hipDeviceProp_t& dp, hipStream_t stream) {
+        Slot& s = Slots[(std::size_t)layer_idx % Slots.size()];
+        if (master.nelem() != s.Quant.nelem()) throw std::invalid_argument("QuantizedWeightCache: shape mismatch");
+        if (s.LayerIdx != layer_idx || s.Version != mVersion) {
+            s.Quant.Stats = master.Stats;  // the copy shares the master's [abs_max, scale]
+            quantize_with_abs_max(s.Quant, s.Quant.scale(), master, master.abs_max(), (long)master.nelem(), dp, stream);
+            s.LayerIdx = layer_idx;
+            s.Version = mVersion;
+            ++mQuantizeCalls;
+        }
+        return s.Quant;
+    }
+
+private:
+    std::vector<Slot> Slots;
+    int mVersion = 0;
+    long mQuantizeCalls = 0;
+};
+
 #endif  // LLMQ_QMM_HPP

@@ -200,6 +200,30 @@ int main(int argc, char** argv) {
         EXPECT(sw_threw, "swiglu_forward with C %% 8 != 0 must throw std::invalid_argument");
     }
 
+    {   // weight side: e4m3 copies rebuilt only when the layer or the optimizer version changes (llama_weights.cpp:434-504)
+        float* wstats = dalloc<float>(2);
+        Tensor master = make(ETensorDType::BF16, dw, {OC, C}, wstats);
+        abs_max(master.abs_max(), master, (long)OC * C, rs.DeviceProp, stream);
+        QuantizedWeightCache cache({make(ETensorDType::FP8_E4M3, dalloc<uint8_t>(hw.size()), {OC, C}),
+                                    make(ETensorDType::FP8_E4M3, dalloc<uint8_t>(hw.size()), {OC, C})});
+        cache.get(0, master, rs.DeviceProp, stream);
+        cache.get(1, master, rs.DeviceProp, stream);
+        Tensor& again = cache.get(0, master, rs.DeviceProp, stream);
+        EXPECT(cache.quantize_calls() == 2, "cached layer was requantized");
+        cache.get(2, master, rs.DeviceProp, stream);          // takes layer 0's slot
+        cache.get(0, master, rs.DeviceProp, stream);
+        EXPECT(cache.quantize_calls() == 4, "evicted layer was not requantized");
+        cache.invalidate();                                   // optimizer step
+        Tensor& fresh = cache.get(1, master, rs.DeviceProp, stream);
+        EXPECT(cache.quantize_calls() == 5, "stale version was not requantized");
+        HIP_OK(hipStreamSynchronize(stream));
+        float ws2[2]; HIP_OK(hipMemcpy(ws2, wstats, 8, hipMemcpyDeviceToHost));
+        EXPECT(std::memcmp(&ws2[0], &aw, 4) == 0 && std::memcmp(&ws2[1], &sw, 4) == 0, "weight cache: abs-max / scale mismatch");
+        EXPECT(fresh.scale() == master.scale() && again.abs_max() == master.abs_max(), "weight cache: Stats not shared with the master");
+        HIP_OK(hipMemcpy(got.data(), fresh.Data, wq.size(), hipMemcpyDeviceToHost));
+        EXPECT(std::memcmp(got.data(), wq.data(), wq.size()) == 0, "weight cache: quantized bytes differ");
+    }
+
     // ---- error behaviour of the shim (reference: gemm_mma.cu:261-263, kernels.cpp:18-24) ----
     bool threw = false;
     try { matmul(out, weight, inp.Quant, no_bias, nullptr, nullptr, nullptr, workspace, OC, BT, C + 64, EMMTranspose::TN, false, stream); }
