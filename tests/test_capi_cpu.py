@@ -73,12 +73,49 @@ def test_invalid_arguments_are_rejected_without_a_gpu(capi):
         capi.check(capi.LLMQ_ERR_RUNTIME)
 
 
+def test_producer_entry_points_reject_bad_arguments_without_a_gpu(capi):
+    """Shape rules of the producers (src/kernels/swiglu.cu:306-318, rope.cu:137, adamw.cu:150) are checked before
+    anything is launched."""
+    L = capi.lib
+    buf = (C.c_char * 4096)()
+    p = (C.addressof(buf) + 15) & ~15
+    INV = capi.LLMQ_ERR_INVALID_ARGUMENT
+    f = C.c_float
+    assert L.llmq_swiglu_forward_bf16(p, p, None, 1, 4, 12, None) == INV and b"divisible by 8" in L.llmq_last_error()
+    assert L.llmq_swiglu_forward_bf16(p, p, None, 1 << 15, 1 << 15, 8, None) == INV and b"too large" in L.llmq_last_error()
+    assert L.llmq_swiglu_forward_quant_bf16(p, None, p, None, 1, 4, 16, None) == INV
+    assert L.llmq_swiglu_backward_bf16(p, p, p, None, 1, 4, 20, None) == INV
+    assert L.llmq_rmsnorm_forward_bf16(p, None, p, p, None, f(1e-6), 1, 4, 12, None) == INV
+    assert L.llmq_rmsnorm_forward_bf16(p, None, p, p, None, f(1e-6), 1, 4, 16392, None) == INV and b"16384" in L.llmq_last_error()
+    assert L.llmq_fused_residual_rmsnorm_forward_bf16(None, p, p, p, p, p, None, f(1e-6), 4, 16, None) == INV
+    assert L.llmq_rmsnorm_backward_bf16(p, p, p, 16, p, p, p, p, p, None, 1, 4, 64, None) == INV and b"scratch" in L.llmq_last_error()
+    assert L.llmq_rmsnorm_backward_scratch_bytes(3584) >= 3584 * 4 and L.llmq_rmsnorm_backward_scratch_bytes(0) == 0
+    assert L.llmq_rope_forward_bf16(p, p, p, None, 1, 4, 2, 1, 12, None) == INV and b"head_dim" in L.llmq_last_error()
+    assert L.llmq_rope_backward_bf16(p, p + 2, p, None, 1, 4, 2, 1, 16, None) == INV
+    assert L.llmq_adamw_update_bf16(p, p, p, 0, p, 0, 12, f(1e-3), f(0.9), f(0.99), 1, f(1e-8), f(0.0), p, None, 1, None) == INV
+    assert L.llmq_adamw_update_bf16(p, p, p, 0, p, 1, 16, f(1e-3), f(0.9), f(0.99), 1, f(1e-8), f(0.0), p, None, 1, None) == INV
+    assert b"moment types" in L.llmq_last_error()
+    assert L.llmq_adamw_update_bf16(p, p, p, 0, p, 0, 16, f(1e-3), f(0.9), f(0.99), 1, f(1e-8), f(0.0), None, None, 1, None) == INV
+
+
+def test_precompute_freqs_cis_on_the_host(capi):
+    """The rope table is host code (src/kernels/rope.cu:15-40): cos / sin of t / theta^(2i/dim) in fp16."""
+    import numpy as np
+    dim, end, theta = 16, 9, 10000.0
+    tab = np.zeros((end, dim), dtype=np.float16)
+    assert capi.lib.llmq_precompute_freqs_cis_f16(tab.ctypes.data, dim, end, C.c_float(theta)) == capi.LLMQ_OK
+    ang = np.arange(end)[:, None] / theta ** (2 * np.arange(dim // 2) / dim)[None, :]
+    assert np.allclose(tab[:, 0::2], np.cos(ang), atol=2.0 ** -10) and np.allclose(tab[:, 1::2], np.sin(ang), atol=2.0 ** -10)
+    assert capi.lib.llmq_precompute_freqs_cis_f16(tab.ctypes.data, 15, end, C.c_float(theta)) == capi.LLMQ_ERR_INVALID_ARGUMENT
+
+
 def test_reference_python_ops_register_without_a_gpu():
     """llmq_amd.ops registers the reference's operator names (src/binding/python/kernels.py:118-165) at import."""
     import torch
     from llmq_amd import ops
     for name in ("abs_max", "quantize_with_abs_max", "quantize_and_transpose_with_abs_max", "transpose", "matmul",
-                 "backward_bias"):
+                 "backward_bias", "swiglu_forward", "swiglu_forward_quant", "swiglu_backward", "rmsnorm_forward",
+                 "fused_residual_rmsnorm_forward", "rmsnorm_backward", "rope_forward", "rope_backward", "adamw_update"):
         assert hasattr(torch.ops.llmq, name)
     assert ops.MODE_NT == 2 and ops.create_cublas_handle() == 0
     with pytest.raises(ValueError):                      # host tensors are rejected before any launch
