@@ -55,6 +55,18 @@ __device__ __forceinline__ uint32_t sr_bf16(float x, uint32_t random) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(p, bf16x2_aw)) & 0xFFFFu;
 }
 
+// 8 consecutive fp32 values as two streaming 16-byte accesses
+__device__ __forceinline__ void load_f32x8(float (&dst)[8], const uint4* p) {
+    const uint4 lo = load_nt(p), hi = load_nt(p + 1);
+    const uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+    for (int k = 0; k < 8; ++k) dst[k] = __uint_as_float(w[k]);
+}
+__device__ __forceinline__ void store_f32x8(uint4* p, const float (&src)[8]) {
+    store_nt(p, make_uint4(__float_as_uint(src[0]), __float_as_uint(src[1]), __float_as_uint(src[2]), __float_as_uint(src[3])));
+    store_nt(p + 1, make_uint4(__float_as_uint(src[4]), __float_as_uint(src[5]), __float_as_uint(src[6]), __float_as_uint(src[7])));
+}
+
 struct AdamArgs {
     float lr, beta1, beta2, c1, c2, eps, wd;
     unsigned seed;
@@ -71,25 +83,23 @@ __global__ __launch_bounds__(THREADS) void adamw_kernel(uint4* __restrict__ para
     uint32_t fold = 0x7F807F80u;
     if (vec < nvec) {
         const float gs = *grad_scale;
-        const uint4 pw = params[vec], gw = grads[vec];
+        const uint4 pw = load_nt(&params[vec]), gw = load_nt(&grads[vec]);
         float m[8], v[8];
         if constexpr (M_BF16) {
-            const uint4 w = reinterpret_cast<const uint4*>(m_mem)[vec];
+            const uint4 w = load_nt(&reinterpret_cast<const uint4*>(m_mem)[vec]);
             const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
             for (int k = 0; k < 4; ++k) { m[2 * k] = bf16_lo(ww[k]); m[2 * k + 1] = bf16_hi(ww[k]); }
         } else {
-            const float4 lo = reinterpret_cast<const float4*>(m_mem)[2 * vec], hi = reinterpret_cast<const float4*>(m_mem)[2 * vec + 1];
-            m[0] = lo.x; m[1] = lo.y; m[2] = lo.z; m[3] = lo.w; m[4] = hi.x; m[5] = hi.y; m[6] = hi.z; m[7] = hi.w;
+            load_f32x8(m, reinterpret_cast<const uint4*>(m_mem) + 2 * vec);
         }
         if constexpr (V_BF16) {
-            const uint4 w = reinterpret_cast<const uint4*>(v_mem)[vec];
+            const uint4 w = load_nt(&reinterpret_cast<const uint4*>(v_mem)[vec]);
             const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
             for (int k = 0; k < 4; ++k) { v[2 * k] = bf16_lo(ww[k]); v[2 * k + 1] = bf16_hi(ww[k]); }
         } else {
-            const float4 lo = reinterpret_cast<const float4*>(v_mem)[2 * vec], hi = reinterpret_cast<const float4*>(v_mem)[2 * vec + 1];
-            v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w; v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+            load_f32x8(v, reinterpret_cast<const uint4*>(v_mem) + 2 * vec);
         }
         const uint32_t pws[4] = {pw.x, pw.y, pw.z, pw.w}, gws[4] = {gw.x, gw.y, gw.z, gw.w};
         uint32_t p_out[8], m_out[8], v_out[8];
@@ -118,21 +128,19 @@ __global__ __launch_bounds__(THREADS) void adamw_kernel(uint4* __restrict__ para
         }
         const uint4 pnew = make_uint4(p_out[0] | (p_out[1] << 16), p_out[2] | (p_out[3] << 16), p_out[4] | (p_out[5] << 16),
                                       p_out[6] | (p_out[7] << 16));
-        params[vec] = pnew;
+        store_nt(&params[vec], pnew);
         if constexpr (ABSMAX) fold = fold_vec(fold, pnew);
         if constexpr (M_BF16) {
-            reinterpret_cast<uint4*>(m_mem)[vec] = make_uint4(m_out[0] | (m_out[1] << 16), m_out[2] | (m_out[3] << 16),
-                                                              m_out[4] | (m_out[5] << 16), m_out[6] | (m_out[7] << 16));
+            store_nt(&reinterpret_cast<uint4*>(m_mem)[vec], make_uint4(m_out[0] | (m_out[1] << 16), m_out[2] | (m_out[3] << 16),
+                                                              m_out[4] | (m_out[5] << 16), m_out[6] | (m_out[7] << 16)));
         } else {
-            reinterpret_cast<float4*>(m_mem)[2 * vec] = make_float4(m[0], m[1], m[2], m[3]);
-            reinterpret_cast<float4*>(m_mem)[2 * vec + 1] = make_float4(m[4], m[5], m[6], m[7]);
+            store_f32x8(reinterpret_cast<uint4*>(m_mem) + 2 * vec, m);
         }
         if constexpr (V_BF16) {
-            reinterpret_cast<uint4*>(v_mem)[vec] = make_uint4(v_out[0] | (v_out[1] << 16), v_out[2] | (v_out[3] << 16),
-                                                              v_out[4] | (v_out[5] << 16), v_out[6] | (v_out[7] << 16));
+            store_nt(&reinterpret_cast<uint4*>(v_mem)[vec], make_uint4(v_out[0] | (v_out[1] << 16), v_out[2] | (v_out[3] << 16),
+                                                              v_out[4] | (v_out[5] << 16), v_out[6] | (v_out[7] << 16)));
         } else {
-            reinterpret_cast<float4*>(v_mem)[2 * vec] = make_float4(v[0], v[1], v[2], v[3]);
-            reinterpret_cast<float4*>(v_mem)[2 * vec + 1] = make_float4(v[4], v[5], v[6], v[7]);
+            store_f32x8(reinterpret_cast<uint4*>(v_mem) + 2 * vec, v);
         }
     }
     if constexpr (ABSMAX) {

@@ -40,6 +40,25 @@ constexpr int kWave = 64;
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xFFFF0000u); }
 
+// Streaming accesses: data read for the last time, or written for a consumer that is not the next kernel, is
+// marked non-temporal so that it does not displace what the next kernel re-reads from the 256 MB last-level
+// cache (measured: abs-max followed by quantize of a 310 MB tensor goes from 151 to 124 us when the quantizer's
+// accesses are non-temporal, because the tensor the abs-max just read is still cached).
+typedef unsigned int llmq_v4u __attribute__((ext_vector_type(4)));
+typedef unsigned int llmq_v2u __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint4 load_nt(const uint4* p) {
+    const llmq_v4u t = __builtin_nontemporal_load(reinterpret_cast<const llmq_v4u*>(p));
+    return make_uint4(t[0], t[1], t[2], t[3]);
+}
+__device__ __forceinline__ void store_nt(uint4* p, const uint4& v) {
+    const llmq_v4u t = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(t, reinterpret_cast<llmq_v4u*>(p));
+}
+__device__ __forceinline__ void store_nt(uint2* p, const uint2& v) {
+    const llmq_v2u t = {v.x, v.y};
+    __builtin_nontemporal_store(t, reinterpret_cast<llmq_v2u*>(p));
+}
+
 // scale = 448 / max(absmax, 1e-10) with an IEEE-correct fp32 division (src/kernels/quant.cu:79).
 __device__ __forceinline__ float quant_scale(float absmax) {
     float a = (absmax > 1e-10f) ? absmax : 1e-10f;  // fmaxf semantics incl. NaN -> 1e-10

@@ -35,12 +35,12 @@ __global__ __launch_bounds__(256) void quantize_kernel(uint2* __restrict__ out, 
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             const int64_t idx = i + u * stride;
-            v[u] = idx < nvec ? in[idx] : make_uint4(0, 0, 0, 0);
+            v[u] = idx < nvec ? load_nt(&in[idx]) : make_uint4(0, 0, 0, 0);
         }
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             const int64_t idx = i + u * stride;
-            if (idx < nvec) out[idx] = encode8<FMT>(v[u], s);
+            if (idx < nvec) store_nt(&out[idx], encode8<FMT>(v[u], s));
         }
     }
     if (tid < ntail) {
@@ -114,7 +114,7 @@ __global__ __launch_bounds__(256) void quantize_transpose_kernel(uint8_t* __rest
         for (int j = 0; j < 4; ++j) {
             const int row = r0 + 4 * rq + j;
             if (row < rows && col < cols) {
-                v[p][j] = *reinterpret_cast<const uint4*>(in + (int64_t)row * cols + col);
+                v[p][j] = load_nt(reinterpret_cast<const uint4*>(in + (int64_t)row * cols + col));
             } else {
                 v[p][j] = make_uint4(0, 0, 0, 0);
             }
@@ -157,7 +157,7 @@ __global__ __launch_bounds__(256) void quantize_transpose_kernel(uint8_t* __rest
             const uint32_t* src = &tile[c * kQtStride + 4 * p];
             uint8_t* dst = out + (int64_t)(c0 + c) * rows + r;
             if (rows_mult16) {
-                *reinterpret_cast<uint4*>(dst) = make_uint4(src[0], src[1], src[2], src[3]);
+                store_nt(reinterpret_cast<uint4*>(dst), make_uint4(src[0], src[1], src[2], src[3]));
             } else {
                 *reinterpret_cast<uint2*>(dst) = make_uint2(src[0], src[1]);
                 if (r + 8 < rows) *reinterpret_cast<uint2*>(dst + 8) = make_uint2(src[2], src[3]);

@@ -64,7 +64,7 @@ __global__ __launch_bounds__(WAVES * 64) void rmsnorm_forward_kernel(uint4* resi
     for (int k = 0; k < NCH; ++k) {
         const int c = lane + kWave * k;
         x[k] = make_uint4(0, 0, 0, 0);
-        if (valid && c < chunks) x[k] = inp1[base + c];
+        if (valid && c < chunks) x[k] = load_nt(&inp1[base + c]);
     }
     if constexpr (RESIDUAL) {
         uint4 y[NCH];
@@ -72,14 +72,14 @@ __global__ __launch_bounds__(WAVES * 64) void rmsnorm_forward_kernel(uint4* resi
         for (int k = 0; k < NCH; ++k) {
             const int c = lane + kWave * k;
             y[k] = make_uint4(0, 0, 0, 0);
-            if (valid && c < chunks) y[k] = inp2[base + c];
+            if (valid && c < chunks) y[k] = load_nt(&inp2[base + c]);
         }
 #pragma unroll
         for (int k = 0; k < NCH; ++k) {
             const int c = lane + kWave * k;
             x[k] = make_uint4(add_pair(x[k].x, y[k].x), add_pair(x[k].y, y[k].y), add_pair(x[k].z, y[k].z),
                               add_pair(x[k].w, y[k].w));
-            if (valid && c < chunks) residual[base + c] = x[k];
+            if (valid && c < chunks) store_nt(&residual[base + c], x[k]);
         }
     }
 
@@ -99,7 +99,7 @@ __global__ __launch_bounds__(WAVES * 64) void rmsnorm_forward_kernel(uint4* resi
             const uint4 o = make_uint4(norm_pair(x[k].x, w.x, s), norm_pair(x[k].y, w.y, s), norm_pair(x[k].z, w.z, s),
                                        norm_pair(x[k].w, w.w, s));
             if (valid) {
-                normed[base + c] = o;
+                store_nt(&normed[base + c], o);
                 if constexpr (ABSMAX) fold = fold_vec(fold, o);
             }
         }
@@ -212,9 +212,9 @@ __global__ __launch_bounds__(256) void rmsnorm_backward_kernel(uint4* dinp, floa
             const int c = c_first + kWave * WPR * k;
             d[k] = x[k] = old[k] = make_uint4(0, 0, 0, 0);
             if (valid && c < chunks) {
-                d[k] = dout[base + c];
-                x[k] = inp[base + c];
-                old[k] = dresidual[base + c];
+                d[k] = load_nt(&dout[base + c]);
+                x[k] = load_nt(&inp[base + c]);
+                old[k] = load_nt(&dresidual[base + c]);
             }
         }
         float dot = 0.f;
@@ -262,7 +262,7 @@ __global__ __launch_bounds__(256) void rmsnorm_backward_kernel(uint4* dinp, floa
                     res[j] = pack_bf16_rn(bf16_lo(ov[j]) + v0, bf16_hi(ov[j]) + v1);
                 }
                 const uint4 o = make_uint4(res[0], res[1], res[2], res[3]);
-                dinp[base + c] = o;
+                store_nt(&dinp[base + c], o);
                 if constexpr (ABSMAX) fold = fold_vec(fold, o);
             }
         }

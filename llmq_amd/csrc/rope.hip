@@ -45,18 +45,23 @@ __device__ __forceinline__ void rotate_pair(uint32_t re, uint32_t im, uint32_t c
 }
 
 template <int DW> struct Words;  // DW dwords moved with one access
-template <> struct Words<2> { typedef uint2 type; };
-template <> struct Words<4> { typedef uint4 type; };
-template <int DW>
+template <> struct Words<2> { typedef unsigned int type __attribute__((ext_vector_type(2))); };
+template <> struct Words<4> { typedef unsigned int type __attribute__((ext_vector_type(4))); };
+// STREAM: non-temporal (the tensor itself; the small factor table is left to the caches)
+template <int DW, bool STREAM>
 __device__ __forceinline__ void load_words(uint32_t (&dst)[DW], const void* p) {
-    const typename Words<DW>::type v = *reinterpret_cast<const typename Words<DW>::type*>(p);
-    __builtin_memcpy(dst, &v, sizeof(v));
+    typedef typename Words<DW>::type V;
+    const V v = STREAM ? __builtin_nontemporal_load(reinterpret_cast<const V*>(p)) : *reinterpret_cast<const V*>(p);
+#pragma unroll
+    for (int k = 0; k < DW; ++k) dst[k] = v[k];
 }
 template <int DW>
 __device__ __forceinline__ void store_words(void* p, const uint32_t (&src)[DW]) {
-    typename Words<DW>::type v;
-    __builtin_memcpy(&v, src, sizeof(v));
-    *reinterpret_cast<typename Words<DW>::type*>(p) = v;
+    typedef typename Words<DW>::type V;
+    V v;
+#pragma unroll
+    for (int k = 0; k < DW; ++k) v[k] = src[k];
+    __builtin_nontemporal_store(v, reinterpret_cast<V*>(p));
 }
 
 // W: d values per lane (4 or 8).  Lane -> (token bt, head h, group of W d values).
@@ -79,13 +84,13 @@ __global__ __launch_bounds__(THREADS) void rope_kernel(uint16_t* out, const uint
         const bool rotated = h < Nq + Nkv;
         if (rotated || ABSMAX || !in_place) {
             uint32_t re[DW], im[DW];
-            load_words<DW>(re, inp + base);
-            load_words<DW>(im, inp + base + head_dim / 2);
+            load_words<DW, true>(re, inp + base);
+            load_words<DW, true>(im, inp + base + head_dim / 2);
             if (rotated) {
                 const uint16_t* f = freqs + (int64_t)t * head_dim + 2 * grp * W;
                 uint32_t cs_lo[DW], cs_hi[DW], cs[W];
-                load_words<DW>(cs_lo, f);
-                load_words<DW>(cs_hi, f + W);
+                load_words<DW, false>(cs_lo, f);
+                load_words<DW, false>(cs_hi, f + W);
 #pragma unroll
                 for (int k = 0; k < DW; ++k) {
                     cs[k] = cs_lo[k];

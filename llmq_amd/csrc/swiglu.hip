@@ -76,8 +76,8 @@ __global__ __launch_bounds__(THREADS) void swiglu_forward_kernel(void* __restric
         up[u] = gate[u] = make_uint4(0, 0, 0, 0);
         if (idx < nchunks) {
             const uint32_t src = input_chunk(idx, chunks_per_row);
-            up[u] = inp[src];
-            gate[u] = inp[src + chunks_per_row];
+            up[u] = load_nt(&inp[src]);
+            gate[u] = load_nt(&inp[src + chunks_per_row]);
         }
     }
     uint32_t acc = 0x7F807F80u;
@@ -87,8 +87,8 @@ __global__ __launch_bounds__(THREADS) void swiglu_forward_kernel(void* __restric
         const uint4 r = swiglu_chunk(up[u], gate[u]);  // zeros for the predicated-off chunks
         if constexpr (MODE == 1) acc = fold_vec(acc, r);
         if (idx < nchunks) {
-            if constexpr (MODE == 2) reinterpret_cast<uint2*>(out)[idx] = encode8<kE4M3>(r, s);
-            else reinterpret_cast<uint4*>(out)[idx] = r;
+            if constexpr (MODE == 2) store_nt(&reinterpret_cast<uint2*>(out)[idx], encode8<kE4M3>(r, s));
+            else store_nt(&reinterpret_cast<uint4*>(out)[idx], r);
         }
     }
     if constexpr (MODE == 1) {
@@ -125,9 +125,9 @@ __global__ __launch_bounds__(THREADS) void swiglu_backward_kernel(uint4* __restr
         d[u] = up[u] = gate[u] = make_uint4(0, 0, 0, 0);
         if (idx < nchunks) {
             const uint32_t src = input_chunk(idx, chunks_per_row);
-            d[u] = dout[idx];
-            up[u] = inp[src];
-            gate[u] = inp[src + chunks_per_row];
+            d[u] = load_nt(&dout[idx]);
+            up[u] = load_nt(&inp[src]);
+            gate[u] = load_nt(&inp[src + chunks_per_row]);
         }
     }
     uint32_t acc = 0x7F807F80u;
@@ -142,8 +142,8 @@ __global__ __launch_bounds__(THREADS) void swiglu_backward_kernel(uint4* __restr
         if constexpr (ABSMAX) acc = fold_vec(fold_vec(acc, g1), g2);
         if (idx < nchunks) {
             const uint32_t dst = input_chunk(idx, chunks_per_row);
-            dinp[dst] = g1;
-            dinp[dst + chunks_per_row] = g2;
+            store_nt(&dinp[dst], g1);
+            store_nt(&dinp[dst + chunks_per_row], g2);
         }
     }
     if constexpr (ABSMAX) {
@@ -164,7 +164,7 @@ static int check_shape(const char* what, int B, int T, int C, int64_t& nchunks) 
     return LLMQ_OK;
 }
 
-constexpr int kFwdUnroll = 4, kBwdUnroll = 2, kAbsmaxThreads = 1024;
+constexpr int kFwdUnroll = 4, kBwdUnroll = 2, kAbsmaxThreads = 512;
 
 static unsigned blocks_for(int64_t nchunks, int threads, int unroll) {
     return (unsigned)((nchunks + (int64_t)threads * unroll - 1) / ((int64_t)threads * unroll));

@@ -50,7 +50,7 @@ __global__ __launch_bounds__(256) void transpose_u8_kernel(uint8_t* __restrict__
         for (int j = 0; j < 4; ++j) {
             const int row = r0 + 4 * (q + 32 * p) + j;
             if (row < rows && col < cols) {
-                v[p][j] = *reinterpret_cast<const uint4*>(src + (int64_t)row * cols + col);
+                v[p][j] = load_nt(reinterpret_cast<const uint4*>(src + (int64_t)row * cols + col));
             } else {
                 v[p][j] = make_uint4(0, 0, 0, 0);
             }
@@ -80,7 +80,7 @@ __global__ __launch_bounds__(256) void transpose_u8_kernel(uint8_t* __restrict__
         const int r = r0 + 16 * p;
         if (c0 + c < cols && r < rows) {
             const uint32_t* s = &tile[c * kTrStride + 4 * p];
-            *reinterpret_cast<uint4*>(dst + (int64_t)(c0 + c) * rows + r) = make_uint4(s[0], s[1], s[2], s[3]);
+            store_nt(reinterpret_cast<uint4*>(dst + (int64_t)(c0 + c) * rows + r), make_uint4(s[0], s[1], s[2], s[3]));
         }
     }
 }
