@@ -767,7 +767,10 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 
         // Epilogue.  acc[i][j][r] is c row 16 i + 4 kg + r of the wave tile and, thanks to the a-tile row
-        // permutation, column 8 l16 + j: a lane owns 8 adjacent columns of each of its 32 rows.
+        // permutation, column 8 l16 + j: a lane owns 8 adjacent columns of each of its 32 rows.  The stores are
+        // non-temporal: the output (up to 620 MB) is not read by this kernel again and would otherwise push
+        // the operands, which the other XCDs still fetch, out of the last-level cache (measured on one box,
+        // alternating builds: -8 % on the gate+up forward, -3.7 % over the six bench shapes).
         int n_blk, m_blk;
         decode(logical, n_blk, m_blk);
         logical += tile_stride;
@@ -840,11 +843,11 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
                             const f32x2_t pr = {v[2 * j], v[2 * j + 1]};
                             packed[j] = __builtin_bit_cast(int, __builtin_convertvector(pr, bf16x2_t));
                         }
-                        *(LLMQ_GLOBAL v4i*)row[r] = packed;
+                        __builtin_nontemporal_store(packed, (LLMQ_GLOBAL v4i*)row[r]);
                     } else {
                         const v4fl lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
-                        *(LLMQ_GLOBAL v4fl*)row[r] = lo;
-                        *(LLMQ_GLOBAL v4fl*)(row[r] + 16) = hi;
+                        __builtin_nontemporal_store(lo, (LLMQ_GLOBAL v4fl*)row[r]);
+                        __builtin_nontemporal_store(hi, (LLMQ_GLOBAL v4fl*)(row[r] + 16));
                     }
                 }
             }
