@@ -101,7 +101,8 @@ template <> struct PairIo<uint16_t> {
     }
     static __device__ __forceinline__ void store(LLMQ_GLOBAL void* p, float v0, float v1) {
         const f32x2_t v = {v0, v1};
-        *(LLMQ_GLOBAL bf16x2_t*)p = __builtin_convertvector(v, bf16x2_t);  // v_cvt_pk_bf16_f32, RNE
+        // v_cvt_pk_bf16_f32 (RNE); outputs are written once and not read again by these kernels: non-temporal
+        __builtin_nontemporal_store(__builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t)), (LLMQ_GLOBAL uint32_t*)p);
     }
 };
 template <> struct PairIo<float> {
@@ -112,7 +113,7 @@ template <> struct PairIo<float> {
     }
     static __device__ __forceinline__ void store(LLMQ_GLOBAL void* p, float v0, float v1) {
         const f32x2_t v = {v0, v1};
-        *(LLMQ_GLOBAL f32x2_t*)p = v;
+        __builtin_nontemporal_store(v, (LLMQ_GLOBAL f32x2_t*)p);
     }
 };
 
@@ -415,7 +416,7 @@ __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(Gemm
 #pragma unroll
             for (int p = 0; p < 4; ++p) {
                 LLMQ_GLOBAL char* row = scalar_ptr((LLMQ_GLOBAL char*)(out + (int64_t)(row0 + i * 32 + p * 8) * g.M));
-                *(LLMQ_GLOBAL v4i*)(row + lane_bytes) = piece[p];
+                __builtin_nontemporal_store(piece[p], (LLMQ_GLOBAL v4i*)(row + lane_bytes));
             }
         }
     };
