@@ -40,7 +40,7 @@ __global__ __launch_bounds__(256) void quantize_kernel(uint2* __restrict__ out, 
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             const int64_t idx = i + u * stride;
-            if (idx < nvec) store_nt(&out[idx], encode8<FMT>(v[u], s));
+            if (idx < nvec) out[idx] = encode8<FMT>(v[u], s);
         }
     }
     if (tid < ntail) {
@@ -157,7 +157,7 @@ __global__ __launch_bounds__(256) void quantize_transpose_kernel(uint8_t* __rest
             const uint32_t* src = &tile[c * kQtStride + 4 * p];
             uint8_t* dst = out + (int64_t)(c0 + c) * rows + r;
             if (rows_mult16) {
-                store_nt(reinterpret_cast<uint4*>(dst), make_uint4(src[0], src[1], src[2], src[3]));
+                *reinterpret_cast<uint4*>(dst) = make_uint4(src[0], src[1], src[2], src[3]);
             } else {
                 *reinterpret_cast<uint2*>(dst) = make_uint2(src[0], src[1]);
                 if (r + 8 < rows) *reinterpret_cast<uint2*>(dst + 8) = make_uint2(src[2], src[3]);

@@ -80,7 +80,7 @@ __global__ __launch_bounds__(256) void transpose_u8_kernel(uint8_t* __restrict__
         const int r = r0 + 16 * p;
         if (c0 + c < cols && r < rows) {
             const uint32_t* s = &tile[c * kTrStride + 4 * p];
-            store_nt(reinterpret_cast<uint4*>(dst + (int64_t)(c0 + c) * rows + r), make_uint4(s[0], s[1], s[2], s[3]));
+            *reinterpret_cast<uint4*>(dst + (int64_t)(c0 + c) * rows + r) = make_uint4(s[0], s[1], s[2], s[3]);
         }
     }
 }
