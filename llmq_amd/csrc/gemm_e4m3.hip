@@ -101,8 +101,7 @@ template <> struct PairIo<uint16_t> {
     }
     static __device__ __forceinline__ void store(LLMQ_GLOBAL void* p, float v0, float v1) {
         const f32x2_t v = {v0, v1};
-        // v_cvt_pk_bf16_f32 (RNE); outputs are written once and not read again by these kernels: non-temporal
-        __builtin_nontemporal_store(__builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t)), (LLMQ_GLOBAL uint32_t*)p);
+        *(LLMQ_GLOBAL bf16x2_t*)p = __builtin_convertvector(v, bf16x2_t);  // v_cvt_pk_bf16_f32, RNE
     }
 };
 template <> struct PairIo<float> {
@@ -113,7 +112,7 @@ template <> struct PairIo<float> {
     }
     static __device__ __forceinline__ void store(LLMQ_GLOBAL void* p, float v0, float v1) {
         const f32x2_t v = {v0, v1};
-        __builtin_nontemporal_store(v, (LLMQ_GLOBAL f32x2_t*)p);
+        *(LLMQ_GLOBAL f32x2_t*)p = v;
     }
 };
 
@@ -768,8 +767,8 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 
         // Epilogue.  acc[i][j][r] is c row 16 i + 4 kg + r of the wave tile and, thanks to the a-tile row
-        // permutation, column 8 l16 + j: a lane owns 8 adjacent columns of each of its 32 rows.  The stores are
-        // non-temporal: the output (up to 620 MB) is not read by this kernel again and would otherwise push
+        // permutation, column 8 l16 + j: a lane owns 8 adjacent columns of each of its 32 rows.  The bf16 stores
+        // are non-temporal: the output (up to 620 MB) is not read by this kernel again and would otherwise push
         // the operands, which the other XCDs still fetch, out of the last-level cache (measured on one box,
         // alternating builds: -8 % on the gate+up forward, -3.7 % over the six bench shapes).
         int n_blk, m_blk;
@@ -847,8 +846,8 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
                         __builtin_nontemporal_store(packed, (LLMQ_GLOBAL v4i*)row[r]);
                     } else {
                         const v4fl lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
-                        __builtin_nontemporal_store(lo, (LLMQ_GLOBAL v4fl*)row[r]);
-                        __builtin_nontemporal_store(hi, (LLMQ_GLOBAL v4fl*)(row[r] + 16));
+                        *(LLMQ_GLOBAL v4fl*)row[r] = lo;  // two instructions interleave 16-byte pieces: left to the L2 to merge
+                        *(LLMQ_GLOBAL v4fl*)(row[r] + 16) = hi;
                     }
                 }
             }
