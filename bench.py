@@ -14,7 +14,8 @@ One JSON line is printed:
   roofline        the GEMM kernel alone: algorithmic FLOP / mean launch duration (HIP events around
                   each GEMM launch inside the timed steps) against the dense FP8 MFMA peak
   quantize        abs-max + quantize (+transpose) launches: algorithmic bytes / event-timed duration
-                  against 8 TB/s
+                  against 8 TB/s, inside the step; quantize.cold_large_tensor holds the same kernels timed
+                  on their own on 310 MB tensors that no cache holds (median of 20 launches)
   cpu_baseline    the multithreaded CPU port of the same path on a bounded sample (host cores of this box)
 Extra fields: roofline.mfma_only_ceiling_TFLOPs (register-only matrix-instruction loops: what the chip sustains
 under its power limit), roofline.traffic (hardware-counter bytes per GEMM launch, from profiles/), hip_graph_replay
@@ -289,6 +290,52 @@ def main():
         del a_m, a_v, a_p, a_g
         swiglu["fused_residual_rmsnorm_forward+abs_max (8 B/el)"] = gbs(
             lambda: K.fused_residual_rmsnorm_forward(r_out, r_norm, r_rms, r_in, r_att, r_w, sw_am, 1e-6), 8 * BT * C, iters=10)
+    # The HBM-bound kernels on their own, cold: 5 warm-up and 20 timed launches each, one pair of events per
+    # launch, rotating through three distinct 310 MB tensors (930 MB, well beyond the 256 MB last-level cache,
+    # so every launch reads from HBM); median and best launch.  The in-step figures above include what the
+    # previous kernel left in the cache and the launch gaps of tensors as small as 59 MB.
+    cold = None
+    if not args.no_graph:
+        n_h = BT * FFN
+        srcs = [t["h"], out["dh"], out["y_up"].view(-1)[:n_h].view(BT, FFN)]
+        q_srcs = [q["h"], q["dy_up"].view(-1)[:n_h].view(BT, FFN), q["dy_up"].view(-1)[n_h:].view(BT, FFN)]
+        am3 = [torch.zeros(1, device=dev) for _ in srcs]
+        for a, s_ in zip(am3, srcs):
+            K.abs_max(a, s_)
+
+        def cold_run(fn, nbytes, warm=5, timed=20):
+            for i in range(warm):
+                fn(i % 3)
+            evs = []
+            for i in range(timed):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                fn((warm + i) % 3)
+                e1.record()
+                evs.append((e0, e1))
+            torch.cuda.synchronize()
+            us = sorted(e0.elapsed_time(e1) * 1e3 for e0, e1 in evs)
+            med = 0.5 * (us[len(us) // 2] + us[(len(us) - 1) // 2])
+            return {"median_us": med, "min_us": us[0], "GBps": nbytes / med / 1e3, "frac_hbm": nbytes / med / 1e3 / HBM_PEAK_GBS,
+                    "best_GBps": nbytes / us[0] / 1e3}
+
+        def pair(i):
+            K.abs_max(am3[i], srcs[i])
+            K.quantize_with_abs_max(q["h"], stats["h"][1:2], srcs[i], am3[i])
+
+        cold = {
+            "what": "20 timed launches after 5 warm-ups, events around each launch, rotating through three 8192 x 18944 "
+                    "tensors (930 MB of sources)",
+            "abs_max (2 B/el)": cold_run(lambda i: K.abs_max(am3[i], srcs[i]), 2 * n_h),
+            "quantize (3 B/el)": cold_run(lambda i: K.quantize_with_abs_max(q["h"], stats["h"][1:2], srcs[i], am3[i]), 3 * n_h),
+            "abs_max + quantize of one tensor (5 B/el)": cold_run(pair, 5 * n_h),
+            "quantize_and_transpose (3 B/el)": cold_run(
+                lambda i: K.quantize_and_transpose_with_abs_max(q["h_t"], None, srcs[i], am3[i]), 3 * n_h),
+            "transpose (2 B/el)": cold_run(lambda i: K.transpose(q["h_t"], q_srcs[i]), 2 * n_h),
+        }
+        K.abs_max(stats["h"][0:1], t["h"])   # restore what the step left in the shared slots
+        K.quantize_with_abs_max(q["h"], stats["h"][1:2], t["h"], stats["h"][0:1])
+        qtr(q["h_t"], "h")
     if args.calibrate_copy:
         src = torch.randint(0, 255, (1 << 30,), dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
@@ -346,7 +393,7 @@ def main():
                      "mean_launch_ms": ks["gemm"]["mean_ms"], "launches": ks["gemm"]["launches"]},
         "quantize": {"bound": "hbm", "kernels": "abs_max + quantize_with_abs_max (5 bytes/element)",
                      "achieved": aq_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": aq_gbs / HBM_PEAK_GBS,
-                     "per_kernel": per_kernel},
+                     "per_kernel": per_kernel, "cold_large_tensor": cold},
         "hip_graph_replay": None if graph_ms is None else {"ms_per_step": graph_ms,
                                                            "value": gemm_flop / (graph_ms * 1e-3) / 1e12},
         "fused_quantize_transpose_step": None if fused_ms is None else {
