@@ -319,23 +319,32 @@ def main():
             return {"median_us": med, "min_us": us[0], "GBps": nbytes / med / 1e3, "frac_hbm": nbytes / med / 1e3 / HBM_PEAK_GBS,
                     "best_GBps": nbytes / us[0] / 1e3}
 
+        q_dsts = q_srcs                                   # three distinct 155 MB outputs as well
+        qt_dsts = [q["h_t"], q["dy_up_t"].view(-1)[:n_h].view(FFN, BT), q["dy_up_t"].view(-1)[n_h:].view(FFN, BT)]
+
         def pair(i):
             K.abs_max(am3[i], srcs[i])
-            K.quantize_with_abs_max(q["h"], stats["h"][1:2], srcs[i], am3[i])
+            K.quantize_with_abs_max(q_dsts[i], stats["h"][1:2], srcs[i], am3[i])
 
         cold = {
             "what": "20 timed launches after 5 warm-ups, events around each launch, rotating through three 8192 x 18944 "
-                    "tensors (930 MB of sources)",
+                    "source tensors (930 MB) and three destinations, so that no launch finds its data in a cache",
             "abs_max (2 B/el)": cold_run(lambda i: K.abs_max(am3[i], srcs[i]), 2 * n_h),
-            "quantize (3 B/el)": cold_run(lambda i: K.quantize_with_abs_max(q["h"], stats["h"][1:2], srcs[i], am3[i]), 3 * n_h),
+            "quantize (3 B/el)": cold_run(lambda i: K.quantize_with_abs_max(q_dsts[i], stats["h"][1:2], srcs[i], am3[i]), 3 * n_h),
             "abs_max + quantize of one tensor (5 B/el)": cold_run(pair, 5 * n_h),
             "quantize_and_transpose (3 B/el)": cold_run(
-                lambda i: K.quantize_and_transpose_with_abs_max(q["h_t"], None, srcs[i], am3[i]), 3 * n_h),
-            "transpose (2 B/el)": cold_run(lambda i: K.transpose(q["h_t"], q_srcs[i]), 2 * n_h),
+                lambda i: K.quantize_and_transpose_with_abs_max(qt_dsts[i], None, srcs[i], am3[i]), 3 * n_h),
+            "transpose (2 B/el)": cold_run(lambda i: K.transpose(qt_dsts[i], q_srcs[(i + 1) % 3]), 2 * n_h),
+            # what a plain streaming copy sustains under the same protocol: the practical ceiling of a
+            # read + write stream on this chip, for reading the fractions above
+            "plain copy kernel, same protocol (2 B/el)": cold_run(lambda i: capi.check(capi.lib.llmq_debug_copy_u8(
+                qt_dsts[i].data_ptr(), q_srcs[(i + 1) % 3].data_ptr(), n_h, torch.cuda.current_stream().cuda_stream)), 2 * n_h),
         }
-        K.abs_max(stats["h"][0:1], t["h"])   # restore what the step left in the shared slots
+        K.abs_max(stats["h"][0:1], t["h"])   # restore what the step left in the buffers used above
         K.quantize_with_abs_max(q["h"], stats["h"][1:2], t["h"], stats["h"][0:1])
         qtr(q["h_t"], "h")
+        K.quantize_with_abs_max(q["dy_up"], stats["dy_up"][1:2], t["dy_up"], stats["dy_up"][0:1])
+        tr(q["dy_up_t"], q["dy_up"])
     if args.calibrate_copy:
         src = torch.randint(0, 255, (1 << 30,), dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)

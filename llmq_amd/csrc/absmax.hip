@@ -23,11 +23,15 @@ namespace llmq {
 constexpr int kAbsmaxThreads = 1024;
 
 // Every lane keeps UNROLL independent 128-bit loads in flight; out-of-range slots of the last trip are
-// predicated to zero instead of falling into a serial tail loop.  The loads are ordinary (cached) ones on
-// purpose: the quantizer that follows re-reads the tensor, and what is still in the 256 MB last-level cache
-// it gets from there (measured on 136-310 MB tensors: with streaming loads here the abs-max alone is 6-10 %
-// faster, the abs-max + quantize pair 8-12 % slower).
-template <int UNROLL>
+// predicated to zero instead of falling into a serial tail loop.
+// STREAM selects the cache policy of the loads; the library uses ordinary (cached) loads for every size.  The
+// quantizer that follows re-reads the tensor, and what is still in the 256 MB last-level cache it gets from
+// there.  For tensors beyond the cache size streaming loads make this kernel 8-10 % faster on its own (its
+// allocating reads no longer push out earlier kernels' not yet written-back outputs), but those write-backs
+// then fall into the quantizer and the matmul that follow: the whole bench step was 0.8 % slower with
+// streaming loads above 224 MiB (alternating builds on one box: abs-max -4.3 us, quantize +2.9 us, matmul
+// +8 us per launch), and slower for every tensor that fits the cache (59 MB: abs-max + quantize 35 -> 38 us).
+template <int UNROLL, bool STREAM>
 __global__ __launch_bounds__(kAbsmaxThreads) void absmax_bf16_kernel(unsigned* __restrict__ result,
                                                           const uint4* __restrict__ in, int64_t nvec,
                                                           const uint16_t* __restrict__ tail, int ntail) {
@@ -39,7 +43,7 @@ __global__ __launch_bounds__(kAbsmaxThreads) void absmax_bf16_kernel(unsigned* _
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             const int64_t idx = i + u * stride;
-            v[u] = idx < nvec ? in[idx] : make_uint4(0, 0, 0, 0);
+            v[u] = idx < nvec ? (STREAM ? load_nt(in + idx) : in[idx]) : make_uint4(0, 0, 0, 0);
         }
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) acc = fold_vec(acc, v[u]);
@@ -74,6 +78,10 @@ __global__ __launch_bounds__(kAbsmaxThreads) void absmax_f32_kernel(unsigned* __
     block_min_to_atomic_max(result, acc, 0x7F800000u, 0);
 }
 
+// tensors above this many bytes would be read with streaming loads: none by default (see absmax_bf16_kernel;
+// llmq_debug_set_absmax_stream_bytes is the hook the measurement above was made with)
+static int64_t g_absmax_stream_bytes = INT64_MAX;
+
 template <typename Kernel, typename Elem>
 static int launch_absmax(Kernel kernel, float* out, const Elem* in, int64_t n, int elems_per_vec, int unroll,
                          hipStream_t stream) {
@@ -102,8 +110,12 @@ static int launch_absmax(Kernel kernel, float* out, const Elem* in, int64_t n, i
 }  // namespace llmq
 
 extern "C" int llmq_abs_max_bf16(float* out, const uint16_t* in, int64_t n, void* stream) {
-    return llmq::launch_absmax(llmq::absmax_bf16_kernel<8>, out, in, n, 8, 8, static_cast<hipStream_t>(stream));
+    if (2 * n > llmq::g_absmax_stream_bytes)
+        return llmq::launch_absmax(llmq::absmax_bf16_kernel<8, true>, out, in, n, 8, 8, static_cast<hipStream_t>(stream));
+    return llmq::launch_absmax(llmq::absmax_bf16_kernel<8, false>, out, in, n, 8, 8, static_cast<hipStream_t>(stream));
 }
+
+extern "C" void llmq_debug_set_absmax_stream_bytes(int64_t bytes) { llmq::g_absmax_stream_bytes = bytes; }
 
 extern "C" int llmq_abs_max_f32(float* out, const float* in, int64_t n, void* stream) {
     return llmq::launch_absmax(llmq::absmax_f32_kernel<8>, out, reinterpret_cast<const uint32_t*>(in), n, 4, 8,
