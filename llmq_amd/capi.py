@@ -67,6 +67,8 @@ lib.llmq_debug_set_gemm_variant.argtypes = [_int, _int]
 lib.llmq_debug_set_gemm_variant.restype = None
 lib.llmq_debug_set_absmax_stream_bytes.argtypes = [_i64]
 lib.llmq_debug_set_absmax_stream_bytes.restype = None
+lib.llmq_debug_set_quantize_unroll.argtypes = [_int]
+lib.llmq_debug_set_quantize_unroll.restype = None
 lib.llmq_debug_set_gemm_persist.argtypes = [_int]
 lib.llmq_debug_set_gemm_persist.restype = None
 lib.llmq_debug_copy_u8.argtypes = [_vp, _vp, _i64, _vp]

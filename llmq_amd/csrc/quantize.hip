@@ -20,6 +20,12 @@
 
 namespace llmq {
 
+// One trip per lane: UNROLL independent 16-byte loads, then UNROLL 8-byte stores.  A workgroup owns a contiguous
+// piece of 256 * UNROLL vectors (lane t takes vectors t, t + 256, ...).  Many small workgroups with two loads
+// per lane sustain the most HBM bandwidth on tensors no cache holds (310 MB source, rotating buffers:
+// UNROLL 8 / 4 / 2 = 5.44 / 5.69 / 5.89 TB/s; a plain copy kernel gets 5.7), hence UNROLL = 2 below.
+static int g_quantize_unroll = 2;  // 2, 4 or 8; llmq_debug_set_quantize_unroll is the hook the comparison was made with
+
 template <int FMT, int UNROLL>
 __global__ __launch_bounds__(256) void quantize_kernel(uint2* __restrict__ out, float* __restrict__ scale_ptr,
                                                        const uint4* __restrict__ in,
@@ -28,20 +34,18 @@ __global__ __launch_bounds__(256) void quantize_kernel(uint2* __restrict__ out, 
                                                        uint8_t* __restrict__ tail_out, int ntail) {
     const float s = quant_scale(*absmax);
     const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     if (tid == 0 && scale_ptr) *scale_ptr = __fdiv_rn(1.f, s);
-    for (int64_t i = tid; i < nvec; i += UNROLL * stride) {
-        uint4 v[UNROLL];
+    const int64_t first = (int64_t)blockIdx.x * (256 * UNROLL) + threadIdx.x;
+    uint4 v[UNROLL];
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            const int64_t idx = i + u * stride;
-            v[u] = idx < nvec ? load_nt(&in[idx]) : make_uint4(0, 0, 0, 0);
-        }
+    for (int u = 0; u < UNROLL; ++u) {
+        const int64_t idx = first + u * 256;
+        v[u] = idx < nvec ? load_nt(&in[idx]) : make_uint4(0, 0, 0, 0);
+    }
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            const int64_t idx = i + u * stride;
-            if (idx < nvec) out[idx] = encode8<FMT>(v[u], s);
-        }
+    for (int u = 0; u < UNROLL; ++u) {
+        const int64_t idx = first + u * 256;
+        if (idx < nvec) out[idx] = encode8<FMT>(v[u], s);
     }
     if (tid < ntail) {
         float y = s * __uint_as_float((uint32_t)tail_in[tid] << 16);
@@ -175,17 +179,21 @@ static int launch_quantize(uint8_t* out, float* scale_ptr, const uint16_t* in, c
     LLMQ_REQUIRE(absmax != nullptr, "quantize_with_abs_max: abs_max pointer is null");
     LLMQ_REQUIRE(n == 0 || (out != nullptr && in != nullptr), "quantize_with_abs_max: null tensor pointer");
     LLMQ_REQUIRE(aligned16(in) && aligned16(out), "quantize_with_abs_max: tensors must be 16-byte aligned");
-    constexpr int UNROLL = 8;
     const int64_t nvec = n / 8;
     const int ntail = (int)(n - nvec * 8);
-    // One trip per lane (UNROLL independent 16-byte loads, then UNROLL 8-byte stores): many short
-    // workgroups sustain more HBM bandwidth here than a persistent grid-stride loop.
-    int64_t blocks = (nvec + 256 * UNROLL - 1) / (256 * UNROLL);
-    if (blocks > 0x7FFFFFFF) blocks = 0x7FFFFFFF;
-    if (blocks < 1) blocks = 1;  // still writes the scale for n == 0
-    hipLaunchKernelGGL((quantize_kernel<FMT, UNROLL>), dim3((unsigned)blocks), dim3(256), 0, stream,
-                       reinterpret_cast<uint2*>(out), scale_ptr, reinterpret_cast<const uint4*>(in), absmax, nvec,
-                       in + nvec * 8, out + nvec * 8, ntail);
+    auto launch = [&](auto kernel, int unroll) -> int {
+        int64_t blocks = (nvec + 256 * unroll - 1) / (256 * unroll);
+        LLMQ_REQUIRE(blocks <= 0x7FFFFFFF, "quantize_with_abs_max: %lld elements are too many", (long long)n);
+        if (blocks < 1) blocks = 1;  // still writes the scale for n == 0
+        hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), 0, stream, reinterpret_cast<uint2*>(out), scale_ptr,
+                           reinterpret_cast<const uint4*>(in), absmax, nvec, in + nvec * 8, out + nvec * 8, ntail);
+        return LLMQ_OK;
+    };
+    int rc;
+    if (g_quantize_unroll == 8) rc = launch(quantize_kernel<FMT, 8>, 8);
+    else if (g_quantize_unroll == 4) rc = launch(quantize_kernel<FMT, 4>, 4);
+    else rc = launch(quantize_kernel<FMT, 2>, 2);
+    if (rc != LLMQ_OK) return rc;
     LLMQ_HIP_TRY(hipGetLastError());
     return LLMQ_OK;
 }
@@ -234,6 +242,7 @@ extern "C" int llmq_quantize_e5m2_bf16(uint8_t* out, float* scale_or_null, const
     return llmq::launch_quantize<llmq::kE5M2>(out, scale_or_null, in, absmax, n, static_cast<hipStream_t>(stream));
 }
 
+extern "C" void llmq_debug_set_quantize_unroll(int v) { llmq::g_quantize_unroll = v; }
 extern "C" void llmq_debug_set_qt_order(int v) { llmq::g_qt_row_major_grid = v; }
 
 namespace llmq {
