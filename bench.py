@@ -264,7 +264,8 @@ def main():
         swiglu = {
             "what": "producers of the projections' inputs with the abs-max of their output computed on the way: "
                     "h = swiglu(y_up) [8192 x 18944], the same as e4m3 codes, its backward, the residual add + rmsnorm [8192 x 3584] "
-                    "and the rmsnorm backward, the AdamW step of a weight",
+                    "and the rmsnorm backward, the AdamW step of a weight; backward_bias on e4m3 gradients and the e5m2 "
+                    "gradient dtype (quantize, matmul)",
             "swiglu_forward+abs_max (6 B/el)": gbs(lambda: K.swiglu_forward(h3, y3, sw_am), 6 * n_act),
             "swiglu_forward_quant (5 B/el)": gbs(lambda: K.swiglu_forward_quant(hq3, sw_sc, y3, sw_am), 5 * n_act),
             "swiglu_backward+abs_max (10 B/el)": gbs(lambda: K.swiglu_backward(dy3, dh3, y3, sw_am), 10 * n_act),
@@ -288,6 +289,21 @@ def main():
         swiglu["adamw_update+abs_max, bf16 moments (14 B/param)"] = gbs(
             lambda: K.adamw_update(a_p, a_g, a_m, a_v, 1e-4, 0.9, 0.95, 2, 1e-8, 0.1, a_gs, None, sw_am, 7), 14 * UP * C)
         del a_m, a_v, a_p, a_g
+        # backward_bias on the quantized gradient of the attention's QKV projection (the 7B model's
+        # [8192 x 4608], e4m3 codes with two scales): the other consumer of the quantized gradient bytes
+        QKV = C + 2 * 512
+        bb_dout = q["dy_up"].view(-1)[:BT * QKV].view(1, BT, QKV)
+        bb_dbias = torch.zeros(QKV, dtype=torch.bfloat16, device=dev)
+        bb_scr = torch.empty(K.get_bias_backward_scratch_size(f8, QKV, BT) // 4, dtype=torch.float32, device=dev)
+        swiglu["backward_bias e4m3 [8192 x 4608] (1 B/el)"] = gbs(
+            lambda: K.backward_bias(bb_dbias, bb_dout, sw_sc, sw_sc, bb_scr), BT * QKV, iters=10)
+        # the e5m2 gradient dtype: quantize to e5m2 and the e4m3 x e5m2 matmul (gate+up dgrad shape)
+        g5 = torch.empty((BT, UP), dtype=torch.float8_e5m2, device=dev)
+        swiglu["quantize to e5m2 [8192 x 37888] (3 B/el)"] = gbs(
+            lambda: K.quantize_with_abs_max(g5, sw_sc, t["dy_up"], stats["dy_up"][0:1]), 3 * BT * UP)
+        e5 = gbs(lambda: K.matmul(out["dx"], q["w_up_t"], g5, None, stats["w_up"][1:2], sw_sc, C, BT, UP, workspace=ws), 1)
+        swiglu["matmul e4m3 x e5m2, gate_up dgrad shape"] = {"TFLOPs": 2.0 * C * BT * UP / e5["mean_us"] / 1e6, "mean_us": e5["mean_us"]}
+        del g5
         swiglu["fused_residual_rmsnorm_forward+abs_max (8 B/el)"] = gbs(
             lambda: K.fused_residual_rmsnorm_forward(r_out, r_norm, r_rms, r_in, r_att, r_w, sw_am, 1e-6), 8 * BT * C, iters=10)
     # The HBM-bound kernels on their own, cold: 5 warm-up and 20 timed launches each, one pair of events per
