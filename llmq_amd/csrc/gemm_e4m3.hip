@@ -78,15 +78,17 @@ __device__ __forceinline__ void xcd_tile_range(int total, int xcd, int& first, i
 }
 
 // Logical tile number -> tile origin: groups of `group` tile-rows, column-major inside a group.
+// Tiles are 256 rows (n) by BM columns (m).
+template <int BM = 256>
 __device__ __forceinline__ void decode_tile256(const GemmArgs& g, int logical, int& n_blk, int& m_blk) {
-    const int tiles_n = g.N / 256, tiles_m = g.M / 256;
+    const int tiles_n = g.N / 256, tiles_m = g.M / BM;
     const int per_group = g.group * tiles_m;
     const int gid = logical / per_group;
     const int first_n = gid * g.group;
     const int gsz = (tiles_n - first_n) < g.group ? (tiles_n - first_n) : g.group;
     const int in_group = logical % per_group;
     n_blk = (first_n + in_group % gsz) * 256;
-    m_blk = (in_group / gsz) * 256;
+    m_blk = (in_group / gsz) * BM;
 }
 
 #define LLMQ_GLOBAL __attribute__((address_space(1)))
@@ -555,11 +557,20 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs g, int spli
 // The workgroup is persistent (one per compute unit, walking its XCD's tile list) and the stream of
 // K-steps and copies runs across tile boundaries.  Needs K to be a multiple of 256: the LDS stage and the
 // fb half of a step are then compile-time functions of the step's parity.
-template <typename OutT, int B_FMT, bool SEG>
+//
+// NJ < 8 narrows the tile along m to 2 * 16 * NJ columns (NJ second-operand fragments per wave instead of 8): a
+// shape whose 256-wide tiles fill the last round of the chip badly can have a tile count that divides evenly
+// (M = 3584: 14 x 32 = 448 tiles of 256 = 1.75 rounds of 256 compute units, but 16 x 32 = 512 tiles of 224 = 2
+// full rounds of 7/8 the work each).  Everything below is written for NJ fragments; only NJ = 8 and 7 are
+// instantiated, the narrow one for bf16 output without bias or accumulation.
+template <typename OutT, int B_FMT, bool SEG, int NJ = 8>
 __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     constexpr int BLK = 256, T = 256, WT = 128, NF = 8;
+    constexpr int WTM = 16 * NJ, BLKM = 2 * WTM;  // columns (first-operand rows) per wave and per tile
     constexpr int P_BYTES = BLK * kBK, STAGE = 2 * P_BYTES;
-    constexpr int ITERS = BLK * 8 / T;  // 16-byte copies per lane, operand and K-step
+    constexpr int ITERS = BLK * 8 / T;    // 16-byte copies per lane and K-step, b rows
+    constexpr int ITERS_Q = BLKM * 8 / T;  // the same for the a rows (= NJ)
+    static_assert(NJ == 8 || (NJ == 7 && !SEG && std::is_same_v<OutT, uint16_t>), "unsupported tile width");
     typedef float v4f __attribute__((ext_vector_type(4)));
 
     __shared__ __attribute__((aligned(16))) uint8_t lds[2 * STAGE];
@@ -575,7 +586,7 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     // XCD's last, partial round are left to a second launch of this kernel (SEG) that cuts each of them
     // into S segments of K (slot s: tile s / S, segment s % S) and writes raw accumulators as a 256 x 256
     // fp32 tile to g.partial for the reduction kernel below: the round then costs 1 / S of a tile.
-    const int total = (g.N / BLK) * (g.M / BLK);
+    const int total = (g.N / BLK) * (g.M / BLKM);
     const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
     int xcd_first, xcd_count;
     xcd_tile_range(total, xcd, xcd_first, xcd_count);
@@ -592,15 +603,21 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         if (g.rem_split > 1) my_tiles = xcd_count / tile_stride;
     }
     if (my_tiles <= 0) return;  // uniform for the whole workgroup, before any barrier
-    auto decode = [&](int logical, int& n_blk, int& m_blk) { decode_tile256(g, logical, n_blk, m_blk); };
+    auto decode = [&](int logical, int& n_blk, int& m_blk) { decode_tile256<BLKM>(g, logical, n_blk, m_blk); };
 
     // copies: lane -> (row tid/8 of a 32-row slab, physical 16-byte chunk tid%8); every address is a
     // wave-uniform base plus a 32-bit lane offset
     const int ld_row = tid / 8;
     const int ld_chunk = (tid & 7) ^ ((ld_row >> 1) & 7);
     const uint32_t p_lane = (uint32_t)ld_row * (uint32_t)g.K + (uint32_t)ld_chunk * 16u;
-    // LDS row rho of the a-tile holds global row (rho/128)*128 + 8*(rho%16) + (rho%128)/16
-    const uint32_t q_lane = (uint32_t)(8 * (ld_row % 16) + ld_row / 16) * (uint32_t)g.K + (uint32_t)ld_chunk * 16u;
+    // LDS row rho of the a-tile is row rho % 16 of fragment f = rho / 16 (wave half f / NJ, fragment f % NJ of it)
+    // and holds global row frag_row(f) + NJ * (rho % 16), so that a lane of the epilogue owns NJ adjacent columns.
+    // A copy slab is two fragments, f = 2 it and 2 it + 1; the second starts one global row after the first,
+    // except where it opens the second wave half (odd NJ only: slab (NJ - 1) / 2), hence a second lane offset.
+    auto frag_row = [](int f) { return WTM * (f / NJ) + f % NJ; };
+    const uint32_t q_lane = (uint32_t)(NJ * (ld_row % 16) + ld_row / 16) * (uint32_t)g.K + (uint32_t)ld_chunk * 16u;
+    const uint32_t q_lane_x =
+        (uint32_t)(NJ * (ld_row % 16) + (ld_row / 16) * (WTM - (NJ - 1))) * (uint32_t)g.K + (uint32_t)ld_chunk * 16u;
     // The copy stream runs two K-steps ahead of the matrix instructions and has its own position: tile
     // number, K offset and the operand bases of that tile already advanced to the K offset.
     int copy_k0 = 0, copy_tile = 0;
@@ -637,11 +654,11 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
             dst = lds_wave + stage_ofs + c * T * 16;
             lane_ofs = p_lane;
         } else {
-            // slab `it` covers LDS rows 32 it .. 32 it + 31 = global rows (it/4)*128 + 2*(it%4) + (those of slab 0)
+            // slab `it` covers LDS rows 32 it .. 32 it + 31: fragments 2 it and 2 it + 1
             const int it = c - ITERS;
-            src = q_cur + (int64_t)((it / 4) * 128 + 2 * (it % 4)) * g.K;
+            src = q_cur + (int64_t)frag_row(2 * it) * g.K;
             dst = lds_wave + stage_ofs + P_BYTES + it * T * 16;
-            lane_ofs = q_lane;
+            lane_ofs = (NJ % 2 == 1 && it == (NJ - 1) / 2) ? q_lane_x : q_lane;
         }
         asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                      :
@@ -652,7 +669,7 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     const int sw = (l16 >> 1) & 7;
     const int c0 = ((2 * kg) ^ sw) * 16, c1 = ((2 * kg + 1) ^ sw) * 16;
     const int p_frag = (wn * WT + l16) * kBK;
-    const int q_frag = P_BYTES + (wm * WT + l16) * kBK;
+    const int q_frag = P_BYTES + (wm * WTM + l16) * kBK;
     auto read_frag = [&](const uint8_t* row) -> v8i {
         const v4i lo = *reinterpret_cast<const v4i*>(row + c0);
         const v4i hi = *reinterpret_cast<const v4i*>(row + c1);
@@ -678,22 +695,23 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
             asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0 cbsz:1" : "=a"(c) : "v"(a), "v"(b) : "memory");
     };
 
-    v4f acc[NF][NF];  // written by the first K-step of every tile
-    v8i fa[4], fb[2][NF];
+    v4f acc[NF][NJ];  // written by the first K-step of every tile
+    v8i fa[4], fb[2][NJ];
 
     // prologue of the stream: the first two K-steps of the first tile
+    constexpr int COPIES = ITERS + ITERS_Q;  // per K-step and lane
 #pragma unroll
-    for (int c = 0; c < 2 * ITERS; ++c) issue_load(c, 0);
+    for (int c = 0; c < COPIES; ++c) issue_load(c, 0);
     advance_copy();
 #pragma unroll
-    for (int c = 0; c < 2 * ITERS; ++c) issue_load(c, STAGE);
+    for (int c = 0; c < COPIES; ++c) issue_load(c, STAGE);
     advance_copy();
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * ITERS) : "memory");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(COPIES) : "memory");
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < 4; ++i) fa[i] = read_frag(lds + p_frag + i * 16 * kBK);
 #pragma unroll
-    for (int j = 0; j < NF; ++j) fb[0][j] = read_frag(lds + q_frag + j * 16 * kBK);
+    for (int j = 0; j < NJ; ++j) fb[0][j] = read_frag(lds + q_frag + j * 16 * kBK);
 
     // One K-step of parity PAR (LDS stage PAR, fb half PAR): rows i = 0..7 of first-operand fragments
     // against all 8 second-operand fragments.  fa rotates through 4 slots (fragment i+4 is read once row i
@@ -710,13 +728,15 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
 #pragma unroll
         for (int i = 0; i < NF; ++i) {
 #pragma unroll
-            for (int j = 0; j < NF; ++j) {
+            for (int j = 0; j < NJ; ++j) {
                 if constexpr (FIRST) mfma_first(acc[i][j], fa[i % 4], fb[PAR][j]);
                 else mfma(acc[i][j], fa[i % 4], fb[PAR][j]);
-                if ((i == 5 || i == 6) && j >= 1 && j <= 6) issue_load(4 + 6 * (i - 5) + (j - 1), PAR * STAGE);
+                if ((i == 5 || i == 6) && j >= 1 && j <= 6) {
+                    if (4 + 6 * (i - 5) + (j - 1) < COPIES) issue_load(4 + 6 * (i - 5) + (j - 1), PAR * STAGE);
+                }
                 if (i >= 5 && (j == 2 || j == 5)) {  // rows 5..7: fragments 2..7 of the next step
                     const int f = 2 * (i - 4) + (j == 5 ? 1 : 0);
-                    fb[1 - PAR][f] = read_frag(nxt + q_frag + f * 16 * kBK);
+                    if (f < NJ) fb[1 - PAR][f] = read_frag(nxt + q_frag + f * 16 * kBK);
                 }
             }
             if (i == 4) {
@@ -728,7 +748,7 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
                     // previous tile's epilogue) sit that epilogue's stores; the counter retires in issue
                     // order, so allowing as many outstanding operations as there were stores is enough.
                     if (pending_stores) {
-                        if constexpr (sizeof(OutT) == 2) asm volatile("s_waitcnt vmcnt(32) lgkmcnt(0)" ::: "memory");
+                        if constexpr (sizeof(OutT) == 2 && NJ == 8) asm volatile("s_waitcnt vmcnt(32) lgkmcnt(0)" ::: "memory");
                         else asm volatile("s_waitcnt vmcnt(63) lgkmcnt(0)" ::: "memory");
                     } else {
                         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
@@ -767,7 +787,8 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 
         // Epilogue.  acc[i][j][r] is c row 16 i + 4 kg + r of the wave tile and, thanks to the a-tile row
-        // permutation, column 8 l16 + j: a lane owns 8 adjacent columns of each of its 32 rows.  The bf16 stores
+        // permutation, column NJ l16 + j: a lane owns NJ adjacent columns of each of its 32 rows (8: one 16-byte
+        // store per row; 7: 14 bytes at a 2-byte aligned address, stored as 12 + 2).  The bf16 stores
         // are non-temporal: the output (up to 620 MB) is not read by this kernel again and would otherwise push
         // the operands, which the other XCDs still fetch, out of the last-level cache (measured on one box,
         // alternating builds: -8 % on the gate+up forward, -3.7 % over the six bench shapes).
@@ -787,14 +808,38 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         }
         const int e_lane = opaque(threadIdx.x) % 64;
         const int el16 = e_lane % 16, ekg = e_lane / 16;
-        const int m_lane = m_blk + wm * WT + 8 * el16;
+        const int m_lane = m_blk + wm * WTM + NJ * el16;
         const uint32_t lane_bytes = ((uint32_t)(4 * ekg) * (uint32_t)ldc + (uint32_t)m_lane) * (uint32_t)sizeof(OutT);
         const int row0 = n_blk + wn * WT;
         auto rows = [&](auto bias_tag, auto acc_tag) {
             constexpr bool BIAS = decltype(bias_tag)::value;
             constexpr bool ACC = decltype(acc_tag)::value;
             typedef float v4fl __attribute__((ext_vector_type(4)));
+            if constexpr (NJ == 7) {
+                static_assert(NJ != 7 || (!BIAS && !ACC), "the narrow tile has the plain epilogue only");
+                typedef int v3i_u __attribute__((ext_vector_type(3), aligned(2)));
+                typedef uint16_t u16_u __attribute__((aligned(2)));
+#pragma unroll
+                for (int i = 0; i < NF; ++i) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        LLMQ_GLOBAL char* dst =
+                            scalar_ptr((LLMQ_GLOBAL char*)(c + (int64_t)(row0 + 16 * i + r) * ldc)) + lane_bytes;
+                        v3i_u packed;
+#pragma unroll
+                        for (int j = 0; j < 3; ++j) {
+                            const f32x2_t pr = {acc[i][2 * j][r] * scale, acc[i][2 * j + 1][r] * scale};
+                            packed[j] = __builtin_bit_cast(int, __builtin_convertvector(pr, bf16x2_t));
+                        }
+                        const f32x2_t last = {acc[i][6][r] * scale, 0.f};
+                        const uint32_t tail = __builtin_bit_cast(uint32_t, __builtin_convertvector(last, bf16x2_t));
+                        *(LLMQ_GLOBAL v3i_u*)dst = packed;
+                        *(LLMQ_GLOBAL u16_u*)(dst + 12) = (uint16_t)tail;
+                    }
+                }
+            } else {
             float bias_v[8];
+            static_assert(NJ == 7 || NJ == 8, "epilogue written for 7 or 8 columns per lane");
             if constexpr (BIAS) {
 #pragma unroll
                 for (int j = 0; j < 8; ++j) bias_v[j] = load_bias(g.bias, g.bias_is_bf16, m_lane + j);
@@ -851,11 +896,13 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
                     }
                 }
             }
+            }  // NJ == 8
         };
         constexpr std::true_type yes{};
         constexpr std::false_type no{};
-        if constexpr (SEG) {
+        if constexpr (SEG || NJ != 8) {
             rows(no, no);
+            pending_stores = !SEG;
         } else if (g.accumulate) {
             if (g.bias) rows(yes, yes);
             else rows(no, yes);
@@ -998,21 +1045,54 @@ static W4Plan plan_w4(int tiles256, int cus, int M, int N, int K, int forced_spl
 template <typename OutT, int B_FMT>
 static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     LLMQ_REQUIRE(g.M > 0 && g.N > 0 && g.K > 0, "matmul: M, N, K must be positive (got %d, %d, %d)", g.M, g.N, g.K);
-    LLMQ_REQUIRE(g.M % 128 == 0 && g.N % 128 == 0 && g.K % 128 == 0,
+    const int cus = cu_count();
+    // The four-wave kernel with 256 x 224 tiles: bf16 output without bias or accumulation, e4m3 b operand.
+    const bool narrow_ok = std::is_same_v<OutT, uint16_t> && B_FMT == 0 && !g.bias && !g.accumulate && g.N % 256 == 0 &&
+                           g.M % 224 == 0 && g.K % (2 * kBK) == 0 && cus % 8 == 0;
+    LLMQ_REQUIRE((g.M % 128 == 0 || narrow_ok) && g.N % 128 == 0 && g.K % 128 == 0,
                  "matmul: M, N, K must be divisible by 128 (got %d, %d, %d)", g.M, g.N, g.K);
     LLMQ_REQUIRE(g.a && g.b && g.c, "matmul: null operand pointer");
     LLMQ_REQUIRE(aligned16(g.a) && aligned16(g.b) && aligned16(g.c) && aligned16(g.bias) && aligned16(workspace),
                  "matmul: all pointers must be 16-byte aligned");
     LLMQ_REQUIRE(workspace != nullptr || workspace_bytes == 0, "matmul: workspace size given without a workspace");
     g.group = 8;
-    const int cus = cu_count();
     int tile = g_gemm_tile;
-    LLMQ_REQUIRE(tile >= 0 && tile <= 3, "matmul: unknown tile selector %d", tile);
+    LLMQ_REQUIRE(tile >= 0 && tile <= 4, "matmul: unknown tile selector %d", tile);
     const bool fits256 = g.N % 256 == 0 && g.M % 256 == 0;
     LLMQ_REQUIRE((tile != 1 && tile != 3) || fits256, "matmul: the 256 x 256 tile needs M and N divisible by 256");
     const bool w4_ok = fits256 && g.K % (2 * kBK) == 0 && cus % 8 == 0;
     if (tile == 3) {
         LLMQ_REQUIRE(w4_ok, "matmul: the four-wave kernel needs K divisible by 256");
+    }
+    // The 256 x 224 tiles are taken when their whole rounds of 7/8-sized tiles beat the rounds of full tiles by
+    // a margin, e.g. M = 3584, N = 8192: 512 tiles in 2 rounds instead of 448 in 1.75, on paper 12.5 % less
+    // time.  Measured (alternating builds on one box): K = 18944 371 -> 357 us, K = 37888 860 -> 820 us, i.e.
+    // 4-5 %: a narrow tile does 7/8 of the matrix work per barrier, copy and fragment-read overhead of a
+    // K-step, and the 192 tiles of a three-quarter round run faster than those of a full one.  Hence the 8 %
+    // the comparison below asks for.  The narrow tiles also serve an M that only 224 divides.
+    if (tile == 4) {
+        LLMQ_REQUIRE(narrow_ok, "matmul: the 256 x 224 tile needs bf16 output without bias or accumulation, N %% 256 == 0, "
+                                "M %% 224 == 0 and K %% 256 == 0");
+    }
+    bool narrow = tile == 4 || g.M % 128 != 0;
+    if (tile == 0 && narrow_ok && w4_ok && g_gemm_splits == 0) {
+        const int64_t t256 = (int64_t)(g.N / 256) * (g.M / 256), t224 = (int64_t)(g.N / 256) * (g.M / 224);
+        const int64_t r256 = (t256 + cus - 1) / cus, r224 = (t224 + cus - 1) / cus;
+        // only where the full tiles' last round would not be cut into K segments anyway (a remainder of 1-2
+        // tiles per XCD), and never for less than a round of tiles
+        const int64_t rem256 = t256 % cus;
+        narrow = t256 >= cus && (rem256 == 0 || rem256 > cus / 8) && (double)r224 * 7.0 * 1.08 < (double)r256 * 8.0;
+    }
+    if constexpr (std::is_same_v<OutT, uint16_t> && B_FMT == 0) {
+        if (narrow) {
+            const int t224 = (g.N / 256) * (g.M / 224);
+            g.rem_split = 1;
+            g.part_per_xcd = 0;
+            const int grid = t224 < cus ? (t224 + 7) / 8 * 8 : cus;
+            hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, 0, false, 7>), dim3((unsigned)grid), dim3(256), 0, stream, g);
+            LLMQ_HIP_TRY(hipGetLastError());
+            return LLMQ_OK;
+        }
     }
     if (tile == 0) {
         // Rounds of workgroups the chip needs: one 256 x 256 tile per compute unit and round (four units

@@ -294,6 +294,52 @@ def test_gemm_random_codes_within_tolerance(K, O, variant, out_f32):
         set_variant((0, 0))
 
 
+@pytest.mark.parametrize("forced", [True, False])
+@pytest.mark.parametrize("mnk", [(224, 256, 256), (448, 512, 512), (3584, 8192, 256), (3584, 8192, 512), (1792, 8448, 768),
+                                 (7168, 4352, 256)])
+def test_gemm_narrow_tile(K, O, mnk, forced):
+    """The four-wave kernel with 256 x 224 tiles (tile selector 4, and whatever the automatic choice takes for
+    these shapes): less than one round of tiles, exactly two rounds, uneven persistent walks; integer operands
+    -> bit exact against the oracle; random codes within the GEMM tolerance; bias / accumulate / fp32 output
+    are refused by the forced selector and served by the other kernels automatically."""
+    M, N, Kd = mnk
+    a, _ = O.fill_int_e4m3(M * Kd, 777, 0)
+    b, _ = O.fill_int_e4m3(N * Kd, 777, 1)
+    a, b = a.reshape(M, Kd), b.reshape(N, Kd)
+    s = float(np.sqrt(np.float32(4.0 / Kd)))
+    mt = M % 64 == 0          # the threaded oracle works on 64-column blocks
+    set_variant((4, 0) if forced else (0, 0))
+    try:
+        want = O.gemm_tn(a, b, sa=s, sb=s, mt=mt)
+        got = run_gemm(K, a, b, M, N, Kd, s, s)
+        assert np.array_equal(host_bits(got), want)
+        got = run_gemm(K, a, b, M, N, Kd, None, None)
+        assert np.array_equal(host_bits(got), O.gemm_tn(a, b, mt=mt))
+        if M * N <= 3584 * 8192 and Kd <= 512:
+            rng = np.random.default_rng(M + Kd)
+            ar = rng.integers(0, 256, (M, Kd)).astype(np.uint8)
+            br = rng.integers(0, 256, (N, Kd)).astype(np.uint8)
+            ar[(ar & 0x7F) == 0x7F] ^= 1
+            br[(br & 0x7F) == 0x7F] ^= 1
+            rows = (0, N) if N <= 512 else (N - 300, N)
+            exact, sumabs = O.gemm_exact(ar, br, rows=rows)
+            g32 = run_gemm(K, ar, br, M, N, Kd, 0.37, 1.0 / 448).float().cpu().numpy()
+            scale = np.float32(np.float32(0.37) * np.float32(1.0 / 448))
+            gemm_check(g32[rows[0]:rows[1]], exact[rows[0]:rows[1]], sumabs[rows[0]:rows[1]], scale, True)
+        _, biasv = O.fill_int_e4m3(M, 777, 2)
+        bias = O.f32_to_bf16(biasv.astype(np.float32))
+        if forced:
+            with pytest.raises(ValueError, match="256 x 224|divisible by 128"):
+                run_gemm(K, a, b, M, N, Kd, s, s, bias)
+            with pytest.raises(ValueError, match="256 x 224|divisible by 128"):
+                run_gemm(K, a, b, M, N, Kd, s, s, out_f32=True)
+        elif M % 128 == 0:
+            got = run_gemm(K, a, b, M, N, Kd, s, s, bias)
+            assert np.array_equal(host_bits(got), O.gemm_tn(a, b, sa=s, sb=s, bias=bias, mt=True))
+    finally:
+        set_variant((0, 0))
+
+
 @pytest.mark.parametrize("variant", [(1, 1, 1), (3, 1), (3, 2), (3, 3), (3, 4)])
 @pytest.mark.parametrize("mnk", [(4352, 4352, 384), (4608, 4096, 256), (8192, 4864, 512), (4352, 4352, 1024),
                                  (4352, 4096, 1024), (4352, 4352, 1536)])
