@@ -105,8 +105,8 @@ int llmq_transpose_u8(uint8_t* dst, const uint8_t* src, int rows, int cols, void
  *     c[n,m] = round( (sum_k b[n,k]*a[m,k]) * (sa*sb) + bias[m] + (accumulate ? c[n,m] : 0) )
  * fp32 accumulation, fp32 epilogue, one rounding to the output type.  sa / sb are device fp32
  * scalars or NULL (= 1).  bias is bf16[M] or NULL.  M, N, K must be multiples of 128 (the
- * precondition of the reference's hand-written kernel, src/kernels/gemm_mma.cu:261-263); without bias
- * and accumulation an M that is a multiple of 224 is served as well, given N and K multiples of 256.
+ * precondition of the reference's hand-written kernel, src/kernels/gemm_mma.cu:261-263); without
+ * accumulation an M that is a multiple of 224 or 192 is served as well, given N and K multiples of 256.
  * Replaces: matmul(nv_bfloat16* c, const __nv_fp8_e4m3* a, const __nv_fp8_e4m3* b,
  *           const nv_bfloat16* bias, const float* scale_a, const float* scale_b, cublasLtHandle_t,
  *           std::byte* ws, size_t ws_size, int M, int N, int K, EMMTranspose::TN, bool accumulate,

@@ -561,8 +561,9 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs g, int spli
 // NJ < 8 narrows the tile along m to 2 * 16 * NJ columns (NJ second-operand fragments per wave instead of 8): a
 // shape whose 256-wide tiles fill the last round of the chip badly can have a tile count that divides evenly
 // (M = 3584: 14 x 32 = 448 tiles of 256 = 1.75 rounds of 256 compute units, but 16 x 32 = 512 tiles of 224 = 2
-// full rounds of 7/8 the work each).  Everything below is written for NJ fragments; only NJ = 8 and 7 are
-// instantiated, the narrow one for bf16 output without bias or accumulation.
+// full rounds of 7/8 the work each; M = 1536, N = 16384: 384 tiles of 256 = 1.5 rounds, 512 tiles of 192 = 2 full
+// rounds of 3/4 the work).  Everything below is written for NJ fragments; NJ = 8, 7 and 6 are instantiated, the
+// narrow ones for bf16 output without accumulation.
 template <typename OutT, int B_FMT, bool SEG, int NJ = 8>
 __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     constexpr int BLK = 256, T = 256, WT = 128, NF = 8;
@@ -570,7 +571,7 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     constexpr int P_BYTES = BLK * kBK, STAGE = 2 * P_BYTES;
     constexpr int ITERS = BLK * 8 / T;    // 16-byte copies per lane and K-step, b rows
     constexpr int ITERS_Q = BLKM * 8 / T;  // the same for the a rows (= NJ)
-    static_assert(NJ == 8 || (NJ == 7 && !SEG && std::is_same_v<OutT, uint16_t>), "unsupported tile width");
+    static_assert(NJ == 8 || ((NJ == 7 || NJ == 6) && !SEG && std::is_same_v<OutT, uint16_t>), "unsupported tile width");
     typedef float v4f __attribute__((ext_vector_type(4)));
 
     __shared__ __attribute__((aligned(16))) uint8_t lds[2 * STAGE];
@@ -731,8 +732,11 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
             for (int j = 0; j < NJ; ++j) {
                 if constexpr (FIRST) mfma_first(acc[i][j], fa[i % 4], fb[PAR][j]);
                 else mfma(acc[i][j], fa[i % 4], fb[PAR][j]);
-                if ((i == 5 || i == 6) && j >= 1 && j <= 6) {
-                    if (4 + 6 * (i - 5) + (j - 1) < COPIES) issue_load(4 + 6 * (i - 5) + (j - 1), PAR * STAGE);
+                // copies 4 .. COPIES - 1: after the middle matrix instructions of rows 5 and 6
+                constexpr int PER_ROW = NJ - 1 < 6 ? NJ - 1 : 6;
+                static_assert(4 + 2 * PER_ROW >= COPIES, "not every copy of a K-step has a place in the schedule");
+                if ((i == 5 || i == 6) && j >= 1 && j <= PER_ROW) {
+                    if (4 + PER_ROW * (i - 5) + (j - 1) < COPIES) issue_load(4 + PER_ROW * (i - 5) + (j - 1), PAR * STAGE);
                 }
                 if (i >= 5 && (j == 2 || j == 5)) {  // rows 5..7: fragments 2..7 of the next step
                     const int f = 2 * (i - 4) + (j == 5 ? 1 : 0);
@@ -748,7 +752,7 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
                     // previous tile's epilogue) sit that epilogue's stores; the counter retires in issue
                     // order, so allowing as many outstanding operations as there were stores is enough.
                     if (pending_stores) {
-                        if constexpr (sizeof(OutT) == 2 && NJ == 8) asm volatile("s_waitcnt vmcnt(32) lgkmcnt(0)" ::: "memory");
+                        if constexpr (sizeof(OutT) == 2 && NJ != 7) asm volatile("s_waitcnt vmcnt(32) lgkmcnt(0)" ::: "memory");
                         else asm volatile("s_waitcnt vmcnt(63) lgkmcnt(0)" ::: "memory");
                     } else {
                         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
@@ -788,7 +792,7 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
 
         // Epilogue.  acc[i][j][r] is c row 16 i + 4 kg + r of the wave tile and, thanks to the a-tile row
         // permutation, column NJ l16 + j: a lane owns NJ adjacent columns of each of its 32 rows (8: one 16-byte
-        // store per row; 7: 14 bytes at a 2-byte aligned address, stored as 12 + 2).  The bf16 stores
+        // store per row; 7: 14 bytes at a 2-byte aligned address, stored as 12 + 2; 6: one 12-byte store).  The bf16 stores
         // are non-temporal: the output (up to 620 MB) is not read by this kernel again and would otherwise push
         // the operands, which the other XCDs still fetch, out of the last-level cache (measured on one box,
         // alternating builds: -8 % on the gate+up forward, -3.7 % over the six bench shapes).
@@ -815,9 +819,19 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
             constexpr bool BIAS = decltype(bias_tag)::value;
             constexpr bool ACC = decltype(acc_tag)::value;
             typedef float v4fl __attribute__((ext_vector_type(4)));
-            if constexpr (NJ == 7) {
-                static_assert(NJ != 7 || (!BIAS && !ACC), "the narrow tile has the plain epilogue only");
-                typedef int v3i_u __attribute__((ext_vector_type(3), aligned(2)));
+            if constexpr (NJ < 8) {
+                static_assert(NJ == 8 || !ACC, "the narrow tiles do not accumulate");
+                float bias_n[NJ];
+                if constexpr (BIAS) {
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j) bias_n[j] = load_bias(g.bias, g.bias_is_bf16, m_lane + j);
+                }
+                auto value = [&](int i, int j, int r) {
+                    float v = acc[i][j][r] * scale;
+                    if constexpr (BIAS) v = v + bias_n[j];
+                    return v;
+                };
+                typedef int v3i_u __attribute__((ext_vector_type(3), aligned(2)));  // 14 l16 (NJ = 7) or 12 l16 bytes
                 typedef uint16_t u16_u __attribute__((aligned(2)));
 #pragma unroll
                 for (int i = 0; i < NF; ++i) {
@@ -828,18 +842,20 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
                         v3i_u packed;
 #pragma unroll
                         for (int j = 0; j < 3; ++j) {
-                            const f32x2_t pr = {acc[i][2 * j][r] * scale, acc[i][2 * j + 1][r] * scale};
+                            const f32x2_t pr = {value(i, 2 * j, r), value(i, 2 * j + 1, r)};
                             packed[j] = __builtin_bit_cast(int, __builtin_convertvector(pr, bf16x2_t));
                         }
-                        const f32x2_t last = {acc[i][6][r] * scale, 0.f};
-                        const uint32_t tail = __builtin_bit_cast(uint32_t, __builtin_convertvector(last, bf16x2_t));
                         *(LLMQ_GLOBAL v3i_u*)dst = packed;
-                        *(LLMQ_GLOBAL u16_u*)(dst + 12) = (uint16_t)tail;
+                        if constexpr (NJ == 7) {
+                            const f32x2_t last = {value(i, NJ - 1, r), 0.f};
+                            const uint32_t tail = __builtin_bit_cast(uint32_t, __builtin_convertvector(last, bf16x2_t));
+                            *(LLMQ_GLOBAL u16_u*)(dst + 12) = (uint16_t)tail;
+                        }
                     }
                 }
             } else {
             float bias_v[8];
-            static_assert(NJ == 7 || NJ == 8, "epilogue written for 7 or 8 columns per lane");
+            static_assert(NJ >= 6 && NJ <= 8, "epilogue written for 6, 7 or 8 columns per lane");
             if constexpr (BIAS) {
 #pragma unroll
                 for (int j = 0; j < 8; ++j) bias_v[j] = load_bias(g.bias, g.bias_is_bf16, m_lane + j);
@@ -900,9 +916,12 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         };
         constexpr std::true_type yes{};
         constexpr std::false_type no{};
-        if constexpr (SEG || NJ != 8) {
+        if constexpr (SEG) {
             rows(no, no);
-            pending_stores = !SEG;
+        } else if constexpr (NJ != 8) {
+            if (g.bias) rows(yes, no);
+            else rows(no, no);
+            pending_stores = true;
         } else if (g.accumulate) {
             if (g.bias) rows(yes, yes);
             else rows(no, yes);
@@ -1046,10 +1065,13 @@ template <typename OutT, int B_FMT>
 static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     LLMQ_REQUIRE(g.M > 0 && g.N > 0 && g.K > 0, "matmul: M, N, K must be positive (got %d, %d, %d)", g.M, g.N, g.K);
     const int cus = cu_count();
-    // The four-wave kernel with 256 x 224 tiles: bf16 output without bias or accumulation, e4m3 b operand.
-    const bool narrow_ok = std::is_same_v<OutT, uint16_t> && B_FMT == 0 && !g.bias && !g.accumulate && g.N % 256 == 0 &&
-                           g.M % 224 == 0 && g.K % (2 * kBK) == 0 && cus % 8 == 0;
-    LLMQ_REQUIRE((g.M % 128 == 0 || narrow_ok) && g.N % 128 == 0 && g.K % 128 == 0,
+    // The four-wave kernel with 256 x 224 or 256 x 192 tiles: bf16 output without accumulation, e4m3 b operand.
+    auto narrow_fits = [&](int width) {
+        return std::is_same_v<OutT, uint16_t> && B_FMT == 0 && !g.accumulate && g.N % 256 == 0 && g.M % width == 0 &&
+               g.K % (2 * kBK) == 0 && cus % 8 == 0;
+    };
+    const bool ok224 = narrow_fits(224), ok192 = narrow_fits(192);
+    LLMQ_REQUIRE((g.M % 128 == 0 || ok224 || ok192) && g.N % 128 == 0 && g.K % 128 == 0,
                  "matmul: M, N, K must be divisible by 128 (got %d, %d, %d)", g.M, g.N, g.K);
     LLMQ_REQUIRE(g.a && g.b && g.c, "matmul: null operand pointer");
     LLMQ_REQUIRE(aligned16(g.a) && aligned16(g.b) && aligned16(g.c) && aligned16(g.bias) && aligned16(workspace),
@@ -1057,39 +1079,53 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
     LLMQ_REQUIRE(workspace != nullptr || workspace_bytes == 0, "matmul: workspace size given without a workspace");
     g.group = 8;
     int tile = g_gemm_tile;
-    LLMQ_REQUIRE(tile >= 0 && tile <= 4, "matmul: unknown tile selector %d", tile);
+    LLMQ_REQUIRE(tile >= 0 && tile <= 5, "matmul: unknown tile selector %d", tile);
     const bool fits256 = g.N % 256 == 0 && g.M % 256 == 0;
     LLMQ_REQUIRE((tile != 1 && tile != 3) || fits256, "matmul: the 256 x 256 tile needs M and N divisible by 256");
     const bool w4_ok = fits256 && g.K % (2 * kBK) == 0 && cus % 8 == 0;
     if (tile == 3) {
         LLMQ_REQUIRE(w4_ok, "matmul: the four-wave kernel needs K divisible by 256");
     }
-    // The 256 x 224 tiles are taken when their whole rounds of 7/8-sized tiles beat the rounds of full tiles by
-    // a margin, e.g. M = 3584, N = 8192: 512 tiles in 2 rounds instead of 448 in 1.75, on paper 12.5 % less
-    // time.  Measured (alternating builds on one box): K = 18944 371 -> 357 us, K = 37888 860 -> 820 us, i.e.
+    // The narrow tiles are taken when their whole rounds of 7/8- or 3/4-sized tiles beat the rounds of full tiles
+    // by a margin, e.g. M = 3584, N = 8192: 512 tiles of 224 in 2 rounds instead of 448 in 1.75, on paper 12.5 %
+    // less time.  Measured (alternating builds on one box): K = 18944 371 -> 357 us, K = 37888 860 -> 820 us, i.e.
     // 4-5 %: a narrow tile does 7/8 of the matrix work per barrier, copy and fragment-read overhead of a
     // K-step, and the 192 tiles of a three-quarter round run faster than those of a full one.  Hence the 8 %
-    // the comparison below asks for.  The narrow tiles also serve an M that only 224 divides.
-    if (tile == 4) {
-        LLMQ_REQUIRE(narrow_ok, "matmul: the 256 x 224 tile needs bf16 output without bias or accumulation, N %% 256 == 0, "
-                                "M %% 224 == 0 and K %% 256 == 0");
-    }
-    bool narrow = tile == 4 || g.M % 128 != 0;
-    if (tile == 0 && narrow_ok && w4_ok && g_gemm_splits == 0) {
-        const int64_t t256 = (int64_t)(g.N / 256) * (g.M / 256), t224 = (int64_t)(g.N / 256) * (g.M / 224);
-        const int64_t r256 = (t256 + cus - 1) / cus, r224 = (t224 + cus - 1) / cus;
+    // (12 % for the 192-wide tile) the comparison below asks for.  The narrow tiles also serve an M that only
+    // 224 or 192 divide.
+    int narrow_nj = 0;
+    if (tile == 4 || tile == 5) {
+        LLMQ_REQUIRE(tile == 4 ? ok224 : ok192,
+                     "matmul: the narrow tile (256 x %d) needs bf16 output without accumulation, N %% 256 == 0, "
+                     "M %% %d == 0 and K %% 256 == 0", tile == 4 ? 224 : 192, tile == 4 ? 224 : 192);
+        narrow_nj = tile == 4 ? 7 : 6;
+    } else if (g.M % 128 != 0) {
+        LLMQ_REQUIRE(tile == 0, "matmul: M = %d needs the narrow tile", g.M);
+        narrow_nj = ok224 ? 7 : 6;
+    } else if (tile == 0 && w4_ok && g_gemm_splits == 0) {
+        const int64_t tn = g.N / 256, t256 = tn * (g.M / 256), rem256 = t256 % cus;
         // only where the full tiles' last round would not be cut into K segments anyway (a remainder of 1-2
         // tiles per XCD), and never for less than a round of tiles
-        const int64_t rem256 = t256 % cus;
-        narrow = t256 >= cus && (rem256 == 0 || rem256 > cus / 8) && (double)r224 * 7.0 * 1.08 < (double)r256 * 8.0;
+        if (t256 >= cus && (rem256 == 0 || rem256 > cus / 8)) {
+            auto rounds = [&](int64_t tiles) { return (double)((tiles + cus - 1) / cus); };
+            double best = rounds(t256) * 8.0;
+            if (ok224 && rounds(tn * (g.M / 224)) * 7.0 * 1.08 < best) {
+                best = rounds(tn * (g.M / 224)) * 7.0 * 1.08;
+                narrow_nj = 7;
+            }
+            if (ok192 && rounds(tn * (g.M / 192)) * 6.0 * 1.12 < best) narrow_nj = 6;
+        }
     }
     if constexpr (std::is_same_v<OutT, uint16_t> && B_FMT == 0) {
-        if (narrow) {
-            const int t224 = (g.N / 256) * (g.M / 224);
+        if (narrow_nj) {
+            const int tiles = (g.N / 256) * (g.M / (32 * narrow_nj));
             g.rem_split = 1;
             g.part_per_xcd = 0;
-            const int grid = t224 < cus ? (t224 + 7) / 8 * 8 : cus;
-            hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, 0, false, 7>), dim3((unsigned)grid), dim3(256), 0, stream, g);
+            const int grid = tiles < cus ? (tiles + 7) / 8 * 8 : cus;
+            if (narrow_nj == 7)
+                hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, 0, false, 7>), dim3((unsigned)grid), dim3(256), 0, stream, g);
+            else
+                hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, 0, false, 6>), dim3((unsigned)grid), dim3(256), 0, stream, g);
             LLMQ_HIP_TRY(hipGetLastError());
             return LLMQ_OK;
         }

@@ -296,19 +296,22 @@ def test_gemm_random_codes_within_tolerance(K, O, variant, out_f32):
 
 @pytest.mark.parametrize("forced", [True, False])
 @pytest.mark.parametrize("mnk", [(224, 256, 256), (448, 512, 512), (3584, 8192, 256), (3584, 8192, 512), (1792, 8448, 768),
-                                 (7168, 4352, 256)])
+                                 (7168, 4352, 256), (192, 256, 256), (576, 512, 512), (1536, 16384, 256), (1536, 8448, 768),
+                                 (4608, 4352, 512)])
 def test_gemm_narrow_tile(K, O, mnk, forced):
-    """The four-wave kernel with 256 x 224 tiles (tile selector 4, and whatever the automatic choice takes for
-    these shapes): less than one round of tiles, exactly two rounds, uneven persistent walks; integer operands
-    -> bit exact against the oracle; random codes within the GEMM tolerance; bias / accumulate / fp32 output
-    are refused by the forced selector and served by the other kernels automatically."""
+    """The four-wave kernel with 256 x 224 and 256 x 192 tiles (tile selectors 4 and 5, and whatever the automatic
+    choice takes for these shapes): less than one round of tiles, exactly two rounds, uneven persistent walks;
+    integer operands -> bit exact against the oracle, with and without bias; random codes within the GEMM
+    tolerance; accumulation and fp32 output are refused by the forced selector and served by the other kernels
+    automatically."""
     M, N, Kd = mnk
+    selector = 4 if M % 224 == 0 else 5
     a, _ = O.fill_int_e4m3(M * Kd, 777, 0)
     b, _ = O.fill_int_e4m3(N * Kd, 777, 1)
     a, b = a.reshape(M, Kd), b.reshape(N, Kd)
     s = float(np.sqrt(np.float32(4.0 / Kd)))
     mt = M % 64 == 0          # the threaded oracle works on 64-column blocks
-    set_variant((4, 0) if forced else (0, 0))
+    set_variant((selector, 0) if forced else (0, 0))
     try:
         want = O.gemm_tn(a, b, sa=s, sb=s, mt=mt)
         got = run_gemm(K, a, b, M, N, Kd, s, s)
@@ -328,14 +331,18 @@ def test_gemm_narrow_tile(K, O, mnk, forced):
             gemm_check(g32[rows[0]:rows[1]], exact[rows[0]:rows[1]], sumabs[rows[0]:rows[1]], scale, True)
         _, biasv = O.fill_int_e4m3(M, 777, 2)
         bias = O.f32_to_bf16(biasv.astype(np.float32))
-        if forced:
-            with pytest.raises(ValueError, match="256 x 224|divisible by 128"):
-                run_gemm(K, a, b, M, N, Kd, s, s, bias)
-            with pytest.raises(ValueError, match="256 x 224|divisible by 128"):
+        got = run_gemm(K, a, b, M, N, Kd, s, s, bias)
+        assert np.array_equal(host_bits(got), O.gemm_tn(a, b, sa=s, sb=s, bias=bias, mt=mt))
+        _, oldv = O.fill_int_e4m3(N * M, 777, 3)
+        old = O.f32_to_bf16(oldv.astype(np.float32)).reshape(N, M)
+        if forced or M % 128 != 0:
+            with pytest.raises(ValueError, match="narrow tile|divisible by 128"):
+                run_gemm(K, a, b, M, N, Kd, s, s, None, old)
+            with pytest.raises(ValueError, match="narrow tile|divisible by 128"):
                 run_gemm(K, a, b, M, N, Kd, s, s, out_f32=True)
-        elif M % 128 == 0:
-            got = run_gemm(K, a, b, M, N, Kd, s, s, bias)
-            assert np.array_equal(host_bits(got), O.gemm_tn(a, b, sa=s, sb=s, bias=bias, mt=True))
+        else:
+            got = run_gemm(K, a, b, M, N, Kd, s, s, bias, old)
+            assert np.array_equal(host_bits(got), O.gemm_tn(a, b, sa=s, sb=s, bias=bias, c_old=old, mt=True))
     finally:
         set_variant((0, 0))
 
