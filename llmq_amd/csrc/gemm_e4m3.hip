@@ -1065,9 +1065,9 @@ template <typename OutT, int B_FMT>
 static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     LLMQ_REQUIRE(g.M > 0 && g.N > 0 && g.K > 0, "matmul: M, N, K must be positive (got %d, %d, %d)", g.M, g.N, g.K);
     const int cus = cu_count();
-    // The four-wave kernel with 256 x 224 or 256 x 192 tiles: bf16 output without accumulation, e4m3 b operand.
+    // The four-wave kernel with 256 x 224 or 256 x 192 tiles: bf16 output without accumulation.
     auto narrow_fits = [&](int width) {
-        return std::is_same_v<OutT, uint16_t> && B_FMT == 0 && !g.accumulate && g.N % 256 == 0 && g.M % width == 0 &&
+        return std::is_same_v<OutT, uint16_t> && !g.accumulate && g.N % 256 == 0 && g.M % width == 0 &&
                g.K % (2 * kBK) == 0 && cus % 8 == 0;
     };
     const bool ok224 = narrow_fits(224), ok192 = narrow_fits(192);
@@ -1116,16 +1116,16 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
             if (ok192 && rounds(tn * (g.M / 192)) * 6.0 * 1.12 < best) narrow_nj = 6;
         }
     }
-    if constexpr (std::is_same_v<OutT, uint16_t> && B_FMT == 0) {
+    if constexpr (std::is_same_v<OutT, uint16_t>) {
         if (narrow_nj) {
             const int tiles = (g.N / 256) * (g.M / (32 * narrow_nj));
             g.rem_split = 1;
             g.part_per_xcd = 0;
             const int grid = tiles < cus ? (tiles + 7) / 8 * 8 : cus;
             if (narrow_nj == 7)
-                hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, 0, false, 7>), dim3((unsigned)grid), dim3(256), 0, stream, g);
+                hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, B_FMT, false, 7>), dim3((unsigned)grid), dim3(256), 0, stream, g);
             else
-                hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, 0, false, 6>), dim3((unsigned)grid), dim3(256), 0, stream, g);
+                hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, B_FMT, false, 6>), dim3((unsigned)grid), dim3(256), 0, stream, g);
             LLMQ_HIP_TRY(hipGetLastError());
             return LLMQ_OK;
         }

@@ -438,11 +438,12 @@ def test_gemm_automatic_split_k(K, O, mnk):
     gemm_check(c1.cpu().numpy(), exact, sumabs, np.float32(np.float32(0.01) * np.float32(0.02)), False)
 
 
-@pytest.mark.parametrize("variant", [(0, 0), (1, 1, 1), (2, 2), (3, 1)])
+@pytest.mark.parametrize("variant", [(0, 0), (1, 1, 1), (2, 2), (3, 1), (4, 0), (5, 0)])
 def test_gemm_e5m2_b_operand(K, O, variant):
     """a e4m3, b e5m2 (src/kernels/kernels.h:92-94): small integers are exact in both formats ->
-    bit-exact against the oracle; random codes within the stated tolerance of the exact product."""
-    M, N, Kd = 512, 768, 768
+    bit-exact against the oracle; random codes within the stated tolerance of the exact product.  Selectors 4
+    and 5 are the narrow tiles (bf16 output only: their fp32 check runs on the automatic choice)."""
+    M, N, Kd = {4: (448, 768, 768), 5: (576, 768, 768)}.get(variant[0], (512, 768, 768))
     rng = np.random.default_rng(91)
     ai, bi = rng.integers(-4, 5, (M, Kd)), rng.integers(-4, 5, (N, Kd))
     enc4 = {v: O.lib().orc_e4m3_encode(float(v)) for v in range(-4, 5)}
@@ -466,9 +467,14 @@ def test_gemm_e5m2_b_operand(K, O, variant):
         br[(br & 0x7C) == 0x7C] ^= 0x40                      # no Inf / NaN codes
         br &= 0xBF                                           # magnitudes below 2: products stay modest
         exact, sumabs = O.gemm_exact(ar, br, b_e5m2=True)
-        c32 = torch.empty((N, M), dtype=torch.float32, device="cuda")
-        K.matmul(c32, dev_u8(ar), dev_u8(br), None, dev_scalar(0.25), None, M, N, Kd, workspace=workspace(), b_e5m2=True)
-        gemm_check(c32.cpu().numpy(), exact, sumabs, 0.25, False)
+        if variant[0] in (4, 5):
+            c16 = torch.empty((N, M), dtype=torch.bfloat16, device="cuda")
+            K.matmul(c16, dev_u8(ar), dev_u8(br), None, dev_scalar(0.25), None, M, N, Kd, workspace=workspace(), b_e5m2=True)
+            gemm_check(c16.float().cpu().numpy(), exact, sumabs, 0.25, True)
+        else:
+            c32 = torch.empty((N, M), dtype=torch.float32, device="cuda")
+            K.matmul(c32, dev_u8(ar), dev_u8(br), None, dev_scalar(0.25), None, M, N, Kd, workspace=workspace(), b_e5m2=True)
+            gemm_check(c32.cpu().numpy(), exact, sumabs, 0.25, False)
     finally:
         set_variant((0, 0))
 
