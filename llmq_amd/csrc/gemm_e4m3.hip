@@ -1061,6 +1061,58 @@ static W4Plan plan_w4(int tiles256, int cus, int M, int N, int K, int forced_spl
     return p;
 }
 
+// Kernel choice for outputs with less than one round of 256 x 256 tiles (weight gradients of narrow layers, small
+// models), from estimated times in microseconds.  The constants come from measurements on this chip: a K-step of the
+// four-wave kernel takes 0.9 us on a nearly idle chip and 1.8 us with every compute unit busy (the chip is power
+// limited: the time grows with the square of the active fraction of the matrix work); a pair of co-resident
+// 128 x 128 tiles advances one K-step in 0.43 to 0.78 us; a launch costs about 4-6 us, the second pass of a K split
+// about 8 us plus its traffic at 4 TB/s.  Candidates: one round of 256-, 224- or 192-wide four-wave tiles, or
+// 128 x 128 tiles with 1..8 K splits.  Checked against measured sweeps (7B / 1.5B / 0.5B weight-gradient shapes):
+// the estimate picks the fastest or second-fastest variant, within 5 % of the fastest.
+struct SmallPlan {
+    int nj;      // 8, 7, 6: four-wave kernel with that many fragment columns per wave; 0: 128 x 128 tiles
+    int splits;  // K splits of the 128 x 128 tiles
+};
+static SmallPlan plan_small(int M, int N, int K, int cus, bool ok256, bool ok224, bool ok192, int64_t ws_bytes) {
+    const double kt = (double)K / kBK;
+    SmallPlan best{0, 1};
+    double best_us = 1e30;
+    auto four_wave = [&](int nj, double penalty) {
+        const int w = 32 * nj;
+        const int64_t tiles = (int64_t)(N / 256) * (M / w);
+        const int64_t rounds = (tiles + cus - 1) / cus;
+        auto step = [&](double f) {
+            const double x = f * w / 256.0;
+            return (0.9 + 0.9 * x * x) * (w / 256.0) * penalty;
+        };
+        const double f_last = (double)(tiles - (rounds - 1) * cus) / cus;
+        const double us = (rounds - 1) * (kt * step(1.0) + 6.0) + kt * step(f_last) + 6.0;
+        if (us < best_us) {
+            best_us = us;
+            best = SmallPlan{nj, 1};
+        }
+    };
+    if (ok256) four_wave(8, 1.0);
+    if (ok224) four_wave(7, 1.05);
+    if (ok192) four_wave(6, 1.08);
+    const int64_t t128 = (int64_t)(N / 128) * (M / 128);
+    const int64_t slice = (int64_t)N * M * 4;
+    for (int sp = 1; sp <= 8; ++sp) {
+        if (M % 128 != 0) break;
+        if (sp > 1 && ((int64_t)sp * slice > ws_bytes || K / sp < 512)) break;
+        const int64_t items = t128 * sp, slots = 2 * (int64_t)cus;
+        const int64_t rounds = (items + slots - 1) / slots;
+        const double f_last = (double)(items - (rounds - 1) * slots) / slots;
+        double us = ((rounds - 1) * 0.78 + 0.43 + 0.35 * f_last) * (kt / sp) + 4.0 * rounds;
+        if (sp > 1) us += 8.0 + (double)N * M * (4.0 * sp + 2.0) / 4e6;
+        if (us < best_us) {
+            best_us = us;
+            best = SmallPlan{0, sp};
+        }
+    }
+    return best;
+}
+
 template <typename OutT, int B_FMT>
 static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     LLMQ_REQUIRE(g.M > 0 && g.N > 0 && g.K > 0, "matmul: M, N, K must be positive (got %d, %d, %d)", g.M, g.N, g.K);
@@ -1093,7 +1145,7 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
     // K-step, and the 192 tiles of a three-quarter round run faster than those of a full one.  Hence the 8 %
     // (12 % for the 192-wide tile) the comparison below asks for.  The narrow tiles also serve an M that only
     // 224 or 192 divide.
-    int narrow_nj = 0;
+    int narrow_nj = 0, small_splits = 0;
     if (tile == 4 || tile == 5) {
         LLMQ_REQUIRE(tile == 4 ? ok224 : ok192,
                      "matmul: the narrow tile (256 x %d) needs bf16 output without accumulation, N %% 256 == 0, "
@@ -1102,6 +1154,16 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
     } else if (g.M % 128 != 0) {
         LLMQ_REQUIRE(tile == 0, "matmul: M = %d needs the narrow tile", g.M);
         narrow_nj = ok224 ? 7 : 6;
+    } else if (tile == 0 && g_gemm_splits == 0 && (int64_t)(g.N / 256) * (g.M / 256) < cus) {
+        const SmallPlan sp = plan_small(g.M, g.N, g.K, cus, w4_ok, ok224, ok192, workspace ? (int64_t)workspace_bytes : 0);
+        if (sp.nj == 8) {
+            tile = 3;
+        } else if (sp.nj) {
+            narrow_nj = sp.nj;
+        } else {
+            tile = 2;
+            small_splits = sp.splits;
+        }
     } else if (tile == 0 && w4_ok && g_gemm_splits == 0) {
         const int64_t tn = g.N / 256, t256 = tn * (g.M / 256), rem256 = t256 % cus;
         // only where the full tiles' last round would not be cut into K segments anyway (a remainder of 1-2
@@ -1146,7 +1208,9 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
     const int64_t ws_splits = (int64_t)(workspace_bytes / (size_t)slice_bytes);
     int splits = tile == 3 ? 1 : g_gemm_splits;  // for the four-wave kernel the knob cuts the last round instead
     LLMQ_REQUIRE(splits >= 0, "matmul: negative split count %d", splits);
-    if (splits == 0) {
+    if (splits == 0 && small_splits > 0) {
+        splits = small_splits;
+    } else if (splits == 0) {
         splits = 1;
         if (2 * tiles <= cus && ws_splits >= 2) {
             int64_t want = cus / tiles;
