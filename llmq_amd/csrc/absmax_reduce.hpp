@@ -60,6 +60,6 @@ __device__ __forceinline__ void block_min_to_atomic_max(unsigned* result, uint32
 }
 
 // Resets an abs-max slot: a one-lane fill kernel rather than a memset node, safe to record into a HIP graph.
-static __global__ void reset_slot_kernel(unsigned* slot) { *slot = 0u; }
+__attribute__((unused)) static __global__ void reset_slot_kernel(unsigned* slot) { *slot = 0u; }
 
 }  // namespace llmq
