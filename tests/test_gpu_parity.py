@@ -347,6 +347,53 @@ def test_gemm_narrow_tile(K, O, mnk, forced):
         set_variant((0, 0))
 
 
+def _dispatch_sweep_cases():
+    """Deterministic pseudo-random shapes for the automatic kernel choice: M from multiples of 128, 192, 224 and
+    256, N from multiples of 128 and 256, K from multiples of 128 and 256, tile counts from a handful to a few
+    rounds of the chip, every epilogue flavour."""
+    rng = np.random.default_rng(2024)
+    cases = []
+    for idx in range(48):
+        unit_m = [128, 192, 224, 256][idx % 4]
+        M = int(unit_m * rng.integers(1, [24, 16, 16, 14][idx % 4]))
+        N = int([128, 256][idx % 2] * rng.integers(1, [40, 24][idx % 2]))
+        Kd = int([128, 256][(idx // 2) % 2] * rng.integers(1, 9))
+        if unit_m in (192, 224) and M % 128:       # only the narrow tiles serve these: they need N, K % 256 == 0
+            N, Kd = -(-N // 256) * 256, -(-Kd // 256) * 256
+            if M % 64:                             # outside the threaded oracle's 64-column blocks: keep it small
+                N, Kd = min(N, 1024), min(Kd, 512)
+        cases.append((M, N, Kd, idx % 3 == 1, idx % 5 == 2, idx % 7 == 3, idx % 4 != 3))
+    return cases
+
+
+@pytest.mark.parametrize("case", _dispatch_sweep_cases())
+def test_gemm_automatic_choice_sweep(K, O, case):
+    """Whatever kernel, tile width and K split the dispatcher picks: integer operands -> bit exact against the
+    oracle (bf16 and fp32 output, bias, accumulation, with and without a workspace)."""
+    M, N, Kd, use_bias, use_old, out_f32, with_ws = case
+    if M % 128 and (use_old or out_f32):
+        use_old = out_f32 = False                  # the narrow tiles take bf16 output without accumulation only
+    a, _ = O.fill_int_e4m3(M * Kd, 31 + M, 0)
+    b, _ = O.fill_int_e4m3(N * Kd, 31 + N, 1)
+    a, b = a.reshape(M, Kd), b.reshape(N, Kd)
+    s = float(np.sqrt(np.float32(4.0 / Kd)))
+    _, biasv = O.fill_int_e4m3(M, 31, 2)
+    _, oldv = O.fill_int_e4m3(N * M, 31, 3)
+    bias = O.f32_to_bf16(biasv.astype(np.float32)) if use_bias else None
+    oldf = oldv.astype(np.float32).reshape(N, M)
+    old = (oldf if out_f32 else O.f32_to_bf16(oldf).reshape(N, M)) if use_old else None
+    want = O.gemm_tn(a, b, sa=s, sb=s, bias=bias, c_old=old, out_f32=out_f32, mt=M % 64 == 0)
+    dt = torch.float32 if out_f32 else torch.bfloat16
+    if old is not None:
+        c = (torch.from_numpy(old).cuda() if out_f32 else dev_bf16(old)).reshape(N, M).clone()
+    else:
+        c = torch.full((N, M), float("nan"), dtype=dt, device="cuda")
+    K.matmul(c, dev_u8(a), dev_u8(b), dev_bf16(bias) if use_bias else None, dev_scalar(s), dev_scalar(s), M, N, Kd,
+             accumulate=use_old, workspace=workspace() if with_ws else None)
+    got = c.cpu().numpy() if out_f32 else host_bits(c)
+    assert np.array_equal(got, want), case
+
+
 @pytest.mark.parametrize("variant", [(1, 1, 1), (3, 1), (3, 2), (3, 3), (3, 4)])
 @pytest.mark.parametrize("mnk", [(4352, 4352, 384), (4608, 4096, 256), (8192, 4864, 512), (4352, 4352, 1024),
                                  (4352, 4096, 1024), (4352, 4352, 1536)])
