@@ -200,31 +200,41 @@ __global__ __launch_bounds__(256) void rmsnorm_backward_kernel(uint4* dinp, floa
         for (int e = 0; e < 8; ++e) dw[k][e] = 0.f;
     uint32_t fold = 0x7F807F80u;
 
-    int parity = 0;
-    for (int row0 = blockIdx.x * ROWS; row0 < N; row0 += gridDim.x * ROWS, parity ^= 1) {  // uniform trip count
-        const int row = row0 + rslot;
-        const bool valid = row < N;
-        const int64_t base = (int64_t)row * chunks;
-        const float r = valid ? rstd[row] : 0.f;
+    // Two register sets in ping-pong: the loads of the row after the current one are issued before the current
+    // row is worked on, so that a wave keeps memory requests in flight through its arithmetic, the workgroup
+    // barrier and its stores (one wave per SIMD pair otherwise alternates between loading and computing).
+    struct RowRegs {
         uint4 d[NCH], x[NCH], old[NCH];
+        float r;
+        bool valid;
+        int64_t base;
+    };
+    auto load_row = [&](RowRegs& q, int row0) {
+        const int row = row0 + rslot;
+        q.valid = row < N;
+        q.base = (int64_t)row * chunks;
+        q.r = q.valid ? rstd[row] : 0.f;
 #pragma unroll
         for (int k = 0; k < NCH; ++k) {
             const int c = c_first + kWave * WPR * k;
-            d[k] = x[k] = old[k] = make_uint4(0, 0, 0, 0);
-            if (valid && c < chunks) {
-                d[k] = load_nt(&dout[base + c]);
-                x[k] = load_nt(&inp[base + c]);
-                old[k] = load_nt(&dresidual[base + c]);
+            q.d[k] = q.x[k] = q.old[k] = make_uint4(0, 0, 0, 0);
+            if (q.valid && c < chunks) {
+                q.d[k] = load_nt(&dout[q.base + c]);
+                q.x[k] = load_nt(&inp[q.base + c]);
+                q.old[k] = load_nt(&dresidual[q.base + c]);
             }
         }
+    };
+    auto work_row = [&](const RowRegs& q, int parity) {
+        const float r = q.r;
         float dot = 0.f;
 #pragma unroll
         for (int k = 0; k < NCH; ++k) {
             const int c = c_first + kWave * WPR * k;
             if (c < chunks) {
                 const uint4 w = weight[c];
-                const uint32_t dv[4] = {d[k].x, d[k].y, d[k].z, d[k].w}, xv[4] = {x[k].x, x[k].y, x[k].z, x[k].w},
-                               wv[4] = {w.x, w.y, w.z, w.w};
+                const uint32_t dv[4] = {q.d[k].x, q.d[k].y, q.d[k].z, q.d[k].w},
+                               xv[4] = {q.x[k].x, q.x[k].y, q.x[k].z, q.x[k].w}, wv[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     dot = dot + (bf16_lo(wv[j]) * bf16_lo(dv[j])) * bf16_lo(xv[j]);
@@ -236,21 +246,22 @@ __global__ __launch_bounds__(256) void rmsnorm_backward_kernel(uint4* dinp, floa
         for (int off = 32; off > 0; off >>= 1) dot = dot + __shfl_xor(dot, off, kWave);
         if constexpr (WPR > 1) {
             // the parts of the waves sharing the row, added in wave order (double-buffered slots: the next
-            // iteration's writes cannot overtake this iteration's reads)
+            // row's writes cannot overtake this row's reads)
             if (lane == 0) dot_part[parity][wave] = dot;
             __syncthreads();
             dot = dot_part[parity][rslot * WPR];
 #pragma unroll
-            for (int q = 1; q < WPR; ++q) dot = dot + dot_part[parity][rslot * WPR + q];
+            for (int p = 1; p < WPR; ++p) dot = dot + dot_part[parity][rslot * WPR + p];
         }
         const float kk = __fdiv_rn(dot, c_float) * r;
 #pragma unroll
         for (int k = 0; k < NCH; ++k) {
             const int c = c_first + kWave * WPR * k;
-            if (valid && c < chunks) {
+            if (q.valid && c < chunks) {
                 const uint4 w = weight[c];
-                const uint32_t dv[4] = {d[k].x, d[k].y, d[k].z, d[k].w}, xv[4] = {x[k].x, x[k].y, x[k].z, x[k].w},
-                               wv[4] = {w.x, w.y, w.z, w.w}, ov[4] = {old[k].x, old[k].y, old[k].z, old[k].w};
+                const uint32_t dv[4] = {q.d[k].x, q.d[k].y, q.d[k].z, q.d[k].w},
+                               xv[4] = {q.x[k].x, q.x[k].y, q.x[k].z, q.x[k].w}, wv[4] = {w.x, w.y, w.z, w.w},
+                               ov[4] = {q.old[k].x, q.old[k].y, q.old[k].z, q.old[k].w};
                 uint32_t res[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
@@ -262,9 +273,20 @@ __global__ __launch_bounds__(256) void rmsnorm_backward_kernel(uint4* dinp, floa
                     res[j] = pack_bf16_rn(bf16_lo(ov[j]) + v0, bf16_hi(ov[j]) + v1);
                 }
                 const uint4 o = make_uint4(res[0], res[1], res[2], res[3]);
-                store_nt(&dinp[base + c], o);
+                store_nt(&dinp[q.base + c], o);
                 if constexpr (ABSMAX) fold = fold_vec(fold, o);
             }
+        }
+    };
+    const int step = gridDim.x * ROWS;
+    RowRegs ra, rb;
+    load_row(ra, blockIdx.x * ROWS);
+    for (int row0 = blockIdx.x * ROWS; row0 < N; row0 += 2 * step) {  // uniform trip count
+        load_row(rb, row0 + step);       // rows past the end load nothing and store nothing
+        work_row(ra, 0);
+        if (row0 + step < N) {           // uniform: the barrier inside is reached by all or none
+            load_row(ra, row0 + 2 * step);
+            work_row(rb, 1);
         }
     }
 
