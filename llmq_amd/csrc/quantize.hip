@@ -54,29 +54,30 @@ __global__ __launch_bounds__(256) void quantize_kernel(uint2* __restrict__ out, 
 }
 
 // fp32 input (master weights / activations of an fp32 model): 4 bytes read + 1 written per element.
-// Each lane converts 4 values per access (16-byte load, 4-byte store), UNROLL accesses in flight.
+// Each lane converts 4 values per access (16-byte load, 4-byte store), UNROLL accesses in flight, a workgroup
+// owning a contiguous piece of 256 * UNROLL vectors, as in the bf16 kernel above.
 template <int FMT, int UNROLL>
 __global__ __launch_bounds__(256) void quantize_f32_kernel(uint32_t* __restrict__ out, float* __restrict__ scale_ptr,
-                                                           const float4* __restrict__ in,
+                                                           const uint4* __restrict__ in,
                                                            const float* __restrict__ absmax, int64_t nvec,
                                                            const float* __restrict__ tail_in,
                                                            uint8_t* __restrict__ tail_out, int ntail) {
     const float s = quant_scale(*absmax);
     const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     if (tid == 0 && scale_ptr) *scale_ptr = __fdiv_rn(1.f, s);
-    for (int64_t i = tid; i < nvec; i += UNROLL * stride) {
-        float4 v[UNROLL];
+    const int64_t first = (int64_t)blockIdx.x * (256 * UNROLL) + threadIdx.x;
+    uint4 v[UNROLL];
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            const int64_t idx = i + u * stride;
-            v[u] = idx < nvec ? in[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
-        }
+    for (int u = 0; u < UNROLL; ++u) {
+        const int64_t idx = first + u * 256;
+        v[u] = idx < nvec ? load_nt(&in[idx]) : make_uint4(0, 0, 0, 0);
+    }
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            const int64_t idx = i + u * stride;
-            if (idx < nvec) out[idx] = encode4<FMT>(s * v[u].x, s * v[u].y, s * v[u].z, s * v[u].w);
-        }
+    for (int u = 0; u < UNROLL; ++u) {
+        const int64_t idx = first + u * 256;
+        if (idx < nvec)
+            out[idx] = encode4<FMT>(s * __uint_as_float(v[u].x), s * __uint_as_float(v[u].y), s * __uint_as_float(v[u].z),
+                                    s * __uint_as_float(v[u].w));
     }
     if (tid < ntail) tail_out[tid] = (uint8_t)(encode4<FMT>(s * tail_in[tid], 0.f, 0.f, 0.f) & 0xFFu);
 }
@@ -208,15 +209,21 @@ static int launch_quantize_f32(uint8_t* out, float* scale_ptr, const float* in, 
     LLMQ_REQUIRE(absmax != nullptr, "quantize_with_abs_max: abs_max pointer is null");
     LLMQ_REQUIRE(n == 0 || (out != nullptr && in != nullptr), "quantize_with_abs_max: null tensor pointer");
     LLMQ_REQUIRE(aligned16(in) && aligned16(out), "quantize_with_abs_max: tensors must be 16-byte aligned");
-    constexpr int UNROLL = 8;
     const int64_t nvec = n / 4;
     const int ntail = (int)(n - nvec * 4);
-    int64_t blocks = (nvec + 256 * UNROLL - 1) / (256 * UNROLL);
-    if (blocks > 0x7FFFFFFF) blocks = 0x7FFFFFFF;
-    if (blocks < 1) blocks = 1;  // still writes the scale for n == 0
-    hipLaunchKernelGGL((quantize_f32_kernel<FMT, UNROLL>), dim3((unsigned)blocks), dim3(256), 0, stream,
-                       reinterpret_cast<uint32_t*>(out), scale_ptr, reinterpret_cast<const float4*>(in), absmax, nvec,
-                       in + nvec * 4, out + nvec * 4, ntail);
+    auto launch = [&](auto kernel, int unroll) -> int {
+        int64_t blocks = (nvec + 256 * unroll - 1) / (256 * unroll);
+        LLMQ_REQUIRE(blocks <= 0x7FFFFFFF, "quantize_with_abs_max: %lld elements are too many", (long long)n);
+        if (blocks < 1) blocks = 1;  // still writes the scale for n == 0
+        hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), 0, stream, reinterpret_cast<uint32_t*>(out), scale_ptr,
+                           reinterpret_cast<const uint4*>(in), absmax, nvec, in + nvec * 4, out + nvec * 4, ntail);
+        return LLMQ_OK;
+    };
+    int rc;
+    if (g_quantize_unroll == 8) rc = launch(quantize_f32_kernel<FMT, 8>, 8);
+    else if (g_quantize_unroll == 4) rc = launch(quantize_f32_kernel<FMT, 4>, 4);
+    else rc = launch(quantize_f32_kernel<FMT, 2>, 2);
+    if (rc != LLMQ_OK) return rc;
     LLMQ_HIP_TRY(hipGetLastError());
     return LLMQ_OK;
 }
