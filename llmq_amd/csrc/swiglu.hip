@@ -210,8 +210,11 @@ extern "C" int llmq_swiglu_forward_quant_bf16(uint8_t* out, float* scale_or_null
     LLMQ_REQUIRE(aligned16(inp) && (reinterpret_cast<uintptr_t>(out) & 7u) == 0,
                  "swiglu_forward_quant: inp must be 16-byte and out 8-byte aligned");
     // an empty tensor still gets its scale written, by the same kernel (grid of one workgroup)
-    const unsigned blocks = nchunks ? blocks_for(nchunks, 256, kFwdUnroll) : 1u;
-    hipLaunchKernelGGL((swiglu_forward_kernel<2, kFwdUnroll, 256>), dim3(blocks), dim3(256), 0, stream, out,
+    // two chunks per operand and lane: 4 % faster than four for this variant (130 against 134 us on [8192 x 18944],
+    // alternating builds, tensors no cache holds); the bf16-output variants measured the other way round
+    constexpr int kQuantUnroll = 2;
+    const unsigned blocks = nchunks ? blocks_for(nchunks, 256, kQuantUnroll) : 1u;
+    hipLaunchKernelGGL((swiglu_forward_kernel<2, kQuantUnroll, 256>), dim3(blocks), dim3(256), 0, stream, out,
                        reinterpret_cast<const uint4*>(inp), nullptr, abs_max, scale_or_null, (uint32_t)nchunks,
                        (uint32_t)(C > 0 ? C / 8 : 1));
     LLMQ_HIP_TRY(hipGetLastError());
