@@ -564,7 +564,8 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs g, int spli
 // full rounds of 7/8 the work each; M = 1536, N = 16384: 384 tiles of 256 = 1.5 rounds, 512 tiles of 192 = 2 full
 // rounds of 3/4 the work).  Everything below is written for NJ fragments; NJ = 8, 7 and 6 are instantiated, the
 // narrow ones for bf16 output without accumulation.
-template <typename OutT, int B_FMT, bool SEG, int NJ = 8>
+// STREAM_OUT: the bf16 stores of the full-width epilogue are non-temporal (see there).
+template <typename OutT, int B_FMT, bool SEG, int NJ = 8, bool STREAM_OUT = true>
 __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     constexpr int BLK = 256, T = 256, WT = 128, NF = 8;
     constexpr int WTM = 16 * NJ, BLKM = 2 * WTM;  // columns (first-operand rows) per wave and per tile
@@ -793,9 +794,11 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         // Epilogue.  acc[i][j][r] is c row 16 i + 4 kg + r of the wave tile and, thanks to the a-tile row
         // permutation, column NJ l16 + j: a lane owns NJ adjacent columns of each of its 32 rows (8: one 16-byte
         // store per row; 7: 14 bytes at a 2-byte aligned address, stored as 12 + 2; 6: one 12-byte store).  The bf16 stores
-        // are non-temporal: the output (up to 620 MB) is not read by this kernel again and would otherwise push
-        // the operands, which the other XCDs still fetch, out of the last-level cache (measured on one box,
-        // alternating builds: -8 % on the gate+up forward, -3.7 % over the six bench shapes).
+        // are non-temporal when operands and output together exceed the 256 MB last-level cache: the output (up to
+        // 620 MB) is not read by this kernel again and would otherwise push the operands, which the other XCDs
+        // still fetch, out of that cache (measured on one box, alternating builds: -3 to -10 % on outputs of
+        // 270-620 MB).  When everything fits, ordinary stores are acknowledged sooner and the wait for them at the
+        // next tile's second barrier is shorter (8192 x 8192 x 3584: 178 -> 167 us, K = 512: 48 -> 43 us).
         int n_blk, m_blk;
         decode(logical, n_blk, m_blk);
         logical += tile_stride;
@@ -904,7 +907,8 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
                             const f32x2_t pr = {v[2 * j], v[2 * j + 1]};
                             packed[j] = __builtin_bit_cast(int, __builtin_convertvector(pr, bf16x2_t));
                         }
-                        __builtin_nontemporal_store(packed, (LLMQ_GLOBAL v4i*)row[r]);
+                        if constexpr (STREAM_OUT) __builtin_nontemporal_store(packed, (LLMQ_GLOBAL v4i*)row[r]);
+                        else *(LLMQ_GLOBAL v4i*)row[r] = packed;
                     } else {
                         const v4fl lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
                         *(LLMQ_GLOBAL v4fl*)row[r] = lo;  // two instructions interleave 16-byte pieces: left to the L2 to merge
@@ -1245,8 +1249,15 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
         g.k_len = plan.k_len;
         g.part_per_xcd = plan.part_per_xcd;
         g.partial = reinterpret_cast<float*>(workspace);
-        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<OutT, B_FMT, false>), dim3((unsigned)plan.grid), dim3(256), 0, stream,
-                           g);
+        // operands and output together within the last-level cache: ordinary output stores (see the epilogue)
+        const bool cached_out = std::is_same_v<OutT, uint16_t> &&
+                                ((int64_t)g.M + g.N) * g.K + (int64_t)g.N * g.M * 2 <= ((int64_t)224 << 20);
+        if (cached_out)
+            hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<OutT, B_FMT, false, 8, false>), dim3((unsigned)plan.grid), dim3(256), 0,
+                               stream, g);
+        else
+            hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<OutT, B_FMT, false>), dim3((unsigned)plan.grid), dim3(256), 0, stream,
+                               g);
         LLMQ_HIP_TRY(hipGetLastError());
         if (plan.rem_split > 1) {
             hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<float, B_FMT, true>), dim3((unsigned)plan.grid), dim3(256), 0,
