@@ -1067,9 +1067,9 @@ static W4Plan plan_w4(int tiles256, int cus, int M, int N, int K, int forced_spl
 
 // Kernel choice for outputs with less than one round of 256 x 256 tiles (weight gradients of narrow layers, small
 // models), from estimated times in microseconds.  The constants come from measurements on this chip: a K-step of the
-// four-wave kernel takes 0.9 us on a nearly idle chip and 1.8 us with every compute unit busy (the chip is power
+// four-wave kernel takes 0.9 us on a nearly idle chip and 1.4 us with every compute unit busy (the chip is power
 // limited: the time grows with the square of the active fraction of the matrix work); a pair of co-resident
-// 128 x 128 tiles advances one K-step in 0.43 to 0.78 us; a launch costs about 4-6 us, the second pass of a K split
+// 128 x 128 tiles advances one K-step in 0.47 to 0.85 us; a launch costs about 4-6 us, the second pass of a K split
 // about 8 us plus its traffic at 4 TB/s.  Candidates: one round of 256-, 224- or 192-wide four-wave tiles, or
 // 128 x 128 tiles with 1..8 K splits.  Checked against measured sweeps (7B / 1.5B / 0.5B weight-gradient shapes):
 // the estimate picks the fastest or second-fastest variant, within 5 % of the fastest.
@@ -1087,7 +1087,7 @@ static SmallPlan plan_small(int M, int N, int K, int cus, bool ok256, bool ok224
         const int64_t rounds = (tiles + cus - 1) / cus;
         auto step = [&](double f) {
             const double x = f * w / 256.0;
-            return (0.9 + 0.9 * x * x) * (w / 256.0) * penalty;
+            return (0.9 + 0.5 * x * x) * (w / 256.0) * penalty;
         };
         const double f_last = (double)(tiles - (rounds - 1) * cus) / cus;
         const double us = (rounds - 1) * (kt * step(1.0) + 6.0) + kt * step(f_last) + 6.0;
@@ -1107,7 +1107,7 @@ static SmallPlan plan_small(int M, int N, int K, int cus, bool ok256, bool ok224
         const int64_t items = t128 * sp, slots = 2 * (int64_t)cus;
         const int64_t rounds = (items + slots - 1) / slots;
         const double f_last = (double)(items - (rounds - 1) * slots) / slots;
-        double us = ((rounds - 1) * 0.78 + 0.43 + 0.35 * f_last) * (kt / sp) + 4.0 * rounds;
+        double us = ((rounds - 1) * 0.85 + 0.47 + 0.38 * f_last) * (kt / sp) + 4.0 * rounds;
         if (sp > 1) us += 8.0 + (double)N * M * (4.0 * sp + 2.0) / 4e6;
         if (us < best_us) {
             best_us = us;
