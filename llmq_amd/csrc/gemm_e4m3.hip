@@ -612,14 +612,27 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     const int ld_row = tid / 8;
     const int ld_chunk = (tid & 7) ^ ((ld_row >> 1) & 7);
     const uint32_t p_lane = (uint32_t)ld_row * (uint32_t)g.K + (uint32_t)ld_chunk * 16u;
-    // LDS row rho of the a-tile is row rho % 16 of fragment f = rho / 16 (wave half f / NJ, fragment f % NJ of it)
-    // and holds global row frag_row(f) + NJ * (rho % 16), so that a lane of the epilogue owns NJ adjacent columns.
-    // A copy slab is two fragments, f = 2 it and 2 it + 1; the second starts one global row after the first,
-    // except where it opens the second wave half (odd NJ only: slab (NJ - 1) / 2), hence a second lane offset.
-    auto frag_row = [](int f) { return WTM * (f / NJ) + f % NJ; };
-    const uint32_t q_lane = (uint32_t)(NJ * (ld_row % 16) + ld_row / 16) * (uint32_t)g.K + (uint32_t)ld_chunk * 16u;
-    const uint32_t q_lane_x =
-        (uint32_t)(NJ * (ld_row % 16) + (ld_row / 16) * (WTM - (NJ - 1))) * (uint32_t)g.K + (uint32_t)ld_chunk * 16u;
+    // LDS row rho of the a-tile is row l = rho % 16 of fragment f = rho / 16 (wave half f / NJ, fragment f % NJ of
+    // it) and holds global row frag_row(f) + frag_step(f) * l.  NJ = 8 and 6: fragment j of a wave half starts at
+    // row j with step NJ, so that a lane of the epilogue owns NJ adjacent columns (16 or 12 bytes of bf16).  NJ = 7:
+    // the first six fragments do the same with step 6 (12 bytes per lane, 4-byte aligned), the seventh takes the
+    // last 16 columns of the wave half one per lane (14 adjacent columns per lane would mean 2-byte aligned
+    // 12 + 2 byte stores, measured 3 us per tile slower).
+    // A copy slab is two fragments, f = 2 it (lanes of its first 16 rows) and 2 it + 1: the lane offset of a slab
+    // follows from the two fragments' steps and the distance of their first rows -- one value for all slabs
+    // with NJ = 8 and 6, three different ones with NJ = 7 (slabs 3 and 6 hold a seventh fragment).
+    auto frag_row = [](int f) {
+        const int j = f % NJ;
+        return WTM * (f / NJ) + ((NJ == 7 && j == 6) ? 96 : j);
+    };
+    auto frag_step = [](int f) { return NJ == 7 ? (f % NJ == 6 ? 1 : 6) : NJ; };
+    auto slab_lane_rows = [&](int it) {  // global row of this lane's LDS row, relative to the slab's first row
+        const int l = ld_row % 16;
+        return ld_row < 16 ? frag_step(2 * it) * l : frag_row(2 * it + 1) - frag_row(2 * it) + frag_step(2 * it + 1) * l;
+    };
+    const uint32_t q_lane = (uint32_t)slab_lane_rows(0) * (uint32_t)g.K + (uint32_t)ld_chunk * 16u;
+    const uint32_t q_lane_3 = (uint32_t)slab_lane_rows(NJ == 7 ? 3 : 0) * (uint32_t)g.K + (uint32_t)ld_chunk * 16u;
+    const uint32_t q_lane_6 = (uint32_t)slab_lane_rows(NJ == 7 ? 6 : 0) * (uint32_t)g.K + (uint32_t)ld_chunk * 16u;
     // The copy stream runs two K-steps ahead of the matrix instructions and has its own position: tile
     // number, K offset and the operand bases of that tile already advanced to the K offset.
     int copy_k0 = 0, copy_tile = 0;
@@ -660,7 +673,7 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
             const int it = c - ITERS;
             src = q_cur + (int64_t)frag_row(2 * it) * g.K;
             dst = lds_wave + stage_ofs + P_BYTES + it * T * 16;
-            lane_ofs = (NJ % 2 == 1 && it == (NJ - 1) / 2) ? q_lane_x : q_lane;
+            lane_ofs = (NJ == 7 && it == 3) ? q_lane_3 : (NJ == 7 && it == 6) ? q_lane_6 : q_lane;
         }
         asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                      :
@@ -793,7 +806,8 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
 
         // Epilogue.  acc[i][j][r] is c row 16 i + 4 kg + r of the wave tile and, thanks to the a-tile row
         // permutation, column NJ l16 + j: a lane owns NJ adjacent columns of each of its 32 rows (8: one 16-byte
-        // store per row; 7: 14 bytes at a 2-byte aligned address, stored as 12 + 2; 6: one 12-byte store).  The bf16 stores
+        // store per row; 6: one 12-byte store; 7: 6 adjacent columns and one of the wave half's last 16, a 12-byte
+        // and a 2-byte store).  The bf16 stores
         // are non-temporal when operands and output together exceed the 256 MB last-level cache: the output (up to
         // 620 MB) is not read by this kernel again and would otherwise push the operands, which the other XCDs
         // still fetch, out of that cache (measured on one box, alternating builds: -3 to -10 % on outputs of
@@ -815,8 +829,10 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         }
         const int e_lane = opaque(threadIdx.x) % 64;
         const int el16 = e_lane % 16, ekg = e_lane / 16;
-        const int m_lane = m_blk + wm * WTM + NJ * el16;
+        const int m_lane = m_blk + wm * WTM + (NJ == 7 ? 6 : NJ) * el16;
         const uint32_t lane_bytes = ((uint32_t)(4 * ekg) * (uint32_t)ldc + (uint32_t)m_lane) * (uint32_t)sizeof(OutT);
+        const int m_lane7 = m_blk + wm * WTM + 96 + el16;  // NJ = 7: the column of the seventh fragment
+        const uint32_t lane_bytes7 = ((uint32_t)(4 * ekg) * (uint32_t)ldc + (uint32_t)m_lane7) * (uint32_t)sizeof(OutT);
         const int row0 = n_blk + wn * WT;
         auto rows = [&](auto bias_tag, auto acc_tag) {
             constexpr bool BIAS = decltype(bias_tag)::value;
@@ -827,21 +843,22 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
                 float bias_n[NJ];
                 if constexpr (BIAS) {
 #pragma unroll
-                    for (int j = 0; j < NJ; ++j) bias_n[j] = load_bias(g.bias, g.bias_is_bf16, m_lane + j);
+                    for (int j = 0; j < NJ; ++j)
+                        bias_n[j] = load_bias(g.bias, g.bias_is_bf16, (NJ == 7 && j == 6) ? m_lane7 : m_lane + j);
                 }
                 auto value = [&](int i, int j, int r) {
                     float v = acc[i][j][r] * scale;
                     if constexpr (BIAS) v = v + bias_n[j];
                     return v;
                 };
-                typedef int v3i_u __attribute__((ext_vector_type(3), aligned(2)));  // 14 l16 (NJ = 7) or 12 l16 bytes
+                typedef int v3i_u __attribute__((ext_vector_type(3), aligned(4)));  // 12 bytes per lane
                 typedef uint16_t u16_u __attribute__((aligned(2)));
 #pragma unroll
                 for (int i = 0; i < NF; ++i) {
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
-                        LLMQ_GLOBAL char* dst =
-                            scalar_ptr((LLMQ_GLOBAL char*)(c + (int64_t)(row0 + 16 * i + r) * ldc)) + lane_bytes;
+                        LLMQ_GLOBAL char* row_ptr = scalar_ptr((LLMQ_GLOBAL char*)(c + (int64_t)(row0 + 16 * i + r) * ldc));
+                        LLMQ_GLOBAL char* dst = row_ptr + lane_bytes;
                         v3i_u packed;
 #pragma unroll
                         for (int j = 0; j < 3; ++j) {
@@ -852,7 +869,7 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
                         if constexpr (NJ == 7) {
                             const f32x2_t last = {value(i, NJ - 1, r), 0.f};
                             const uint32_t tail = __builtin_bit_cast(uint32_t, __builtin_convertvector(last, bf16x2_t));
-                            *(LLMQ_GLOBAL u16_u*)(dst + 12) = (uint16_t)tail;
+                            *(LLMQ_GLOBAL u16_u*)(row_ptr + lane_bytes7) = (uint16_t)tail;
                         }
                     }
                 }
