@@ -732,8 +732,8 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     // against all 8 second-operand fragments.  fa rotates through 4 slots (fragment i+4 is read once row i
     // has been issued; rows 4..7 fetch the next step's first four from the other stage); the next step's
     // second-operand fragments go into the other half of fb, two per row in rows 4..7 (after the barrier).  The 16 copies of
-    // the step after next go into the stage this step releases: 4 right after the barrier, then one after
-    // each of the six middle matrix instructions of rows 5 and 6.
+    // the step after next go into the stage this step releases: 4 right after the barrier, the rest spread
+    // evenly over the matrix instructions of rows 5..7.
     bool pending_stores = false;  // an epilogue without accumulation has just issued its stores
     auto k_step = [&](auto par_tag, auto first_tag) {
         constexpr int PAR = decltype(par_tag)::value;
@@ -746,11 +746,16 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
             for (int j = 0; j < NJ; ++j) {
                 if constexpr (FIRST) mfma_first(acc[i][j], fa[i % 4], fb[PAR][j]);
                 else mfma(acc[i][j], fa[i % 4], fb[PAR][j]);
-                // copies 4 .. COPIES - 1: after the middle matrix instructions of rows 5 and 6
-                constexpr int PER_ROW = NJ - 1 < 6 ? NJ - 1 : 6;
-                static_assert(4 + 2 * PER_ROW >= COPIES, "not every copy of a K-step has a place in the schedule");
-                if ((i == 5 || i == 6) && j >= 1 && j <= PER_ROW) {
-                    if (4 + PER_ROW * (i - 5) + (j - 1) < COPIES) issue_load(4 + PER_ROW * (i - 5) + (j - 1), PAR * STAGE);
+                // copies 4 .. COPIES - 1: spread evenly over the matrix instructions of rows 5..7 (with NJ = 8 after
+                // every second one).  The CU's one address unit takes 16 cycles per copy instruction and the four
+                // waves issue theirs at the same time; a denser burst backs up into the waves' instruction issue
+                // and stalls the matrix instructions behind it (one copy per instruction over rows 5 and 6: 4 %
+                // slower over six large shapes; all sixteen right after the barrier: 11 %).
+                constexpr int SPREAD = COPIES - 4, SLOTS = 3 * NJ;
+                static_assert(SPREAD <= SLOTS, "not every copy of a K-step has a place in the schedule");
+                if (i >= 5) {
+                    const int p = (i - 5) * NJ + j;
+                    if ((p + 1) * SPREAD / SLOTS > p * SPREAD / SLOTS) issue_load(4 + p * SPREAD / SLOTS, PAR * STAGE);
                 }
                 if (i >= 5 && (j == 2 || j == 5)) {  // rows 5..7: fragments 2..7 of the next step
                     const int f = 2 * (i - 4) + (j == 5 ? 1 : 0);
