@@ -17,6 +17,8 @@ One JSON line is printed:
                   against 8 TB/s, inside the step; quantize.cold_large_tensor holds the same kernels timed
                   on their own on 310 MB tensors that no cache holds (median of 20 launches)
   cpu_baseline    the multithreaded CPU port of the same path on a bounded sample (host cores of this box)
+  gemm_error      max-abs and relative-Frobenius error of each of the six GEMMs against the exact product of the same
+                  e4m3 operands (sampled outputs; computed with the CPU oracle beside the CPU baseline)
 Extra fields: roofline.mfma_only_ceiling_TFLOPs (register-only matrix-instruction loops: what the chip sustains
 under its power limit), roofline.traffic (hardware-counter bytes per GEMM launch, from profiles/), hip_graph_replay
 (the same step replayed from a HIP graph), fused_quantize_transpose_step (the step with the single-read
@@ -107,6 +109,8 @@ def main():
 
     def gemm(c, a, b, sa, sb, M, N, Kd):
         timed("gemm", 2.0 * M * N * Kd, lambda: K.matmul(c, a, b, None, sa, sb, M, N, Kd, workspace=ws))
+        if record[0]:
+            timers["gemm"][-1] += ("M%d_N%d_K%d" % (M, N, Kd),)
 
     def tr(dst, src):
         timed("transpose", 2 * src.numel(), lambda: K.transpose(dst, src))
@@ -179,6 +183,18 @@ def main():
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     record[0] = False
+
+    # Samples for the error report (gemm_error): operands, scales and sampled outputs of the six GEMMs are taken
+    # now, while the buffers hold the step's values; the oracle evaluates them in the CPU leg at the end.
+    error_samples = None
+    if not args.no_cpu_baseline:
+        gemms = [("gate_up fwd", out["y_up"], q["w_up"], q["x"], "w_up", "x"),
+                 ("down fwd", out["y_down"], q["w_down"], q["h"], "w_down", "h"),
+                 ("down dgrad", out["dh"], q["w_down_t"], q["dy_down"], "w_down", "dy_down"),
+                 ("down wgrad", out["dw_down"], q["h_t"], q["dy_down_t"], "h", "dy_down"),
+                 ("gate_up dgrad", out["dx"], q["w_up_t"], q["dy_up"], "w_up", "dy_up"),
+                 ("gate_up wgrad", out["dw_up"], q["x_t"], q["dy_up_t"], "x", "dy_up")]
+        error_samples = collect_gemm_samples(gemms, stats, np, torch)
 
     # The same step recorded once into a HIP graph and replayed (the reference replays its transformer
     # block from a graph as well, src/models/llama_model.cpp:49-71): removes the launch gaps.
@@ -353,7 +369,7 @@ def main():
             "transpose (2 B/el)": cold_run(lambda i: K.transpose(qt_dsts[i], q_srcs[(i + 1) % 3]), 2 * n_h),
             # what a plain streaming copy sustains under the same protocol: the practical ceiling of a
             # read + write stream on this chip, for reading the fractions above
-            "plain copy kernel, same protocol (2 B/el)": cold_run(lambda i: capi.check(capi.lib.llmq_debug_copy_u8(
+            "plain copy kernel, same protocol (2 B/el)": cold_run(lambda i: capi.check(capi.testaid().llmq_debug_copy_u8(
                 qt_dsts[i].data_ptr(), q_srcs[(i + 1) % 3].data_ptr(), n_h, torch.cuda.current_stream().cuda_stream)), 2 * n_h),
         }
         K.abs_max(stats["h"][0:1], t["h"])   # restore what the step left in the buffers used above
@@ -364,9 +380,36 @@ def main():
     if args.calibrate_copy:
         src = torch.randint(0, 255, (1 << 30,), dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
-        capi.check(capi.lib.llmq_debug_copy_u8(dst.data_ptr(), src.data_ptr(), src.numel(),
+        capi.check(capi.testaid().llmq_debug_copy_u8(dst.data_ptr(), src.data_ptr(), src.numel(),
                                                torch.cuda.current_stream().cuda_stream))
         torch.cuda.synchronize()
+    # Secondary: the matmul alone on the layer shapes of BASELINE.json's other configurations (Qwen2.5-0.5B block,
+    # 8192 tokens; Qwen2.5-1.5B MLP, 16384 tokens), forward / dgrad / wgrad, bf16 output, best of 3 x 5 launches.
+    secondary = None
+    if not args.no_graph:
+        secondary = {"what": "matmul only, e4m3 operands of the given shape (matmul M, N, K), bf16 output, best of 3 x 5 "
+                             "launches; TFLOP/s and fraction of the dense FP8 peak"}
+        layers = {"0.5B qkv": (8192, 896, 1152), "0.5B o_proj": (8192, 896, 896), "0.5B gate_up": (8192, 896, 9728),
+                  "0.5B down": (8192, 4864, 896), "1.5B gate_up": (16384, 1536, 17920), "1.5B down": (16384, 8960, 1536)}
+        one1 = torch.ones(1, device=dev)
+        for lname, (bt, cin, oc) in layers.items():
+            for kind, (M_, N_, K_) in (("fwd", (oc, bt, cin)), ("dgrad", (cin, bt, oc)), ("wgrad", (cin, oc, bt))):
+                a_op = q["dy_up"].view(-1)[:M_ * K_].view(M_, K_)       # any resident codes of the right size
+                b_op = q["dy_up_t"].view(-1)[:N_ * K_].view(N_, K_)
+                c_op = out["y_up"].view(-1)[:N_ * M_].view(N_, M_)
+                best = 1e30
+                for _ in range(3):
+                    K.matmul(c_op, a_op, b_op, None, one1, one1, M_, N_, K_, workspace=ws)
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    for _ in range(5):
+                        K.matmul(c_op, a_op, b_op, None, one1, one1, M_, N_, K_, workspace=ws)
+                    e1.record()
+                    torch.cuda.synchronize()
+                    best = min(best, e0.elapsed_time(e1) / 5 * 1e3)
+                tf = 2.0 * M_ * N_ * K_ / best / 1e6
+                secondary["%s %s (%d, %d, %d)" % (lname, kind, M_, N_, K_)] = {
+                    "us": best, "TFLOPs": tf, "frac_fp8_peak": tf / FP8_PEAK_TFLOPS}
     step_ms = (t1 - t0) * 1e3 / args.steps
 
     # What the matrix cores sustain with no memory traffic at all: a register-only MFMA loop on random
@@ -375,21 +418,37 @@ def main():
     st = torch.cuda.current_stream().cuda_stream
     ceiling = {}
     for label, rnd in (("constant_operands", 0), ("random_operands", 1), ("random_operands_16x16x128", 2)):
-        capi.check(capi.lib.llmq_debug_mfma_ceiling(scratch.data_ptr(), 256, 20000, rnd, st))
+        capi.check(capi.testaid().llmq_debug_mfma_ceiling(scratch.data_ptr(), 256, 20000, rnd, st))
         ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         ev0.record()
         reps, iters = 6, 50000
         for _ in range(reps):
-            capi.check(capi.lib.llmq_debug_mfma_ceiling(scratch.data_ptr(), 256, iters, rnd, st))
+            capi.check(capi.testaid().llmq_debug_mfma_ceiling(scratch.data_ptr(), 256, iters, rnd, st))
         ev1.record()
         torch.cuda.synchronize()
         ceiling[label] = 256.0 * 8 * iters * 8 * 131072.0 * reps / (ev0.elapsed_time(ev1) * 1e-3) / 1e12
 
     def summarize(name):
         evs = timers.get(name, [])
-        ms = [s.elapsed_time(f) for s, f, _ in evs]
-        work = sum(w for _, _, w in evs)
+        ms = [e[0].elapsed_time(e[1]) for e in evs]
+        work = sum(e[2] for e in evs)
         return {"launches": len(evs), "mean_ms": sum(ms) / max(len(ms), 1), "total_ms": sum(ms), "work": work}
+
+    def median(v):
+        v = sorted(v)
+        return 0.5 * (v[len(v) // 2] + v[(len(v) - 1) // 2])
+
+    # per GEMM shape of the step: median and best launch over the timed steps
+    shape_ms = {}
+    for ev in timers.get("gemm", []):
+        shape_ms.setdefault(ev[3], []).append((ev[0].elapsed_time(ev[1]), ev[2]))
+    per_shape = {n: {"median_us": median([m for m, _ in v]) * 1e3, "min_us": min(m for m, _ in v) * 1e3,
+                     "TFLOPs_at_median": v[0][1] / (median([m for m, _ in v]) * 1e-3) / 1e12,
+                     "frac_at_median": v[0][1] / (median([m for m, _ in v]) * 1e-3) / 1e12 / FP8_PEAK_TFLOPS}
+                 for n, v in shape_ms.items()}
+    gemm_flop_sum = sum(v[0][1] for v in shape_ms.values())
+    tflops_median = gemm_flop_sum / (sum(p["median_us"] for p in per_shape.values()) * 1e-6) / 1e12
+    tflops_best = gemm_flop_sum / (sum(p["min_us"] for p in per_shape.values()) * 1e-6) / 1e12
 
     ks = {n: summarize(n) for n in ("gemm", "abs_max", "quantize", "quantize_transpose", "transpose")}
     gemm_tflops_kernel = ks["gemm"]["work"] / (ks["gemm"]["total_ms"] * 1e-3) / 1e12
@@ -415,7 +474,9 @@ def main():
                      "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": gemm_tflops_kernel / FP8_PEAK_TFLOPS,
                      "traffic": measured_traffic(), "mfma_only_ceiling_TFLOPs": ceiling,
                      "frac_of_mfma_only_ceiling": gemm_tflops_kernel / max(ceiling["random_operands"], ceiling["random_operands_16x16x128"]),
-                     "mean_launch_ms": ks["gemm"]["mean_ms"], "launches": ks["gemm"]["launches"]},
+                     "mean_launch_ms": ks["gemm"]["mean_ms"], "launches": ks["gemm"]["launches"],
+                     "achieved_at_median_launch": tflops_median, "achieved_at_best_launch": tflops_best,
+                     "per_shape": per_shape},
         "quantize": {"bound": "hbm", "kernels": "abs_max + quantize_with_abs_max (5 bytes/element)",
                      "achieved": aq_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": aq_gbs / HBM_PEAK_GBS,
                      "per_kernel": per_kernel, "cold_large_tensor": cold},
@@ -425,12 +486,16 @@ def main():
             "ms_per_step": fused_ms, "value": gemm_flop / (fused_ms * 1e-3) / 1e12,
             "note": "extension: single-read quantize + transposed copy for weights and output gradients"},
         "vendor_gemm": vendor,
+        "secondary_gemm_shapes": secondary,
         "producers": swiglu,
         "library": capi.version(),
     }
 
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(t, np, torch, args.cpu_seconds)
+        # the six GEMMs of the step against the exact product of the same e4m3 operands (oracle as the checker,
+        # part of this CPU leg, outside every timed region)
+        result["gemm_error"] = gemm_error_report(error_samples, np)
     print(json.dumps(result))
 
 
@@ -445,6 +510,44 @@ def measured_traffic():
     except OSError:
         pass
     return None
+
+
+def collect_gemm_samples(gemms, stats, np, torch, samples=8192):
+    """Host copies of what the error report needs: per GEMM the operand codes, the fp32 factor sa*sb and
+    `samples` seeded output coordinates with the device results there."""
+    taken = []
+    for i, (name, c, a_op, b_op, sa_name, sb_name) in enumerate(gemms):
+        N, M = c.shape
+        rng = np.random.default_rng(100 + i)
+        idx_n = rng.integers(0, N, samples).astype(np.int32)
+        idx_m = rng.integers(0, M, samples).astype(np.int32)
+        got = c[torch.from_numpy(idx_n).long().cuda(), torch.from_numpy(idx_m).long().cuda()].float().cpu().numpy()
+        taken.append({"name": name, "M": M, "N": N, "a": a_op.view(torch.uint8).cpu().numpy(),
+                      "b": b_op.view(torch.uint8).cpu().numpy(), "idx_n": idx_n, "idx_m": idx_m, "got": got.astype(np.float64),
+                      "scale": float(np.float32(stats[sa_name][1].item()) * np.float32(stats[sb_name][1].item()))})
+    return taken
+
+
+def gemm_error_report(taken, np):
+    """Per GEMM of the step: max-abs and relative-Frobenius error of the bf16 device result against the exact
+    (fp64) product of the same e4m3 operands times the fp32 factor sa*sb, on seeded output coordinates (the
+    reference's acceptance loop prints the same two figures, src/testing/test-gemm.cpp:114-148), and the worst
+    ratio of an element's error to the stated bound 2^-8 |ref| + 2^-11 sa sb sum|a b|."""
+    from oracle import pyoracle as O
+    report = {"what": "bf16 result vs exact fp64 product of the same e4m3 operands x (sa*sb), %d sampled outputs per "
+                      "GEMM; bound = 2^-8 |ref| + 2^-11 sa sb sum_k|a_k b_k|, relative Frobenius limit 2.5e-3"
+                      % taken[0]["idx_n"].size}
+    for s in taken:
+        ex, sabs = O.gemm_exact_sampled(s["a"], s["b"], s["idx_n"], s["idx_m"])
+        ref = ex * s["scale"]
+        err = np.abs(s["got"] - ref)
+        bound = 2.0 ** -8 * np.abs(ref) + 2.0 ** -11 * s["scale"] * sabs + 1e-300
+        fro = float(np.sqrt((err ** 2).sum() / (ref ** 2).sum()))
+        report[s["name"]] = {"M": s["M"], "N": s["N"], "K": int(s["a"].shape[1]), "max_abs": float(err.max()),
+                             "rel_frobenius": fro, "max_abs_ref": float(np.abs(ref).max()),
+                             "worst_err_over_bound": float((err / bound).max()),
+                             "within_tolerance": bool((err <= bound).all() and fro <= 2.5e-3)}
+    return report
 
 
 def cpu_baseline(t, np, torch, budget_s):

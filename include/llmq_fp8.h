@@ -23,6 +23,10 @@
 #ifdef __cplusplus
 extern "C" {
 #endif
+/* The library is built with hidden visibility: the functions declared here are its whole exported surface. */
+#if defined(__GNUC__)
+#pragma GCC visibility push(default)
+#endif
 
 #define LLMQ_OK 0
 #define LLMQ_ERR_INVALID_ARGUMENT 1 /* shape / alignment / null-pointer precondition violated */
@@ -288,6 +292,9 @@ int llmq_adamw_update_bf16(uint16_t* params, const uint16_t* grads, void* m, int
                            float weight_decay, const float* grad_scale, float* abs_max_or_null, unsigned int seed,
                            void* stream);
 
+#if defined(__GNUC__)
+#pragma GCC visibility pop
+#endif
 #ifdef __cplusplus
 }
 #endif

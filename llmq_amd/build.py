@@ -1,6 +1,11 @@
-"""Builds libllmq_fp8.so (the C-ABI library with the gfx950 kernels) with hipcc, in-tree.
+"""Builds the gfx950 libraries with hipcc, in-tree.
 
     python -m llmq_amd.build          # rebuild everything
+
+lib/libllmq_fp8.so          the product: the C ABI of include/llmq_fp8.h and nothing else (hidden visibility)
+lib/libllmq_fp8_testaid.so  for tests and bench.py only: the GEMM file compiled with LLMQ_TEST_HOOKS (the parity
+                            tests force every kernel instantiation through llmq_debug_set_gemm_variant) plus the
+                            measurement aids of calibrate.hip (plain copy kernel, register-only MFMA loop)
 """
 import os
 import subprocess
@@ -12,12 +17,17 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "csrc", "build")
 LIB = os.path.join(HERE, "lib", "libllmq_fp8.so")
+TESTAID_LIB = os.path.join(HERE, "lib", "libllmq_fp8_testaid.so")
 
-SOURCES = ["runtime.hip", "absmax.hip", "quantize.hip", "transpose.hip", "gemm_e4m3.hip", "bias.hip", "swiglu.hip", "rmsnorm.hip", "rope.hip", "adamw.hip", "calibrate.hip"]
+SOURCES = ["runtime.hip", "absmax.hip", "quantize.hip", "transpose.hip", "gemm_e4m3.hip", "bias.hip", "swiglu.hip",
+           "rmsnorm.hip", "rope.hip", "adamw.hip"]
+# (source, object name, extra flags)
+TESTAID_UNITS = [("gemm_e4m3.hip", "gemm_e4m3_hooks.o", ["-DLLMQ_TEST_HOOKS"]), ("calibrate.hip", "calibrate.o", []),
+                 ("runtime.hip", "runtime.o", [])]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++20", "-fPIC",
+    "--offload-arch=gfx950", "-O3", "-std=c++20", "-fPIC", "-fvisibility=hidden",
     "-ffp-contract=off",                       # the epilogue and the quantize multiply are defined op by op
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-mllvm", "-enable-post-misched=0",       # keep the hand-specified interleave of the GEMM K loop
@@ -26,9 +36,10 @@ FLAGS = [
 ]
 
 
-def _compile(src):
-    obj = os.path.join(OBJ, src.replace(".hip", ".o"))
-    cmd = [HIPCC] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+def _compile(unit):
+    src, obj_name, extra = unit
+    obj = os.path.join(OBJ, obj_name)
+    cmd = [HIPCC] + FLAGS + extra + ["-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     out = "\n".join(l for l in (r.stdout + r.stderr).splitlines()
                     if "packed-fp32-ops" not in l and "is not a recognized feature" not in l)
@@ -37,18 +48,26 @@ def _compile(src):
     return obj, out
 
 
+def _link(lib, objs):
+    subprocess.check_call([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,-Bsymbolic",
+                           "-Wl,--version-script=" + os.path.join(CSRC, "exports.map"), "-o", lib] + objs)
+
+
 def build(verbose=True):
     os.makedirs(OBJ, exist_ok=True)
     os.makedirs(os.path.dirname(LIB), exist_ok=True)
-    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
-        results = list(ex.map(_compile, SOURCES))
-    for obj, out in results:
+    units = [(s, s.replace(".hip", ".o"), []) for s in SOURCES]
+    extra_units = [u for u in TESTAID_UNITS if u[1] not in {n for _, n, _ in units}]
+    with ThreadPoolExecutor(max_workers=8) as ex:
+        results = dict(zip([u[1] for u in units + extra_units], ex.map(_compile, units + extra_units)))
+    for obj, out in results.values():
         if verbose and out.strip():
             print(out)
-    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + [o for o, _ in results]
-    subprocess.check_call(cmd)
+    _link(LIB, [results[n][0] for _, n, _ in units])
+    _link(TESTAID_LIB, [results[n][0] for _, n, _ in TESTAID_UNITS])
     if verbose:
         print("built", LIB)
+        print("built", TESTAID_LIB)
     return LIB
 
 

@@ -63,18 +63,6 @@ lib.llmq_rope_backward_bf16.argtypes = lib.llmq_rope_forward_bf16.argtypes
 lib.llmq_precompute_freqs_cis_f16.argtypes = [_vp, _int, _int, C.c_float]
 lib.llmq_adamw_update_bf16.argtypes = [_vp, _vp, _vp, _int, _vp, _int, _i64, C.c_float, C.c_float, C.c_float, _int, C.c_float,
                                        C.c_float, _vp, _vp, C.c_uint, _vp]
-lib.llmq_debug_set_gemm_variant.argtypes = [_int, _int]
-lib.llmq_debug_set_gemm_variant.restype = None
-lib.llmq_debug_set_absmax_stream_bytes.argtypes = [_i64]
-lib.llmq_debug_set_absmax_stream_bytes.restype = None
-lib.llmq_debug_set_quantize_unroll.argtypes = [_int]
-lib.llmq_debug_set_quantize_unroll.restype = None
-lib.llmq_debug_set_gemm_persist.argtypes = [_int]
-lib.llmq_debug_set_gemm_persist.restype = None
-lib.llmq_debug_copy_u8.argtypes = [_vp, _vp, _i64, _vp]
-lib.llmq_debug_copy_u8.restype = _int
-lib.llmq_debug_mfma_ceiling.argtypes = [_vp, _int, _int, _int, _vp]
-lib.llmq_debug_mfma_ceiling.restype = _int
 for _name in EXPORTS[3:]:
     getattr(lib, _name).restype = _int
 lib.llmq_backward_bias_scratch_bytes.restype = _i64
@@ -82,11 +70,41 @@ lib.llmq_rmsnorm_backward_scratch_bytes.restype = _i64
 
 LLMQ_OK, LLMQ_ERR_INVALID_ARGUMENT, LLMQ_ERR_RUNTIME = 0, 1, 2
 
+TESTAID_PATH = os.path.join(_HERE, "lib", "libllmq_fp8_testaid.so")
+_testaid = None
 
-def check(code):
+
+def testaid():
+    """The test-aid library (tests and bench.py only; never needed by a user of the path): the four matmul
+    entry points from a build of the GEMM file whose kernel selection can be forced
+    (llmq_debug_set_gemm_variant / llmq_debug_set_gemm_persist), and the measurement aids llmq_debug_copy_u8
+    (plain copy kernel) and llmq_debug_mfma_ceiling (register-only matrix-instruction loop)."""
+    global _testaid
+    if _testaid is None:
+        if not os.path.exists(TESTAID_PATH):
+            raise ImportError("%s is missing: build it with `python -m llmq_amd.build`" % TESTAID_PATH)
+        t = C.CDLL(TESTAID_PATH)
+        t.llmq_last_error.restype = C.c_char_p
+        for name in ("llmq_gemm_tn_e4m3_bf16", "llmq_gemm_tn_e4m3_f32", "llmq_gemm_tn_e4m3_e5m2_bf16",
+                     "llmq_gemm_tn_e4m3_e5m2_f32"):
+            getattr(t, name).argtypes = getattr(lib, name).argtypes
+            getattr(t, name).restype = _int
+        t.llmq_debug_set_gemm_variant.argtypes = [_int, _int]
+        t.llmq_debug_set_gemm_variant.restype = None
+        t.llmq_debug_set_gemm_persist.argtypes = [_int]
+        t.llmq_debug_set_gemm_persist.restype = None
+        t.llmq_debug_copy_u8.argtypes = [_vp, _vp, _i64, _vp]
+        t.llmq_debug_copy_u8.restype = _int
+        t.llmq_debug_mfma_ceiling.argtypes = [_vp, _int, _int, _int, _vp]
+        t.llmq_debug_mfma_ceiling.restype = _int
+        _testaid = t
+    return _testaid
+
+
+def check(code, from_lib=None):
     if code == LLMQ_OK:
         return
-    msg = lib.llmq_last_error().decode("utf-8", "replace")
+    msg = (from_lib or lib).llmq_last_error().decode("utf-8", "replace")
     if code == LLMQ_ERR_INVALID_ARGUMENT:
         raise ValueError(msg)
     raise RuntimeError(msg)

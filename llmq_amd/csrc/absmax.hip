@@ -78,10 +78,6 @@ __global__ __launch_bounds__(kAbsmaxThreads) void absmax_f32_kernel(unsigned* __
     block_min_to_atomic_max(result, acc, 0x7F800000u, 0);
 }
 
-// tensors above this many bytes would be read with streaming loads: none by default (see absmax_bf16_kernel;
-// llmq_debug_set_absmax_stream_bytes is the hook the measurement above was made with)
-static int64_t g_absmax_stream_bytes = INT64_MAX;
-
 template <typename Kernel, typename Elem>
 static int launch_absmax(Kernel kernel, float* out, const Elem* in, int64_t n, int elems_per_vec, int unroll,
                          hipStream_t stream) {
@@ -110,12 +106,8 @@ static int launch_absmax(Kernel kernel, float* out, const Elem* in, int64_t n, i
 }  // namespace llmq
 
 extern "C" int llmq_abs_max_bf16(float* out, const uint16_t* in, int64_t n, void* stream) {
-    if (2 * n > llmq::g_absmax_stream_bytes)
-        return llmq::launch_absmax(llmq::absmax_bf16_kernel<8, true>, out, in, n, 8, 8, static_cast<hipStream_t>(stream));
     return llmq::launch_absmax(llmq::absmax_bf16_kernel<8, false>, out, in, n, 8, 8, static_cast<hipStream_t>(stream));
 }
-
-extern "C" void llmq_debug_set_absmax_stream_bytes(int64_t bytes) { llmq::g_absmax_stream_bytes = bytes; }
 
 extern "C" int llmq_abs_max_f32(float* out, const float* in, int64_t n, void* stream) {
     return llmq::launch_absmax(llmq::absmax_f32_kernel<8>, out, reinterpret_cast<const uint32_t*>(in), n, 4, 8,

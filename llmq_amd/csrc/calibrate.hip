@@ -90,7 +90,7 @@ __global__ __launch_bounds__(512) void mfma_ceiling_kernel(float* out, int iters
 
 }  // namespace llmq
 
-extern "C" int llmq_debug_copy_u8(uint8_t* dst, const uint8_t* src, int64_t n, void* stream) {
+extern "C" __attribute__((visibility("default"))) int llmq_debug_copy_u8(uint8_t* dst, const uint8_t* src, int64_t n, void* stream) {
     using namespace llmq;
     LLMQ_REQUIRE(dst && src && n > 0 && n % 16 == 0, "copy: need non-null pointers and a positive multiple of 16 bytes");
     LLMQ_REQUIRE(aligned16(dst) && aligned16(src), "copy: pointers must be 16-byte aligned");
@@ -107,7 +107,7 @@ extern "C" int llmq_debug_copy_u8(uint8_t* dst, const uint8_t* src, int64_t n, v
 // 8 * 131072 flop per wave (= blocks * 8 * iters * 1048576 flop).  mode: 0 = 32x32x64 instruction with
 // constant operands, 1 = 32x32x64 with random operands, 2 = 16x16x128 with random operands.
 // scratch: blocks * 512 floats.
-extern "C" int llmq_debug_mfma_ceiling(float* scratch, int blocks, int iters, int mode, void* stream) {
+extern "C" __attribute__((visibility("default"))) int llmq_debug_mfma_ceiling(float* scratch, int blocks, int iters, int mode, void* stream) {
     using namespace llmq;
     LLMQ_REQUIRE(scratch != nullptr && blocks > 0 && iters > 0 && iters % 2 == 0 && mode >= 0 && mode <= 2,
                  "mfma_ceiling: bad arguments");
@@ -118,3 +118,7 @@ extern "C" int llmq_debug_mfma_ceiling(float* scratch, int blocks, int iters, in
     LLMQ_HIP_TRY(hipGetLastError());
     return LLMQ_OK;
 }
+
+// What the library's launch plans take as the number of accelerator dies and compute units of the current device.
+extern "C" __attribute__((visibility("default"))) int llmq_debug_xcd_count(void) { return llmq::xcd_count(); }
+extern "C" __attribute__((visibility("default"))) int llmq_debug_cu_count(void) { return llmq::cu_count(); }

@@ -33,6 +33,9 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 // Number of compute units of the current device (cached per device id).
 int cu_count();
+// Number of accelerator dies (XCDs) the device's compute units are spread over; workgroup ids are dealt to them
+// round-robin and each has an L2 of its own, which the tile walks are laid out for.
+int xcd_count();
 
 constexpr int kWave = 64;
 

@@ -39,6 +39,7 @@
 // layers) split K over gridDim.y: every split writes its raw fp32 accumulators to a slice of the
 // caller's workspace, and a second kernel adds the slices in a fixed order and applies the epilogue, so
 // the result does not depend on scheduling.
+#include <atomic>
 #include <type_traits>
 
 #include "common.hpp"
@@ -68,11 +69,12 @@ struct GemmArgs {
     int k_len;       // split-K only: K elements per split (multiple of 128; four-wave kernel: of 256)
     int rem_split;   // four-wave kernel: K segments per tile of an XCD's last, partial round (1 = none)
     int part_per_xcd;  // four-wave kernel: partial tiles reserved per XCD in `partial`
+    int xcds;          // accelerator dies of the device (workgroup ids are dealt to them round-robin)
 };
 
-// XCD x owns a contiguous range of the logical tile sequence (the first total % 8 XCDs one tile more).
-__device__ __forceinline__ void xcd_tile_range(int total, int xcd, int& first, int& count) {
-    const int xq = total / 8, xr = total % 8;
+// XCD x owns a contiguous range of the logical tile sequence (the first total % xcds XCDs one tile more).
+__device__ __forceinline__ void xcd_tile_range(int total, int xcds, int xcd, int& first, int& count) {
+    const int xq = total / xcds, xr = total % xcds;
     first = xcd * xq + (xcd < xr ? xcd : xr);
     count = xq + (xcd < xr ? 1 : 0);
 }
@@ -142,6 +144,15 @@ __device__ __forceinline__ void sched_group() {
     if constexpr (N > 0) __builtin_amdgcn_sched_group_barrier(MASK, N, 0);
 }
 
+// Compile-time loop: f(integral_constant<int, B>{}), ..., f(integral_constant<int, E - 1>{}).
+template <int B, int E, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (B < E) {
+        f(std::integral_constant<int, B>{});
+        static_for<B + 1, E>(f);
+    }
+}
+
 // SPLIT: blockIdx.y selects a K range of g.k_len elements and the raw accumulators go to g.partial.
 // B_FMT: fp8 format of the b operand (0 = e4m3, 1 = e5m2, the reference's gradient dtype option); b rows are
 // the first operand of the matrix instruction, whose format field takes this value directly.
@@ -173,8 +184,8 @@ __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(Gemm
     // Tile order: XCD x (workgroups are dealt to XCDs round-robin) owns a contiguous range of the
     // "logical" tile sequence, which walks column-major groups of g.group tile-rows.
     const int total = tiles_n * tiles_m;
-    const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
-    const int xq = (PERSIST ? total : (int)gridDim.x) / 8, xr = (PERSIST ? total : (int)gridDim.x) % 8;
+    const int xcd = blockIdx.x % g.xcds, slot = blockIdx.x / g.xcds;
+    const int xq = (PERSIST ? total : (int)gridDim.x) / g.xcds, xr = (PERSIST ? total : (int)gridDim.x) % g.xcds;
     const int xcd_first = xcd * xq + (xcd < xr ? xcd : xr);
     auto decode = [&](int logical, int& n_blk, int& m_blk) {
         const int per_group = g.group * tiles_m;
@@ -188,7 +199,7 @@ __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(Gemm
     int my_tiles = 1, tile_stride = 0;
     if constexpr (PERSIST) {
         const int xcd_count = xq + (xcd < xr ? 1 : 0);
-        tile_stride = gridDim.x / 8;
+        tile_stride = gridDim.x / g.xcds;
         my_tiles = slot < xcd_count ? (xcd_count - slot + tile_stride - 1) / tile_stride : 0;
         if (my_tiles == 0) return;  // uniform for the whole workgroup, before any barrier
     }
@@ -589,10 +600,10 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     // into S segments of K (slot s: tile s / S, segment s % S) and writes raw accumulators as a 256 x 256
     // fp32 tile to g.partial for the reduction kernel below: the round then costs 1 / S of a tile.
     const int total = (g.N / BLK) * (g.M / BLKM);
-    const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
+    const int xcd = blockIdx.x % g.xcds, slot = blockIdx.x / g.xcds;
     int xcd_first, xcd_count;
-    xcd_tile_range(total, xcd, xcd_first, xcd_count);
-    const int tile_stride = gridDim.x / 8;
+    xcd_tile_range(total, g.xcds, xcd, xcd_first, xcd_count);
+    const int tile_stride = gridDim.x / g.xcds;
     int my_tiles, k_first = 0, k_total = g.K;
     if constexpr (SEG) {
         const int rem = xcd_count % tile_stride;
@@ -633,52 +644,97 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     const uint32_t q_lane = (uint32_t)slab_lane_rows(0) * (uint32_t)g.K + (uint32_t)ld_chunk * 16u;
     const uint32_t q_lane_3 = (uint32_t)slab_lane_rows(NJ == 7 ? 3 : 0) * (uint32_t)g.K + (uint32_t)ld_chunk * 16u;
     const uint32_t q_lane_6 = (uint32_t)slab_lane_rows(NJ == 7 ? 6 : 0) * (uint32_t)g.K + (uint32_t)ld_chunk * 16u;
-    // The copy stream runs two K-steps ahead of the matrix instructions and has its own position: tile
-    // number, K offset and the operand bases of that tile already advanced to the K offset.
+    // The copy stream runs two K-steps ahead of the matrix instructions and has its own position: tile number
+    // and K offset.  A copy's global address is "scalar base of its slab in the current tile + 32-bit lane
+    // offset": the 16 slab bases change once per tile, the K offset lives in the lane offsets (one vector add
+    // per K-step), so a copy costs two instructions in the K loop: the write of M0 (LDS destination) and the
+    // copy itself.
     int copy_k0 = 0, copy_tile = 0;
-    const uint8_t *p_cur, *q_cur;
-    auto tile_bases = [&](int logical, const uint8_t*& pb, const uint8_t*& qb) {
+    const uint8_t* p_base[ITERS];
+    const uint8_t* q_base[ITERS_Q];
+    uint32_t vp = p_lane, vq = q_lane, vq3 = q_lane_3, vq6 = q_lane_6;
+    auto tile_bases = [&](int logical) {
         int nb, mb;
         decode(logical, nb, mb);
-        pb = g.b + (int64_t)nb * g.K + k_first;
-        qb = g.a + (int64_t)mb * g.K + k_first;
+        const uint8_t* pb = g.b + (int64_t)nb * g.K + k_first;
+        const uint8_t* qb = g.a + (int64_t)mb * g.K + k_first;
+        // pinned in scalar registers here, once per tile (otherwise the compiler sinks the additions to the
+        // copies and repeats them in every K-step)
+#pragma unroll
+        for (int c = 0; c < ITERS; ++c) {
+            p_base[c] = pb + (int64_t)(32 * c) * g.K;
+            asm volatile("" : "+s"(p_base[c]));
+        }
+#pragma unroll
+        for (int it = 0; it < ITERS_Q; ++it) {
+            q_base[it] = qb + (int64_t)frag_row(2 * it) * g.K;
+            asm volatile("" : "+s"(q_base[it]));
+        }
     };
-    tile_bases(xcd_first + slot, p_cur, q_cur);
+    tile_bases(xcd_first + slot);
     // after the copies of one K-step; past the last tile the stream re-reads that tile's first K-steps
     // (harmless, and no step needs a special case)
     auto advance_copy = [&]() {
         copy_k0 += kBK;
-        p_cur += kBK;
-        q_cur += kBK;
+        vp += kBK;
+        vq += kBK;
+        if constexpr (NJ == 7) {
+            vq3 += kBK;
+            vq6 += kBK;
+        }
         if (copy_k0 == k_total) {
             copy_k0 = 0;
+            vp -= (uint32_t)k_total;
+            vq -= (uint32_t)k_total;
+            if constexpr (NJ == 7) {
+                vq3 -= (uint32_t)k_total;
+                vq6 -= (uint32_t)k_total;
+            }
             if (copy_tile + 1 < my_tiles) ++copy_tile;
-            tile_bases(xcd_first + slot + copy_tile * tile_stride, p_cur, q_cur);
+            tile_bases(xcd_first + slot + copy_tile * tile_stride);
         }
     };
-    // Copy number c of a K-step, c = 0 .. 2*ITERS-1: first the b-rows slabs, then the a-rows slabs.  Written
-    // as an asm statement to get the addressing form "scalar base + 32-bit lane offset" (no vector address
-    // arithmetic between the matrix instructions); M0 carries the LDS destination of the wave.
+    // Copy number c of a K-step, c = 0 .. COPIES-1: first the b-rows slabs, then the a-rows slabs, as two asm
+    // statements.  set_m0 computes the LDS destination of the wave's part of the slab into M0 and hands it to the
+    // compiler as a value living in M0; issue_copy consumes that value.  Both are modelled operands, so the compiler
+    // keeps M0 intact between the two.  The hardware needs one instruction between a write of M0 and the copy that
+    // uses it: the callers place a matrix instruction or an LDS read there (issue_copy_nop carries an s_nop of its
+    // own for places that have none).  The compiler does not know that issue_copy is a memory instruction reading
+    // scalar registers and would not keep the 5 wait states such an instruction needs after a vector instruction
+    // wrote one of them (v_readlane reloading a spilled scalar): the kernel is written so that no scalar is spilled,
+    // and tests/test_asm_hazards.py checks the generated code for both distances.
     const uint32_t lds_wave = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds + wave * 1024;
-    const int64_t slab_p = (int64_t)32 * g.K;
-    auto issue_load = [&](int c, int stage_ofs) {
-        const uint8_t* src;
-        uint32_t dst, lane_ofs;
+    // c_tag / stage_tag: integral constants (copy number, byte offset of the LDS stage): the compile-time part of
+    // the destination is an immediate of the add
+    auto set_m0 = [&](auto c_tag, auto stage_tag) -> uint32_t {
+        constexpr int C = decltype(c_tag)::value, STAGE_OFS = decltype(stage_tag)::value;
+        constexpr int DST = C < ITERS ? STAGE_OFS + C * T * 16 : STAGE_OFS + P_BYTES + (C - ITERS) * T * 16;
+        uint32_t tok;
+        asm volatile("s_add_i32 %0, %1, %2" : "={m0}"(tok) : "s"(lds_wave), "n"(DST));
+        return tok;
+    };
+    auto copy_src = [&](int c, const uint8_t*& src, uint32_t& lane_ofs) {
         if (c < ITERS) {
-            src = p_cur + c * slab_p;
-            dst = lds_wave + stage_ofs + c * T * 16;
-            lane_ofs = p_lane;
+            src = p_base[c];
+            lane_ofs = vp;
         } else {
-            // slab `it` covers LDS rows 32 it .. 32 it + 31: fragments 2 it and 2 it + 1
-            const int it = c - ITERS;
-            src = q_cur + (int64_t)frag_row(2 * it) * g.K;
-            dst = lds_wave + stage_ofs + P_BYTES + it * T * 16;
-            lane_ofs = (NJ == 7 && it == 3) ? q_lane_3 : (NJ == 7 && it == 6) ? q_lane_6 : q_lane;
+            const int it = c - ITERS;  // slab `it` covers LDS rows 32 it .. 32 it + 31: fragments 2 it and 2 it + 1
+            src = q_base[it];
+            lane_ofs = (NJ == 7 && it == 3) ? vq3 : (NJ == 7 && it == 6) ? vq6 : vq;
         }
-        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                     :
-                     : "v"(lane_ofs), "s"(src), "s"(dst)
-                     : "memory", "m0");
+    };
+    auto issue_copy = [&](int c, uint32_t tok) {
+        const uint8_t* src;
+        uint32_t lane_ofs;
+        copy_src(c, src, lane_ofs);
+        asm volatile("global_load_lds_dwordx4 %0, %1" : : "v"(lane_ofs), "s"(src), "{m0}"(tok) : "memory");
+    };
+    auto issue_copy_nop = [&](auto c_tag, auto stage_tag) {
+        const uint8_t* src;
+        uint32_t lane_ofs;
+        copy_src(decltype(c_tag)::value, src, lane_ofs);
+        const uint32_t tok = set_m0(c_tag, stage_tag);
+        asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(lane_ofs), "s"(src), "{m0}"(tok) : "memory");
     };
 
     const int sw = (l16 >> 1) & 7;
@@ -715,11 +771,9 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
 
     // prologue of the stream: the first two K-steps of the first tile
     constexpr int COPIES = ITERS + ITERS_Q;  // per K-step and lane
-#pragma unroll
-    for (int c = 0; c < COPIES; ++c) issue_load(c, 0);
+    static_for<0, COPIES>([&](auto c) { issue_copy_nop(c, std::integral_constant<int, 0>{}); });
     advance_copy();
-#pragma unroll
-    for (int c = 0; c < COPIES; ++c) issue_load(c, STAGE);
+    static_for<0, COPIES>([&](auto c) { issue_copy_nop(c, std::integral_constant<int, STAGE>{}); });
     advance_copy();
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(COPIES) : "memory");
     __syncthreads();
@@ -740,29 +794,33 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         constexpr bool FIRST = decltype(first_tag)::value;
         const uint8_t* cur = lds + PAR * STAGE;
         const uint8_t* nxt = lds + (1 - PAR) * STAGE;
-#pragma unroll
-        for (int i = 0; i < NF; ++i) {
-#pragma unroll
-            for (int j = 0; j < NJ; ++j) {
+        constexpr std::integral_constant<int, PAR * STAGE> refill{};  // the stage this step releases
+        // copies 4 .. COPIES - 1: spread evenly over the matrix instructions of rows 5..7 (with NJ = 8 after every
+        // second one); the write of M0 for a copy sits in front of the matrix instruction the copy follows.  The
+        // CU's one address unit takes 16 cycles per copy instruction and the four waves issue theirs at the same
+        // time; a denser burst backs up into the waves' instruction issue and stalls the matrix instructions
+        // behind it (one copy per instruction over rows 5 and 6: 4 % slower over six large shapes; all sixteen right
+        // after the barrier: 11 %).
+        constexpr int SPREAD = COPIES - 4, SLOTS = 3 * NJ;
+        static_assert(SPREAD <= SLOTS, "not every copy of a K-step has a place in the schedule");
+        static_for<0, NF>([&](auto i_tag) {
+            constexpr int i = decltype(i_tag)::value;
+            static_for<0, NJ>([&](auto j_tag) {
+                constexpr int j = decltype(j_tag)::value;
+                constexpr int p = (i - 5) * NJ + j;  // slot in rows 5..7
+                constexpr bool COPY_HERE = i >= 5 && ((p + 1) * SPREAD / SLOTS > p * SPREAD / SLOTS);
+                constexpr int COPY_C = COPY_HERE ? 4 + p * SPREAD / SLOTS : 0;
+                uint32_t tok = 0;
+                if constexpr (COPY_HERE) tok = set_m0(std::integral_constant<int, COPY_C>{}, refill);
                 if constexpr (FIRST) mfma_first(acc[i][j], fa[i % 4], fb[PAR][j]);
                 else mfma(acc[i][j], fa[i % 4], fb[PAR][j]);
-                // copies 4 .. COPIES - 1: spread evenly over the matrix instructions of rows 5..7 (with NJ = 8 after
-                // every second one).  The CU's one address unit takes 16 cycles per copy instruction and the four
-                // waves issue theirs at the same time; a denser burst backs up into the waves' instruction issue
-                // and stalls the matrix instructions behind it (one copy per instruction over rows 5 and 6: 4 %
-                // slower over six large shapes; all sixteen right after the barrier: 11 %).
-                constexpr int SPREAD = COPIES - 4, SLOTS = 3 * NJ;
-                static_assert(SPREAD <= SLOTS, "not every copy of a K-step has a place in the schedule");
-                if (i >= 5) {
-                    const int p = (i - 5) * NJ + j;
-                    if ((p + 1) * SPREAD / SLOTS > p * SPREAD / SLOTS) issue_load(4 + p * SPREAD / SLOTS, PAR * STAGE);
+                if constexpr (COPY_HERE) issue_copy(COPY_C, tok);
+                if constexpr (i >= 5 && (j == 2 || j == 5)) {  // rows 5..7: fragments 2..7 of the next step
+                    constexpr int f = 2 * (i - 4) + (j == 5 ? 1 : 0);
+                    if constexpr (f < NJ) fb[1 - PAR][f] = read_frag(nxt + q_frag + f * 16 * kBK);
                 }
-                if (i >= 5 && (j == 2 || j == 5)) {  // rows 5..7: fragments 2..7 of the next step
-                    const int f = 2 * (i - 4) + (j == 5 ? 1 : 0);
-                    if (f < NJ) fb[1 - PAR][f] = read_frag(nxt + q_frag + f * 16 * kBK);
-                }
-            }
-            if (i == 4) {
+            });
+            if constexpr (i == 4) {
                 // every read of the current stage has been issued (the last one after row 3); once they
                 // have returned and all waves are here the stage may be overwritten, and the next stage
                 // (copied one step ago) is complete
@@ -780,14 +838,28 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
                     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
                 }
                 __syncthreads();
-#pragma unroll
-                for (int c = 0; c < 4; ++c) issue_load(c, PAR * STAGE);
-                fb[1 - PAR][0] = read_frag(nxt + q_frag);
-                fb[1 - PAR][1] = read_frag(nxt + q_frag + 16 * kBK);
+                // copies 0..3, each with one of the four LDS reads of the next step's first two second-operand
+                // fragments between the write of M0 and the copy
+                const uint8_t* r0 = nxt + q_frag;
+                const uint8_t* r1 = nxt + q_frag + 16 * kBK;
+                uint32_t tok = set_m0(std::integral_constant<int, 0>{}, refill);
+                const v4i lo0 = *reinterpret_cast<const v4i*>(r0 + c0);
+                issue_copy(0, tok);
+                tok = set_m0(std::integral_constant<int, 1>{}, refill);
+                const v4i hi0 = *reinterpret_cast<const v4i*>(r0 + c1);
+                issue_copy(1, tok);
+                tok = set_m0(std::integral_constant<int, 2>{}, refill);
+                const v4i lo1 = *reinterpret_cast<const v4i*>(r1 + c0);
+                issue_copy(2, tok);
+                tok = set_m0(std::integral_constant<int, 3>{}, refill);
+                const v4i hi1 = *reinterpret_cast<const v4i*>(r1 + c1);
+                issue_copy(3, tok);
+                fb[1 - PAR][0] = __builtin_shufflevector(lo0, hi0, 0, 1, 2, 3, 4, 5, 6, 7);
+                fb[1 - PAR][1] = __builtin_shufflevector(lo1, hi1, 0, 1, 2, 3, 4, 5, 6, 7);
             }
-            if (i < 4) fa[i % 4] = read_frag(cur + p_frag + (i + 4) * 16 * kBK);
+            if constexpr (i < 4) fa[i % 4] = read_frag(cur + p_frag + (i + 4) * 16 * kBK);
             else fa[i % 4] = read_frag(nxt + p_frag + (i - 4) * 16 * kBK);
-        }
+        });
         advance_copy();
     };
 
@@ -973,7 +1045,7 @@ __global__ __launch_bounds__(256) void w4_segment_reduce_kernel(GemmArgs g, int 
     const int band = blockIdx.x % 32, tr = blockIdx.x / 32;
     const int t = tr % rem_max, xcd = tr / rem_max;
     int xcd_first, xcd_count;
-    xcd_tile_range((g.N / 256) * (g.M / 256), xcd, xcd_first, xcd_count);
+    xcd_tile_range((g.N / 256) * (g.M / 256), g.xcds, xcd, xcd_first, xcd_count);
     const int rem = xcd_count % tile_stride;
     if (t >= rem) return;
     int n_blk, m_blk;
@@ -1028,11 +1100,16 @@ static int launch_pipe(const GemmArgs& g, int splits, int persistent_grid, hipSt
     return LLMQ_OK;
 }
 
-// Tuning / test hooks: 0 = automatic.  tile: 1 = 256 x 256 tile with 8 waves, 2 = 128 x 128 tile with
-// 4 waves.  splits: forced number of K splits (needs a workspace).
-int g_gemm_tile = 0;
-int g_gemm_splits = 0;
-int g_gemm_persist = -1;  // -1 = automatic, 0 = never, 1 = whenever possible
+// Kernel selection overrides, 0 / -1 = automatic.  They exist only in the test-aid build of this file
+// (LLMQ_TEST_HOOKS), where the parity tests force every kernel instantiation in turn; in the product library
+// they are constants and the dispatch below is a function of its arguments alone.  tile: 1 = 256 x 256 tile with
+// 8 waves, 2 = 128 x 128 tile with 4 waves, 3 = four-wave kernel, 4 / 5 = its 224- / 192-wide tiles.  splits:
+// forced number of K splits (needs a workspace).  persist: -1 = automatic, 0 = never, 1 = whenever possible.
+#ifdef LLMQ_TEST_HOOKS
+static std::atomic<int> g_gemm_tile{0}, g_gemm_splits{0}, g_gemm_persist{-1};
+#else
+constexpr int g_gemm_tile = 0, g_gemm_splits = 0, g_gemm_persist = -1;
+#endif
 
 // Launch plan of the four-wave kernel.  A persistent grid of `grid` workgroups (grid / 8 per XCD) walks
 // tiles256 tiles.  When the last round of an XCD holds only a few tiles, those can be cut into rem_split K
@@ -1045,18 +1122,18 @@ int g_gemm_persist = -1;  // -1 = automatic, 0 = never, 1 = whenever possible
 struct W4Plan {
     int grid, rem_split, k_len, part_per_xcd, rem_max;
 };
-static W4Plan plan_w4(int tiles256, int cus, int M, int N, int K, int forced_split, size_t workspace_bytes) {
-    W4Plan p{tiles256 < cus ? (tiles256 + 7) / 8 * 8 : cus, 1, K, 0, 0};
+static W4Plan plan_w4(int tiles256, int cus, int xcds, int M, int N, int K, int forced_split, size_t workspace_bytes) {
+    W4Plan p{tiles256 < cus ? (tiles256 + xcds - 1) / xcds * xcds : cus, 1, K, 0, 0};
     if (forced_split == 1) return p;
-    const int stride = cus / 8;
-    const int xq = tiles256 / 8, xr = tiles256 % 8;
+    const int stride = cus / xcds;
+    const int xq = tiles256 / xcds, xr = tiles256 % xcds;
     // tiles in the last round of the XCDs (those with one tile more and the others)
     const int rem_hi = xr ? (xq + 1) % stride : 0, rem_lo = xq % stride;
     const int rem_max = rem_hi > rem_lo ? rem_hi : rem_lo;
     if (rem_max == 0) return p;
     const int pairs = K / (2 * kBK);  // segments are whole pairs of K-steps
     const int64_t ws_tiles = (int64_t)(workspace_bytes / (size_t)(256 * 256 * 4));
-    const int rem_total = xr * rem_hi + (8 - xr) * rem_lo;
+    const int rem_total = xr * rem_hi + (xcds - xr) * rem_lo;
     const double stream_us = (double)rem_total * 512.0 * K / (((double)M + N) * K <= 192e6 ? 10e6 : 3.5e6);
     const double tile_us = (double)K / 164.0;
     const double whole_us = tile_us > stream_us ? tile_us : stream_us;
@@ -1065,7 +1142,7 @@ static W4Plan plan_w4(int tiles256, int cus, int M, int N, int K, int forced_spl
     for (int s = 2; s <= stride / rem_max && s <= pairs; ++s) {
         const int seg_pairs = (pairs + s - 1) / s;
         if ((s - 1) * seg_pairs >= pairs) continue;  // would leave the last segment empty
-        if ((int64_t)8 * rem_max * s > ws_tiles) break;
+        if ((int64_t)xcds * rem_max * s > ws_tiles) break;
         if (forced_split > 1) {
             if (s == forced_split) best = s;
             continue;
@@ -1142,11 +1219,13 @@ static SmallPlan plan_small(int M, int N, int K, int cus, bool ok256, bool ok224
 template <typename OutT, int B_FMT>
 static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     LLMQ_REQUIRE(g.M > 0 && g.N > 0 && g.K > 0, "matmul: M, N, K must be positive (got %d, %d, %d)", g.M, g.N, g.K);
-    const int cus = cu_count();
+    const int cus = cu_count(), xcds = xcd_count();
+    g.xcds = xcds;
+    const int force_tile = g_gemm_tile, force_splits = g_gemm_splits, force_persist = g_gemm_persist;
     // The four-wave kernel with 256 x 224 or 256 x 192 tiles: bf16 output without accumulation.
     auto narrow_fits = [&](int width) {
         return std::is_same_v<OutT, uint16_t> && !g.accumulate && g.N % 256 == 0 && g.M % width == 0 &&
-               g.K % (2 * kBK) == 0 && cus % 8 == 0;
+               g.K % (2 * kBK) == 0 && cus % xcds == 0;
     };
     const bool ok224 = narrow_fits(224), ok192 = narrow_fits(192);
     LLMQ_REQUIRE((g.M % 128 == 0 || ok224 || ok192) && g.N % 128 == 0 && g.K % 128 == 0,
@@ -1156,11 +1235,11 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
                  "matmul: all pointers must be 16-byte aligned");
     LLMQ_REQUIRE(workspace != nullptr || workspace_bytes == 0, "matmul: workspace size given without a workspace");
     g.group = 8;
-    int tile = g_gemm_tile;
+    int tile = force_tile;
     LLMQ_REQUIRE(tile >= 0 && tile <= 5, "matmul: unknown tile selector %d", tile);
     const bool fits256 = g.N % 256 == 0 && g.M % 256 == 0;
     LLMQ_REQUIRE((tile != 1 && tile != 3) || fits256, "matmul: the 256 x 256 tile needs M and N divisible by 256");
-    const bool w4_ok = fits256 && g.K % (2 * kBK) == 0 && cus % 8 == 0;
+    const bool w4_ok = fits256 && g.K % (2 * kBK) == 0 && cus % xcds == 0;
     if (tile == 3) {
         LLMQ_REQUIRE(w4_ok, "matmul: the four-wave kernel needs K divisible by 256");
     }
@@ -1180,7 +1259,7 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
     } else if (g.M % 128 != 0) {
         LLMQ_REQUIRE(tile == 0, "matmul: M = %d needs the narrow tile", g.M);
         narrow_nj = ok224 ? 7 : 6;
-    } else if (tile == 0 && g_gemm_splits == 0 && (int64_t)(g.N / 256) * (g.M / 256) < cus) {
+    } else if (tile == 0 && force_splits == 0 && (int64_t)(g.N / 256) * (g.M / 256) < cus) {
         const SmallPlan sp = plan_small(g.M, g.N, g.K, cus, w4_ok, ok224, ok192, workspace ? (int64_t)workspace_bytes : 0);
         if (sp.nj == 8) {
             tile = 3;
@@ -1190,11 +1269,11 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
             tile = 2;
             small_splits = sp.splits;
         }
-    } else if (tile == 0 && w4_ok && g_gemm_splits == 0) {
+    } else if (tile == 0 && w4_ok && force_splits == 0) {
         const int64_t tn = g.N / 256, t256 = tn * (g.M / 256), rem256 = t256 % cus;
         // only where the full tiles' last round would not be cut into K segments anyway (a remainder of 1-2
         // tiles per XCD), and never for less than a round of tiles
-        if (t256 >= cus && (rem256 == 0 || rem256 > cus / 8)) {
+        if (t256 >= cus && (rem256 == 0 || rem256 > cus / xcds)) {
             auto rounds = [&](int64_t tiles) { return (double)((tiles + cus - 1) / cus); };
             double best = rounds(t256) * 8.0;
             if (ok224 && rounds(tn * (g.M / 224)) * 7.0 * 1.08 < best) {
@@ -1209,7 +1288,7 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
             const int tiles = (g.N / 256) * (g.M / (32 * narrow_nj));
             g.rem_split = 1;
             g.part_per_xcd = 0;
-            const int grid = tiles < cus ? (tiles + 7) / 8 * 8 : cus;
+            const int grid = tiles < cus ? (tiles + xcds - 1) / xcds * xcds : cus;
             if (narrow_nj == 7)
                 hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, B_FMT, false, 7>), dim3((unsigned)grid), dim3(256), 0, stream, g);
             else
@@ -1232,7 +1311,7 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
     const int64_t tiles = tile != 2 ? (int64_t)(g.N / 256) * (g.M / 256) : (int64_t)(g.N / 128) * (g.M / 128);
     const int64_t slice_bytes = (int64_t)g.N * g.M * 4;
     const int64_t ws_splits = (int64_t)(workspace_bytes / (size_t)slice_bytes);
-    int splits = tile == 3 ? 1 : g_gemm_splits;  // for the four-wave kernel the knob cuts the last round instead
+    int splits = tile == 3 ? 1 : force_splits;  // for the four-wave kernel the knob cuts the last round instead
     LLMQ_REQUIRE(splits >= 0, "matmul: negative split count %d", splits);
     if (splits == 0 && small_splits > 0) {
         splits = small_splits;
@@ -1258,14 +1337,14 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
     // Persistent walk (one workgroup per compute unit) for the large tile when there is more than one
     // round of tiles; its cross-tile copy stream needs at least two K-steps.
     int persistent_grid = 0;
-    const bool can_persist = tile == 1 && splits == 1 && g.K >= 2 * kBK && cus % 8 == 0;
-    if (can_persist && (g_gemm_persist == 1 || (g_gemm_persist < 0 && tiles > cus))) persistent_grid = cus;
+    const bool can_persist = tile == 1 && splits == 1 && g.K >= 2 * kBK && cus % xcds == 0;
+    if (can_persist && (force_persist == 1 || (force_persist < 0 && tiles > cus))) persistent_grid = cus;
     // The four-wave kernel takes every large-tile launch it can (K a multiple of 256, no K split).
-    if ((tile == 3 || (tile == 1 && g_gemm_tile == 0 && w4_ok)) && splits == 1) {
+    if ((tile == 3 || (tile == 1 && force_tile == 0 && w4_ok)) && splits == 1) {
         const int tiles256 = (g.N / 256) * (g.M / 256);
-        W4Plan plan = plan_w4(tiles256, cus, g.M, g.N, g.K, tile == 3 ? g_gemm_splits : 0, workspace ? workspace_bytes : 0);
-        LLMQ_REQUIRE(tile != 3 || g_gemm_splits <= 1 || plan.rem_split == g_gemm_splits,
-                     "matmul: cannot cut the last round into %d segments (K = %d, workspace %zu bytes)", g_gemm_splits,
+        W4Plan plan = plan_w4(tiles256, cus, xcds, g.M, g.N, g.K, tile == 3 ? force_splits : 0, workspace ? workspace_bytes : 0);
+        LLMQ_REQUIRE(tile != 3 || force_splits <= 1 || plan.rem_split == force_splits,
+                     "matmul: cannot cut the last round into %d segments (K = %d, workspace %zu bytes)", force_splits,
                      g.K, workspace_bytes);
         g.rem_split = plan.rem_split;
         g.k_len = plan.k_len;
@@ -1285,8 +1364,8 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
             hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<float, B_FMT, true>), dim3((unsigned)plan.grid), dim3(256), 0,
                                stream, g);
             LLMQ_HIP_TRY(hipGetLastError());
-            hipLaunchKernelGGL((w4_segment_reduce_kernel<OutT>), dim3((unsigned)(8 * plan.rem_max * 32)), dim3(256), 0,
-                               stream, g, plan.grid / 8, plan.rem_max);
+            hipLaunchKernelGGL((w4_segment_reduce_kernel<OutT>), dim3((unsigned)(xcds * plan.rem_max * 32)), dim3(256), 0,
+                               stream, g, plan.grid / xcds, plan.rem_max);
             LLMQ_HIP_TRY(hipGetLastError());
         }
         return LLMQ_OK;
@@ -1300,7 +1379,7 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
 extern "C" int llmq_gemm_tn_e4m3_bf16(uint16_t* c, const uint8_t* a, const uint8_t* b, const uint16_t* bias_or_null,
                                       const float* sa_or_null, const float* sb_or_null, void* workspace_or_null,
                                       size_t workspace_bytes, int M, int N, int K, int accumulate, void* stream) {
-    llmq::GemmArgs g{c, a, b, bias_or_null, sa_or_null, sb_or_null, M, N, K, 1, accumulate, 8, nullptr, 0, 1, 0};
+    llmq::GemmArgs g{c, a, b, bias_or_null, sa_or_null, sb_or_null, M, N, K, 1, accumulate, 8, nullptr, 0, 1, 0, 8};
     return llmq::gemm_dispatch<uint16_t, 0>(g, workspace_or_null, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
@@ -1308,7 +1387,7 @@ extern "C" int llmq_gemm_tn_e4m3_f32(float* c, const uint8_t* a, const uint8_t* 
                                      int bias_is_bf16, const float* sa_or_null, const float* sb_or_null,
                                      void* workspace_or_null, size_t workspace_bytes, int M, int N, int K,
                                      int accumulate, void* stream) {
-    llmq::GemmArgs g{c, a, b, bias_or_null, sa_or_null, sb_or_null, M, N, K, bias_is_bf16, accumulate, 8, nullptr, 0, 1, 0};
+    llmq::GemmArgs g{c, a, b, bias_or_null, sa_or_null, sb_or_null, M, N, K, bias_is_bf16, accumulate, 8, nullptr, 0, 1, 0, 8};
     return llmq::gemm_dispatch<float, 0>(g, workspace_or_null, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
@@ -1316,7 +1395,7 @@ extern "C" int llmq_gemm_tn_e4m3_e5m2_bf16(uint16_t* c, const uint8_t* a, const 
                                            const uint16_t* bias_or_null, const float* sa_or_null, const float* sb_or_null,
                                            void* workspace_or_null, size_t workspace_bytes, int M, int N, int K,
                                            int accumulate, void* stream) {
-    llmq::GemmArgs g{c, a, b_e5m2, bias_or_null, sa_or_null, sb_or_null, M, N, K, 1, accumulate, 8, nullptr, 0, 1, 0};
+    llmq::GemmArgs g{c, a, b_e5m2, bias_or_null, sa_or_null, sb_or_null, M, N, K, 1, accumulate, 8, nullptr, 0, 1, 0, 8};
     return llmq::gemm_dispatch<uint16_t, 1>(g, workspace_or_null, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
@@ -1324,13 +1403,15 @@ extern "C" int llmq_gemm_tn_e4m3_e5m2_f32(float* c, const uint8_t* a, const uint
                                           int bias_is_bf16, const float* sa_or_null, const float* sb_or_null,
                                           void* workspace_or_null, size_t workspace_bytes, int M, int N, int K,
                                           int accumulate, void* stream) {
-    llmq::GemmArgs g{c, a, b_e5m2, bias_or_null, sa_or_null, sb_or_null, M, N, K, bias_is_bf16, accumulate, 8, nullptr, 0, 1, 0};
+    llmq::GemmArgs g{c, a, b_e5m2, bias_or_null, sa_or_null, sb_or_null, M, N, K, bias_is_bf16, accumulate, 8, nullptr, 0, 1, 0, 8};
     return llmq::gemm_dispatch<float, 1>(g, workspace_or_null, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
-// Tuning / test hooks (not part of the drop-in surface).
-extern "C" void llmq_debug_set_gemm_variant(int tile, int splits) {
+#ifdef LLMQ_TEST_HOOKS
+// Test-aid build only (not part of the drop-in surface, absent from the product library).
+extern "C" __attribute__((visibility("default"))) void llmq_debug_set_gemm_variant(int tile, int splits) {
     llmq::g_gemm_tile = tile;
     llmq::g_gemm_splits = splits;
 }
-extern "C" void llmq_debug_set_gemm_persist(int v) { llmq::g_gemm_persist = v; }
+extern "C" __attribute__((visibility("default"))) void llmq_debug_set_gemm_persist(int v) { llmq::g_gemm_persist = v; }
+#endif

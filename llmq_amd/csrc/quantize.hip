@@ -24,7 +24,7 @@ namespace llmq {
 // piece of 256 * UNROLL vectors (lane t takes vectors t, t + 256, ...).  Many small workgroups with two loads
 // per lane sustain the most HBM bandwidth on tensors no cache holds (310 MB source, rotating buffers:
 // UNROLL 8 / 4 / 2 = 5.44 / 5.69 / 5.89 TB/s; a plain copy kernel gets 5.7), hence UNROLL = 2 below.
-static int g_quantize_unroll = 2;  // 2, 4 or 8; llmq_debug_set_quantize_unroll is the hook the comparison was made with
+constexpr int kQuantizeUnroll = 2;
 
 template <int FMT, int UNROLL>
 __global__ __launch_bounds__(256) void quantize_kernel(uint2* __restrict__ out, float* __restrict__ scale_ptr,
@@ -171,8 +171,6 @@ __global__ __launch_bounds__(256) void quantize_transpose_kernel(uint8_t* __rest
     }
 }
 
-int g_qt_row_major_grid = 1;
-
 template <int FMT>
 static int launch_quantize(uint8_t* out, float* scale_ptr, const uint16_t* in, const float* absmax, int64_t n,
                            hipStream_t stream) {
@@ -190,10 +188,7 @@ static int launch_quantize(uint8_t* out, float* scale_ptr, const uint16_t* in, c
                            reinterpret_cast<const uint4*>(in), absmax, nvec, in + nvec * 8, out + nvec * 8, ntail);
         return LLMQ_OK;
     };
-    int rc;
-    if (g_quantize_unroll == 8) rc = launch(quantize_kernel<FMT, 8>, 8);
-    else if (g_quantize_unroll == 4) rc = launch(quantize_kernel<FMT, 4>, 4);
-    else rc = launch(quantize_kernel<FMT, 2>, 2);
+    const int rc = launch(quantize_kernel<FMT, kQuantizeUnroll>, kQuantizeUnroll);
     if (rc != LLMQ_OK) return rc;
     LLMQ_HIP_TRY(hipGetLastError());
     return LLMQ_OK;
@@ -219,10 +214,7 @@ static int launch_quantize_f32(uint8_t* out, float* scale_ptr, const float* in, 
                            reinterpret_cast<const uint4*>(in), absmax, nvec, in + nvec * 4, out + nvec * 4, ntail);
         return LLMQ_OK;
     };
-    int rc;
-    if (g_quantize_unroll == 8) rc = launch(quantize_f32_kernel<FMT, 8>, 8);
-    else if (g_quantize_unroll == 4) rc = launch(quantize_f32_kernel<FMT, 4>, 4);
-    else rc = launch(quantize_f32_kernel<FMT, 2>, 2);
+    const int rc = launch(quantize_f32_kernel<FMT, kQuantizeUnroll>, kQuantizeUnroll);
     if (rc != LLMQ_OK) return rc;
     LLMQ_HIP_TRY(hipGetLastError());
     return LLMQ_OK;
@@ -249,9 +241,6 @@ extern "C" int llmq_quantize_e5m2_bf16(uint8_t* out, float* scale_or_null, const
     return llmq::launch_quantize<llmq::kE5M2>(out, scale_or_null, in, absmax, n, static_cast<hipStream_t>(stream));
 }
 
-extern "C" void llmq_debug_set_quantize_unroll(int v) { llmq::g_quantize_unroll = v; }
-extern "C" void llmq_debug_set_qt_order(int v) { llmq::g_qt_row_major_grid = v; }
-
 namespace llmq {
 
 template <int FMT, bool BOTH>
@@ -270,7 +259,7 @@ static int launch_quantize_transpose(uint8_t* out, uint8_t* out_plain, float* sc
     const unsigned gy = empty ? 1u : (unsigned)((rows + kQtRows - 1) / kQtRows);
     // Wide tiles (256-byte row segments on the read side) once there are enough of them to fill the chip.
     const int64_t wide_tiles = (int64_t)((cols + 127) / 128) * gy;
-    const bool rm = g_qt_row_major_grid != 0;
+    const bool rm = true;  // workgroups walk along the input rows (see the kernel); the other order serves grids beyond 65535
     const int r = empty ? 0 : rows, c = empty ? 0 : cols;
     if (!empty && cols >= 128 && wide_tiles >= 2LL * cu_count()) {
         const unsigned gx = (unsigned)((cols + 127) / 128);

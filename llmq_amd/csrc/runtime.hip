@@ -31,6 +31,20 @@ int cu_count() {
     return cached[dev];
 }
 
+int xcd_count() {
+    static int cached[64];
+    static std::mutex mu;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 8;
+    std::lock_guard<std::mutex> lock(mu);
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeNumberOfXccs, dev) != hipSuccess || n <= 0) n = 8;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
 }  // namespace llmq
 
 extern "C" const char* llmq_last_error(void) { return llmq::tl_error; }

@@ -103,11 +103,7 @@ __global__ __launch_bounds__(256) void transpose_u8_generic_kernel(uint8_t* __re
     }
 }
 
-int g_transpose_row_major_grid = 1;
-
 }  // namespace llmq
-
-extern "C" void llmq_debug_set_transpose_order(int v) { llmq::g_transpose_row_major_grid = v; }
 
 extern "C" int llmq_transpose_u8(uint8_t* dst, const uint8_t* src, int rows, int cols, void* stream) {
     using namespace llmq;
@@ -118,7 +114,7 @@ extern "C" int llmq_transpose_u8(uint8_t* dst, const uint8_t* src, int rows, int
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (rows % 16 == 0 && cols % 16 == 0 && aligned16(src) && aligned16(dst)) {
         const unsigned gc = (unsigned)((cols + kTrCols - 1) / kTrCols), gr = (unsigned)((rows + kTrRows - 1) / kTrRows);
-        if (g_transpose_row_major_grid && gc <= 65535u) {
+        if (gc <= 65535u) {
             hipLaunchKernelGGL(transpose_u8_kernel<true>, dim3(gr, gc), dim3(256), 0, st, dst, src, rows, cols);
         } else {
             hipLaunchKernelGGL(transpose_u8_kernel<false>, dim3(gc, gr), dim3(256), 0, st, dst, src, rows, cols);

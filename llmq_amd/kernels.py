@@ -111,12 +111,14 @@ def transpose(dst, src, stream=0):
     capi.check(capi.lib.llmq_transpose_u8(d, s, src.shape[0], src.shape[1], _stream(stream)))
 
 
-def matmul(c, a, b, bias, scale_a, scale_b, M, N, K, accumulate=False, stream=0, workspace=None, b_e5m2=False):
+def matmul(c, a, b, bias, scale_a, scale_b, M, N, K, accumulate=False, stream=0, workspace=None, b_e5m2=False, _lib=None):
     """TN matmul in the convention of the reference's kernels.h: row-major a[M,K], b[N,K] (e4m3) give
     row-major c[N,M] = (b @ a.T) * scale_a * scale_b (+ bias[M]) (+ c).  c: bf16 or fp32.
     workspace: optional device byte tensor (the reference passes a 32 MiB one); it enables the
     split-K path for outputs with too few tiles to fill the chip.  b may hold e5m2 codes (the gradient
-    dtype option): a float8_e5m2 tensor, or uint8 with b_e5m2=True."""
+    dtype option): a float8_e5m2 tensor, or uint8 with b_e5m2=True.  _lib: tests pass the test-aid build of
+    the same entry points (capi.testaid()) to force a kernel variant; everyone else leaves it alone."""
+    L = _lib or capi.lib
     pws, ws_bytes = None, 0
     if workspace is not None:
         pws = _dev(workspace, "workspace", (torch.uint8, torch.int8, torch.float32))
@@ -133,15 +135,15 @@ def matmul(c, a, b, bias, scale_a, scale_b, M, N, K, accumulate=False, stream=0,
         pbias = _dev(bias, "bias", (torch.bfloat16,), optional=True)
         if bias is not None and bias.numel() != M:
             raise ValueError("bias must have M elements")
-        fn = capi.lib.llmq_gemm_tn_e4m3_e5m2_bf16 if b_e5m2 else capi.lib.llmq_gemm_tn_e4m3_bf16
-        capi.check(fn(pc, pa, pb, pbias, sa, sb, pws, ws_bytes, M, N, K, int(accumulate), _stream(stream)))
+        fn = L.llmq_gemm_tn_e4m3_e5m2_bf16 if b_e5m2 else L.llmq_gemm_tn_e4m3_bf16
+        capi.check(fn(pc, pa, pb, pbias, sa, sb, pws, ws_bytes, M, N, K, int(accumulate), _stream(stream)), L)
     else:
         pbias = _dev(bias, "bias", (torch.bfloat16, torch.float32), optional=True)
         if bias is not None and bias.numel() != M:
             raise ValueError("bias must have M elements")
         is_bf16 = int(bias is not None and bias.dtype == torch.bfloat16)
-        fn = capi.lib.llmq_gemm_tn_e4m3_e5m2_f32 if b_e5m2 else capi.lib.llmq_gemm_tn_e4m3_f32
-        capi.check(fn(pc, pa, pb, pbias, is_bf16, sa, sb, pws, ws_bytes, M, N, K, int(accumulate), _stream(stream)))
+        fn = L.llmq_gemm_tn_e4m3_e5m2_f32 if b_e5m2 else L.llmq_gemm_tn_e4m3_f32
+        capi.check(fn(pc, pa, pb, pbias, is_bf16, sa, sb, pws, ws_bytes, M, N, K, int(accumulate), _stream(stream)), L)
 
 
 _BIAS_FMT = {torch.float8_e4m3fn: 0, torch.float8_e5m2: 1, torch.bfloat16: 2}

@@ -29,6 +29,19 @@ def test_every_declared_symbol_is_exported(capi):
     assert sorted(capi.EXPORTS) == names
 
 
+def test_product_library_exports_exactly_the_header(capi):
+    """The dynamic symbol table of libllmq_fp8.so is the set of functions include/llmq_fp8.h declares: no tuning
+    knobs, no measurement aids, no C++ internals (those live in the test-aid library, see llmq_amd/build.py)."""
+    import subprocess
+    out = subprocess.run(["nm", "-D", "--defined-only", capi.LIB_PATH], capture_output=True, text=True, check=True).stdout
+    exported = sorted(line.split()[-1] for line in out.splitlines() if line.strip())
+    assert exported == declared_symbols()
+    out = subprocess.run(["nm", "-D", "--defined-only", capi.TESTAID_PATH], capture_output=True, text=True, check=True).stdout
+    aid = {line.split()[-1] for line in out.splitlines() if line.strip()}
+    assert {"llmq_debug_set_gemm_variant", "llmq_debug_set_gemm_persist", "llmq_debug_copy_u8",
+            "llmq_debug_mfma_ceiling"} <= aid
+
+
 def test_version_and_arch(capi):
     assert capi.target_arch() == "gfx950"
     assert capi.version()

@@ -4,11 +4,13 @@ the C ABI, every intermediate compared with the CPU oracle: abs-max, scales and 
 GEMM outputs within the stated tolerance on a deterministic sample of output coordinates plus whole
 boundary rows/columns.  Inputs are seeded: small tensors come from the oracle's counter-based
 generator, large ones from a seeded torch generator on the device (same bytes feed both sides)."""
+import os
+
 import numpy as np
 import pytest
 import torch
 
-from gpu_util import dev_bf16, gemm_check, host_bits
+from gpu_util import dev_bf16, gemm_check, host_bits, report_gemm_error
 
 pytestmark = pytest.mark.gpu
 F8 = torch.float8_e4m3fn
@@ -118,6 +120,8 @@ def check_gemm(O, c, a_codes, b_codes, sa, sb, seed, name, c_old=None):
     scale = np.float32(np.float32(sa) * np.float32(sb))
     mx, fro = gemm_check(got, ex, sabs, scale, c.dtype == torch.bfloat16, extra=extra)
     print("%-28s [%5d x %5d] max-abs err %.3e  rel-Frobenius %.3e" % (name, N, M, mx, fro))
+    cfg = os.environ.get("PYTEST_CURRENT_TEST", "").split("::")[-1].split(" ")[0]
+    report_gemm_error(cfg, name, N, M, a_codes.shape[1], mx, fro, "%d sampled outputs incl. boundary rows/columns" % idx_n.size)
     return mx, fro
 
 

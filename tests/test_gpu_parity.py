@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 import torch
 
-from gpu_util import dev_bf16, dev_scalar, dev_u8, gemm_check, host_bits
+from gpu_util import dev_bf16, dev_scalar, dev_u8, gemm_check, host_bits, report_gemm_error
 
 pytestmark = pytest.mark.gpu
 
@@ -179,13 +179,27 @@ def test_quantize_fp32_input_bit_exact(K, O, fmt, n):
 
 
 # --------------------------------------------------------------------------------------------- GEMM
+_FORCED = {"lib": None}
+
+
 def set_variant(v):
     """v = (tile, splits[, persistent]): tile 0 = automatic, 1 = 256 x 256 (8 waves), 2 = 128 x 128, 3 = 256 x 256
-    (4 waves, 16x16x128 matrix instruction); splits 0 =
-    automatic; persistent -1 = automatic, 0 = one workgroup per tile, 1 = persistent tile walk."""
+    (4 waves, 16x16x128 matrix instruction), 4 / 5 = its 224- / 192-wide tiles; splits 0 = automatic; persistent
+    -1 = automatic, 0 = one workgroup per tile, 1 = persistent tile walk.  The product library has no such
+    switch: a forced variant runs on the test-aid build of the same GEMM source (capi.testaid()), the automatic
+    choice (0, 0) on the product library."""
     from llmq_amd import capi
-    capi.lib.llmq_debug_set_gemm_variant(v[0], v[1])
-    capi.lib.llmq_debug_set_gemm_persist(v[2] if len(v) > 2 else -1)
+    forced = tuple(v) not in ((0, 0), (0, 0, -1))
+    if forced or _FORCED["lib"] is not None:
+        t = capi.testaid()
+        t.llmq_debug_set_gemm_variant(v[0], v[1])
+        t.llmq_debug_set_gemm_persist(v[2] if len(v) > 2 else -1)
+    _FORCED["lib"] = capi.testaid() if forced else None
+
+
+def mm(K, *args, **kw):
+    """K.matmul on whichever library set_variant selected."""
+    return K.matmul(*args, _lib=_FORCED["lib"], **kw)
 
 
 # (tile selector, K splits[, persistent walk]); for the four-wave kernel (tile 3) the second number cuts the
@@ -228,7 +242,7 @@ def run_gemm(K, a, b, M, N, Kd, sa, sb, bias_bits=None, old=None, out_f32=False)
     else:
         c = torch.full((N, M), float("nan"), dtype=dt, device="cuda")
     bias = dev_bf16(bias_bits) if bias_bits is not None else None
-    K.matmul(c, dev_u8(a), dev_u8(b), bias, dev_scalar(sa) if sa is not None else None,
+    mm(K, c, dev_u8(a), dev_u8(b), bias, dev_scalar(sa) if sa is not None else None,
              dev_scalar(sb) if sb is not None else None, M, N, Kd, accumulate=old is not None, workspace=workspace())
     torch.cuda.synchronize()
     return c
@@ -388,7 +402,7 @@ def test_gemm_automatic_choice_sweep(K, O, case):
         c = (torch.from_numpy(old).cuda() if out_f32 else dev_bf16(old)).reshape(N, M).clone()
     else:
         c = torch.full((N, M), float("nan"), dtype=dt, device="cuda")
-    K.matmul(c, dev_u8(a), dev_u8(b), dev_bf16(bias) if use_bias else None, dev_scalar(s), dev_scalar(s), M, N, Kd,
+    mm(K, c, dev_u8(a), dev_u8(b), dev_bf16(bias) if use_bias else None, dev_scalar(s), dev_scalar(s), M, N, Kd,
              accumulate=use_old, workspace=workspace() if with_ws else None)
     got = c.cpu().numpy() if out_f32 else host_bits(c)
     assert np.array_equal(got, want), case
@@ -446,7 +460,7 @@ def test_gemm_four_wave_large_repeatable(K, O, variant, mnk):
         first = None
         for rep in range(8):
             c = torch.full((N, M), float("nan"), dtype=torch.float32, device="cuda")
-            K.matmul(c, ad, bd, None, sa, None, M, N, Kd, workspace=workspace())
+            mm(K, c, ad, bd, None, sa, None, M, N, Kd, workspace=workspace())
             torch.cuda.synchronize()
             if first is None:
                 first = c
@@ -504,7 +518,7 @@ def test_gemm_e5m2_b_operand(K, O, variant):
     try:
         want = O.gemm_tn(a, b, sa=s, sb=s, bias=bias, mt=True, b_e5m2=True)
         c = torch.full((N, M), float("nan"), dtype=torch.bfloat16, device="cuda")
-        K.matmul(c, dev_u8(a), dev_u8(b).view(torch.float8_e5m2), dev_bf16(bias), dev_scalar(s), dev_scalar(s), M, N, Kd,
+        mm(K, c, dev_u8(a), dev_u8(b).view(torch.float8_e5m2), dev_bf16(bias), dev_scalar(s), dev_scalar(s), M, N, Kd,
                  workspace=workspace())
         assert np.array_equal(host_bits(c), want)
         # same integers: the e5m2 result must equal the int64 product, i.e. differ from reading b as e4m3
@@ -516,11 +530,11 @@ def test_gemm_e5m2_b_operand(K, O, variant):
         exact, sumabs = O.gemm_exact(ar, br, b_e5m2=True)
         if variant[0] in (4, 5):
             c16 = torch.empty((N, M), dtype=torch.bfloat16, device="cuda")
-            K.matmul(c16, dev_u8(ar), dev_u8(br), None, dev_scalar(0.25), None, M, N, Kd, workspace=workspace(), b_e5m2=True)
+            mm(K, c16, dev_u8(ar), dev_u8(br), None, dev_scalar(0.25), None, M, N, Kd, workspace=workspace(), b_e5m2=True)
             gemm_check(c16.float().cpu().numpy(), exact, sumabs, 0.25, True)
         else:
             c32 = torch.empty((N, M), dtype=torch.float32, device="cuda")
-            K.matmul(c32, dev_u8(ar), dev_u8(br), None, dev_scalar(0.25), None, M, N, Kd, workspace=workspace(), b_e5m2=True)
+            mm(K, c32, dev_u8(ar), dev_u8(br), None, dev_scalar(0.25), None, M, N, Kd, workspace=workspace(), b_e5m2=True)
             gemm_check(c32.cpu().numpy(), exact, sumabs, 0.25, False)
     finally:
         set_variant((0, 0))
@@ -618,7 +632,7 @@ def test_config1_forward_pipeline(K, O):
     K.abs_max(stats[2:3], wd)
     K.quantize_with_abs_max(xq, stats[1:2], xd, stats[0:1])
     K.quantize_with_abs_max(wq, stats[3:4], wd, stats[2:3])
-    K.matmul(y, wq, xq, None, stats[3:4], stats[1:2], OC, BT, C)       # forward_qmm call, llama_model.cpp:44
+    mm(K, y, wq, xq, None, stats[3:4], stats[1:2], OC, BT, C)       # forward_qmm call, llama_model.cpp:44
     torch.cuda.synchronize()
     st = stats.cpu().numpy()
     ax, aw = O.abs_max_bf16(x), O.abs_max_bf16(w)
@@ -633,6 +647,7 @@ def test_config1_forward_pipeline(K, O):
     got = y.float().cpu().numpy()[idx_n, idx_m]
     scale = np.float32(dw * dx)
     max_abs, fro = gemm_check(got, ex, sabs, scale, True)
+    report_gemm_error("config1", "forward y", BT, OC, C, max_abs, fro, "%d sampled outputs incl. boundary rows/columns" % idx_n.size)
     # closeness to the unquantised product, as a sanity check of the whole path (fp8 noise ~ 3-4 %)
     ref = (O.bf16_to_f32(x)[idx_n[:2000]].astype(np.float64) * O.bf16_to_f32(w)[idx_m[:2000]].astype(np.float64)).sum(1)
     rel = np.linalg.norm(got[:2000] - ref) / np.linalg.norm(ref)
