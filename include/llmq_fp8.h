@@ -169,6 +169,20 @@ int llmq_backward_bias_bf16(uint16_t* dbias, const void* dout, int dout_format, 
                             const float* sb_or_null, float* scratch, size_t scratch_bytes, int BT, int OC, void* stream);
 
 /*
+ * llmq_backward_bias_bf16 for callers that cannot allocate or carry a scratch buffer (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference, whose
+ * callers take the scratch from their bump allocator.  Same arguments minus the scratch, same result bit for bit:
+ * the band sums go to an array built into the library's device code (LLMQ_BACKWARD_BIAS_STATIC_SCRATCH_BYTES per
+ * GPU, held until the process ends); the call allocates and frees nothing.  A shape whose band sums
+ * (llmq_backward_bias_scratch_bytes) exceed that size is refused with LLMQ_ERR_INVALID_ARGUMENT.  All calls on one
+ * GPU share the array: calls that overlap there (different streams, no ordering between them) race; the array
+ * needs no clearing between calls (every call overwrites what it reads).
+ */
+#define LLMQ_BACKWARD_BIAS_STATIC_SCRATCH_BYTES ((size_t)16 << 20)
+int llmq_backward_bias_bf16_static_scratch(uint16_t* dbias, const void* dout, int dout_format, const float* sa_or_null,
+                                           const float* sb_or_null, int BT, int OC, void* stream);
+
+/*
  * SwiGLU producers adjacent to the quantized matmuls.  inp: row-major [B*T, 2*C] bf16, each row [up(C) | gate(C)].
  *     s = 1 / (1 + exp(-gate));   out[bt, c] = bf16((up * gate) * s)
  * abs_max_or_null: if non-NULL, reset and then set to max |out| over the rounded bf16 outputs (NaNs ignored),

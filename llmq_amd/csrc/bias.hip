@@ -13,6 +13,8 @@
 // a chunk are combined through LDS, and the band's partial sums go to the caller's scratch buffer
 // [bands][OC].  A second small kernel adds the bands in index order, applies the scale and updates
 // dbias.
+#include <mutex>
+
 #include "common.hpp"
 
 namespace llmq {
@@ -142,6 +144,41 @@ static int bias_bands(int rows, int chunks) {
     return bands < 1 ? 1 : bands;
 }
 
+// Scratch of the entry point that allocates nothing: band sums [bands][OC] as in the caller-provided buffer of
+// llmq_backward_bias_bf16.  Every GPU the library runs on holds its own copy of this array at its own address
+// until the process ends; host code reaches it only through the address hipGetSymbolAddress returns with that
+// GPU current (the array's name is a host-side stand-in, not a device address).
+constexpr size_t kStaticBiasScratchBytes = LLMQ_BACKWARD_BIAS_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) float static_bias_scratch[kStaticBiasScratchBytes / sizeof(float)];
+
+// Device address of static_bias_scratch on the current device (looked up once per device), or nullptr with the
+// error recorded.
+static float* static_bias_scratch_ptr() {
+    static float* cached[64];
+    static std::mutex mu;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) {
+        hip_fail(e, "hipGetDevice");
+        return nullptr;
+    }
+    if (dev < 0 || dev >= 64) {
+        set_error(LLMQ_ERR_RUNTIME, "backward_bias: device index %d out of range", dev);
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(mu);
+    if (cached[dev] == nullptr) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(static_bias_scratch));
+        if (e != hipSuccess || p == nullptr) {
+            hip_fail(e, "hipGetSymbolAddress(static_bias_scratch)");
+            return nullptr;
+        }
+        cached[dev] = static_cast<float*>(p);
+    }
+    return cached[dev];
+}
+
 }  // namespace llmq
 
 extern "C" int64_t llmq_backward_bias_scratch_bytes(int BT, int OC, int dout_format) {
@@ -191,4 +228,19 @@ extern "C" int llmq_backward_bias_bf16(uint16_t* dbias, const void* dout, int do
                        sa_or_null, sb_or_null);
     LLMQ_HIP_TRY(hipGetLastError());
     return LLMQ_OK;
+}
+
+extern "C" int llmq_backward_bias_bf16_static_scratch(uint16_t* dbias, const void* dout, int dout_format,
+                                                      const float* sa_or_null, const float* sb_or_null, int BT, int OC,
+                                                      void* stream) {
+    using namespace llmq;
+    const int64_t need = llmq_backward_bias_scratch_bytes(BT, OC, dout_format);
+    LLMQ_REQUIRE(need <= (int64_t)kStaticBiasScratchBytes,
+                 "backward_bias (static scratch): [%d x %d] needs %lld bytes of band sums, the built-in scratch holds %zu; "
+                 "use llmq_backward_bias_bf16 with a caller-provided buffer",
+                 BT, OC, (long long)need, kStaticBiasScratchBytes);
+    float* scratch = static_bias_scratch_ptr();
+    if (scratch == nullptr) return LLMQ_ERR_RUNTIME;
+    return llmq_backward_bias_bf16(dbias, dout, dout_format, sa_or_null, sb_or_null, scratch, kStaticBiasScratchBytes, BT,
+                                   OC, stream);
 }

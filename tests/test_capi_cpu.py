@@ -80,6 +80,9 @@ def test_invalid_arguments_are_rejected_without_a_gpu(capi):
     assert b"scratch buffer too small" in L.llmq_last_error()
     assert L.llmq_backward_bias_bf16(p, p, 7, None, None, p, 1 << 20, 8, 64, None) == INV
     assert L.llmq_backward_bias_scratch_bytes(8192, 1152, 0) >= 1152 * 4
+    # the variant with built-in scratch refuses what its array cannot hold, before any GPU call
+    assert L.llmq_backward_bias_bf16_static_scratch(p, p, 0, None, None, 64, 5 << 20, None) == INV
+    assert b"built-in scratch" in L.llmq_last_error()
     with pytest.raises(ValueError):
         capi.check(INV)
     with pytest.raises(RuntimeError):
