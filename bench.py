@@ -51,6 +51,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain 1 GiB copy kernel (reference point for hardware traffic counters)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="rough budget of the CPU baseline sample")
+    ap.add_argument("--hbm-kernels-only", action="store_true",
+                    help="run only the cold-tensor section of the HBM-bound kernels (abs-max, quantize, quantize+transpose, "
+                         "transpose, plain copy) and print its figures: the workload of the profiles named hbm_kernels__*")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (--gpus 1); multi-GPU sharding is a design note, "
@@ -176,6 +179,8 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    if args.hbm_kernels_only:
+        args.steps, args.no_graph, args.no_cpu_baseline = 1, True, True   # nothing but the cold section below
     record[0] = True
     t0 = time.perf_counter()
     for _ in range(args.steps):
@@ -326,8 +331,7 @@ def main():
     # launch, rotating through three distinct 310 MB tensors (930 MB, well beyond the 256 MB last-level cache,
     # so every launch reads from HBM); median and best launch.  The in-step figures above include what the
     # previous kernel left in the cache and the launch gaps of tensors as small as 59 MB.
-    cold = None
-    if not args.no_graph:
+    def cold_section():
         n_h = BT * FFN
         srcs = [t["h"], out["dh"], out["y_up"].view(-1)[:n_h].view(BT, FFN)]
         q_srcs = [q["h"], q["dy_up"].view(-1)[:n_h].view(BT, FFN), q["dy_up"].view(-1)[n_h:].view(BT, FFN)]
@@ -377,6 +381,12 @@ def main():
         qtr(q["h_t"], "h")
         K.quantize_with_abs_max(q["dy_up"], stats["dy_up"][1:2], t["dy_up"], stats["dy_up"][0:1])
         tr(q["dy_up_t"], q["dy_up"])
+        return cold
+
+    cold = cold_section() if (not args.no_graph or args.hbm_kernels_only) else None
+    if args.hbm_kernels_only:
+        print(json.dumps({"hbm_kernels_cold_large_tensor": cold, "peak_GBps": HBM_PEAK_GBS}))
+        return
     if args.calibrate_copy:
         src = torch.randint(0, 255, (1 << 30,), dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)

@@ -87,6 +87,12 @@ int llmq_quantize_e5m2_f32(uint8_t* out, float* scale_or_null, const float* in, 
 int llmq_quantize_transpose_e4m3_bf16(uint8_t* out, float* scale_or_null, const uint16_t* in,
                                       const float* absmax, int rows, int cols, void* stream);
 
+/* fp32-input variant of the above (fp32 master weights / fp32 model dtype); same arithmetic.
+ * Replaces: quantize_and_transpose_with_abs_max(__nv_fp8_e4m3* out, float* scale_ptr, const float* in,
+ *           const float* abs_max, int rows, int cols, ...)  src/kernels/kernels.h:261, src/kernels/quant.cu:135-149,175-189. */
+int llmq_quantize_transpose_e4m3_f32(uint8_t* out, float* scale_or_null, const float* in, const float* absmax, int rows,
+                                     int cols, void* stream);
+
 /*
  * Extension with no counterpart in the reference (it reads the tensor twice instead: quantize_with_abs_max
  * followed by transpose of the codes, src/models/llama_model.cpp:310-331): one read of in[rows, cols] produces
@@ -108,9 +114,10 @@ int llmq_transpose_u8(uint8_t* dst, const uint8_t* src, int rows, int cols, void
  * a[M,K] and b[N,K] (both e4m3, K contiguous) it writes ROW-MAJOR c[N,M]:
  *     c[n,m] = round( (sum_k b[n,k]*a[m,k]) * (sa*sb) + bias[m] + (accumulate ? c[n,m] : 0) )
  * fp32 accumulation, fp32 epilogue, one rounding to the output type.  sa / sb are device fp32
- * scalars or NULL (= 1).  bias is bf16[M] or NULL.  M, N, K must be multiples of 128 (the
- * precondition of the reference's hand-written kernel, src/kernels/gemm_mma.cu:261-263); without
- * accumulation an M that is a multiple of 224 or 192 is served as well, given N and K multiples of 256.
+ * scalars or NULL (= 1).  bias is bf16[M] or NULL.  Any M, N >= 1; K must be a multiple of 16 (16-byte aligned
+ * operand rows, the rule of the reference's default backend, src/kernels/matmul.cpp:55-57).  The fast kernels take
+ * K % 128 == 0 with M % 128 == 0 (bf16 output without accumulation: also M % 224 == 0 or M % 192 == 0) and all but
+ * the last N % 128 rows of c; a general-shape kernel serves those rows and every other shape.
  * Replaces: matmul(nv_bfloat16* c, const __nv_fp8_e4m3* a, const __nv_fp8_e4m3* b,
  *           const nv_bfloat16* bias, const float* scale_a, const float* scale_b, cublasLtHandle_t,
  *           std::byte* ws, size_t ws_size, int M, int N, int K, EMMTranspose::TN, bool accumulate,
@@ -298,13 +305,28 @@ int llmq_precompute_freqs_cis_f16(uint16_t* freqs_cis_host, int dim, int end, fl
  * Replaces: adamw_update(nv_bfloat16* params, const nv_bfloat16* grads, {float|nv_bfloat16}* m, {float|nv_bfloat16}* v,
  *           size_t num_parameters, float learning_rate, float beta1, float beta2, int t, float eps, float weight_decay,
  *           const float* grad_scale, float* abs_max, unsigned int seed, cudaStream_t)
- *           src/kernels/kernels.h:225-235, src/kernels/adamw.cu:18-195.  Not provided: fp32 parameters and the
- *           fp8 first moment with block scales (kernels.h:221,237).
+ *           src/kernels/kernels.h:225-235, src/kernels/adamw.cu:18-195.  Not provided: fp32 parameters
+ *           (kernels.h:221); the e4m3 first moment is llmq_adamw_update_bf16_fp8m below.
  */
 int llmq_adamw_update_bf16(uint16_t* params, const uint16_t* grads, void* m, int m_dtype, void* v, int v_dtype,
                            int64_t num_parameters, float learning_rate, float beta1, float beta2, int t, float eps,
                            float weight_decay, const float* grad_scale, float* abs_max_or_null, unsigned int seed,
                            void* stream);
+
+/*
+ * The same update with the first moment kept as e4m3 codes and one fp32 scale per 128 consecutive elements
+ * (m_scales: ceil(num_parameters / 128) floats), second moment bf16.  m is read as (float)code * m_scales[i / 128];
+ * every block of 128 new values gets the scale absmax / 448 (1 when its absmax is not above 1e-10) and is written
+ * with the reference's stochastic rounding to e4m3 (values outside [2^-6, 448] in magnitude: round to nearest).
+ * Replaces: adamw_update(nv_bfloat16* params, const nv_bfloat16* grads, __nv_fp8_e4m3* m, nv_bfloat16* v,
+ *           size_t num_parameters, float learning_rate, float beta1, float beta2, int t, float eps, float weight_decay,
+ *           const float* grad_scale, float* m_scales, float* abs_max, unsigned int seed, cudaStream_t)
+ *           src/kernels/kernels.h:237-239, src/kernels/adamw.cu:22-66,191-195.
+ */
+int llmq_adamw_update_bf16_fp8m(uint16_t* params, const uint16_t* grads, uint8_t* m_e4m3, float* m_scales, uint16_t* v_bf16,
+                                int64_t num_parameters, float learning_rate, float beta1, float beta2, int t, float eps,
+                                float weight_decay, const float* grad_scale, float* abs_max_or_null, unsigned int seed,
+                                void* stream);
 
 #if defined(__GNUC__)
 #pragma GCC visibility pop

@@ -196,11 +196,19 @@ inline void quantize_and_transpose_with_abs_max(__hip_fp8_e4m3* out, float* scal
     llmq_detail::check(llmq_quantize_transpose_e4m3_bf16(llmq_detail::u8(out), scale_ptr, llmq_detail::u16(in), abs_max,
                                                          rows, cols, stream));
 }
+// fp32 input (src/kernels/kernels.h:261)
+inline void quantize_and_transpose_with_abs_max(__hip_fp8_e4m3* out, float* scale_ptr, const float* in, const float* abs_max,
+                                                int rows, int cols, const hipDeviceProp_t&, hipStream_t stream) {
+    llmq_detail::check(llmq_quantize_transpose_e4m3_f32(llmq_detail::u8(out), scale_ptr, in, abs_max, rows, cols, stream));
+}
 inline void quantize_and_transpose_with_abs_max(Tensor& out, float* scale_ptr, const Tensor& in, const float* abs_max,
                                                 int rows, int cols, const hipDeviceProp_t& dp, hipStream_t stream) {
     if (out.DType == ETensorDType::FP8_E4M3 && in.DType == ETensorDType::BF16)
         quantize_and_transpose_with_abs_max(out.get<__hip_fp8_e4m3>(), scale_ptr, in.get<__hip_bfloat16>(), abs_max, rows,
                                             cols, dp, stream);
+    else if (out.DType == ETensorDType::FP8_E4M3 && in.DType == ETensorDType::FP32)
+        quantize_and_transpose_with_abs_max(out.get<__hip_fp8_e4m3>(), scale_ptr, in.get<float>(), abs_max, rows, cols, dp,
+                                            stream);
     else llmq_detail::unsupported(__func__, out, in);
 }
 
@@ -469,7 +477,8 @@ inline void rope_backward(__hip_bfloat16* dinp, const __hip_bfloat16* dout, cons
 }
 
 // ---- adamw (reference: src/kernels/kernels.h:225-235, src/kernels/adamw.cu) ----------------------------------------
-// bf16 parameters and gradients; moments fp32/fp32, bf16/fp32 or bf16/bf16.  abs_max is merged, not reset.
+// bf16 parameters and gradients; moments fp32/fp32, bf16/fp32, bf16/bf16 or e4m3 (block scales)/bf16.  abs_max is
+// merged, not reset.
 inline void adamw_update(__hip_bfloat16* params, const __hip_bfloat16* grads, float* m, float* v, std::size_t num_parameters,
                          float learning_rate, float beta1, float beta2, int t, float eps, float weight_decay,
                          const float* grad_scale, float* abs_max, unsigned int seed, hipStream_t stream) {
@@ -490,6 +499,16 @@ inline void adamw_update(__hip_bfloat16* params, const __hip_bfloat16* grads, __
     llmq_detail::check(llmq_adamw_update_bf16(llmq_detail::u16(params), llmq_detail::u16(grads), m, 1, v, 1,
                                               (std::int64_t)num_parameters, learning_rate, beta1, beta2, t, eps, weight_decay,
                                               grad_scale, abs_max, seed, stream));
+}
+// e4m3 first moment with one fp32 scale per 128 elements (m_scales), bf16 second moment (kernels.h:237-239)
+inline void adamw_update(__hip_bfloat16* params, const __hip_bfloat16* grads, __hip_fp8_e4m3* m, __hip_bfloat16* v,
+                         std::size_t num_parameters, float learning_rate, float beta1, float beta2, int t, float eps,
+                         float weight_decay, const float* grad_scale, float* m_scales, float* abs_max, unsigned int seed,
+                         hipStream_t stream) {
+    llmq_detail::check(llmq_adamw_update_bf16_fp8m(llmq_detail::u16(params), llmq_detail::u16(grads),
+                                                   reinterpret_cast<std::uint8_t*>(m), m_scales, llmq_detail::u16(v),
+                                                   (std::int64_t)num_parameters, learning_rate, beta1, beta2, t, eps,
+                                                   weight_decay, grad_scale, abs_max, seed, stream));
 }
 
 #endif  // LLMQ_KERNELS_HPP

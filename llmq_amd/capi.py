@@ -17,14 +17,14 @@ LIB_PATH = os.path.join(_HERE, "lib", "libllmq_fp8.so")
 EXPORTS = [
     "llmq_last_error", "llmq_version", "llmq_target_arch",
     "llmq_abs_max_bf16", "llmq_abs_max_f32",
-    "llmq_quantize_e4m3_bf16", "llmq_quantize_e5m2_bf16", "llmq_quantize_transpose_e4m3_bf16",
+    "llmq_quantize_e4m3_bf16", "llmq_quantize_e5m2_bf16", "llmq_quantize_transpose_e4m3_bf16", "llmq_quantize_transpose_e4m3_f32",
     "llmq_transpose_u8", "llmq_gemm_tn_e4m3_bf16", "llmq_gemm_tn_e4m3_f32", "llmq_gemm_tn_e4m3_e5m2_bf16", "llmq_gemm_tn_e4m3_e5m2_f32",
     "llmq_backward_bias_bf16", "llmq_backward_bias_scratch_bytes", "llmq_backward_bias_bf16_static_scratch", "llmq_quantize_both_bf16", "llmq_quantize_e4m3_f32", "llmq_quantize_e5m2_f32",
     "llmq_swiglu_forward_bf16", "llmq_swiglu_forward_quant_bf16", "llmq_swiglu_backward_bf16",
     "llmq_rmsnorm_forward_bf16", "llmq_fused_residual_rmsnorm_forward_bf16",
     "llmq_rmsnorm_backward_bf16", "llmq_rmsnorm_backward_scratch_bytes",
     "llmq_rope_forward_bf16", "llmq_rope_backward_bf16", "llmq_precompute_freqs_cis_f16",
-    "llmq_adamw_update_bf16",
+    "llmq_adamw_update_bf16", "llmq_adamw_update_bf16_fp8m",
 ]
 
 if not os.path.exists(LIB_PATH):
@@ -41,6 +41,7 @@ lib.llmq_abs_max_f32.argtypes = [_vp, _vp, _i64, _vp]
 lib.llmq_quantize_e4m3_bf16.argtypes = [_vp, _vp, _vp, _vp, _i64, _vp]
 lib.llmq_quantize_e5m2_bf16.argtypes = [_vp, _vp, _vp, _vp, _i64, _vp]
 lib.llmq_quantize_transpose_e4m3_bf16.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _vp]
+lib.llmq_quantize_transpose_e4m3_f32.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _vp]
 lib.llmq_quantize_e4m3_f32.argtypes = [_vp, _vp, _vp, _vp, _i64, _vp]
 lib.llmq_quantize_e5m2_f32.argtypes = [_vp, _vp, _vp, _vp, _i64, _vp]
 lib.llmq_quantize_both_bf16.argtypes = [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp]
@@ -62,6 +63,8 @@ lib.llmq_rmsnorm_backward_scratch_bytes.argtypes = [_int]
 lib.llmq_rope_forward_bf16.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _vp]
 lib.llmq_rope_backward_bf16.argtypes = lib.llmq_rope_forward_bf16.argtypes
 lib.llmq_precompute_freqs_cis_f16.argtypes = [_vp, _int, _int, C.c_float]
+lib.llmq_adamw_update_bf16_fp8m.argtypes = [_vp, _vp, _vp, _vp, _vp, _i64, C.c_float, C.c_float, C.c_float, _int, C.c_float,
+                                            C.c_float, _vp, _vp, C.c_uint, _vp]
 lib.llmq_adamw_update_bf16.argtypes = [_vp, _vp, _vp, _int, _vp, _int, _i64, C.c_float, C.c_float, C.c_float, _int, C.c_float,
                                        C.c_float, _vp, _vp, C.c_uint, _vp]
 for _name in EXPORTS[3:]:

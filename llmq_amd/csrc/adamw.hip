@@ -23,6 +23,7 @@
 
 #include "common.hpp"
 #include "absmax_reduce.hpp"
+#include "fp8_encode.hpp"
 
 namespace llmq {
 
@@ -114,7 +115,7 @@ __global__ __launch_bounds__(THREADS) void adamw_kernel(uint4* __restrict__ para
             const float v_new = __builtin_fmaf(a.beta2, v[e], __builtin_fmaf(-a.beta2, g2, g2));
             const uint32_t random = squirrel_noise_5(first + e, a.seed);
             const float m_hat = m_new * a.c1, v_hat = v_new * a.c2;
-            const float quot = __fdiv_rn(m_hat, __fsqrt_rn(v_hat) + a.eps);
+            const float quot = __fdiv_rn(m_hat, sqrt_rn(v_hat) + a.eps);
             const float p_new = __builtin_fmaf(-a.lr, __builtin_fmaf(a.wd, p_old, quot), p_old);
             p_out[e] = sr_bf16(p_new, random);
             m[e] = m_new;
@@ -142,6 +143,97 @@ __global__ __launch_bounds__(THREADS) void adamw_kernel(uint4* __restrict__ para
         } else {
             store_f32x8(reinterpret_cast<uint4*>(v_mem) + 2 * vec, v);
         }
+    }
+    if constexpr (ABSMAX) {
+        const uint32_t lo = fold & 0xFFFFu, hi = fold >> 16;
+        block_min_to_atomic_max(absmax_out, lo < hi ? lo : hi, 0x7F80u, 16);
+    }
+}
+
+// fp32 -> e4m3 code with the reference's stochastic rounding (squirrel_noise.cuh:58-75): outside [2^-6, 448] in
+// magnitude plain round-to-nearest; inside, the 20 bits below e4m3's three mantissa bits are filled with ones
+// (the conversion then rounds away from zero) when they exceed the 20-bit threshold, else cleared.
+__device__ __forceinline__ float sr_e4m3_prepare(float x, uint32_t random) {
+    const float ax = __builtin_fabsf(x);
+    if (ax > 448.f || ax < 0.015625f || x != x) return x;
+    uint32_t bits = __float_as_uint(x);
+    bits = (bits & 0xFFFFFu) > (random & 0xFFFFFu) ? (bits | 0xFFFFFu) : (bits & ~0xFFFFFu);
+    return __uint_as_float(bits);
+}
+
+// First moment as e4m3 codes with one fp32 scale per 128 consecutive elements, second moment bf16
+// (src/kernels/adamw.cu:22-66).  A lane takes 8 parameters, so 16 consecutive lanes share a block scale: the block's
+// abs-max of the new first moment is combined with four xor-shuffles inside each group of 16 lanes.  Lanes beyond
+// the tensor contribute 0 to it.
+template <bool ABSMAX, int THREADS>
+__global__ __launch_bounds__(THREADS) void adamw_fp8m_kernel(uint4* __restrict__ params, const uint4* __restrict__ grads,
+                                                             uint2* __restrict__ m_codes, float* __restrict__ m_scales,
+                                                             uint4* __restrict__ v_mem, int64_t nvec, AdamArgs a,
+                                                             const float* __restrict__ grad_scale,
+                                                             unsigned* __restrict__ absmax_out) {
+    const int64_t vec = (int64_t)blockIdx.x * THREADS + threadIdx.x;
+    const bool active = vec < nvec;
+    uint32_t fold = 0x7F807F80u;
+    float m[8];
+    float blk_max = 0.f;
+    uint32_t p_out[8], v_out[8];
+    if (active) {
+        const float gs = *grad_scale;
+        const uint4 pw = load_nt(&params[vec]), gw = load_nt(&grads[vec]), vw = load_nt(&v_mem[vec]);
+        const uint2 mw = m_codes[vec];
+        const float old_scale = m_scales[vec / 16];
+        const uint32_t pws[4] = {pw.x, pw.y, pw.z, pw.w}, gws[4] = {gw.x, gw.y, gw.z, gw.w}, vws[4] = {vw.x, vw.y, vw.z, vw.w};
+        const uint32_t mws[2] = {mw.x, mw.y};
+        const uint32_t first = (uint32_t)(vec * 8);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const f32x2_aw pair = (e & 2) ? __builtin_amdgcn_cvt_pk_f32_fp8((int)mws[e / 4], true)
+                                          : __builtin_amdgcn_cvt_pk_f32_fp8((int)mws[e / 4], false);
+            const float m_old = pair[e & 1] * old_scale;
+            const float p_old = (e & 1) ? bf16_hi(pws[e / 2]) : bf16_lo(pws[e / 2]);
+            const float v_old = (e & 1) ? bf16_hi(vws[e / 2]) : bf16_lo(vws[e / 2]);
+            const float grad = gs * ((e & 1) ? bf16_hi(gws[e / 2]) : bf16_lo(gws[e / 2]));
+            const float m_new = __builtin_fmaf(a.beta1, m_old, __builtin_fmaf(-a.beta1, grad, grad));
+            const float g2 = grad * grad;
+            const float v_new = __builtin_fmaf(a.beta2, v_old, __builtin_fmaf(-a.beta2, g2, g2));
+            const uint32_t random = squirrel_noise_5(first + e, a.seed);
+            const float m_hat = m_new * a.c1, v_hat = v_new * a.c2;
+            const float quot = __fdiv_rn(m_hat, sqrt_rn(v_hat) + a.eps);
+            const float p_new = __builtin_fmaf(-a.lr, __builtin_fmaf(a.wd, p_old, quot), p_old);
+            p_out[e] = sr_bf16(p_new, random);
+            v_out[e] = sr_bf16(v_new, rotl32(random, 20));
+            m[e] = m_new;
+            const float ma = __builtin_fabsf(m_new);
+            blk_max = blk_max < ma ? ma : blk_max;  // a NaN never replaces the maximum
+        }
+    }
+    // abs-max of the 128-element block: all lanes take part in the shuffles
+#pragma unroll
+    for (int d = 1; d < 16; d *= 2) {
+        const float other = __shfl_xor(blk_max, d, 16);
+        blk_max = blk_max < other ? other : blk_max;
+    }
+    if (active) {
+        float factor = 1.f, scale = 1.f;
+        if (blk_max > 1e-10f) {
+            factor = __fdiv_rn(448.f, blk_max);
+            scale = __fdiv_rn(1.f, factor);
+        }
+        if (vec % 16 == 0) m_scales[vec / 16] = scale;
+        const uint32_t base = squirrel_noise_5((uint32_t)(vec * 8), 51245u);
+        float y[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) y[e] = sr_e4m3_prepare(m[e] * factor, e == 0 ? base : rotl32(base, (7 * e) % 32));
+        uint2 codes;
+        codes.x = encode4<kE4M3>(y[0], y[1], y[2], y[3]);
+        codes.y = encode4<kE4M3>(y[4], y[5], y[6], y[7]);
+        m_codes[vec] = codes;
+        const uint4 pnew = make_uint4(p_out[0] | (p_out[1] << 16), p_out[2] | (p_out[3] << 16), p_out[4] | (p_out[5] << 16),
+                                      p_out[6] | (p_out[7] << 16));
+        store_nt(&params[vec], pnew);
+        if constexpr (ABSMAX) fold = fold_vec(fold, pnew);
+        store_nt(&v_mem[vec], make_uint4(v_out[0] | (v_out[1] << 16), v_out[2] | (v_out[3] << 16), v_out[4] | (v_out[5] << 16),
+                                         v_out[6] | (v_out[7] << 16)));
     }
     if constexpr (ABSMAX) {
         const uint32_t lo = fold & 0xFFFFu, hi = fold >> 16;
@@ -187,6 +279,37 @@ extern "C" int llmq_adamw_update_bf16(uint16_t* params, const uint16_t* grads, v
     else if (v_dtype == 0) LLMQ_ADAM(true, false);
     else LLMQ_ADAM(true, true);
 #undef LLMQ_ADAM
+    LLMQ_HIP_TRY(hipGetLastError());
+    return LLMQ_OK;
+}
+
+// e4m3 first moment with one fp32 scale per 128 elements, bf16 second moment.
+extern "C" int llmq_adamw_update_bf16_fp8m(uint16_t* params, const uint16_t* grads, uint8_t* m_e4m3, float* m_scales,
+                                           uint16_t* v_bf16, int64_t num_parameters, float learning_rate, float beta1,
+                                           float beta2, int t, float eps, float weight_decay, const float* grad_scale,
+                                           float* abs_max_or_null, unsigned int seed, void* stream_) {
+    using namespace llmq;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    LLMQ_REQUIRE(num_parameters >= 0, "adamw_update: negative parameter count %lld", (long long)num_parameters);
+    LLMQ_REQUIRE(num_parameters % 8 == 0, "adamw_update: num_parameters must be divisible by 8 (got %lld)",
+                 (long long)num_parameters);
+    LLMQ_REQUIRE(grad_scale != nullptr, "adamw_update: grad_scale pointer is null");
+    if (num_parameters == 0) return LLMQ_OK;
+    LLMQ_REQUIRE(params && grads && m_e4m3 && m_scales && v_bf16, "adamw_update: null tensor pointer");
+    LLMQ_REQUIRE(aligned16(params) && aligned16(grads) && aligned16(v_bf16) && (reinterpret_cast<uintptr_t>(m_e4m3) & 7u) == 0,
+                 "adamw_update: tensors must be 16-byte aligned (the e4m3 moment 8-byte)");
+    const float c1 = 1.0f / (1.0f - powf(beta1, (float)t)), c2 = 1.0f / (1.0f - powf(beta2, (float)t));
+    const AdamArgs a{learning_rate, beta1, beta2, c1, c2, eps, weight_decay, seed};
+    const int64_t nvec = num_parameters / 8;
+    LLMQ_REQUIRE((nvec + 255) / 256 <= 0x7FFFFFFF, "adamw_update: tensor too large");
+    auto launch = [&](auto kernel, int threads) {
+        hipLaunchKernelGGL(kernel, dim3((unsigned)((nvec + threads - 1) / threads)), dim3(threads), 0, stream,
+                           reinterpret_cast<uint4*>(params), reinterpret_cast<const uint4*>(grads), reinterpret_cast<uint2*>(m_e4m3),
+                           m_scales, reinterpret_cast<uint4*>(v_bf16), nvec, a, grad_scale,
+                           reinterpret_cast<unsigned*>(abs_max_or_null));
+    };
+    if (abs_max_or_null) launch(adamw_fp8m_kernel<true, 1024>, 1024);
+    else launch(adamw_fp8m_kernel<false, 256>, 256);
     LLMQ_HIP_TRY(hipGetLastError());
     return LLMQ_OK;
 }

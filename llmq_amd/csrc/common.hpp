@@ -70,4 +70,20 @@ __device__ __forceinline__ float quant_scale(float absmax) {
     return __fdiv_rn(448.f, a);
 }
 
+// Correctly rounded fp32 square root.  The hardware instruction (what sqrtf / __fsqrt_rn compile to on gfx950) is
+// within one ulp but not always the nearest value (probed: sqrt(0x370b7c3f) returns 0x3b3cf75c, the nearest is
+// 0x3b3cf75d), and the parity claims of the kernels that use a square root are bit for bit.  The neighbours of the
+// hardware result are tested with exact residuals: s is the nearest value iff x - (s - ulp) * s > 0 and
+// x - (s + ulp) * s <= 0.
+__device__ __forceinline__ float sqrt_rn(float x) {
+    float s = __builtin_sqrtf(x);
+    if (s > 0.f && s < __builtin_huge_valf()) {
+        const float down = __uint_as_float(__float_as_uint(s) - 1u), up = __uint_as_float(__float_as_uint(s) + 1u);
+        const float r_down = __builtin_fmaf(-down, s, x), r_up = __builtin_fmaf(-up, s, x);
+        if (r_down <= 0.f) s = down;
+        if (r_up > 0.f) s = up;
+    }
+    return s;
+}
+
 }  // namespace llmq

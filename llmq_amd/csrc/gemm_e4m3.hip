@@ -70,6 +70,7 @@ struct GemmArgs {
     int rem_split;   // four-wave kernel: K segments per tile of an XCD's last, partial round (1 = none)
     int part_per_xcd;  // four-wave kernel: partial tiles reserved per XCD in `partial`
     int xcds;          // accelerator dies of the device (workgroup ids are dealt to them round-robin)
+    int n_first;       // general-shape kernel: first c row of the region it covers (rows n_first .. N - 1)
 };
 
 // XCD x owns a contiguous range of the logical tile sequence (the first total % xcds XCDs one tile more).
@@ -576,8 +577,11 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs g, int spli
 // rounds of 3/4 the work).  Everything below is written for NJ fragments; NJ = 8, 7 and 6 are instantiated, the
 // narrow ones for bf16 output without accumulation.
 // STREAM_OUT: the bf16 stores of the full-width epilogue are non-temporal (see there).
-template <typename OutT, int B_FMT, bool SEG, int NJ = 8, bool STREAM_OUT = true>
+// ODDK: the number of K-steps per tile is odd (K an odd multiple of 128, at least 384; not with SEG): the LDS stage
+// and fb half of a tile's first step then alternate from tile to tile, and the tile loop carries both orders.
+template <typename OutT, int B_FMT, bool SEG, int NJ = 8, bool STREAM_OUT = true, bool ODDK = false>
 __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
+    static_assert(!(SEG && ODDK), "K segments are whole pairs of K-steps");
     constexpr int BLK = 256, T = 256, WT = 128, NF = 8;
     constexpr int WTM = 16 * NJ, BLKM = 2 * WTM;  // columns (first-operand rows) per wave and per tile
     constexpr int P_BYTES = BLK * kBK, STAGE = 2 * P_BYTES;
@@ -706,11 +710,14 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     const uint32_t lds_wave = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds + wave * 1024;
     // c_tag / stage_tag: integral constants (copy number, byte offset of the LDS stage): the compile-time part of
     // the destination is an immediate of the add
+    // ODDK: the stage is a run-time value (stage_rt, see the tile loop) and stage_tag is 0.
+    uint32_t lds_wave_stage = lds_wave;  // ODDK: lds_wave + byte offset of the stage the current K-step releases
     auto set_m0 = [&](auto c_tag, auto stage_tag) -> uint32_t {
         constexpr int C = decltype(c_tag)::value, STAGE_OFS = decltype(stage_tag)::value;
         constexpr int DST = C < ITERS ? STAGE_OFS + C * T * 16 : STAGE_OFS + P_BYTES + (C - ITERS) * T * 16;
         uint32_t tok;
-        asm volatile("s_add_i32 %0, %1, %2" : "={m0}"(tok) : "s"(lds_wave), "n"(DST));
+        if constexpr (ODDK) asm volatile("s_add_i32 %0, %1, %2" : "={m0}"(tok) : "s"(lds_wave_stage), "n"(DST));
+        else asm volatile("s_add_i32 %0, %1, %2" : "={m0}"(tok) : "s"(lds_wave), "n"(DST));
         return tok;
     };
     auto copy_src = [&](int c, const uint8_t*& src, uint32_t& lane_ofs) {
@@ -789,12 +796,18 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     // the step after next go into the stage this step releases: 4 right after the barrier, the rest spread
     // evenly over the matrix instructions of rows 5..7.
     bool pending_stores = false;  // an epilogue without accumulation has just issued its stores
-    auto k_step = [&](auto par_tag, auto first_tag) {
+    [[maybe_unused]] int stage_rt = 0;  // ODDK: byte offset of the LDS stage of the current K-step
+    // par_tag: LDS stage of the step; fp_tag: the half of fb that holds its second-operand fragments (the same
+    // as the stage unless ODDK, see the tile loop).
+    auto k_step = [&](auto par_tag, auto fp_tag, auto first_tag) {
         constexpr int PAR = decltype(par_tag)::value;
+        constexpr int FP = decltype(fp_tag)::value;
         constexpr bool FIRST = decltype(first_tag)::value;
-        const uint8_t* cur = lds + PAR * STAGE;
-        const uint8_t* nxt = lds + (1 - PAR) * STAGE;
-        constexpr std::integral_constant<int, PAR * STAGE> refill{};  // the stage this step releases
+        // the stage this step computes from and then releases to the copies; with ODDK a run-time value
+        const uint8_t* cur = lds + (ODDK ? stage_rt : PAR * STAGE);
+        const uint8_t* nxt = lds + (ODDK ? STAGE - stage_rt : (1 - PAR) * STAGE);
+        constexpr std::integral_constant<int, ODDK ? 0 : PAR * STAGE> refill{};
+        if constexpr (ODDK) lds_wave_stage = lds_wave + (uint32_t)stage_rt;
         // copies 4 .. COPIES - 1: spread evenly over the matrix instructions of rows 5..7 (with NJ = 8 after every
         // second one); the write of M0 for a copy sits in front of the matrix instruction the copy follows.  The
         // CU's one address unit takes 16 cycles per copy instruction and the four waves issue theirs at the same
@@ -812,12 +825,12 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
                 constexpr int COPY_C = COPY_HERE ? 4 + p * SPREAD / SLOTS : 0;
                 uint32_t tok = 0;
                 if constexpr (COPY_HERE) tok = set_m0(std::integral_constant<int, COPY_C>{}, refill);
-                if constexpr (FIRST) mfma_first(acc[i][j], fa[i % 4], fb[PAR][j]);
-                else mfma(acc[i][j], fa[i % 4], fb[PAR][j]);
+                if constexpr (FIRST) mfma_first(acc[i][j], fa[i % 4], fb[FP][j]);
+                else mfma(acc[i][j], fa[i % 4], fb[FP][j]);
                 if constexpr (COPY_HERE) issue_copy(COPY_C, tok);
                 if constexpr (i >= 5 && (j == 2 || j == 5)) {  // rows 5..7: fragments 2..7 of the next step
                     constexpr int f = 2 * (i - 4) + (j == 5 ? 1 : 0);
-                    if constexpr (f < NJ) fb[1 - PAR][f] = read_frag(nxt + q_frag + f * 16 * kBK);
+                    if constexpr (f < NJ) fb[1 - FP][f] = read_frag(nxt + q_frag + f * 16 * kBK);
                 }
             });
             if constexpr (i == 4) {
@@ -854,13 +867,14 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
                 tok = set_m0(std::integral_constant<int, 3>{}, refill);
                 const v4i hi1 = *reinterpret_cast<const v4i*>(r1 + c1);
                 issue_copy(3, tok);
-                fb[1 - PAR][0] = __builtin_shufflevector(lo0, hi0, 0, 1, 2, 3, 4, 5, 6, 7);
-                fb[1 - PAR][1] = __builtin_shufflevector(lo1, hi1, 0, 1, 2, 3, 4, 5, 6, 7);
+                fb[1 - FP][0] = __builtin_shufflevector(lo0, hi0, 0, 1, 2, 3, 4, 5, 6, 7);
+                fb[1 - FP][1] = __builtin_shufflevector(lo1, hi1, 0, 1, 2, 3, 4, 5, 6, 7);
             }
             if constexpr (i < 4) fa[i % 4] = read_frag(cur + p_frag + (i + 4) * 16 * kBK);
             else fa[i % 4] = read_frag(nxt + p_frag + (i - 4) * 16 * kBK);
         });
         advance_copy();
+        if constexpr (ODDK) stage_rt = STAGE - stage_rt;
     };
 
     using std::integral_constant;
@@ -868,14 +882,31 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     constexpr integral_constant<int, 1> P1{};
     constexpr integral_constant<bool, true> Y{};
     constexpr integral_constant<bool, false> NO{};
-    const int KT = k_total / kBK;  // even
+    const int KT = k_total / kBK;  // even, or odd and at least 3 with ODDK
     int logical = xcd_first + slot;
     for (int t = 0; t < my_tiles; ++t) {
-        k_step(P0, Y);
-        k_step(P1, NO);
-        for (int kt = 2; kt < KT; kt += 2) {
-            k_step(P0, NO);
-            k_step(P1, NO);
+        if constexpr (!ODDK) {
+            k_step(P0, P0, Y);
+            k_step(P1, P1, NO);
+            for (int kt = 2; kt < KT; kt += 2) {
+                k_step(P0, P0, NO);
+                k_step(P1, P1, NO);
+            }
+        } else {
+            // An odd number of K-steps: the LDS stage of a tile's first step alternates from tile to tile, so the
+            // stage is a run-time value here (stage_rt, toggled by every step; the tags only name the fb half).  The
+            // last step leaves the next tile's first second-operand fragments in fb half 1; they are moved to half
+            // 0, where every tile starts.
+            k_step(P0, P0, Y);
+            k_step(P1, P1, NO);
+            for (int kt = 3; kt < KT; kt += 2) {
+                k_step(P0, P0, NO);
+                k_step(P1, P1, NO);
+            }
+            k_step(P0, P0, NO);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) fb[0][j] = fb[1][j];
         }
         // the compiler does not know the statements above are matrix instructions: give the last ones time
         // to retire before their results are read (generously: four times the instruction's 32 cycles)
@@ -1078,6 +1109,78 @@ __global__ __launch_bounds__(256) void w4_segment_reduce_kernel(GemmArgs g, int 
     }
 }
 
+// ---- general shapes ---------------------------------------------------------------------------------
+// Any M, N >= 1 and any K that is a multiple of 16 (the 16-byte row alignment the reference's default backend asks
+// for, src/kernels/matmul.cpp:55-57): 64 x 64 output tile per workgroup, 4 waves of 32 x 32 (one
+// v_mfma_f32_32x32x64_f8f6f4 per K-step of 64), rows and K chunks beyond the operands read as zeros, every output
+// element stored on its own.  It serves what the tiled kernels above cannot: an M or K off their lattice (the whole
+// output) and the last N % 128 rows of an otherwise regular output (rows g.n_first .. N - 1).  Simple rather than fast:
+// operands go through registers into a single LDS stage (row stride 80 bytes: the 16-byte reads of 32 consecutive
+// rows spread over all banks), the next K-step's global loads are in flight while the current one is computed.
+template <typename OutT, int B_FMT>
+__global__ __launch_bounds__(256) void gemm_tn_e4m3_edge_kernel(GemmArgs g) {
+    constexpr int TILE = 64, KS = 64, ROW = 80;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * TILE * ROW];
+    const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+    const int wn = wave / 2, wm = wave % 2, l32 = lane % 32, kg = lane / 32;
+    const int n0 = g.n_first + blockIdx.y * TILE, m0 = blockIdx.x * TILE;
+    // copies: thread -> (row tid / 4, 16-byte chunk tid % 4) of both operand tiles
+    const int ld_row = tid / 4, ld_chunk = tid % 4;
+    const bool b_ok = n0 + ld_row < g.N, a_ok = m0 + ld_row < g.M;
+    const uint8_t* b_src = g.b + (int64_t)(b_ok ? n0 + ld_row : 0) * g.K + ld_chunk * 16;
+    const uint8_t* a_src = g.a + (int64_t)(a_ok ? m0 + ld_row : 0) * g.K + ld_chunk * 16;
+    const v4i zero = {0, 0, 0, 0};
+    auto fetch = [&](int k0, v4i& vb, v4i& va) {
+        const bool k_ok = k0 + ld_chunk * 16 < g.K;  // K is a multiple of 16: a chunk is inside or outside as a whole
+        vb = (b_ok && k_ok) ? *reinterpret_cast<const v4i*>(b_src + k0) : zero;
+        va = (a_ok && k_ok) ? *reinterpret_cast<const v4i*>(a_src + k0) : zero;
+    };
+    uint8_t* b_dst = lds + ld_row * ROW + ld_chunk * 16;
+    uint8_t* a_dst = lds + TILE * ROW + ld_row * ROW + ld_chunk * 16;
+    const uint8_t* b_frag = lds + (wn * 32 + l32) * ROW + kg * 32;
+    const uint8_t* a_frag = lds + TILE * ROW + (wm * 32 + l32) * ROW + kg * 32;
+    v16f acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    v4i vb, va;
+    fetch(0, vb, va);
+    for (int k0 = 0; k0 < g.K; k0 += KS) {
+        __syncthreads();  // the previous step's fragment reads are done
+        *reinterpret_cast<v4i*>(b_dst) = vb;
+        *reinterpret_cast<v4i*>(a_dst) = va;
+        __syncthreads();
+        if (k0 + KS < g.K) fetch(k0 + KS, vb, va);
+        const v4i b_lo = *reinterpret_cast<const v4i*>(b_frag), b_hi = *reinterpret_cast<const v4i*>(b_frag + 16);
+        const v4i a_lo = *reinterpret_cast<const v4i*>(a_frag), a_hi = *reinterpret_cast<const v4i*>(a_frag + 16);
+        const v8i fb_ = __builtin_shufflevector(b_lo, b_hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        const v8i fa_ = __builtin_shufflevector(a_lo, a_hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb_, fa_, acc, B_FMT, 0, 0, 0, 0, 0);
+    }
+    // accumulator register r: c row 8 * (r / 4) + 4 * kg + r % 4 of the wave's 32 x 32 block, column l32
+    float scale = g.sa ? *g.sa : 1.f;
+    if (g.sb) scale = scale * *g.sb;
+    const int m = m0 + wm * 32 + l32;
+    if (m >= g.M) return;
+    const float bias = g.bias ? load_bias(g.bias, g.bias_is_bf16, m) : 0.f;
+    OutT* c = reinterpret_cast<OutT*>(g.c);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int n = n0 + wn * 32 + 8 * (r / 4) + 4 * kg + r % 4;
+        if (n >= g.N) continue;
+        float v = acc[r] * scale;
+        if (g.bias) v = v + bias;
+        OutT* dst = c + (int64_t)n * g.M + m;
+        if constexpr (std::is_same_v<OutT, uint16_t>) {
+            if (g.accumulate) v = v + __uint_as_float((uint32_t)*dst << 16);
+            const f32x2_t pr = {v, 0.f};
+            *dst = (uint16_t)(__builtin_bit_cast(uint32_t, __builtin_convertvector(pr, bf16x2_t)) & 0xFFFFu);  // RNE
+        } else {
+            if (g.accumulate) v = v + *dst;
+            *dst = v;
+        }
+    }
+}
+
 // ---- host side ------------------------------------------------------------------------------------
 template <int BLK_N, int BLK_M, int WV_N, int WV_M, typename OutT, int B_FMT>
 static int launch_pipe(const GemmArgs& g, int splits, int persistent_grid, hipStream_t stream) {
@@ -1124,7 +1227,7 @@ struct W4Plan {
 };
 static W4Plan plan_w4(int tiles256, int cus, int xcds, int M, int N, int K, int forced_split, size_t workspace_bytes) {
     W4Plan p{tiles256 < cus ? (tiles256 + xcds - 1) / xcds * xcds : cus, 1, K, 0, 0};
-    if (forced_split == 1) return p;
+    if (forced_split == 1 || K % (2 * kBK) != 0) return p;  // segments are whole pairs of K-steps
     const int stride = cus / xcds;
     const int xq = tiles256 / xcds, xr = tiles256 % xcds;
     // tiles in the last round of the XCDs (those with one tile more and the others)
@@ -1216,32 +1319,72 @@ static SmallPlan plan_small(int M, int N, int K, int cus, bool ok256, bool ok224
     return best;
 }
 
+// One launch of the four-wave kernel's main variant (no K segments); odd_k selects the instance for an odd number of
+// K-steps.
+template <typename OutT, int B_FMT, int NJ, bool STREAM_OUT>
+static void launch_w4(bool odd_k, int grid, const GemmArgs& g, hipStream_t stream) {
+    if (odd_k)
+        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<OutT, B_FMT, false, NJ, STREAM_OUT, true>), dim3((unsigned)grid), dim3(256), 0,
+                           stream, g);
+    else
+        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<OutT, B_FMT, false, NJ, STREAM_OUT, false>), dim3((unsigned)grid), dim3(256), 0,
+                           stream, g);
+}
+
 template <typename OutT, int B_FMT>
 static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     LLMQ_REQUIRE(g.M > 0 && g.N > 0 && g.K > 0, "matmul: M, N, K must be positive (got %d, %d, %d)", g.M, g.N, g.K);
     const int cus = cu_count(), xcds = xcd_count();
     g.xcds = xcds;
     const int force_tile = g_gemm_tile, force_splits = g_gemm_splits, force_persist = g_gemm_persist;
-    // The four-wave kernel with 256 x 224 or 256 x 192 tiles: bf16 output without accumulation.
-    auto narrow_fits = [&](int width) {
-        return std::is_same_v<OutT, uint16_t> && !g.accumulate && g.N % 256 == 0 && g.M % width == 0 &&
-               g.K % (2 * kBK) == 0 && cus % xcds == 0;
-    };
-    const bool ok224 = narrow_fits(224), ok192 = narrow_fits(192);
-    LLMQ_REQUIRE((g.M % 128 == 0 || ok224 || ok192) && g.N % 128 == 0 && g.K % 128 == 0,
-                 "matmul: M, N, K must be divisible by 128 (got %d, %d, %d)", g.M, g.N, g.K);
+    LLMQ_REQUIRE(g.K % 16 == 0, "matmul: K must be a multiple of 16 (rows of the fp8 operands are 16-byte aligned), got %d",
+                 g.K);
     LLMQ_REQUIRE(g.a && g.b && g.c, "matmul: null operand pointer");
     LLMQ_REQUIRE(aligned16(g.a) && aligned16(g.b) && aligned16(g.c) && aligned16(g.bias) && aligned16(workspace),
                  "matmul: all pointers must be 16-byte aligned");
     LLMQ_REQUIRE(workspace != nullptr || workspace_bytes == 0, "matmul: workspace size given without a workspace");
+    // The tiled kernels below work on a lattice: K a multiple of 128, M a multiple of 128 (or, for bf16 output
+    // without accumulation, of 224 or 192) and N a multiple of 128 (256 for the narrow tiles).  Everything else goes
+    // to the general-shape kernel: the whole output when M or K is off the lattice or N is below 128, otherwise the
+    // last N % 128 rows while the tiled kernels take the rows before them (rows of c are independent, so the
+    // split needs nothing but the row count).
+    auto launch_edge = [&](int n_first) -> int {
+        GemmArgs e = g;
+        e.n_first = n_first;
+        const dim3 grid((unsigned)((g.M + 63) / 64), (unsigned)((g.N - n_first + 63) / 64));
+        hipLaunchKernelGGL((gemm_tn_e4m3_edge_kernel<OutT, B_FMT>), grid, dim3(256), 0, stream, e);
+        LLMQ_HIP_TRY(hipGetLastError());
+        return LLMQ_OK;
+    };
+    // K-step counts the four-wave kernel walks: even, or odd from 3 up
+    const bool odd_k = g.K % (2 * kBK) == kBK;
+    const bool w4_k = g.K % kBK == 0 && (!odd_k || g.K >= 3 * kBK);
+    const bool narrow_out = std::is_same_v<OutT, uint16_t> && !g.accumulate && w4_k && cus % xcds == 0;
+    const bool m_narrow = narrow_out && (g.M % 224 == 0 || g.M % 192 == 0);  // served by 256-row tiles only
+    const bool on_lattice = g.K % kBK == 0 && (g.M % 128 == 0 || m_narrow) && g.N >= (g.M % 128 == 0 ? 128 : 256);
+    if (!on_lattice) {
+        LLMQ_REQUIRE(force_tile == 0 && force_splits == 0,
+                     "matmul: M, N, K = %d, %d, %d are off the lattice of the forced kernel variant", g.M, g.N, g.K);
+        return launch_edge(0);
+    }
+    const int n_tail = g.N % (g.M % 128 == 0 ? 128 : 256);
+    if (n_tail != 0) {
+        LLMQ_REQUIRE(force_tile == 0 && force_splits == 0,
+                     "matmul: M, N, K = %d, %d, %d are off the lattice of the forced kernel variant", g.M, g.N, g.K);
+        const int rc = launch_edge(g.N - n_tail);
+        if (rc != LLMQ_OK) return rc;
+        g.N -= n_tail;
+    }
+    auto narrow_fits = [&](int width) { return narrow_out && g.N % 256 == 0 && g.M % width == 0; };
+    const bool ok224 = narrow_fits(224), ok192 = narrow_fits(192);
     g.group = 8;
     int tile = force_tile;
     LLMQ_REQUIRE(tile >= 0 && tile <= 5, "matmul: unknown tile selector %d", tile);
     const bool fits256 = g.N % 256 == 0 && g.M % 256 == 0;
     LLMQ_REQUIRE((tile != 1 && tile != 3) || fits256, "matmul: the 256 x 256 tile needs M and N divisible by 256");
-    const bool w4_ok = fits256 && g.K % (2 * kBK) == 0 && cus % xcds == 0;
+    const bool w4_ok = fits256 && w4_k && cus % xcds == 0;
     if (tile == 3) {
-        LLMQ_REQUIRE(w4_ok, "matmul: the four-wave kernel needs K divisible by 256");
+        LLMQ_REQUIRE(w4_ok, "matmul: the four-wave kernel needs K divisible by 128 and at least 256");
     }
     // The narrow tiles are taken when their whole rounds of 7/8- or 3/4-sized tiles beat the rounds of full tiles
     // by a margin, e.g. M = 3584, N = 8192: 512 tiles of 224 in 2 rounds instead of 448 in 1.75, on paper 12.5 %
@@ -1254,7 +1397,7 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
     if (tile == 4 || tile == 5) {
         LLMQ_REQUIRE(tile == 4 ? ok224 : ok192,
                      "matmul: the narrow tile (256 x %d) needs bf16 output without accumulation, N %% 256 == 0, "
-                     "M %% %d == 0 and K %% 256 == 0", tile == 4 ? 224 : 192, tile == 4 ? 224 : 192);
+                     "M %% %d == 0 and K %% 128 == 0, K >= 256", tile == 4 ? 224 : 192, tile == 4 ? 224 : 192);
         narrow_nj = tile == 4 ? 7 : 6;
     } else if (g.M % 128 != 0) {
         LLMQ_REQUIRE(tile == 0, "matmul: M = %d needs the narrow tile", g.M);
@@ -1289,10 +1432,8 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
             g.rem_split = 1;
             g.part_per_xcd = 0;
             const int grid = tiles < cus ? (tiles + xcds - 1) / xcds * xcds : cus;
-            if (narrow_nj == 7)
-                hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, B_FMT, false, 7>), dim3((unsigned)grid), dim3(256), 0, stream, g);
-            else
-                hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, B_FMT, false, 6>), dim3((unsigned)grid), dim3(256), 0, stream, g);
+            if (narrow_nj == 7) launch_w4<uint16_t, B_FMT, 7, true>(odd_k, grid, g, stream);
+            else launch_w4<uint16_t, B_FMT, 6, true>(odd_k, grid, g, stream);
             LLMQ_HIP_TRY(hipGetLastError());
             return LLMQ_OK;
         }
@@ -1353,12 +1494,12 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
         // operands and output together within the last-level cache: ordinary output stores (see the epilogue)
         const bool cached_out = std::is_same_v<OutT, uint16_t> &&
                                 ((int64_t)g.M + g.N) * g.K + (int64_t)g.N * g.M * 2 <= ((int64_t)224 << 20);
-        if (cached_out)
-            hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<OutT, B_FMT, false, 8, false>), dim3((unsigned)plan.grid), dim3(256), 0,
-                               stream, g);
-        else
-            hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<OutT, B_FMT, false>), dim3((unsigned)plan.grid), dim3(256), 0, stream,
-                               g);
+        if constexpr (std::is_same_v<OutT, uint16_t>) {
+            if (cached_out) launch_w4<uint16_t, B_FMT, 8, false>(odd_k, plan.grid, g, stream);
+            else launch_w4<uint16_t, B_FMT, 8, true>(odd_k, plan.grid, g, stream);
+        } else {
+            launch_w4<OutT, B_FMT, 8, true>(odd_k, plan.grid, g, stream);
+        }
         LLMQ_HIP_TRY(hipGetLastError());
         if (plan.rem_split > 1) {
             hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<float, B_FMT, true>), dim3((unsigned)plan.grid), dim3(256), 0,
@@ -1379,7 +1520,7 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
 extern "C" int llmq_gemm_tn_e4m3_bf16(uint16_t* c, const uint8_t* a, const uint8_t* b, const uint16_t* bias_or_null,
                                       const float* sa_or_null, const float* sb_or_null, void* workspace_or_null,
                                       size_t workspace_bytes, int M, int N, int K, int accumulate, void* stream) {
-    llmq::GemmArgs g{c, a, b, bias_or_null, sa_or_null, sb_or_null, M, N, K, 1, accumulate, 8, nullptr, 0, 1, 0, 8};
+    llmq::GemmArgs g{c, a, b, bias_or_null, sa_or_null, sb_or_null, M, N, K, 1, accumulate, 8, nullptr, 0, 1, 0, 8, 0};
     return llmq::gemm_dispatch<uint16_t, 0>(g, workspace_or_null, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
@@ -1387,7 +1528,7 @@ extern "C" int llmq_gemm_tn_e4m3_f32(float* c, const uint8_t* a, const uint8_t* 
                                      int bias_is_bf16, const float* sa_or_null, const float* sb_or_null,
                                      void* workspace_or_null, size_t workspace_bytes, int M, int N, int K,
                                      int accumulate, void* stream) {
-    llmq::GemmArgs g{c, a, b, bias_or_null, sa_or_null, sb_or_null, M, N, K, bias_is_bf16, accumulate, 8, nullptr, 0, 1, 0, 8};
+    llmq::GemmArgs g{c, a, b, bias_or_null, sa_or_null, sb_or_null, M, N, K, bias_is_bf16, accumulate, 8, nullptr, 0, 1, 0, 8, 0};
     return llmq::gemm_dispatch<float, 0>(g, workspace_or_null, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
@@ -1395,7 +1536,7 @@ extern "C" int llmq_gemm_tn_e4m3_e5m2_bf16(uint16_t* c, const uint8_t* a, const 
                                            const uint16_t* bias_or_null, const float* sa_or_null, const float* sb_or_null,
                                            void* workspace_or_null, size_t workspace_bytes, int M, int N, int K,
                                            int accumulate, void* stream) {
-    llmq::GemmArgs g{c, a, b_e5m2, bias_or_null, sa_or_null, sb_or_null, M, N, K, 1, accumulate, 8, nullptr, 0, 1, 0, 8};
+    llmq::GemmArgs g{c, a, b_e5m2, bias_or_null, sa_or_null, sb_or_null, M, N, K, 1, accumulate, 8, nullptr, 0, 1, 0, 8, 0};
     return llmq::gemm_dispatch<uint16_t, 1>(g, workspace_or_null, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
@@ -1403,7 +1544,7 @@ extern "C" int llmq_gemm_tn_e4m3_e5m2_f32(float* c, const uint8_t* a, const uint
                                           int bias_is_bf16, const float* sa_or_null, const float* sb_or_null,
                                           void* workspace_or_null, size_t workspace_bytes, int M, int N, int K,
                                           int accumulate, void* stream) {
-    llmq::GemmArgs g{c, a, b_e5m2, bias_or_null, sa_or_null, sb_or_null, M, N, K, bias_is_bf16, accumulate, 8, nullptr, 0, 1, 0, 8};
+    llmq::GemmArgs g{c, a, b_e5m2, bias_or_null, sa_or_null, sb_or_null, M, N, K, bias_is_bf16, accumulate, 8, nullptr, 0, 1, 0, 8, 0};
     return llmq::gemm_dispatch<float, 1>(g, workspace_or_null, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 

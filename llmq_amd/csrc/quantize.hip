@@ -15,6 +15,8 @@
 // wave; the transposing kernel stages a [64 or 128 cols] x [256 rows] tile of fp8 codes in LDS
 // (row stride 65 dwords: conflict-free for both the dword writes and the dword reads) so that the
 // stores along the transposed rows are 256-byte contiguous per 16 lanes.
+#include <type_traits>
+
 #include "common.hpp"
 #include "fp8_encode.hpp"
 
@@ -89,11 +91,12 @@ constexpr int kQtStride = 65;      // LDS row stride in dwords (64 dwords of pay
 // NCH = number of 8-column chunks per tile: the tile is [kQtRows rows] x [8*NCH cols].
 // BOTH: the untransposed codes are written as well (out_plain[r*cols + c]), from the same single read of
 // the input: 8 bytes per lane and row, 8*NCH contiguous bytes per row segment.
-template <int FMT, int NCH, bool ROW_MAJOR_GRID, bool BOTH>
+// InT: uint16_t (bf16 patterns) or float (the fp32-input overload, src/kernels/quant.cu:135-149; not with BOTH).
+template <int FMT, int NCH, bool ROW_MAJOR_GRID, bool BOTH, typename InT = uint16_t>
 __global__ __launch_bounds__(256) void quantize_transpose_kernel(uint8_t* __restrict__ out,
                                                                  uint8_t* __restrict__ out_plain,
                                                                  float* __restrict__ scale_ptr,
-                                                                 const uint16_t* __restrict__ in,
+                                                                 const InT* __restrict__ in,
                                                                  const float* __restrict__ absmax, int rows,
                                                                  int cols, int rows_mult16) {
     constexpr int TC = 8 * NCH;
@@ -111,7 +114,37 @@ __global__ __launch_bounds__(256) void quantize_transpose_kernel(uint8_t* __rest
     const int q = t / NCH;
     const int col = c0 + 8 * chunk;
 
-    uint4 v[PASSES][4];
+    constexpr bool F32 = std::is_same_v<InT, float>;
+    static_assert(!(F32 && BOTH), "the plain + transposed variant takes bf16 input");
+    if constexpr (F32) {
+        // 8 columns of a row are two 16-byte pieces; one pass of 4 rows at a time keeps the registers modest
+#pragma unroll
+        for (int p = 0; p < PASSES; ++p) {
+            const int rq = q + QPP * p;
+            uint4 lo[4], hi[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int row = r0 + 4 * rq + j;
+                if (row < rows && col < cols) {
+                    const uint4* src = reinterpret_cast<const uint4*>(in + (int64_t)row * cols + col);
+                    lo[j] = load_nt(src);
+                    hi[j] = load_nt(src + 1);
+                } else {
+                    lo[j] = hi[j] = make_uint4(0, 0, 0, 0);
+                }
+            }
+            auto val = [&](int j, int c) -> float {  // column c (0..7) of row j
+                const uint4& w = c < 4 ? lo[j] : hi[j];
+                const uint32_t bits = (c & 3) == 0 ? w.x : (c & 3) == 1 ? w.y : (c & 3) == 2 ? w.z : w.w;
+                return __uint_as_float(bits);
+            };
+#pragma unroll
+            for (int c = 0; c < 8; ++c)
+                tile[(8 * chunk + c) * kQtStride + rq] = encode4<FMT>(s * val(0, c), s * val(1, c), s * val(2, c), s * val(3, c));
+        }
+    }
+    uint4 v[F32 ? 1 : PASSES][4];
+    if constexpr (!F32) {
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
         const int rq = q + QPP * p;
@@ -125,8 +158,9 @@ __global__ __launch_bounds__(256) void quantize_transpose_kernel(uint8_t* __rest
             }
         }
     }
+    }
 #pragma unroll
-    for (int p = 0; p < PASSES; ++p) {
+    for (int p = 0; p < (F32 ? 0 : PASSES); ++p) {
         const int rq = q + QPP * p;
         const uint32_t w[4][4] = {{v[p][0].x, v[p][0].y, v[p][0].z, v[p][0].w},
                                   {v[p][1].x, v[p][1].y, v[p][1].z, v[p][1].w},
@@ -243,8 +277,8 @@ extern "C" int llmq_quantize_e5m2_bf16(uint8_t* out, float* scale_or_null, const
 
 namespace llmq {
 
-template <int FMT, bool BOTH>
-static int launch_quantize_transpose(uint8_t* out, uint8_t* out_plain, float* scale_or_null, const uint16_t* in,
+template <int FMT, bool BOTH, typename InT = uint16_t>
+static int launch_quantize_transpose(uint8_t* out, uint8_t* out_plain, float* scale_or_null, const InT* in,
                                      const float* absmax, int rows, int cols, hipStream_t st) {
     LLMQ_REQUIRE(rows >= 0 && cols >= 0, "quantize_and_transpose_with_abs_max: negative shape %d x %d", rows, cols);
     LLMQ_REQUIRE(rows % 8 == 0 && cols % 8 == 0,
@@ -264,18 +298,18 @@ static int launch_quantize_transpose(uint8_t* out, uint8_t* out_plain, float* sc
     if (!empty && cols >= 128 && wide_tiles >= 2LL * cu_count()) {
         const unsigned gx = (unsigned)((cols + 127) / 128);
         if (rm && gx <= 65535u)
-            hipLaunchKernelGGL((quantize_transpose_kernel<FMT, 16, true, BOTH>), dim3(gy, gx), dim3(256), 0, st, out,
+            hipLaunchKernelGGL((quantize_transpose_kernel<FMT, 16, true, BOTH, InT>), dim3(gy, gx), dim3(256), 0, st, out,
                                out_plain, scale_or_null, in, absmax, r, c, rows_mult16);
         else
-            hipLaunchKernelGGL((quantize_transpose_kernel<FMT, 16, false, BOTH>), dim3(gx, gy), dim3(256), 0, st, out,
+            hipLaunchKernelGGL((quantize_transpose_kernel<FMT, 16, false, BOTH, InT>), dim3(gx, gy), dim3(256), 0, st, out,
                                out_plain, scale_or_null, in, absmax, r, c, rows_mult16);
     } else {
         const unsigned gx = empty ? 1u : (unsigned)((cols + 63) / 64);
         if (rm && gx <= 65535u)
-            hipLaunchKernelGGL((quantize_transpose_kernel<FMT, 8, true, BOTH>), dim3(gy, gx), dim3(256), 0, st, out,
+            hipLaunchKernelGGL((quantize_transpose_kernel<FMT, 8, true, BOTH, InT>), dim3(gy, gx), dim3(256), 0, st, out,
                                out_plain, scale_or_null, in, absmax, r, c, rows_mult16);
         else
-            hipLaunchKernelGGL((quantize_transpose_kernel<FMT, 8, false, BOTH>), dim3(gx, gy), dim3(256), 0, st, out,
+            hipLaunchKernelGGL((quantize_transpose_kernel<FMT, 8, false, BOTH, InT>), dim3(gx, gy), dim3(256), 0, st, out,
                                out_plain, scale_or_null, in, absmax, r, c, rows_mult16);
     }
     LLMQ_HIP_TRY(hipGetLastError());
@@ -288,6 +322,12 @@ extern "C" int llmq_quantize_transpose_e4m3_bf16(uint8_t* out, float* scale_or_n
                                                  const float* absmax, int rows, int cols, void* stream) {
     return llmq::launch_quantize_transpose<llmq::kE4M3, false>(out, nullptr, scale_or_null, in, absmax, rows, cols,
                                                                static_cast<hipStream_t>(stream));
+}
+
+extern "C" int llmq_quantize_transpose_e4m3_f32(uint8_t* out, float* scale_or_null, const float* in, const float* absmax,
+                                                int rows, int cols, void* stream) {
+    return llmq::launch_quantize_transpose<llmq::kE4M3, false, float>(out, nullptr, scale_or_null, in, absmax, rows, cols,
+                                                                      static_cast<hipStream_t>(stream));
 }
 
 extern "C" int llmq_quantize_both_bf16(uint8_t* out, uint8_t* out_transposed, float* scale_or_null, const uint16_t* in,

@@ -88,7 +88,7 @@ __global__ __launch_bounds__(WAVES * 64) void rmsnorm_forward_kernel(uint4* resi
     for (int k = 0; k < NCH; ++k) acc = squares(squares(squares(squares(acc, x[k].x), x[k].y), x[k].z), x[k].w);
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) acc = acc + __shfl_xor(acc, off, kWave);
-    const float s = __fdiv_rn(1.0f, __fsqrt_rn(__fdiv_rn(acc, c_float) + epsilon));
+    const float s = __fdiv_rn(1.0f, sqrt_rn(__fdiv_rn(acc, c_float) + epsilon));
 
     uint32_t fold = 0x7F807F80u;
 #pragma unroll

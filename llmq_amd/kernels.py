@@ -74,14 +74,15 @@ def quantize_with_abs_max(out, scale, x, abs_max, stream=0):
 
 
 def quantize_and_transpose_with_abs_max(out, scale, x, abs_max, stream=0):
-    """x: [rows, cols] bf16 -> out: [cols, rows] e4m3."""
+    """x: [rows, cols] bf16 or fp32 -> out: [cols, rows] e4m3."""
     if x.dim() != 2 or out.dim() != 2 or out.shape[0] != x.shape[1] or out.shape[1] != x.shape[0]:
         raise ValueError("x must be [rows, cols] and out [cols, rows]")
     o = _dev(out, "out", (torch.float8_e4m3fn, torch.uint8))
     s = _dev(scale, "scale", (torch.float32,), optional=True)
-    i = _dev(x, "x", (torch.bfloat16,))
+    i = _dev(x, "x", (torch.bfloat16, torch.float32))
     a = _dev(abs_max, "abs_max", (torch.float32,))
-    capi.check(capi.lib.llmq_quantize_transpose_e4m3_bf16(o, s, i, a, x.shape[0], x.shape[1], _stream(stream)))
+    fn = capi.lib.llmq_quantize_transpose_e4m3_f32 if x.dtype == torch.float32 else capi.lib.llmq_quantize_transpose_e4m3_bf16
+    capi.check(fn(o, s, i, a, x.shape[0], x.shape[1], _stream(stream)))
 
 
 def quantize_with_abs_max_and_transpose(out, out_t, scale, x, abs_max, stream=0):
@@ -310,11 +311,21 @@ def precompute_freqs_cis(dim, end, theta):
 
 def adamw_update(params, grads, m, v, learning_rate, beta1, beta2, t, eps, weight_decay, grad_scale, m_scales=None,
                  abs_max=None, seed=0, stream=0):
-    """In-place AdamW step on bf16 params with fp32 or bf16 moments and stochastic rounding (reference:
-    src/binding/kernel_binding.cpp:536-551).  grad_scale: fp32 device scalar.  abs_max, if given, is merged
-    with max |new params| (not reset).  m_scales (the fp8 first moment's block scales) is not supported."""
-    if m_scales is not None:
-        raise ValueError("adamw_update: the fp8 first moment with block scales is not supported")
+    """In-place AdamW step on bf16 params with stochastic rounding (reference:
+    src/binding/kernel_binding.cpp:536-551).  Moments: fp32 / fp32, bf16 / fp32, bf16 / bf16, or an e4m3 first
+    moment (float8_e4m3fn or uint8 codes) with m_scales, one fp32 scale per 128 elements, and a bf16 second moment.
+    grad_scale: fp32 device scalar.  abs_max, if given, is merged with max |new params| (not reset)."""
+    if m_scales is not None or m.dtype in (torch.float8_e4m3fn, torch.uint8):
+        n = params.numel()
+        if m_scales is None or any(x.numel() != n for x in (grads, m, v)) or m_scales.numel() < (n + 127) // 128:
+            raise ValueError("adamw_update: the e4m3 first moment needs m_scales with one entry per 128 elements")
+        capi.check(capi.lib.llmq_adamw_update_bf16_fp8m(
+            _dev(params, "params", (torch.bfloat16,)), _dev(grads, "grads", (torch.bfloat16,)),
+            _dev(m, "m", (torch.float8_e4m3fn, torch.uint8)), _dev(m_scales, "m_scales", (torch.float32,)),
+            _dev(v, "v", (torch.bfloat16,)), n, float(learning_rate), float(beta1), float(beta2), int(t), float(eps),
+            float(weight_decay), _dev(grad_scale, "grad_scale", (torch.float32,)),
+            _dev(abs_max, "abs_max", (torch.float32,), optional=True), int(seed) & 0xFFFFFFFF, _stream(stream)))
+        return
     n = params.numel()
     if any(x.numel() != n for x in (grads, m, v)):
         raise ValueError("adamw_update: shape mismatch")

@@ -603,6 +603,78 @@ float orc_adamw_update_bf16(uint16_t* params, const uint16_t* grads, void* m_mem
     return amax;
 }
 
+/*
+ * fp32 -> e4m3 with the reference's stochastic rounding (squirrel_noise.cuh:58-75): values beyond +-448 and below
+ * 2^-6 in magnitude are converted with round-to-nearest; otherwise the low 20 bits of the fp32 pattern (everything
+ * below the three mantissa bits e4m3 keeps) are compared with a 20-bit threshold: above it they are filled with
+ * ones (the conversion then rounds away from zero), else cleared (the value is an e4m3 number already).
+ */
+uint8_t orc_stochastic_round_e4m3(float x, uint32_t random) {
+    const float ax = fabsf(x);
+    if (ax > 448.f || ax < 0.015625f) return orc_e4m3_encode(x);
+    if (x != x) return orc_e4m3_encode(x);
+    uint32_t bits = f32_bits(x);
+    bits = (bits & 0xFFFFFu) > (random & 0xFFFFFu) ? (bits | 0xFFFFFu) : (bits & ~0xFFFFFu);
+    return orc_e4m3_encode(bits_f32(bits));
+}
+
+/*
+ * AdamW with the first moment kept as e4m3 codes and one fp32 scale per 128 consecutive elements, bf16 second
+ * moment (src/kernels/adamw.cu:22-66,69-113, the overload of src/kernels/kernels.h:237-240).  m is read as
+ * (float)code * scale[i / 128]; after the update each block of 128 new values gets the scale absmax / 448 (1 when
+ * the block's absmax is not above 1e-10) and is written as stochastic_round_e4m3(m * (448 / absmax)) with the
+ * hash of the first index of the element's 8-vector and seed 51245, rotated left by 7 per position.  The update
+ * itself, the parameters and v are as in orc_adamw_update_bf16 with bf16 moments.  A last block shorter than 128
+ * takes the absmax of the elements it has.  Returns max |new parameter|.
+ */
+float orc_adamw_update_bf16_fp8m(uint16_t* params, const uint16_t* grads, uint8_t* m_codes, float* m_scales, uint16_t* v_mem,
+                                 int64_t n, float lr, float beta1, float beta2, int t, float eps, float wd, float grad_scale,
+                                 uint32_t seed) {
+    const float c1 = 1.0f / (1.0f - powf(beta1, (float)t)), c2 = 1.0f / (1.0f - powf(beta2, (float)t));
+    float amax = 0.f;
+    float m_new_blk[128];
+    for (int64_t b0 = 0; b0 < n; b0 += 128) {
+        const int len = (int)(n - b0 < 128 ? n - b0 : 128);
+        const float old_scale = m_scales[b0 / 128];
+        float blk_max = 0.f;
+        for (int k = 0; k < len; ++k) {
+            const int64_t i = b0 + k;
+            volatile float m_old = orc_e4m3_decode(m_codes[i]) * old_scale;
+            const float v_old = orc_bf16_to_f32(v_mem[i]);
+            const float p_old = orc_bf16_to_f32(params[i]);
+            volatile float grad = grad_scale * orc_bf16_to_f32(grads[i]);
+            const float m_new = fmaf(beta1, m_old, fmaf(-beta1, grad, grad));
+            volatile float g2 = grad * grad;
+            const float v_new = fmaf(beta2, v_old, fmaf(-beta2, g2, g2));
+            const uint32_t random = orc_squirrel_noise_5((uint32_t)i, seed);
+            volatile float m_hat = m_new * c1, v_hat = v_new * c2;
+            volatile float den = sqrtf(v_hat) + eps;
+            volatile float quot = m_hat / den;
+            const float p_new = fmaf(-lr, fmaf(wd, p_old, quot), p_old);
+            params[i] = orc_stochastic_round_bf16(p_new, random);
+            const float pa = fabsf(orc_bf16_to_f32(params[i]));
+            if (pa > amax) amax = pa;
+            v_mem[i] = orc_stochastic_round_bf16(v_new, rotl32(random, 20));
+            m_new_blk[k] = m_new;
+            const float ma = fabsf(m_new);
+            if (blk_max < ma) blk_max = ma;   /* std::max(abs_max, fabs(x)): a NaN never replaces the maximum */
+        }
+        volatile float factor = 1.f, scale = 1.f;
+        if (blk_max > 1e-10f) {
+            factor = 448.f / blk_max;
+            scale = 1.f / factor;
+        }
+        m_scales[b0 / 128] = scale;
+        for (int k = 0; k < len; ++k) {
+            const int64_t i = b0 + k;
+            const uint32_t base = orc_squirrel_noise_5((uint32_t)(i - i % 8), 51245u);
+            volatile float y = m_new_blk[k] * factor;
+            m_codes[i] = orc_stochastic_round_e4m3(y, rotl32(base, 7 * (int)(i % 8)));
+        }
+    }
+    return amax;
+}
+
 /* ------------------------------------------------------------------------------------------------
  * Deterministic synthetic tensors: a counter-based generator (one 64-bit mix per element index),
  * so any slice can be produced independently and the same bytes feed the CPU and the GPU side.

@@ -118,6 +118,15 @@ def lib():
     L.orc_adamw_update_bf16.restype = C.c_float
     L.orc_adamw_update_bf16.argtypes = [u16p, u16p, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int64, C.c_float, C.c_float,
                                         C.c_float, C.c_int, C.c_float, C.c_float, C.c_float, C.c_uint32]
+    L.orc_adamw_update_bf16_fp8m.restype = C.c_float
+    L.orc_adamw_update_bf16_fp8m.argtypes = [u16p, u16p, C.POINTER(C.c_uint8), C.POINTER(C.c_float), u16p, C.c_int64, C.c_float,
+                                             C.c_float, C.c_float, C.c_int, C.c_float, C.c_float, C.c_float, C.c_uint32]
+    L.orc_stochastic_round_e4m3.restype = C.c_uint8
+    L.orc_stochastic_round_e4m3.argtypes = [C.c_float, C.c_uint32]
+    L.orc_stochastic_round_bf16.restype = C.c_uint16
+    L.orc_stochastic_round_bf16.argtypes = [C.c_float, C.c_uint32]
+    L.orc_squirrel_noise_5.restype = C.c_uint32
+    L.orc_squirrel_noise_5.argtypes = [C.c_uint32, C.c_uint32]
     _lib = L
     return L
 
@@ -388,3 +397,17 @@ def adamw_update(params, grads, m, v, lr, beta1, beta2, t, eps, wd, grad_scale, 
     am = lib().orc_adamw_update_bf16(_p(p, C.c_uint16), _p(g, C.c_uint16), mm.ctypes.data, md, vv.ctypes.data, vd, p.size,
                                      lr, beta1, beta2, t, eps, wd, grad_scale, seed)
     return p, mm, vv, np.float32(am)
+
+
+def adamw_update_fp8m(params, grads, m_codes, m_scales, v, lr, beta1, beta2, t, eps, wd, grad_scale, seed):
+    """AdamW with e4m3 first moment + one fp32 scale per 128 elements, bf16 second moment.  params, grads, v: bf16
+    bits; m_codes: uint8; m_scales: float32 [ceil(n / 128)].  Returns new (params, m_codes, m_scales, v, abs-max of
+    the new params); inputs are not modified."""
+    p = np.array(params, dtype=np.uint16, copy=True)
+    g = np.ascontiguousarray(grads, dtype=np.uint16)
+    mc = np.array(m_codes, dtype=np.uint8, copy=True)
+    ms = np.array(m_scales, dtype=np.float32, copy=True)
+    vv = np.array(v, dtype=np.uint16, copy=True)
+    am = lib().orc_adamw_update_bf16_fp8m(_p(p, C.c_uint16), _p(g, C.c_uint16), _p(mc, C.c_uint8), _p(ms, C.c_float),
+                                          _p(vv, C.c_uint16), p.size, lr, beta1, beta2, t, eps, wd, grad_scale, seed)
+    return p, mc, ms, vv, np.float32(am)

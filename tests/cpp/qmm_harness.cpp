@@ -224,11 +224,11 @@ int main(int argc, char** argv) {
         EXPECT(std::memcmp(got.data(), wq.data(), wq.size()) == 0, "weight cache: quantized bytes differ");
     }
 
-    // ---- error behaviour of the shim (reference: gemm_mma.cu:261-263, kernels.cpp:18-24) ----
+    // ---- error behaviour of the shim (reference: matmul.cpp:55-57, kernels.cpp:18-24) ----
     bool threw = false;
-    try { matmul(out, weight, inp.Quant, no_bias, nullptr, nullptr, nullptr, workspace, OC, BT, C + 64, EMMTranspose::TN, false, stream); }
+    try { matmul(out, weight, inp.Quant, no_bias, nullptr, nullptr, nullptr, workspace, OC, BT, C + 8, EMMTranspose::TN, false, stream); }
     catch (const std::invalid_argument&) { threw = true; }
-    EXPECT(threw, "matmul with K %% 128 != 0 must throw std::invalid_argument");
+    EXPECT(threw, "matmul with K %% 16 != 0 (operand rows not 16-byte aligned) must throw std::invalid_argument");
     threw = false;
     try { matmul(out, weight, inp.Quant, no_bias, nullptr, nullptr, nullptr, workspace, OC, BT, C, EMMTranspose::NN, false, stream); }
     catch (const std::invalid_argument&) { threw = true; }

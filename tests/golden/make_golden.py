@@ -19,6 +19,17 @@ gemm_kat.npz     two GEMM cases in the library's convention c[N, M] = b[N, K] . 
                  "rnd":  random non-NaN codes and arbitrary scales; the exact sum of products and the sum of their
                          magnitudes in float64 (every product of two e4m3 values is exact in float64 and so is a
                          sum of 256 of them), to be met within the stated GEMM tolerance.
+adamw_kat.npz    known answers for the optimizer's integer hash and stochastic rounding, and two whole AdamW steps
+                 (bf16 / bf16 moments; e4m3 first moment with 128-element block scales):
+                 "hash":  SquirrelNoise5 (src/kernels/squirrel_noise.cuh:15-36) for a list of (position, seed), with
+                          Python integers reduced mod 2^32 after every step;
+                 "sr":    stochastic rounding of fp32 patterns to bf16 and to e4m3 (squirrel_noise.cuh:47-75) for a
+                          list of (pattern, random): the threshold comparison on Python integers, the final
+                          conversion by the nearest-code search used for fp8_encode.npz (bf16: integer RNE);
+                 "step":  src/kernels/adamw.cu:22-113 on 384 parameters: every fp32 operation through float64 with one
+                          final rounding (innocuous for +, *, /, sqrt, Figueroa), the three fused multiply-adds in exact
+                          rational arithmetic rounded once to fp32; the parameter line is evaluated in its contracted
+                          form fma(-lr, fma(wd, p, q), p), which the reference leaves to its compiler.
 producers.npz    small inputs and float64 results of swiglu (src/kernels/swiglu.cu:20-36), rmsnorm
                  (src/kernels/rmsnorm.cu:22-83) and the rotary embedding (src/kernels/rope.cu:42-100), straight
                  from their formulas; implementations computing in fp32 and rounding to bf16 meet them within
@@ -178,9 +189,180 @@ def make_producers():
     np.savez_compressed(os.path.join(HERE, "producers.npz"), **out)
 
 
+
+# ---------------------------------------------------------------------------------------- AdamW known answers
+M32 = 0xFFFFFFFF
+
+
+def squirrel_noise_5(position, seed):
+    b = position & M32
+    b = (b * 0xd2a80a3f) & M32
+    b = (b + seed) & M32
+    b ^= b >> 9
+    b = (b + 0xa884f197) & M32
+    b ^= b >> 11
+    b = (b * 0x6C736F4B) & M32
+    b ^= b >> 13
+    b = (b + 0xB79F3ABB) & M32
+    b ^= b >> 15
+    b = (b * 0x1b56c4f5) & M32
+    b ^= b >> 17
+    return b
+
+
+def rotl(x, k):
+    k %= 32
+    return ((x << k) | (x >> (32 - k))) & M32 if k else x
+
+
+def f32(x):
+    return float(np.float32(x))
+
+
+def bits_of(x):
+    return int(np.float32(x).view(np.uint32))
+
+
+def float_of(bits):
+    return float(np.uint32(bits).view(np.float32))
+
+
+def bf16_rne_bits(pattern):
+    """fp32 pattern -> bf16 pattern, round to nearest even (finite values)."""
+    return ((pattern + 0x7FFF + ((pattern >> 16) & 1)) >> 16) & 0xFFFF
+
+
+def sr_bf16(x, random):
+    b = bits_of(x)
+    b = (b | 0xFFFF) if (b & 0xFFFF) > (random & 0xFFFF) else (b & ~0xFFFF & M32)
+    return bf16_rne_bits(b)
+
+
+def e4m3_nearest(y):
+    return int(encode_nearest(np.array([y], dtype=np.float32), E4M3)[0])
+
+
+def sr_e4m3(x, random):
+    x = f32(x)
+    if abs(x) > 448.0 or abs(x) < 0.015625:
+        return e4m3_nearest(x)
+    b = bits_of(x)
+    b = (b | 0xFFFFF) if (b & 0xFFFFF) > (random & 0xFFFFF) else (b & ~0xFFFFF & M32)
+    return e4m3_nearest(float_of(b))
+
+
+def round_fraction_to_f32(q):
+    """Exact rational -> nearest fp32 (ties to even), normal range."""
+    from fractions import Fraction
+    if q == 0:
+        return 0.0
+    sign = -1 if q < 0 else 1
+    q = abs(q)
+    e = q.numerator.bit_length() - q.denominator.bit_length()
+    if Fraction(2) ** e > q:
+        e -= 1
+    assert Fraction(2) ** e <= q < Fraction(2) ** (e + 1) and -126 <= e <= 127
+    scaled = q / Fraction(2) ** (e - 23)          # in [2^23, 2^24)
+    n, rem = divmod(scaled.numerator, scaled.denominator)
+    twice = 2 * rem
+    if twice > scaled.denominator or (twice == scaled.denominator and n & 1):
+        n += 1
+    return sign * float(Fraction(n) * Fraction(2) ** (e - 23))
+
+
+def fma32(a, b, c):
+    from fractions import Fraction
+    return round_fraction_to_f32(Fraction(f32(a)) * Fraction(f32(b)) + Fraction(f32(c)))
+
+
+def adamw_step(p_bits, g_bits, m_in, v_bits, fp8m, m_scales, lr, beta1, beta2, t, eps, wd, gs, seed):
+    """One AdamW step on Python numbers.  m_in: bf16 patterns, or e4m3 codes when fp8m."""
+    dec4 = decode_table(E4M3)
+    lr, beta1, beta2, eps, wd, gs = (f32(x) for x in (lr, beta1, beta2, eps, wd, gs))
+    c1 = f32(1.0 / f32(1.0 - f32(np.float32(beta1) ** np.float32(t))))
+    c2 = f32(1.0 / f32(1.0 - f32(np.float32(beta2) ** np.float32(t))))
+    n = len(p_bits)
+    p_out, v_out, m_new = [], [], []
+    for i in range(n):
+        p_old = float_of(int(p_bits[i]) << 16)
+        v_old = float_of(int(v_bits[i]) << 16)
+        if fp8m:
+            m_old = f32(float(dec4[int(m_in[i])]) * f32(m_scales[i // 128]))
+        else:
+            m_old = float_of(int(m_in[i]) << 16)
+        grad = f32(gs * float_of(int(g_bits[i]) << 16))
+        mn = fma32(beta1, m_old, fma32(-beta1, grad, grad))
+        g2 = f32(grad * grad)
+        vn = fma32(beta2, v_old, fma32(-beta2, g2, g2))
+        random = squirrel_noise_5(i, seed)
+        m_hat, v_hat = f32(mn * c1), f32(vn * c2)
+        den = f32(f32(np.sqrt(np.float64(v_hat))) + eps)
+        quot = f32(m_hat / den)
+        pn = fma32(-lr, fma32(wd, p_old, quot), p_old)
+        p_out.append(sr_bf16(pn, random))
+        v_out.append(sr_bf16(vn, rotl(random, 20)))
+        m_new.append(mn)
+    if not fp8m:
+        m_out = [sr_bf16(m_new[i], rotl(squirrel_noise_5(i - i % 8, 51245), 7 * (i % 8))) for i in range(n)]
+        return p_out, m_out, None, v_out
+    m_out, scales = [], []
+    for b0 in range(0, n, 128):
+        blk = m_new[b0:b0 + 128]
+        amax = max(abs(x) for x in blk)
+        factor, scale = 1.0, 1.0
+        if amax > f32(1e-10):
+            factor = f32(448.0 / amax)
+            scale = f32(1.0 / factor)
+        scales.append(scale)
+        for k, x in enumerate(blk):
+            i = b0 + k
+            m_out.append(sr_e4m3(f32(x * factor), rotl(squirrel_noise_5(i - i % 8, 51245), 7 * (i % 8))))
+    return p_out, m_out, scales, v_out
+
+
+def make_adamw_kat():
+    rng = np.random.default_rng(20250)
+    out = {}
+    pos = np.concatenate([[0, 1, 2, 7, 8, 255, 256, 0x7FFFFFFF, 0x80000000, 0xFFFFFFFF],
+                          rng.integers(0, 1 << 32, 54)]).astype(np.uint32)
+    seeds = np.concatenate([[0, 1, 51245, 0xFFFFFFFF], rng.integers(0, 1 << 32, 60)]).astype(np.uint32)
+    out["hash_position"], out["hash_seed"] = pos, seeds
+    out["hash_value"] = np.array([squirrel_noise_5(int(a), int(b)) for a, b in zip(pos, seeds)], dtype=np.uint32)
+    # stochastic rounding: patterns near thresholds and random ones
+    vals = np.concatenate([rng.standard_normal(200) * 10.0 ** rng.uniform(-4, 3, 200),
+                           [0.0, -0.0, 448.0, 449.0, -500.0, 0.015625, 0.0156, -0.0157, 1.0, 1.0625, 447.9, 3e-5]]).astype(np.float32)
+    rnd = rng.integers(0, 1 << 32, vals.size).astype(np.uint32)
+    rnd[:8] = [0, 0xFFFF, 0xFFFFF, 0xFFFFFFFF, 0x8000, 0x80000, 1, 0xFFFE]
+    out["sr_pattern"], out["sr_random"] = vals.view(np.uint32), rnd
+    out["sr_bf16"] = np.array([sr_bf16(float(v), int(r)) for v, r in zip(vals, rnd)], dtype=np.uint16)
+    out["sr_e4m3"] = np.array([sr_e4m3(float(v), int(r)) for v, r in zip(vals, rnd)], dtype=np.uint8)
+    # whole steps
+    n = 384
+    p = f32_to_bf16_rne((rng.standard_normal(n) * 0.05).astype(np.float32))
+    g = f32_to_bf16_rne((rng.standard_normal(n) * 1e-2).astype(np.float32))
+    v = f32_to_bf16_rne((rng.uniform(0, 1, n) ** 4 * 1e-4).astype(np.float32))
+    hyper = dict(lr=3e-3, beta1=0.9, beta2=0.95, t=3, eps=1e-8, wd=0.1, gs=0.5, seed=1234567)
+    out["step_hyper"] = np.array([hyper[k] for k in ("lr", "beta1", "beta2", "t", "eps", "wd", "gs", "seed")], dtype=np.float64)
+    out["step_p"], out["step_g"], out["step_v"] = p, g, v
+    m16 = f32_to_bf16_rne((rng.standard_normal(n) * 5e-3).astype(np.float32))
+    po, mo, _, vo = adamw_step(p, g, m16, v, False, None, **hyper)
+    out["bf16_m"], out["bf16_p_out"], out["bf16_m_out"], out["bf16_v_out"] = m16, np.array(po, np.uint16), np.array(mo, np.uint16), np.array(vo, np.uint16)
+    m8 = rng.integers(0, 256, n).astype(np.uint8)
+    m8[(m8 & 0x7F) == 0x7F] ^= 1
+    m8[256:384] = 0                                   # a block whose new moment comes from the gradient alone
+    g8 = g.copy()
+    g8[256:320] = 0                                   # half of it exactly zero
+    ms = np.array([2.5e-5, 1.0 / 448, 1.0], dtype=np.float32)
+    po, mo, so, vo = adamw_step(p, g8, m8, v, True, ms, **hyper)
+    out["fp8_g"], out["fp8_m"], out["fp8_scales"] = g8, m8, ms
+    out["fp8_p_out"], out["fp8_m_out"], out["fp8_v_out"] = np.array(po, np.uint16), np.array(mo, np.uint8), np.array(vo, np.uint16)
+    out["fp8_scales_out"] = np.array(so, dtype=np.float32)
+    np.savez_compressed(os.path.join(HERE, "adamw_kat.npz"), **out)
+
 if __name__ == "__main__":
     make_fp8_encode()
     make_gemm_kat()
     make_producers()
-    for f in ("fp8_encode.npz", "gemm_kat.npz", "producers.npz"):
+    make_adamw_kat()
+    for f in ("fp8_encode.npz", "gemm_kat.npz", "producers.npz", "adamw_kat.npz"):
         print(f, os.path.getsize(os.path.join(HERE, f)), "bytes")

@@ -62,10 +62,11 @@ def test_invalid_arguments_are_rejected_without_a_gpu(capi):
     assert L.llmq_transpose_u8(p, p, 16, 16, None) == INV                    # in place
     assert L.llmq_transpose_u8(None, p, 16, 16, None) == INV
     assert L.llmq_transpose_u8(p, p, 0, 16, None) == capi.LLMQ_OK            # empty: nothing to do
-    # GEMM: the 128-divisibility rule of the reference's custom kernel (gemm_mma.cu:261-263)
-    assert L.llmq_gemm_tn_e4m3_bf16(p, p, p, None, None, None, None, 0, 128, 128, 64, 0, None) == INV
-    assert b"divisible by 128" in L.llmq_last_error()
-    assert L.llmq_gemm_tn_e4m3_bf16(p, p, p, None, None, None, None, 0, 100, 128, 128, 0, None) == INV
+    # GEMM: rows of the fp8 operands must be 16-byte aligned (src/kernels/matmul.cpp:55-57), i.e. K % 16 == 0;
+    # M and N are free
+    assert L.llmq_gemm_tn_e4m3_bf16(p, p, p, None, None, None, None, 0, 128, 128, 72, 0, None) == INV
+    assert b"multiple of 16" in L.llmq_last_error()
+    assert L.llmq_gemm_tn_e4m3_bf16(p, p, p, None, None, None, None, 0, 0, 128, 128, 0, None) == INV
     assert L.llmq_gemm_tn_e4m3_bf16(p, None, p, None, None, None, None, 0, 128, 128, 128, 0, None) == INV
     assert L.llmq_gemm_tn_e4m3_bf16(p, p + 8, p, None, None, None, None, 0, 128, 128, 128, 0, None) == INV
     assert b"aligned" in L.llmq_last_error()

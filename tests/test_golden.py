@@ -26,7 +26,7 @@ def within_bf16_rounding(bits, exact, slack):
 
 
 def test_fixture_files_are_present():
-    for f in ("fp8_encode.npz", "gemm_kat.npz", "producers.npz", "make_golden.py"):
+    for f in ("fp8_encode.npz", "gemm_kat.npz", "producers.npz", "adamw_kat.npz", "make_golden.py"):
         assert os.path.exists(os.path.join(GOLDEN, f)), f
 
 
@@ -99,3 +99,30 @@ def test_rope(O):
         want = g[key].reshape(out.shape)
         assert within_bf16_rounding(out, want, 2.0 ** -22 * mag)
         assert np.array_equal(out[:, Nq + Nkv:], qkv[:, Nq + Nkv:])      # value heads: copied bit for bit
+
+
+def test_adamw_hash_and_stochastic_rounding_known_answers(O):
+    """SquirrelNoise5 and the stochastic roundings against vectors written with Python integers
+    (src/kernels/squirrel_noise.cuh:15-75)."""
+    g = load("adamw_kat.npz")
+    L = O.lib()
+    for pos, seed, want in zip(g["hash_position"], g["hash_seed"], g["hash_value"]):
+        assert L.orc_squirrel_noise_5(int(pos), int(seed)) == int(want)
+    vals = g["sr_pattern"].view(np.float32)
+    for x, r, w16, w8 in zip(vals, g["sr_random"], g["sr_bf16"], g["sr_e4m3"]):
+        assert L.orc_stochastic_round_bf16(float(x), int(r)) == int(w16), (x, r)
+        assert L.orc_stochastic_round_e4m3(float(x), int(r)) == int(w8), (x, r)
+
+
+def test_adamw_whole_step_known_answers(O):
+    """One AdamW step on 384 parameters, bf16 / bf16 moments and e4m3 first moment with block scales, against the
+    exact-rational evaluation of tests/golden/make_golden.py (src/kernels/adamw.cu:22-113)."""
+    g = load("adamw_kat.npz")
+    lr, b1, b2, t, eps, wd, gs, seed = g["step_hyper"]
+    p, m, v, _ = O.adamw_update(g["step_p"], g["step_g"], g["bf16_m"], g["step_v"], lr, b1, b2, int(t), eps, wd, gs, int(seed))
+    assert np.array_equal(p, g["bf16_p_out"]) and np.array_equal(m, g["bf16_m_out"]) and np.array_equal(v, g["bf16_v_out"])
+    p, mc, ms, v, _ = O.adamw_update_fp8m(g["step_p"], g["fp8_g"], g["fp8_m"], g["fp8_scales"], g["step_v"], lr, b1, b2, int(t),
+                                          eps, wd, gs, int(seed))
+    assert np.array_equal(p, g["fp8_p_out"]) and np.array_equal(v, g["fp8_v_out"])
+    assert np.array_equal(ms.view(np.uint32), g["fp8_scales_out"].view(np.uint32))
+    assert np.array_equal(mc, g["fp8_m_out"])

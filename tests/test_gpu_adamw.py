@@ -109,3 +109,68 @@ def test_adamw_argument_errors(K):
         K.adamw_update(z(16), z(16), z(16, torch.float32), z(16), 1e-3, 0.9, 0.99, 1, 1e-8, 0.0, gs)
     with pytest.raises(ValueError, match="shape mismatch"):
         K.adamw_update(z(16), z(8), z(16), z(16), 1e-3, 0.9, 0.99, 1, 1e-8, 0.0, gs)
+
+
+# ------------------------------------------------------------------ e4m3 first moment with block scales
+def make_fp8m(O, n, seed):
+    rng = np.random.default_rng(seed)
+    f = lambda a: O.f32_to_bf16(a.astype(np.float32))
+    params, grads = f(rng.standard_normal(n) * 0.05), f(rng.standard_normal(n) * 2e-3)
+    v = f(rng.random(n) * 1e-5 + 1e-8)
+    m = rng.integers(0, 256, n).astype(np.uint8)
+    m[(m & 0x7F) == 0x7F] ^= 1
+    nb = (n + 127) // 128
+    scales = (10.0 ** rng.uniform(-6, -2, nb)).astype(np.float32)
+    if nb > 2:                      # a block that stays exactly zero (scale 1 path) and one with a tiny moment
+        m[128:256] = 0
+        grads[128:256] = 0
+        scales[2] = 1e-30
+    return params, grads, m, scales, v
+
+
+@pytest.mark.parametrize("n", [8, 128, 1000, 8192 + 72, 1 << 20])
+def test_adamw_fp8_first_moment_bit_exact(K, O, n):
+    """adamw_update with an e4m3 first moment and one scale per 128 elements (src/kernels/kernels.h:237-239,
+    adamw.cu:22-66): parameters, codes, scales, second moment and abs-max bit exact against the oracle, including
+    a last block shorter than 128, an all-zero block and a vanishing one."""
+    params, grads, m, scales, v = make_fp8m(O, n, 11 + n % 5)
+    hp = dict(lr=3e-4, beta1=0.9, beta2=0.95, t=5, eps=1e-8, wd=0.1, gs=0.625, seed=0xBEEF + n)
+    wp, wm, ws, wv, wam = O.adamw_update_fp8m(params, grads, m, scales, v, hp["lr"], hp["beta1"], hp["beta2"], hp["t"],
+                                              hp["eps"], hp["wd"], hp["gs"], hp["seed"])
+    dp, dg, dv = dev_bf16(params), dev_bf16(grads), dev_bf16(v)
+    dm, ds = torch.from_numpy(m).cuda(), torch.from_numpy(scales).cuda()
+    gs = torch.tensor([hp["gs"]], dtype=torch.float32, device="cuda")
+    am = torch.zeros(1, dtype=torch.float32, device="cuda")
+    K.adamw_update(dp, dg, dm, dv, hp["lr"], hp["beta1"], hp["beta2"], hp["t"], hp["eps"], hp["wd"], gs, ds, am, hp["seed"])
+    assert np.array_equal(host_bits(dp), wp) and np.array_equal(host_bits(dv), wv)
+    assert np.array_equal(ds.cpu().numpy().view(np.uint32), ws.view(np.uint32))
+    assert np.array_equal(dm.cpu().numpy(), wm)
+    assert am.cpu().numpy().view(np.uint32)[0] == np.float32(wam).view(np.uint32)
+    # the stored moment dequantizes to within one e4m3 step (2^-3 relative) of the exact new moment
+    if n >= 1024:
+        dec = O.e4m3_table()
+        got = dec[wm].astype(np.float64) * np.repeat(ws, 128)[:n]
+        m_old = dec[m].astype(np.float64) * np.repeat(scales, 128)[:n]
+        g = O.bf16_to_f32(grads).astype(np.float64) * hp["gs"]
+        exact = hp["beta1"] * m_old + (1 - hp["beta1"]) * g
+        blk = np.repeat(ws.astype(np.float64) * 448, 128)[:n]              # block abs-max
+        assert np.all(np.abs(got - exact) <= 0.126 * np.abs(exact) + blk * 2.0 ** -9 + 1e-30)
+
+
+def test_adamw_golden_known_answers(K):
+    """The library against the numpy / exact-rational vectors of tests/golden/adamw_kat.npz: pins the hash bits,
+    rotations, thresholds and block scales with no oracle in the loop."""
+    import os
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "adamw_kat.npz"), allow_pickle=False)
+    lr, b1, b2, t, eps, wd, gsv, seed = (float(x) for x in g["step_hyper"])
+    gs = torch.tensor([gsv], dtype=torch.float32, device="cuda")
+    dp, dg, dm, dv = dev_bf16(g["step_p"]), dev_bf16(g["step_g"]), dev_bf16(g["bf16_m"]), dev_bf16(g["step_v"])
+    K.adamw_update(dp, dg, dm, dv, lr, b1, b2, int(t), eps, wd, gs, None, None, int(seed))
+    assert np.array_equal(host_bits(dp), g["bf16_p_out"]) and np.array_equal(host_bits(dm), g["bf16_m_out"])
+    assert np.array_equal(host_bits(dv), g["bf16_v_out"])
+    dp, dg, dv = dev_bf16(g["step_p"]), dev_bf16(g["fp8_g"]), dev_bf16(g["step_v"])
+    dm, ds = torch.from_numpy(g["fp8_m"]).cuda(), torch.from_numpy(g["fp8_scales"]).cuda()
+    K.adamw_update(dp, dg, dm, dv, lr, b1, b2, int(t), eps, wd, gs, ds, None, int(seed))
+    assert np.array_equal(host_bits(dp), g["fp8_p_out"]) and np.array_equal(host_bits(dv), g["fp8_v_out"])
+    assert np.array_equal(ds.cpu().numpy().view(np.uint32), g["fp8_scales_out"].view(np.uint32))
+    assert np.array_equal(dm.cpu().numpy(), g["fp8_m_out"])

@@ -129,6 +129,24 @@ def test_quantize_transpose_bit_exact(K, O, shape):
     assert np.array_equal(host_bits(out2), want.T)
 
 
+@pytest.mark.parametrize("shape", QT_SHAPES)
+def test_quantize_transpose_fp32_input_bit_exact(K, O, shape):
+    """fp32-input overload (src/kernels/kernels.h:261): the bytes of the fp32 quantizer, transposed; NaN, +-Inf,
+    signed zeros and denormals included."""
+    rows, cols = shape
+    rng = np.random.default_rng(rows * 3 + cols)
+    x = (rng.standard_normal((rows, cols)) * 10.0 ** rng.uniform(-6, 2, (rows, cols))).astype(np.float32)
+    flat = x.reshape(-1)
+    flat[:6] = [0.0, -0.0, np.inf, -np.inf, np.nan, 1e-40]
+    am = float(np.abs(flat[np.isfinite(flat)]).max())
+    want, d = O.quantize_f32(x, am)
+    out = torch.empty((cols, rows), dtype=torch.float8_e4m3fn, device="cuda")
+    scale = torch.zeros(1, device="cuda")
+    K.quantize_and_transpose_with_abs_max(out, scale, torch.from_numpy(x).cuda(), dev_scalar(am))
+    assert np.array_equal(host_bits(out), want.T)
+    assert scale.item() == d
+
+
 @pytest.mark.parametrize("fmt", [torch.float8_e4m3fn, torch.float8_e5m2])
 @pytest.mark.parametrize("shape", QT_SHAPES)
 def test_quantize_plain_and_transposed_in_one_read(K, O, shape, fmt):
@@ -217,8 +235,8 @@ def workspace():
 def skip_unsupported(variant, M, N, Kd):
     if variant[0] in (1, 3) and (M % 256 or N % 256):
         pytest.skip("the 256 x 256 tile needs multiples of 256")
-    if variant[0] == 3 and Kd % 256:
-        pytest.skip("the four-wave kernel needs K divisible by 256")
+    if variant[0] == 3 and Kd % 256 and (Kd < 384 or variant[1] > 1):
+        pytest.skip("the four-wave kernel takes an odd number of K-steps from 3 up, and cuts only even ones into segments")
     if variant[0] == 3 and variant[1] > 1:
         # mirrors the launch plan: 32 workgroups per XCD, segments of whole pairs of K-steps, none empty,
         # and one 256 KiB partial tile per segment in the 32 MiB workspace
@@ -349,14 +367,16 @@ def test_gemm_narrow_tile(K, O, mnk, forced):
         assert np.array_equal(host_bits(got), O.gemm_tn(a, b, sa=s, sb=s, bias=bias, mt=mt))
         _, oldv = O.fill_int_e4m3(N * M, 777, 3)
         old = O.f32_to_bf16(oldv.astype(np.float32)).reshape(N, M)
-        if forced or M % 128 != 0:
-            with pytest.raises(ValueError, match="narrow tile|divisible by 128"):
+        if forced:
+            with pytest.raises(ValueError, match="narrow tile|off the lattice"):
                 run_gemm(K, a, b, M, N, Kd, s, s, None, old)
-            with pytest.raises(ValueError, match="narrow tile|divisible by 128"):
+            with pytest.raises(ValueError, match="narrow tile|off the lattice"):
                 run_gemm(K, a, b, M, N, Kd, s, s, out_f32=True)
-        else:
+        else:   # accumulation and fp32 output: the other tiled kernels, or the general-shape kernel when M % 128 != 0
             got = run_gemm(K, a, b, M, N, Kd, s, s, bias, old)
-            assert np.array_equal(host_bits(got), O.gemm_tn(a, b, sa=s, sb=s, bias=bias, c_old=old, mt=True))
+            assert np.array_equal(host_bits(got), O.gemm_tn(a, b, sa=s, sb=s, bias=bias, c_old=old, mt=mt))
+            got32 = run_gemm(K, a, b, M, N, Kd, s, s, out_f32=True)
+            assert np.array_equal(got32.cpu().numpy(), O.gemm_tn(a, b, sa=s, sb=s, out_f32=True, mt=mt))
     finally:
         set_variant((0, 0))
 
@@ -364,7 +384,8 @@ def test_gemm_narrow_tile(K, O, mnk, forced):
 def _dispatch_sweep_cases():
     """Deterministic pseudo-random shapes for the automatic kernel choice: M from multiples of 128, 192, 224 and
     256, N from multiples of 128 and 256, K from multiples of 128 and 256, tile counts from a handful to a few
-    rounds of the chip, every epilogue flavour."""
+    rounds of the chip, every epilogue flavour (an M off the 128 lattice with accumulation or fp32 output, or with
+    an N off the 256 lattice, ends on the general-shape kernel in whole or for its last rows)."""
     rng = np.random.default_rng(2024)
     cases = []
     for idx in range(48):
@@ -372,10 +393,8 @@ def _dispatch_sweep_cases():
         M = int(unit_m * rng.integers(1, [24, 16, 16, 14][idx % 4]))
         N = int([128, 256][idx % 2] * rng.integers(1, [40, 24][idx % 2]))
         Kd = int([128, 256][(idx // 2) % 2] * rng.integers(1, 9))
-        if unit_m in (192, 224) and M % 128:       # only the narrow tiles serve these: they need N, K % 256 == 0
-            N, Kd = -(-N // 256) * 256, -(-Kd // 256) * 256
-            if M % 64:                             # outside the threaded oracle's 64-column blocks: keep it small
-                N, Kd = min(N, 1024), min(Kd, 512)
+        if M % 64:                                 # outside the threaded oracle's 64-column blocks: keep it small
+            N, Kd = min(N, 1024), min(Kd, 512)
         cases.append((M, N, Kd, idx % 3 == 1, idx % 5 == 2, idx % 7 == 3, idx % 4 != 3))
     return cases
 
@@ -385,8 +404,6 @@ def test_gemm_automatic_choice_sweep(K, O, case):
     """Whatever kernel, tile width and K split the dispatcher picks: integer operands -> bit exact against the
     oracle (bf16 and fp32 output, bias, accumulation, with and without a workspace)."""
     M, N, Kd, use_bias, use_old, out_f32, with_ws = case
-    if M % 128 and (use_old or out_f32):
-        use_old = out_f32 = False                  # the narrow tiles take bf16 output without accumulation only
     a, _ = O.fill_int_e4m3(M * Kd, 31 + M, 0)
     b, _ = O.fill_int_e4m3(N * Kd, 31 + N, 1)
     a, b = a.reshape(M, Kd), b.reshape(N, Kd)
@@ -549,6 +566,63 @@ def test_gemm_matches_swapped_operand_transpose(K, O):
     c1 = run_gemm(K, a, b, M, N, Kd, 0.01, 0.5, out_f32=True)
     c2 = run_gemm(K, b, a, N, M, Kd, 0.5, 0.01, out_f32=True)
     assert torch.allclose(c1, c2.T, rtol=1e-5, atol=1e-4)
+
+
+GENERAL_SHAPES = [(144, 272, 400), (1152, 8192, 896), (896, 2048, 896), (1024, 512, 896), (512, 256, 384),
+                  (256, 1000, 512), (3584, 300, 256), (8, 8, 16), (1, 1, 16), (130, 70, 48), (200, 264, 1024), (448, 520, 640)]
+
+
+@pytest.mark.parametrize("mnk", GENERAL_SHAPES)
+def test_gemm_general_shapes(K, O, mnk):
+    """The reference's default backend serves every FP8 shape with 16-byte aligned rows
+    (src/kernels/matmul.cpp:55-57, 160-184).  Here: M, K off the 128 lattice or N below 128 -> the general-shape
+    kernel; a ragged N on top of regular M, K -> tiled kernels for the rows before the last N % 128, general-shape
+    kernel for those; K an odd multiple of 128 -> the four-wave kernel's odd-K instances ((1152, 8192, 896) and
+    (896, 2048, 896) on its 192- and 224-wide tiles, (1024, 512, 896) on the full tile).  Integer operands -> bit
+    exact against the oracle for bf16 / fp32 output with bias and accumulation; random codes within the tolerance."""
+    M, N, Kd = mnk
+    a, _ = O.fill_int_e4m3(M * Kd, 2024, 0)
+    b, _ = O.fill_int_e4m3(N * Kd, 2024, 1)
+    a, b = a.reshape(M, Kd), b.reshape(N, Kd)
+    s = float(np.sqrt(np.float32(4.0 / Kd)))
+    _, biasv = O.fill_int_e4m3(M, 2024, 2)
+    _, oldv = O.fill_int_e4m3(N * M, 2024, 3)
+    bias = O.f32_to_bf16(biasv.astype(np.float32))
+    old = O.f32_to_bf16(oldv.astype(np.float32)).reshape(N, M)
+    mt = M % 64 == 0
+    for use_bias, use_old in [(False, False), (True, False), (True, True)]:
+        want = O.gemm_tn(a, b, sa=s, sb=s, bias=bias if use_bias else None, c_old=old if use_old else None, mt=mt)
+        got = run_gemm(K, a, b, M, N, Kd, s, s, bias if use_bias else None, old if use_old else None)
+        assert np.array_equal(host_bits(got), want), (use_bias, use_old)
+    got32 = run_gemm(K, a, b, M, N, Kd, s, s, out_f32=True)
+    assert np.array_equal(got32.cpu().numpy(), O.gemm_tn(a, b, sa=s, sb=s, out_f32=True, mt=mt))
+    got32 = run_gemm(K, a, b, M, N, Kd, None, None, bias, oldv.astype(np.float32), out_f32=True)
+    want32 = O.gemm_tn(a, b, bias=bias, c_old=oldv.astype(np.float32).reshape(N, M), out_f32=True, mt=mt)
+    assert np.array_equal(got32.cpu().numpy(), want32)
+    if M * N <= 1 << 21:
+        rng = np.random.default_rng(M + N + Kd)
+        ar = rng.integers(0, 256, (M, Kd)).astype(np.uint8)
+        br = rng.integers(0, 256, (N, Kd)).astype(np.uint8)
+        ar[(ar & 0x7F) == 0x7F] ^= 1
+        br[(br & 0x7F) == 0x7F] ^= 1
+        exact, sumabs = O.gemm_exact(ar, br)
+        g16 = run_gemm(K, ar, br, M, N, Kd, 0.37, 1.0 / 448).float().cpu().numpy()
+        gemm_check(g16, exact, sumabs, np.float32(np.float32(0.37) * np.float32(1.0 / 448)), True)
+        # e5m2 second operand on the same shapes
+        br5 = br.copy()
+        br5[(br5 & 0x7C) == 0x7C] ^= 0x40
+        br5 &= 0xBF
+        exact5, sumabs5 = O.gemm_exact(ar, br5, b_e5m2=True)
+        c5 = torch.empty((N, M), dtype=torch.float32, device="cuda")
+        mm(K, c5, dev_u8(ar), dev_u8(br5), None, dev_scalar(0.25), None, M, N, Kd, workspace=workspace(), b_e5m2=True)
+        gemm_check(c5.cpu().numpy(), exact5, sumabs5, 0.25, False)
+
+
+def test_gemm_rejects_unaligned_k(K):
+    a = torch.zeros((128, 72), dtype=torch.uint8, device="cuda")
+    c = torch.zeros((128, 128), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ValueError, match="multiple of 16"):
+        mm(K, c, a, a, None, None, None, 128, 128, 72)
 
 
 # ------------------------------------------------------------------------------------ backward_bias
