@@ -22,7 +22,8 @@ One JSON line is printed:
 Extra fields: roofline.mfma_only_ceiling_TFLOPs (register-only matrix-instruction loops: what the chip sustains
 under its power limit), roofline.traffic (hardware-counter bytes per GEMM launch, from profiles/), hip_graph_replay
 (the same step replayed from a HIP graph), fused_quantize_transpose_step (the step with the single-read
-quantize + transposed-copy extension), vendor_gemm (torch._scaled_mm, i.e. hipBLASLt, on the six GEMM shapes,
+quantize + transposed-copy extension), direct_gradient_layout_step (that step with the gate+up weight gradient
+reading the output gradient in its stored layout, matmul mode TT, instead of a transposed copy), vendor_gemm (torch._scaled_mm, i.e. hipBLASLt, on the six GEMM shapes,
 alternating with this library's GEMM: context for the roofline fraction, not part of the path).
 """
 import argparse
@@ -110,8 +111,8 @@ def main():
         timed("abs_max", 2 * n, lambda: K.abs_max(stats[name][0:1], t[name]))
         timed("quantize", 3 * n, lambda: K.quantize_with_abs_max(q[name], stats[name][1:2], t[name], stats[name][0:1]))
 
-    def gemm(c, a, b, sa, sb, M, N, Kd):
-        timed("gemm", 2.0 * M * N * Kd, lambda: K.matmul(c, a, b, None, sa, sb, M, N, Kd, workspace=ws))
+    def gemm(c, a, b, sa, sb, M, N, Kd, b_kmajor=False):
+        timed("gemm", 2.0 * M * N * Kd, lambda: K.matmul(c, a, b, None, sa, sb, M, N, Kd, workspace=ws, b_kmajor=b_kmajor))
         if record[0]:
             timers["gemm"][-1] += ("M%d_N%d_K%d" % (M, N, Kd),)
 
@@ -174,6 +175,29 @@ def main():
         qtr(q["x_t"], "x")
         gemm(out["dw_up"], q["x_t"], q["dy_up_t"], stats["x"][1:2], stats["dy_up"][1:2], C, UP, BT)
 
+    def step_direct():
+        """step_fused with the gate+up weight gradient reading the quantized output gradient dY[BT, UP] where it
+        lies (matmul mode TT, K-major second operand): no transposed copy of the step's largest tensor.  The down
+        projection's weight gradient keeps the copy: there the copy (29 M elements) costs less than the mode's
+        slower K loop does on that GEMM."""
+        timed("abs_max", 0, lambda: K.abs_max(stats["w_up"][0:1], t["w_up"]))
+        both("w_up", q["w_up_t"])
+        timed("abs_max", 0, lambda: K.abs_max(stats["w_down"][0:1], t["w_down"]))
+        both("w_down", q["w_down_t"])
+        absmax_and_quantize("x")
+        gemm(out["y_up"], q["w_up"], q["x"], stats["w_up"][1:2], stats["x"][1:2], UP, BT, C)
+        absmax_and_quantize("h")
+        gemm(out["y_down"], q["w_down"], q["h"], stats["w_down"][1:2], stats["h"][1:2], C, BT, FFN)
+        timed("abs_max", 0, lambda: K.abs_max(stats["dy_down"][0:1], t["dy_down"]))
+        both("dy_down", q["dy_down_t"])
+        gemm(out["dh"], q["w_down_t"], q["dy_down"], stats["w_down"][1:2], stats["dy_down"][1:2], FFN, BT, C)
+        qtr(q["h_t"], "h")
+        gemm(out["dw_down"], q["h_t"], q["dy_down_t"], stats["h"][1:2], stats["dy_down"][1:2], FFN, C, BT)
+        absmax_and_quantize("dy_up")
+        gemm(out["dx"], q["w_up_t"], q["dy_up"], stats["w_up"][1:2], stats["dy_up"][1:2], C, BT, UP)
+        qtr(q["x_t"], "x")
+        gemm(out["dw_up"], q["x_t"], q["dy_up"], stats["x"][1:2], stats["dy_up"][1:2], C, UP, BT, b_kmajor=True)
+
     gemm_flop = 3 * (2.0 * UP * BT * C) + 3 * (2.0 * C * BT * FFN)
 
     for _ in range(args.warmup):
@@ -215,15 +239,27 @@ def main():
             graph.replay()
         torch.cuda.synchronize()
         graph_ms = (time.perf_counter() - g0) * 1e3 / args.steps
-    fused_ms = None
+    # The two extension sequences, timed in alternation (three rounds of args.steps steps each, median round), so that
+    # clock and temperature drift over the run touches both alike.  The gate+up dW of the direct-layout sequence must
+    # equal the materialised route's bit for bit.
+    fused_ms, direct_ms, direct_identical = None, None, None
     if not args.no_graph:
+        def ms_of(fn):
+            torch.cuda.synchronize()
+            f0 = time.perf_counter()
+            for _ in range(args.steps):
+                fn()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - f0) * 1e3 / args.steps
         step_fused()
+        want_dw = out["dw_up"].clone()
+        step_direct()
         torch.cuda.synchronize()
-        f0 = time.perf_counter()
-        for _ in range(args.steps):
-            step_fused()
-        torch.cuda.synchronize()
-        fused_ms = (time.perf_counter() - f0) * 1e3 / args.steps
+        direct_identical = bool(torch.equal(out["dw_up"], want_dw))
+        del want_dw
+        rounds = [(ms_of(step_fused), ms_of(step_direct)) for _ in range(3)]
+        fused_ms = sorted(r[0] for r in rounds)[1]
+        direct_ms = sorted(r[1] for r in rounds)[1]
     vendor = None
     if not args.no_graph and hasattr(torch, "_scaled_mm"):
         one = torch.ones(1, device=dev)
@@ -495,6 +531,11 @@ def main():
         "fused_quantize_transpose_step": None if fused_ms is None else {
             "ms_per_step": fused_ms, "value": gemm_flop / (fused_ms * 1e-3) / 1e12,
             "note": "extension: single-read quantize + transposed copy for weights and output gradients"},
+        "direct_gradient_layout_step": None if direct_ms is None else {
+            "ms_per_step": direct_ms, "value": gemm_flop / (direct_ms * 1e-3) / 1e12,
+            "dw_identical_to_materialised_route": direct_identical,
+            "note": "extension: fused_quantize_transpose_step without the transposed copy of dY[8192, 37888]; the "
+                    "gate+up weight gradient reads dY in its stored layout (matmul mode TT)"},
         "vendor_gemm": vendor,
         "secondary_gemm_shapes": secondary,
         "producers": swiglu,

@@ -133,6 +133,26 @@ int llmq_gemm_tn_e4m3_bf16(uint16_t* c, const uint8_t* a, const uint8_t* b, cons
                            size_t workspace_bytes, int M, int N, int K, int accumulate, void* stream);
 
 /*
+ * The same matmul with the operand layout selected by the reference's EMMTranspose mode (src/kernels/kernels.h:22:
+ * TT = 0, TN = 1, NT = 2, NN = 3; in its column-major reading, src/kernels/matmul.cpp:66-67).  With row-major storage:
+ *   TN  a[M, K], b[N, K]            (both K contiguous: llmq_gemm_tn_e4m3_bf16 / llmq_gemm_tn_e4m3_e5m2_bf16)
+ *   TT  a[M, K], b[K, N]            (b K-major: the output gradient dY[BT, OC] in its stored layout as the second
+ *                                    operand of the weight gradient, so that no transposed copy of it is needed)
+ * The reference's FP8 path takes TN only (it materialises the transposes, src/models/llama_model.cpp:309-339) and
+ * modes NT / NN (a stored [K, M]) are not provided here either.  TT: N and K multiples of 256, M a multiple of 256
+ * (without accumulation also of 224); other shapes return LLMQ_ERR_INVALID_ARGUMENT and the caller takes the
+ * transposing route.  b_format: 0 = e4m3, 1 = e5m2.  Results are bit-identical to mode TN on the transposed copy.
+ */
+#define LLMQ_MODE_TT 0
+#define LLMQ_MODE_TN 1
+#define LLMQ_MODE_NT 2
+#define LLMQ_MODE_NN 3
+int llmq_gemm_e4m3_bf16_mode(uint16_t* c, const uint8_t* a, const uint8_t* b, const uint16_t* bias_or_null,
+                             const float* sa_or_null, const float* sb_or_null, void* workspace_or_null,
+                             size_t workspace_bytes, int M, int N, int K, int mode, int b_format, int accumulate,
+                             void* stream);
+
+/*
  * fp32-output variant (wgrad into fp32 gradients).  bias may be fp32[M] (bias_is_bf16 == 0) or
  * bf16[M] (bias_is_bf16 != 0) or NULL.
  * Replaces: matmul(float* c, const __nv_fp8_e4m3*, const __nv_fp8_e4m3*, const float* bias, ...)

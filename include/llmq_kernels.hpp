@@ -137,6 +137,12 @@ inline void require_tn(EMMTranspose mode) {
     if (mode != EMMTranspose::TN)
         throw std::invalid_argument("matmul: FP8 operands are only supported in TN layout (both K-contiguous)");
 }
+// bf16 output: TN, and TT (b stored [K, N]; restricted shapes, see llmq_gemm_e4m3_bf16_mode)
+inline int mode_code(EMMTranspose mode) {
+    if (mode == EMMTranspose::TN) return LLMQ_MODE_TN;
+    if (mode == EMMTranspose::TT) return LLMQ_MODE_TT;
+    throw std::invalid_argument("matmul: FP8 operands are supported in modes TN and TT only");
+}
 template <class... T> [[noreturn]] void unsupported(const char* func, const T&... t) {
     std::string msg = std::string(func) + ": unsupported dtypes. Got [";
     ((msg += (t.empty() ? std::string("<null>") : std::string(dtype_to_str(t.DType))) + ", "), ...);
@@ -247,10 +253,9 @@ inline void matmul(__hip_bfloat16* c, const __hip_fp8_e4m3* a, const __hip_fp8_e
                    const float* scale_a, const float* scale_b, llmqBlasHandle_t, std::byte* workspace,
                    std::size_t workspace_size, int M, int N, int K, EMMTranspose mode, bool accumulate,
                    hipStream_t stream, EMatmulBackend = EMatmulBackend::Custom) {
-    llmq_detail::require_tn(mode);
-    llmq_detail::check(llmq_gemm_tn_e4m3_bf16(llmq_detail::u16(c), llmq_detail::u8(a), llmq_detail::u8(b),
-                                              llmq_detail::u16(bias), scale_a, scale_b, workspace, workspace_size, M, N,
-                                              K, accumulate, stream));
+    llmq_detail::check(llmq_gemm_e4m3_bf16_mode(llmq_detail::u16(c), llmq_detail::u8(a), llmq_detail::u8(b),
+                                                llmq_detail::u16(bias), scale_a, scale_b, workspace, workspace_size, M, N,
+                                                K, llmq_detail::mode_code(mode), 0, accumulate, stream));
 }
 inline void matmul(float* c, const __hip_fp8_e4m3* a, const __hip_fp8_e4m3* b, const float* bias, const float* scale_a,
                    const float* scale_b, llmqBlasHandle_t, std::byte* workspace, std::size_t workspace_size, int M,
@@ -273,10 +278,9 @@ inline void matmul(__hip_bfloat16* c, const __hip_fp8_e4m3* a, const __hip_fp8_e
                    const float* scale_a, const float* scale_b, llmqBlasHandle_t, std::byte* workspace,
                    std::size_t workspace_size, int M, int N, int K, EMMTranspose mode, bool accumulate,
                    hipStream_t stream, EMatmulBackend = EMatmulBackend::Custom) {
-    llmq_detail::require_tn(mode);
-    llmq_detail::check(llmq_gemm_tn_e4m3_e5m2_bf16(llmq_detail::u16(c), llmq_detail::u8(a), llmq_detail::u8(b),
-                                                   llmq_detail::u16(bias), scale_a, scale_b, workspace, workspace_size,
-                                                   M, N, K, accumulate, stream));
+    llmq_detail::check(llmq_gemm_e4m3_bf16_mode(llmq_detail::u16(c), llmq_detail::u8(a), llmq_detail::u8(b),
+                                                llmq_detail::u16(bias), scale_a, scale_b, workspace, workspace_size, M, N,
+                                                K, llmq_detail::mode_code(mode), 1, accumulate, stream));
 }
 inline void matmul(float* c, const __hip_fp8_e4m3* a, const __hip_fp8_e5m2* b, const __hip_bfloat16* bias,
                    const float* scale_a, const float* scale_b, llmqBlasHandle_t, std::byte* workspace,

@@ -24,6 +24,18 @@ struct QmmRunState {
     // Extension: quantize the output gradient and produce its transpose from one read of dout.Value (saves one
     // read and one launch per layer; the transposed gradient then lives on the stack during the dgrad as well).
     bool FuseGradTranspose = false;
+    // Extension: the weight-gradient matmul reads the quantized output gradient in its stored layout [B*T, OC]
+    // (matmul mode TT) instead of a transposed copy, wherever direct_grad_layout_applies() says the shape allows
+    // it and the copy costs more than the mode's slower K loop; elsewhere backward_qmm behaves as without the flag.
+    bool DirectGradLayout = false;
+    // Mode TT serves whole 256-wide tiles and bf16 output.  Measured on Qwen2.5-7B shapes at 8192 tokens: the K-major
+    // operand slows the matmul by 4-6 %, the transposed copy costs 2 * B*T * OC bytes of HBM traffic; the copy is
+    // the larger cost while C, the matmul's row count, stays below about 10^4.
+    static bool direct_grad_layout_applies(int B, int T, int C, int OC, ETensorDType dweight_dtype, bool accumulate) {
+        const long BT = (long)B * T;
+        return dweight_dtype == ETensorDType::BF16 && OC % 256 == 0 && BT % 256 == 0 &&
+               (C % 256 == 0 || (C % 224 == 0 && !accumulate)) && C <= 8192;
+    }
     std::vector<std::byte*> Live;
 
     Tensor temp_alloc(ETensorDType dtype, const std::vector<long>& shape) {
@@ -43,9 +55,11 @@ struct QmmRunState {
         t.Data = nullptr;
     }
     // Bytes of stack backward_qmm needs for one layer (the dry run of llama_run_state.cpp:362-390).
-    static std::size_t backward_temp_bytes(int B, int T, int C, int OC, bool fuse_grad_transpose = false) {
+    static std::size_t backward_temp_bytes(int B, int T, int C, int OC, bool fuse_grad_transpose = false,
+                                           bool direct_grad = false) {
         auto up = [](std::size_t b) { return (b + 4095) / 4096 * 4096; };
         const std::size_t wt = up((std::size_t)C * OC), at = up((std::size_t)C * B * T), gt = up((std::size_t)OC * B * T);
+        if (direct_grad) return wt > at ? wt : at;
         if (fuse_grad_transpose) return gt + (wt > at ? wt : at);
         return wt > at + gt ? wt : at + gt;
     }
@@ -72,8 +86,10 @@ inline void backward_qmm(Tensor& dinp, Tensor& dweight, Tensor dbias, Quantizabl
                          int C, int OC, bool reuse_inp, hipStream_t stream) {
     if (weight.DType != ETensorDType::FP8_E4M3)
         throw std::invalid_argument("backward_qmm: this build implements the FP8 (e4m3 weight) branch only");
+    const bool direct_grad = rs.DirectGradLayout &&
+                             QmmRunState::direct_grad_layout_applies(B, T, C, OC, dweight.DType, accumulate_gradient);
     Tensor grad_tp{};
-    if (rs.FuseGradTranspose) {
+    if (rs.FuseGradTranspose && !direct_grad) {
         grad_tp = rs.temp_alloc(dout.Quant.DType, {OC, (long)B * T});
         quantize_with_abs_max_and_transpose(dout.Quant, grad_tp, dout.Quant.scale(), dout.Value, dout.Quant.abs_max(),
                                             B * T, OC, rs.DeviceProp, stream);
@@ -91,7 +107,7 @@ inline void backward_qmm(Tensor& dinp, Tensor& dweight, Tensor dbias, Quantizabl
     rs.temp_free(weight_tp);
 
     Tensor activation_tp = rs.temp_alloc(inp_q.DType, {C, (long)B * T});
-    if (!rs.FuseGradTranspose) grad_tp = rs.temp_alloc(dout.Quant.DType, {OC, (long)B * T});
+    if (!rs.FuseGradTranspose && !direct_grad) grad_tp = rs.temp_alloc(dout.Quant.DType, {OC, (long)B * T});
     if (reuse_inp) {
         transpose(activation_tp, inp_q, B * T, C, stream);
     } else {
@@ -99,13 +115,21 @@ inline void backward_qmm(Tensor& dinp, Tensor& dweight, Tensor dbias, Quantizabl
         quantize_and_transpose_with_abs_max(activation_tp, activation_tp.scale(), inp.Value, inp.Quant.abs_max(),
                                             B * T, C, rs.DeviceProp, stream);
     }
-    if (!rs.FuseGradTranspose) transpose(grad_tp, dout.Quant, B * T, OC, stream);
-    matmul(dweight, activation_tp, grad_tp, no_bias, inp_q.scale(), dout.Quant.scale(), rs.BlasHandle, rs.Workspace, C,
-           OC, B * T, EMMTranspose::TN, accumulate_gradient, stream, rs.MatmulBackend);
+    if (direct_grad) {
+        // the quantized gradient in its stored layout [B*T, OC] is the K-major second operand (mode TT): no transposed copy
+        matmul(dweight, activation_tp, dout.Quant, no_bias, inp_q.scale(), dout.Quant.scale(), rs.BlasHandle, rs.Workspace, C,
+               OC, B * T, EMMTranspose::TT, accumulate_gradient, stream, rs.MatmulBackend);
+    } else {
+        if (!rs.FuseGradTranspose) transpose(grad_tp, dout.Quant, B * T, OC, stream);
+        matmul(dweight, activation_tp, grad_tp, no_bias, inp_q.scale(), dout.Quant.scale(), rs.BlasHandle, rs.Workspace, C,
+               OC, B * T, EMMTranspose::TN, accumulate_gradient, stream, rs.MatmulBackend);
+    }
     if (!dbias.empty()) {
         backward_bias(dbias, dout.Quant, inp_q.scale(), dout.Quant.scale(), bias_buffer, B, T, OC, rs.DeviceProp, stream);
     }
-    if (rs.FuseGradTranspose) {
+    if (direct_grad) {
+        rs.temp_free(activation_tp);
+    } else if (rs.FuseGradTranspose) {
         rs.temp_free(activation_tp);
         rs.temp_free(grad_tp);
     } else {

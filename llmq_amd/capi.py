@@ -18,7 +18,7 @@ EXPORTS = [
     "llmq_last_error", "llmq_version", "llmq_target_arch",
     "llmq_abs_max_bf16", "llmq_abs_max_f32",
     "llmq_quantize_e4m3_bf16", "llmq_quantize_e5m2_bf16", "llmq_quantize_transpose_e4m3_bf16", "llmq_quantize_transpose_e4m3_f32",
-    "llmq_transpose_u8", "llmq_gemm_tn_e4m3_bf16", "llmq_gemm_tn_e4m3_f32", "llmq_gemm_tn_e4m3_e5m2_bf16", "llmq_gemm_tn_e4m3_e5m2_f32",
+    "llmq_transpose_u8", "llmq_gemm_tn_e4m3_bf16", "llmq_gemm_e4m3_bf16_mode", "llmq_gemm_tn_e4m3_f32", "llmq_gemm_tn_e4m3_e5m2_bf16", "llmq_gemm_tn_e4m3_e5m2_f32",
     "llmq_backward_bias_bf16", "llmq_backward_bias_scratch_bytes", "llmq_backward_bias_bf16_static_scratch", "llmq_quantize_both_bf16", "llmq_quantize_e4m3_f32", "llmq_quantize_e5m2_f32",
     "llmq_swiglu_forward_bf16", "llmq_swiglu_forward_quant_bf16", "llmq_swiglu_backward_bf16",
     "llmq_rmsnorm_forward_bf16", "llmq_fused_residual_rmsnorm_forward_bf16",
@@ -47,6 +47,7 @@ lib.llmq_quantize_e5m2_f32.argtypes = [_vp, _vp, _vp, _vp, _i64, _vp]
 lib.llmq_quantize_both_bf16.argtypes = [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp]
 lib.llmq_transpose_u8.argtypes = [_vp, _vp, _int, _int, _vp]
 lib.llmq_gemm_tn_e4m3_bf16.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, C.c_size_t, _int, _int, _int, _int, _vp]
+lib.llmq_gemm_e4m3_bf16_mode.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, C.c_size_t, _int, _int, _int, _int, _int, _int, _vp]
 lib.llmq_gemm_tn_e4m3_f32.argtypes = [_vp, _vp, _vp, _vp, _int, _vp, _vp, _vp, C.c_size_t, _int, _int, _int, _int, _vp]
 lib.llmq_gemm_tn_e4m3_e5m2_bf16.argtypes = lib.llmq_gemm_tn_e4m3_bf16.argtypes
 lib.llmq_gemm_tn_e4m3_e5m2_f32.argtypes = lib.llmq_gemm_tn_e4m3_f32.argtypes

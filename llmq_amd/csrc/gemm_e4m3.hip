@@ -550,6 +550,17 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs g, int spli
     PairIo<OutT>::store((LLMQ_GLOBAL OutT*)dst, v0, v1);
 }
 
+// Position of 16-byte chunk c (0..7) of LDS row r (128 bytes, one K-step of one operand row) is c ^ frag_swizzle(r).
+// A fragment read (ds_read_b128) has lane 16 kg + l read chunk 2 kg + h of row l.  The LDS serves such a read in four
+// cycles of 16 lanes over its 64 banks, and the lanes of a cycle are not consecutive (measured with two-lane probes
+// and the bank-conflict counter): {0-3, 12-15, 20-23, 24-27}, {4-11, 16-19, 28-31}, and the same plus 32.  A cycle so
+// holds every row l once: rows 0-3 and 12-15 with one chunk number, rows 4-11 with that number ^ 2.  Rows of equal
+// parity share banks; xor-ing the chunk with l / 2 alone would put rows 0-3, 12-15 and rows 4-11 of a cycle on the
+// same banks (a two-way conflict on every read: 8 instead of 4 cycles), the extra flip of bit 1 for rows 4-11 undoes it.
+__device__ __forceinline__ int frag_swizzle(int row) {
+    return ((row >> 1) & 7) ^ ((((row >> 2) ^ (row >> 3)) & 1) << 1);
+}
+
 // ---- four-wave variant ----------------------------------------------------------------------------
 // Same 256 x 256 x 128 workgroup tile, LDS layout, copies and tile order as above, with a different
 // division of labour: 4 waves (one per SIMD, up to 512 registers each) of 128 x 128 outputs and the
@@ -579,9 +590,18 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs g, int spli
 // STREAM_OUT: the bf16 stores of the full-width epilogue are non-temporal (see there).
 // ODDK: the number of K-steps per tile is odd (K an odd multiple of 128, at least 384; not with SEG): the LDS stage
 // and fb half of a tile's first step then alternate from tile to tile, and the tile loop carries both orders.
-template <typename OutT, int B_FMT, bool SEG, int NJ = 8, bool STREAM_OUT = true, bool ODDK = false>
+// KMB: the b operand is stored K-major, row-major [K, N] (the reference's mode TT: the output gradient dY[BT, OC] as
+// the weight gradient's second operand, without a transposed copy).  Its tile of a K-step is then 128 rows (k) of
+// 256 bytes (n) in LDS, 16-byte chunk g of row k stored at position g ^ swz(k), swz(k) = (k & 7) | ((k >> 5) & 1) << 3,
+// and the fragments come out of LDS through the transposing read ds_read_b64_tr_b8: per group of 16 lanes it takes
+// 8 rows x 16 bytes (lanes 2r and 2r + 1 give the addresses of the two 8-byte halves of row r) and hands lane i
+// the 8 bytes of column i, i.e. 8 consecutive k of one n; four of them fill a fragment (32 k per lane, in the
+// same k order as the other operand's two 16-byte reads).  The swizzle spreads the 8 rows of one read, and the
+// two lane groups that share an LDS pass, over all banks.
+template <typename OutT, int B_FMT, bool SEG, int NJ = 8, bool STREAM_OUT = true, bool ODDK = false, bool KMB = false>
 __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     static_assert(!(SEG && ODDK), "K segments are whole pairs of K-steps");
+    static_assert(!(KMB && (SEG || ODDK)), "the K-major operand mode is built for whole tiles and even K-step counts");
     constexpr int BLK = 256, T = 256, WT = 128, NF = 8;
     constexpr int WTM = 16 * NJ, BLKM = 2 * WTM;  // columns (first-operand rows) per wave and per tile
     constexpr int P_BYTES = BLK * kBK, STAGE = 2 * P_BYTES;
@@ -625,8 +645,15 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     // copies: lane -> (row tid/8 of a 32-row slab, physical 16-byte chunk tid%8); every address is a
     // wave-uniform base plus a 32-bit lane offset
     const int ld_row = tid / 8;
-    const int ld_chunk = (tid & 7) ^ ((ld_row >> 1) & 7);
-    const uint32_t p_lane = (uint32_t)ld_row * (uint32_t)g.K + (uint32_t)ld_chunk * 16u;
+    const int ld_chunk = (tid & 7) ^ frag_swizzle(ld_row);
+    // b tile copies.  Normal layout: slab c = rows 32 c .. 32 c + 31 of the tile, lane -> (row, chunk) as above.
+    // K-major layout: slab c = k rows 16 c .. 16 c + 15, lane -> (row tid / 16, physical chunk tid % 16) reading
+    // global chunk (tid % 16) ^ swz(k); bit 3 of swz depends on the slab ((c >> 1) & 1), hence two lane offsets.
+    const int kb_row = tid / 16, kb_chunk = (tid & 15) ^ (kb_row & 7);
+    const uint32_t p_lane = KMB ? (uint32_t)kb_row * (uint32_t)g.N + (uint32_t)kb_chunk * 16u
+                                : (uint32_t)ld_row * (uint32_t)g.K + (uint32_t)ld_chunk * 16u;
+    const uint32_t p_lane_hi = (uint32_t)kb_row * (uint32_t)g.N + (uint32_t)(kb_chunk ^ 8) * 16u;  // KMB, slabs 2, 3, 6, 7
+    const uint32_t p_step = KMB ? (uint32_t)kBK * (uint32_t)g.N : (uint32_t)kBK;  // lane offset advance per K-step
     // LDS row rho of the a-tile is row l = rho % 16 of fragment f = rho / 16 (wave half f / NJ, fragment f % NJ of
     // it) and holds global row frag_row(f) + frag_step(f) * l.  NJ = 8 and 6: fragment j of a wave half starts at
     // row j with step NJ, so that a lane of the epilogue owns NJ adjacent columns (16 or 12 bytes of bf16).  NJ = 7:
@@ -656,17 +683,17 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     int copy_k0 = 0, copy_tile = 0;
     const uint8_t* p_base[ITERS];
     const uint8_t* q_base[ITERS_Q];
-    uint32_t vp = p_lane, vq = q_lane, vq3 = q_lane_3, vq6 = q_lane_6;
+    uint32_t vp = p_lane, vp_hi = p_lane_hi, vq = q_lane, vq3 = q_lane_3, vq6 = q_lane_6;
     auto tile_bases = [&](int logical) {
         int nb, mb;
         decode(logical, nb, mb);
-        const uint8_t* pb = g.b + (int64_t)nb * g.K + k_first;
+        const uint8_t* pb = KMB ? g.b + (int64_t)k_first * g.N + nb : g.b + (int64_t)nb * g.K + k_first;
         const uint8_t* qb = g.a + (int64_t)mb * g.K + k_first;
         // pinned in scalar registers here, once per tile (otherwise the compiler sinks the additions to the
         // copies and repeats them in every K-step)
 #pragma unroll
         for (int c = 0; c < ITERS; ++c) {
-            p_base[c] = pb + (int64_t)(32 * c) * g.K;
+            p_base[c] = KMB ? pb + (int64_t)(16 * c) * g.N : pb + (int64_t)(32 * c) * g.K;
             asm volatile("" : "+s"(p_base[c]));
         }
 #pragma unroll
@@ -680,7 +707,8 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     // (harmless, and no step needs a special case)
     auto advance_copy = [&]() {
         copy_k0 += kBK;
-        vp += kBK;
+        vp += p_step;
+        if constexpr (KMB) vp_hi += p_step;
         vq += kBK;
         if constexpr (NJ == 7) {
             vq3 += kBK;
@@ -688,7 +716,8 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         }
         if (copy_k0 == k_total) {
             copy_k0 = 0;
-            vp -= (uint32_t)k_total;
+            vp = p_lane;
+            if constexpr (KMB) vp_hi = p_lane_hi;
             vq -= (uint32_t)k_total;
             if constexpr (NJ == 7) {
                 vq3 -= (uint32_t)k_total;
@@ -723,7 +752,7 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     auto copy_src = [&](int c, const uint8_t*& src, uint32_t& lane_ofs) {
         if (c < ITERS) {
             src = p_base[c];
-            lane_ofs = vp;
+            lane_ofs = (KMB && ((c >> 1) & 1)) ? vp_hi : vp;
         } else {
             const int it = c - ITERS;  // slab `it` covers LDS rows 32 it .. 32 it + 31: fragments 2 it and 2 it + 1
             src = q_base[it];
@@ -744,7 +773,7 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(lane_ofs), "s"(src), "{m0}"(tok) : "memory");
     };
 
-    const int sw = (l16 >> 1) & 7;
+    const int sw = frag_swizzle(l16);
     const int c0 = ((2 * kg) ^ sw) * 16, c1 = ((2 * kg + 1) ^ sw) * 16;
     const int p_frag = (wn * WT + l16) * kBK;
     const int q_frag = P_BYTES + (wm * WTM + l16) * kBK;
@@ -752,6 +781,27 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         const v4i lo = *reinterpret_cast<const v4i*>(row + c0);
         const v4i hi = *reinterpret_cast<const v4i*>(row + c1);
         return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    };
+    // b fragment i (rows 16 i .. 16 i + 15 of the wave's 128 rows of c) from the stage at `stage`.  K-major: this
+    // lane supplies the address of half (l16 & 1) of k row 32 kg + 8 q + l16 / 2 for the q-th of four transposing
+    // reads; the row's chunk 8 wn + i sits at position (8 wn + i) ^ swz(k), and with swz(k) = l16 / 2 | (kg & 1) << 3
+    // for every q that is kb_base ^ (16 i) in bytes: one xor per fragment, the four reads differ by 8 rows = 2048.
+    typedef int v2i_lds __attribute__((ext_vector_type(2)));
+    const uint32_t kb_base = (uint32_t)((32 * kg + l16 / 2) * 256 + (l16 & 1) * 8) + (uint32_t)(((8 * wn) ^ ((kg & 1) << 3)) * 16) +
+                             (uint32_t)((l16 / 2) * 16);
+    auto read_frag_b = [&](const uint8_t* stage, int i) -> v8i {
+        if constexpr (KMB) {
+            const uint8_t* p = stage + (opaque((int)kb_base) ^ (16 * i));
+            typedef __attribute__((address_space(3))) v2i_lds* lds_v2i;
+            const v2i_lds r0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i)(p));
+            const v2i_lds r1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i)(p + 2048));
+            const v2i_lds r2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i)(p + 4096));
+            const v2i_lds r3 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i)(p + 6144));
+            const v8i f = {r0[0], r0[1], r1[0], r1[1], r2[0], r2[1], r3[0], r3[1]};
+            return f;
+        } else {
+            return read_frag(stage + p_frag + i * 16 * kBK);
+        }
     };
 
     // The matrix instruction as an asm statement with the accumulator tied in place in the accumulation
@@ -785,7 +835,7 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(COPIES) : "memory");
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < 4; ++i) fa[i] = read_frag(lds + p_frag + i * 16 * kBK);
+    for (int i = 0; i < 4; ++i) fa[i] = read_frag_b(lds, i);
 #pragma unroll
     for (int j = 0; j < NJ; ++j) fb[0][j] = read_frag(lds + q_frag + j * 16 * kBK);
 
@@ -870,8 +920,8 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
                 fb[1 - FP][0] = __builtin_shufflevector(lo0, hi0, 0, 1, 2, 3, 4, 5, 6, 7);
                 fb[1 - FP][1] = __builtin_shufflevector(lo1, hi1, 0, 1, 2, 3, 4, 5, 6, 7);
             }
-            if constexpr (i < 4) fa[i % 4] = read_frag(cur + p_frag + (i + 4) * 16 * kBK);
-            else fa[i % 4] = read_frag(nxt + p_frag + (i - 4) * 16 * kBK);
+            if constexpr (i < 4) fa[i % 4] = read_frag_b(cur, i + 4);
+            else fa[i % 4] = read_frag_b(nxt, i - 4);
         });
         advance_copy();
         if constexpr (ODDK) stage_rt = STAGE - stage_rt;
@@ -1515,7 +1565,52 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
     return launch_pipe<128, 128, 2, 2, OutT, B_FMT>(g, splits, 0, stream);
 }
 
+// b stored K-major, [K, N] row-major (the reference's mode TT): the four-wave kernel's KMB instances, whole tiles only.
+template <int B_FMT>
+static int gemm_dispatch_b_kmajor(GemmArgs g, hipStream_t stream) {
+    LLMQ_REQUIRE(g.M > 0 && g.N > 0 && g.K > 0, "matmul: M, N, K must be positive (got %d, %d, %d)", g.M, g.N, g.K);
+    const int cus = cu_count(), xcds = xcd_count();
+    g.xcds = xcds;
+    g.group = 8;
+    LLMQ_REQUIRE(g.a && g.b && g.c, "matmul: null operand pointer");
+    LLMQ_REQUIRE(aligned16(g.a) && aligned16(g.b) && aligned16(g.c) && aligned16(g.bias),
+                 "matmul: all pointers must be 16-byte aligned");
+    const bool m224 = g.M % 256 != 0 && g.M % 224 == 0 && !g.accumulate;
+    LLMQ_REQUIRE(g.N % 256 == 0 && g.K % 256 == 0 && (g.M % 256 == 0 || m224) && cus % xcds == 0,
+                 "matmul: the K-major second operand (mode TT) needs N %% 256 == 0, K %% 256 == 0 and M %% 256 == 0 (without "
+                 "accumulation also M %% 224 == 0); got M, N, K = %d, %d, %d", g.M, g.N, g.K);
+    const int tiles = (g.N / 256) * (m224 ? g.M / 224 : g.M / 256);
+    const int grid = tiles < cus ? (tiles + xcds - 1) / xcds * xcds : cus;
+    const bool cached_out = ((int64_t)g.M + g.N) * g.K + (int64_t)g.N * g.M * 2 <= ((int64_t)224 << 20);
+    if (m224)
+        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, B_FMT, false, 7, true, false, true>), dim3((unsigned)grid), dim3(256),
+                           0, stream, g);
+    else if (cached_out)
+        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, B_FMT, false, 8, false, false, true>), dim3((unsigned)grid), dim3(256),
+                           0, stream, g);
+    else
+        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, B_FMT, false, 8, true, false, true>), dim3((unsigned)grid), dim3(256),
+                           0, stream, g);
+    LLMQ_HIP_TRY(hipGetLastError());
+    return LLMQ_OK;
+}
+
 }  // namespace llmq
+
+extern "C" int llmq_gemm_e4m3_bf16_mode(uint16_t* c, const uint8_t* a, const uint8_t* b, const uint16_t* bias_or_null,
+                                        const float* sa_or_null, const float* sb_or_null, void* workspace_or_null,
+                                        size_t workspace_bytes, int M, int N, int K, int mode, int b_format, int accumulate,
+                                        void* stream) {
+    using namespace llmq;
+    LLMQ_REQUIRE(b_format == 0 || b_format == 1, "matmul: unknown fp8 format %d of the second operand", b_format);
+    GemmArgs g{c, a, b, bias_or_null, sa_or_null, sb_or_null, M, N, K, 1, accumulate, 8, nullptr, 0, 1, 0, 8, 0};
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (mode == LLMQ_MODE_TN)
+        return b_format ? gemm_dispatch<uint16_t, 1>(g, workspace_or_null, workspace_bytes, st)
+                        : gemm_dispatch<uint16_t, 0>(g, workspace_or_null, workspace_bytes, st);
+    LLMQ_REQUIRE(mode == LLMQ_MODE_TT, "matmul: FP8 operands are served in modes TN and TT (got mode %d)", mode);
+    return b_format ? gemm_dispatch_b_kmajor<1>(g, st) : gemm_dispatch_b_kmajor<0>(g, st);
+}
 
 extern "C" int llmq_gemm_tn_e4m3_bf16(uint16_t* c, const uint8_t* a, const uint8_t* b, const uint16_t* bias_or_null,
                                       const float* sa_or_null, const float* sb_or_null, void* workspace_or_null,

@@ -112,7 +112,8 @@ def transpose(dst, src, stream=0):
     capi.check(capi.lib.llmq_transpose_u8(d, s, src.shape[0], src.shape[1], _stream(stream)))
 
 
-def matmul(c, a, b, bias, scale_a, scale_b, M, N, K, accumulate=False, stream=0, workspace=None, b_e5m2=False, _lib=None):
+def matmul(c, a, b, bias, scale_a, scale_b, M, N, K, accumulate=False, stream=0, workspace=None, b_e5m2=False, _lib=None,
+           b_kmajor=False):
     """TN matmul in the convention of the reference's kernels.h: row-major a[M,K], b[N,K] (e4m3) give
     row-major c[N,M] = (b @ a.T) * scale_a * scale_b (+ bias[M]) (+ c).  c: bf16 or fp32.
     workspace: optional device byte tensor (the reference passes a 32 MiB one); it enables the
@@ -120,6 +121,21 @@ def matmul(c, a, b, bias, scale_a, scale_b, M, N, K, accumulate=False, stream=0,
     dtype option): a float8_e5m2 tensor, or uint8 with b_e5m2=True.  _lib: tests pass the test-aid build of
     the same entry points (capi.testaid()) to force a kernel variant; everyone else leaves it alone."""
     L = _lib or capi.lib
+    if b_kmajor:
+        # the reference's mode TT: b stored [K, N] row-major (e.g. the output gradient dY[BT, OC] as the second
+        # operand of the weight gradient, without its transposed copy); bf16 output, whole 256-tiles only
+        if c.dtype != torch.bfloat16:
+            raise ValueError("matmul: the K-major second operand is served with bf16 output only")
+        pa = _dev(a, "a", (torch.float8_e4m3fn, torch.uint8))
+        pb = _dev(b, "b", (torch.float8_e4m3fn, torch.float8_e5m2, torch.uint8))
+        if a.numel() != M * K or b.numel() != N * K or c.numel() != N * M:
+            raise ValueError("operand sizes do not match M, N, K")
+        pbias = _dev(bias, "bias", (torch.bfloat16,), optional=True)
+        capi.check(capi.lib.llmq_gemm_e4m3_bf16_mode(
+            _dev(c, "c", (torch.bfloat16,)), pa, pb, pbias, _dev(scale_a, "scale_a", (torch.float32,), optional=True),
+            _dev(scale_b, "scale_b", (torch.float32,), optional=True), None, 0, M, N, K, 0,
+            int(bool(b_e5m2) or b.dtype == torch.float8_e5m2), int(accumulate), _stream(stream)))
+        return
     pws, ws_bytes = None, 0
     if workspace is not None:
         pws = _dev(workspace, "workspace", (torch.uint8, torch.int8, torch.float32))

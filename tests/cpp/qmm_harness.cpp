@@ -64,12 +64,19 @@ int main(int argc, char** argv) {
     const int BT = argc > 1 ? std::atoi(argv[1]) : 1024, C = argc > 2 ? std::atoi(argv[2]) : 896, OC = argc > 3 ? std::atoi(argv[3]) : 1152;
     const bool reuse_inp = argc > 4 && std::atoi(argv[4]) != 0;
     const bool fuse = argc > 5 && std::atoi(argv[5]) != 0;   // gradient quantize + transpose from one read
+    // 1: bf16 weight gradient; 2: also ask for the gradient's stored layout as the wgrad's K-major operand
+    const int dw_mode = argc > 6 ? std::atoi(argv[6]) : 0;
+    const bool dw_bf16 = dw_mode >= 1, direct = dw_mode == 2;
     const int B = 1, T = BT;
-    std::printf("qmm_harness BT=%d C=%d OC=%d reuse_inp=%d fuse=%d\n", BT, C, OC, (int)reuse_inp, (int)fuse);
+    std::printf("qmm_harness BT=%d C=%d OC=%d reuse_inp=%d fuse=%d dweight=%s direct_grad_layout=%d\n", BT, C, OC, (int)reuse_inp,
+                (int)fuse, dw_bf16 ? "bf16" : "fp32", (int)direct);
     hipStream_t stream; HIP_OK(hipStreamCreate(&stream));
     QmmRunState rs; HIP_OK(hipGetDeviceProperties(&rs.DeviceProp, 0));
     rs.FuseGradTranspose = fuse;
-    rs.Capacity = QmmRunState::backward_temp_bytes(B, T, C, OC, fuse);
+    rs.DirectGradLayout = direct;
+    const bool direct_applies = direct && QmmRunState::direct_grad_layout_applies(B, T, C, OC, dw_bf16 ? ETensorDType::BF16 : ETensorDType::FP32, false);
+    std::printf("direct gradient layout applies: %d\n", (int)direct_applies);
+    rs.Capacity = QmmRunState::backward_temp_bytes(B, T, C, OC, fuse, direct_applies);
     rs.Arena = dalloc<std::byte>(rs.Capacity);
 
     std::vector<uint16_t> hx((std::size_t)BT * C), hw((std::size_t)OC * C), hdy((std::size_t)BT * OC);
@@ -89,7 +96,8 @@ int main(int argc, char** argv) {
     Tensor weight = make(ETensorDType::FP8_E4M3, dalloc<uint8_t>(hw.size()), {OC, C}, stats + 2);
     Tensor out = make(ETensorDType::BF16, dalloc<uint16_t>((std::size_t)BT * OC), {BT, OC});
     Tensor dinp = make(ETensorDType::BF16, dalloc<uint16_t>((std::size_t)BT * C), {BT, C});
-    Tensor dweight = make(ETensorDType::FP32, dalloc<float>((std::size_t)OC * C), {OC, C});
+    Tensor dweight = dw_bf16 ? make(ETensorDType::BF16, dalloc<uint16_t>((std::size_t)OC * C), {OC, C})
+                             : make(ETensorDType::FP32, dalloc<float>((std::size_t)OC * C), {OC, C});
     Tensor no_bias{};
     // matmul workspace sized like the reference's (src/training/model.cpp:69)
     Tensor workspace = make(ETensorDType::BYTE, dalloc<uint8_t>(32u << 20), {32L << 20});
@@ -131,17 +139,19 @@ int main(int argc, char** argv) {
     HIP_OK(hipMemcpy(got.data(), dout.Quant.Data, gq.size(), hipMemcpyDeviceToHost));
     EXPECT(std::memcmp(got.data(), gq.data(), gq.size()) == 0, "dy quantized bytes differ");
 
-    std::vector<uint16_t> hy((std::size_t)BT * OC), hdx((std::size_t)BT * C); std::vector<float> hdw((std::size_t)OC * C);
+    std::vector<uint16_t> hy((std::size_t)BT * OC), hdx((std::size_t)BT * C), hdw16; std::vector<float> hdw;
+    if (dw_bf16) hdw16.resize((std::size_t)OC * C); else hdw.resize((std::size_t)OC * C);
     HIP_OK(hipMemcpy(hy.data(), out.Data, hy.size() * 2, hipMemcpyDeviceToHost));
     HIP_OK(hipMemcpy(hdx.data(), dinp.Data, hdx.size() * 2, hipMemcpyDeviceToHost));
-    HIP_OK(hipMemcpy(hdw.data(), dweight.Data, hdw.size() * 4, hipMemcpyDeviceToHost));
+    if (dw_bf16) HIP_OK(hipMemcpy(hdw16.data(), dweight.Data, hdw16.size() * 2, hipMemcpyDeviceToHost));
+    else HIP_OK(hipMemcpy(hdw.data(), dweight.Data, hdw.size() * 4, hipMemcpyDeviceToHost));
     std::vector<uint8_t> wqt(wq.size()), xqt(xq.size()), gqt(gq.size());
     orc_transpose_u8(wqt.data(), wq.data(), OC, C);
     orc_transpose_u8(xqt.data(), xq.data(), BT, C);
     orc_transpose_u8(gqt.data(), gq.data(), BT, OC);
     check_gemm("forward", hy, {}, BT, OC, wq.data(), xq.data(), C, sw * sx);
     check_gemm("dgrad", hdx, {}, BT, C, wqt.data(), gq.data(), OC, sw * sg);
-    check_gemm("wgrad", {}, hdw, OC, C, xqt.data(), gqt.data(), BT, sx * sg);
+    check_gemm("wgrad", hdw16, hdw, OC, C, xqt.data(), gqt.data(), BT, sx * sg);
 
     {   // dbias += sx*sg * column sums of the quantized gradient (llama_model.cpp:334-336)
         std::vector<uint16_t> hdb(OC), want(hdb0);

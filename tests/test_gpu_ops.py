@@ -70,6 +70,30 @@ def test_matmul_torch_convention(P, O):
         P.matmul(c, ad, bd[:, :256].contiguous(), None, None, None, 0, ws, P.MODE_NT, False)
 
 
+def test_matmul_mode_tt_reads_the_first_operand_in_k_major_storage(P, O):
+    """Mode TT in the torch sense: c[M,N] = a[K,M]^T @ b[N,K]^T.  The same codes handed over as a[M,K] in mode NT
+    give the same result to the tolerance, and both are checked against the exact product."""
+    M, N, Kd = 512, 256, 768
+    rng = np.random.default_rng(14)
+    a = rng.integers(0, 0x7E, (M, Kd)).astype(np.uint8) | (rng.integers(0, 2, (M, Kd)).astype(np.uint8) << 7)
+    b = rng.integers(0, 0x7E, (N, Kd)).astype(np.uint8)
+    ad = torch.from_numpy(a).cuda().view(torch.float8_e4m3fn)
+    at = torch.from_numpy(np.ascontiguousarray(a.T)).cuda().view(torch.float8_e4m3fn)      # [K, M]
+    bd = torch.from_numpy(b).cuda().view(torch.float8_e4m3fn)
+    sa, sb = torch.tensor([0.25], device="cuda"), torch.tensor([0.125], device="cuda")
+    bias = torch.randn(N, device="cuda", dtype=torch.bfloat16)
+    ws = torch.empty(32 << 20, dtype=torch.uint8, device="cuda")
+    c = torch.full((M, N), float("nan"), device="cuda", dtype=torch.bfloat16)
+    P.matmul(c, at, bd, bias, sa, sb, 0, ws, P.MODE_TT, False)
+    exact, sumabs = O.gemm_exact(b, a)
+    extra = bias.float().cpu().numpy().astype(np.float64)[None, :]
+    gemm_check(c.float().cpu().numpy(), exact, sumabs, np.float32(0.25 * 0.125), True, extra=extra)
+    with pytest.raises(ValueError):                                            # fp32 output is not served in this mode
+        P.matmul(torch.empty((M, N), device="cuda"), at, bd, None, None, None, 0, ws, P.MODE_TT, False)
+    with pytest.raises(ValueError):                                            # a is [K, M]: handing over [M, K] mismatches c
+        P.matmul(c, ad, bd, None, None, None, 0, ws, P.MODE_TT, False)
+
+
 def test_backward_bias_through_ops(P):
     torch.manual_seed(0)
     B, T, OC = 8, 16, 512                                                    # test_kernels.py:837-853

@@ -618,6 +618,67 @@ def test_gemm_general_shapes(K, O, mnk):
         gemm_check(c5.cpu().numpy(), exact5, sumabs5, 0.25, False)
 
 
+@pytest.mark.parametrize("mnk", [(256, 256, 256), (512, 768, 512), (448, 512, 768), (1024, 2048, 1024), (2304, 512, 2816),
+                                 (3584, 4096, 512)])
+def test_gemm_second_operand_in_k_major_layout(K, O, mnk):
+    """Mode TT of the reference's matmul signature (src/kernels/kernels.h:22, matmul.cpp:66-67): b stored [K, N]
+    row-major, read through transposing LDS reads instead of a materialised transpose (what backward_qmm does with
+    the output gradient, src/models/llama_model.cpp:331-333).  Integer operands -> bit exact against the oracle,
+    with bias and accumulation; random codes (e5m2 included) within the tolerance of the exact product and
+    bit-identical to mode TN on the transposed copy when that runs on the same kernel family (same sums in the same
+    order; the 8-wave kernel's other matrix instruction groups K differently)."""
+    M, N, Kd = mnk
+    a, _ = O.fill_int_e4m3(M * Kd, 606, 0)
+    b, _ = O.fill_int_e4m3(N * Kd, 606, 1)
+    a, b = a.reshape(M, Kd), b.reshape(N, Kd)
+    bt = np.ascontiguousarray(b.T)                      # [K, N]: what the caller holds
+    s = float(np.sqrt(np.float32(4.0 / Kd)))
+    _, biasv = O.fill_int_e4m3(M, 606, 2)
+    _, oldv = O.fill_int_e4m3(N * M, 606, 3)
+    bias = O.f32_to_bf16(biasv.astype(np.float32))
+    old = O.f32_to_bf16(oldv.astype(np.float32)).reshape(N, M)
+    mt = M % 64 == 0
+    cases = [(False, False), (True, False)] + ([(True, True)] if M % 256 == 0 else [])
+    for use_bias, use_old in cases:
+        want = O.gemm_tn(a, b, sa=s, sb=s, bias=bias if use_bias else None, c_old=old if use_old else None, mt=mt)
+        c = dev_bf16(old).reshape(N, M).clone() if use_old else torch.full((N, M), float("nan"), dtype=torch.bfloat16, device="cuda")
+        K.matmul(c, dev_u8(a), dev_u8(bt), dev_bf16(bias) if use_bias else None, dev_scalar(s), dev_scalar(s), M, N, Kd,
+                 accumulate=use_old, b_kmajor=True)
+        assert np.array_equal(host_bits(c), want), (use_bias, use_old)
+    rng = np.random.default_rng(M + Kd)
+    for e5m2 in (False, True):
+        ar = rng.integers(0, 256, (M, Kd)).astype(np.uint8)
+        br = rng.integers(0, 256, (N, Kd)).astype(np.uint8)
+        ar[(ar & 0x7F) == 0x7F] ^= 1
+        if e5m2:
+            br[(br & 0x7C) == 0x7C] ^= 0x40
+            br &= 0xBF
+        else:
+            br[(br & 0x7F) == 0x7F] ^= 1
+        c_tn = torch.empty((N, M), dtype=torch.bfloat16, device="cuda")
+        c_tt = torch.empty((N, M), dtype=torch.bfloat16, device="cuda")
+        K.matmul(c_tt, dev_u8(ar), dev_u8(np.ascontiguousarray(br.T)), None, dev_scalar(0.37), dev_scalar(1.0 / 448), M, N, Kd,
+                 b_e5m2=e5m2, b_kmajor=True)
+        exact, sumabs = O.gemm_exact(ar, br, b_e5m2=e5m2)
+        gemm_check(c_tt.float().cpu().numpy(), exact, sumabs, np.float32(np.float32(0.37) * np.float32(1.0 / 448)), True)
+        set_variant((4, 0) if M % 256 else (3, 1))       # mode TN on the same kernel family: the same sums in the same order
+        try:
+            mm(K, c_tn, dev_u8(ar), dev_u8(br), None, dev_scalar(0.37), dev_scalar(1.0 / 448), M, N, Kd, b_e5m2=e5m2)
+        finally:
+            set_variant((0, 0))
+        assert torch.equal(c_tn.view(torch.int16), c_tt.view(torch.int16)), e5m2
+
+
+def test_gemm_k_major_operand_rejects_what_it_cannot_serve(K):
+    a = torch.zeros((256, 384), dtype=torch.uint8, device="cuda")
+    b = torch.zeros((384, 256), dtype=torch.uint8, device="cuda")
+    c = torch.zeros((256, 256), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ValueError, match="mode TT"):
+        K.matmul(c, a, b, None, None, None, 256, 256, 384, b_kmajor=True)      # K % 256 != 0
+    with pytest.raises(ValueError, match="bf16 output"):
+        K.matmul(c.float(), a, b, None, None, None, 256, 256, 384, b_kmajor=True)
+
+
 def test_gemm_rejects_unaligned_k(K):
     a = torch.zeros((128, 72), dtype=torch.uint8, device="cuda")
     c = torch.zeros((128, 128), dtype=torch.bfloat16, device="cuda")
