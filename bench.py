@@ -411,6 +411,11 @@ def main():
             # read + write stream on this chip, for reading the fractions above
             "plain copy kernel, same protocol (2 B/el)": cold_run(lambda i: capi.check(capi.testaid().llmq_debug_copy_u8(
                 qt_dsts[i].data_ptr(), q_srcs[(i + 1) % 3].data_ptr(), n_h, torch.cuda.current_stream().cuda_stream)), 2 * n_h),
+            # the same access pattern with the reads only (310 MB: what abs-max streams) and with the writes only
+            "plain read-only kernel, same protocol (2 B/el)": cold_run(lambda i: capi.check(capi.testaid().llmq_debug_stream_u8(
+                am3[i].data_ptr(), srcs[i].data_ptr(), 2 * n_h, 0, torch.cuda.current_stream().cuda_stream)), 2 * n_h),
+            "plain write-only kernel, same protocol (1 B/el)": cold_run(lambda i: capi.check(capi.testaid().llmq_debug_stream_u8(
+                qt_dsts[i].data_ptr(), None, n_h, 1, torch.cuda.current_stream().cuda_stream)), n_h),
         }
         K.abs_max(stats["h"][0:1], t["h"])   # restore what the step left in the buffers used above
         K.quantize_with_abs_max(q["h"], stats["h"][1:2], t["h"], stats["h"][0:1])

@@ -82,8 +82,8 @@ _testaid = None
 def testaid():
     """The test-aid library (tests and bench.py only; never needed by a user of the path): the four matmul
     entry points from a build of the GEMM file whose kernel selection can be forced
-    (llmq_debug_set_gemm_variant / llmq_debug_set_gemm_persist), and the measurement aids llmq_debug_copy_u8
-    (plain copy kernel) and llmq_debug_mfma_ceiling (register-only matrix-instruction loop)."""
+    (llmq_debug_set_gemm_variant / llmq_debug_set_gemm_persist), and the measurement aids llmq_debug_copy_u8 and llmq_debug_stream_u8
+    (plain copy, read-only and write-only kernels) and llmq_debug_mfma_ceiling (register-only matrix-instruction loop)."""
     global _testaid
     if _testaid is None:
         if not os.path.exists(TESTAID_PATH):
@@ -100,6 +100,8 @@ def testaid():
         t.llmq_debug_set_gemm_persist.restype = None
         t.llmq_debug_copy_u8.argtypes = [_vp, _vp, _i64, _vp]
         t.llmq_debug_copy_u8.restype = _int
+        t.llmq_debug_stream_u8.argtypes = [_vp, _vp, _i64, _int, _vp]
+        t.llmq_debug_stream_u8.restype = _int
         t.llmq_debug_mfma_ceiling.argtypes = [_vp, _int, _int, _int, _vp]
         t.llmq_debug_mfma_ceiling.restype = _int
         _testaid = t

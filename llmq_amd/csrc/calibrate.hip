@@ -2,6 +2,9 @@
 //
 //  * llmq_debug_copy_u8: a plain streaming copy whose HBM bytes are known exactly (n read + n
 //    written); hardware traffic counters of the real kernels are scaled by what they read for it.
+//  * llmq_debug_read_u8 / llmq_debug_fill_u8: the same access pattern with only the reads (folded into one
+//    word per lane that is never stored) resp. only the writes: what a read-only stream (abs-max) and a
+//    write-only stream sustain, beside the copy's figure for a read + write stream.
 //  * llmq_debug_mfma_ceiling: a loop of fp8 matrix instructions on register operands with no memory
 //    traffic at all, 8 waves per compute unit.  With constant operands it runs at the nominal clock;
 //    with random fp8 operands that change every iteration (what a real K loop feeds the matrix cores)
@@ -23,6 +26,32 @@ __global__ __launch_bounds__(256) void copy_calibration_kernel(uint4* __restrict
     for (int u = 0; u < 4; ++u) {
         const int64_t i = base + u * stride;
         if (i < nvec) dst[i] = src[i];
+    }
+}
+
+__global__ __launch_bounds__(256) void read_calibration_kernel(uint32_t* __restrict__ sink, const uint4* __restrict__ src,
+                                                               int64_t nvec) {
+    const int64_t base = ((int64_t)blockIdx.x * 256 + threadIdx.x);
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    uint4 v[4];
+#pragma unroll 4
+    for (int u = 0; u < 4; ++u) {
+        const int64_t i = base + u * stride;
+        v[u] = i < nvec ? src[i] : make_uint4(0, 0, 0, 0);
+    }
+    uint32_t x = 0;
+#pragma unroll 4
+    for (int u = 0; u < 4; ++u) x |= (v[u].x & v[u].y) ^ (v[u].z & v[u].w);
+    if (x == 0xDEADBEEFu) sink[0] = x;   // practically never true (and harmless if it is): keeps the loads alive
+}
+
+__global__ __launch_bounds__(256) void fill_calibration_kernel(uint4* __restrict__ dst, int64_t nvec, uint32_t value) {
+    const int64_t base = ((int64_t)blockIdx.x * 256 + threadIdx.x);
+    const int64_t stride = (int64_t)gridDim.x * 256;
+#pragma unroll 4
+    for (int u = 0; u < 4; ++u) {
+        const int64_t i = base + u * stride;
+        if (i < nvec) dst[i] = make_uint4(value, value + (uint32_t)i, value, value);
     }
 }
 
@@ -99,6 +128,21 @@ extern "C" __attribute__((visibility("default"))) int llmq_debug_copy_u8(uint8_t
     LLMQ_REQUIRE(blocks <= 0x7FFFFFFF, "copy: too large");
     hipLaunchKernelGGL(copy_calibration_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
                        reinterpret_cast<uint4*>(dst), reinterpret_cast<const uint4*>(src), nvec);
+    LLMQ_HIP_TRY(hipGetLastError());
+    return LLMQ_OK;
+}
+
+// mode 0: read n bytes of src (dst: at least 4 bytes, never written); mode 1: write n bytes of dst (src unused).
+extern "C" __attribute__((visibility("default"))) int llmq_debug_stream_u8(uint8_t* dst, const uint8_t* src, int64_t n, int mode, void* stream) {
+    using namespace llmq;
+    LLMQ_REQUIRE(dst && n > 0 && n % 16 == 0 && (mode == 1 || src), "stream: need non-null pointers and a positive multiple of 16 bytes");
+    LLMQ_REQUIRE(aligned16(dst) && aligned16(src) && (mode == 0 || mode == 1), "stream: 16-byte aligned pointers, mode 0 or 1");
+    const int64_t nvec = n / 16;
+    const int64_t blocks = (nvec + 1023) / 1024;
+    LLMQ_REQUIRE(blocks <= 0x7FFFFFFF, "stream: too large");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (mode == 0) hipLaunchKernelGGL(read_calibration_kernel, dim3((unsigned)blocks), dim3(256), 0, st, reinterpret_cast<uint32_t*>(dst), reinterpret_cast<const uint4*>(src), nvec);
+    else hipLaunchKernelGGL(fill_calibration_kernel, dim3((unsigned)blocks), dim3(256), 0, st, reinterpret_cast<uint4*>(dst), nvec, 0x38383838u);
     LLMQ_HIP_TRY(hipGetLastError());
     return LLMQ_OK;
 }

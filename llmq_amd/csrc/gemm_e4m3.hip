@@ -849,6 +849,12 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     [[maybe_unused]] int stage_rt = 0;  // ODDK: byte offset of the LDS stage of the current K-step
     // par_tag: LDS stage of the step; fp_tag: the half of fb that holds its second-operand fragments (the same
     // as the stage unless ODDK, see the tile loop).
+#ifndef LLMQ_TWO_BARRIERS
+#define LLMQ_TWO_BARRIERS 1
+#endif
+    // copies of this step that are in flight at the step's barrier and need not have landed (they refill the
+    // stage this step computes from)
+    constexpr int kYoung = LLMQ_TWO_BARRIERS ? ITERS_Q : 0;
     auto k_step = [&](auto par_tag, auto fp_tag, auto first_tag) {
         constexpr int PAR = decltype(par_tag)::value;
         constexpr int FP = decltype(fp_tag)::value;
@@ -864,15 +870,31 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         // time; a denser burst backs up into the waves' instruction issue and stalls the matrix instructions
         // behind it (one copy per instruction over rows 5 and 6: 4 % slower over six large shapes; all sixteen right
         // after the barrier: 11 %).
+#if LLMQ_TWO_BARRIERS
+        // The a-rows half of this stage was read in the previous step (fb of this step is in registers): once
+        // every wave is here it may be refilled, half a step before the b-rows half.
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __syncthreads();
+        constexpr int Q_SLOTS = 4 * NJ, SPREAD = ITERS - 4, SLOTS = 3 * NJ;
+#else
         constexpr int SPREAD = COPIES - 4, SLOTS = 3 * NJ;
+#endif
         static_assert(SPREAD <= SLOTS, "not every copy of a K-step has a place in the schedule");
         static_for<0, NF>([&](auto i_tag) {
             constexpr int i = decltype(i_tag)::value;
             static_for<0, NJ>([&](auto j_tag) {
                 constexpr int j = decltype(j_tag)::value;
                 constexpr int p = (i - 5) * NJ + j;  // slot in rows 5..7
+#if LLMQ_TWO_BARRIERS
+                constexpr int pq = i * NJ + j;  // slot in rows 0..3
+                constexpr bool Q_HERE = i < 4 && ((pq + 1) * ITERS_Q / Q_SLOTS > pq * ITERS_Q / Q_SLOTS);
+                constexpr bool P_HERE = i >= 5 && ((p + 1) * SPREAD / SLOTS > p * SPREAD / SLOTS);
+                constexpr bool COPY_HERE = Q_HERE || P_HERE;
+                constexpr int COPY_C = Q_HERE ? ITERS + pq * ITERS_Q / Q_SLOTS : P_HERE ? 4 + p * SPREAD / SLOTS : 0;
+#else
                 constexpr bool COPY_HERE = i >= 5 && ((p + 1) * SPREAD / SLOTS > p * SPREAD / SLOTS);
                 constexpr int COPY_C = COPY_HERE ? 4 + p * SPREAD / SLOTS : 0;
+#endif
                 uint32_t tok = 0;
                 if constexpr (COPY_HERE) tok = set_m0(std::integral_constant<int, COPY_C>{}, refill);
                 if constexpr (FIRST) mfma_first(acc[i][j], fa[i % 4], fb[FP][j]);
@@ -892,13 +914,13 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
                     // previous tile's epilogue) sit that epilogue's stores; the counter retires in issue
                     // order, so allowing as many outstanding operations as there were stores is enough.
                     if (pending_stores) {
-                        if constexpr (sizeof(OutT) == 2 && NJ != 7) asm volatile("s_waitcnt vmcnt(32) lgkmcnt(0)" ::: "memory");
+                        if constexpr (sizeof(OutT) == 2 && NJ != 7) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(32 + kYoung) : "memory");
                         else asm volatile("s_waitcnt vmcnt(63) lgkmcnt(0)" ::: "memory");
                     } else {
-                        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kYoung) : "memory");
                     }
                 } else {
-                    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kYoung) : "memory");
                 }
                 __syncthreads();
                 // copies 0..3, each with one of the four LDS reads of the next step's first two second-operand
