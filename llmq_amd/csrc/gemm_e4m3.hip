@@ -842,19 +842,26 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     // One K-step of parity PAR (LDS stage PAR, fb half PAR): rows i = 0..7 of first-operand fragments
     // against all 8 second-operand fragments.  fa rotates through 4 slots (fragment i+4 is read once row i
     // has been issued; rows 4..7 fetch the next step's first four from the other stage); the next step's
-    // second-operand fragments go into the other half of fb, two per row in rows 4..7 (after the barrier).  The 16 copies of
-    // the step after next go into the stage this step releases: 4 right after the barrier, the rest spread
-    // evenly over the matrix instructions of rows 5..7.
+    // second-operand fragments go into the other half of fb, two per row in rows 4..7 (after the barrier).
+    // The 16 copies of the step after next go into the stage this step computes from, each half as soon as it is
+    // free.  The a-rows half was read into fb during the previous step: a barrier at the start of the step releases
+    // it, and its copies follow every fourth matrix instruction of rows 0..3.  The b-rows half is read until row 3:
+    // the barrier after row 4 releases it (and confirms that the other stage has landed); 4 copies right after that
+    // barrier, the rest spread over rows 5..7.  A copy so has 5 to 13 rows of matrix instructions (256 cycles each) to
+    // land before the barrier that needs it.  With a single barrier per step and all copies in rows 4..7 (4 to 8
+    // rows to land) the waves spent 10 % of their cycles waiting at that barrier for data from beyond the L2; the
+    // second barrier made six large shapes 6 % faster (2.90 -> 3.08 PFLOP/s, one box, alternating launches).
+    // Measured against it and not kept: all eight b-rows fragments of a step in registers, so that the whole stage is
+    // released at the start of the step and the landing barrier moves to row 6 (copies have 7 to 14 rows): 1-4 % slower,
+    // the 32 extra live registers push address registers into scratch around the tile epilogue.  Shorter copy windows
+    // (rows 0..2 for the a-rows half, rows 5..6 or row 5 for the b-rows half): 0.3-1 % slower.
     bool pending_stores = false;  // an epilogue without accumulation has just issued its stores
     [[maybe_unused]] int stage_rt = 0;  // ODDK: byte offset of the LDS stage of the current K-step
     // par_tag: LDS stage of the step; fp_tag: the half of fb that holds its second-operand fragments (the same
     // as the stage unless ODDK, see the tile loop).
-#ifndef LLMQ_TWO_BARRIERS
-#define LLMQ_TWO_BARRIERS 1
-#endif
-    // copies of this step that are in flight at the step's barrier and need not have landed (they refill the
-    // stage this step computes from)
-    constexpr int kYoung = LLMQ_TWO_BARRIERS ? ITERS_Q : 0;
+    // kYoung: copies of this step that are in flight at the step's second barrier and need not have landed (they
+    // refill the a-rows half of the stage this step computes from)
+    constexpr int kYoung = ITERS_Q;
     auto k_step = [&](auto par_tag, auto fp_tag, auto first_tag) {
         constexpr int PAR = decltype(par_tag)::value;
         constexpr int FP = decltype(fp_tag)::value;
@@ -864,37 +871,27 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         const uint8_t* nxt = lds + (ODDK ? STAGE - stage_rt : (1 - PAR) * STAGE);
         constexpr std::integral_constant<int, ODDK ? 0 : PAR * STAGE> refill{};
         if constexpr (ODDK) lds_wave_stage = lds_wave + (uint32_t)stage_rt;
-        // copies 4 .. COPIES - 1: spread evenly over the matrix instructions of rows 5..7 (with NJ = 8 after every
-        // second one); the write of M0 for a copy sits in front of the matrix instruction the copy follows.  The
-        // CU's one address unit takes 16 cycles per copy instruction and the four waves issue theirs at the same
-        // time; a denser burst backs up into the waves' instruction issue and stalls the matrix instructions
-        // behind it (one copy per instruction over rows 5 and 6: 4 % slower over six large shapes; all sixteen right
-        // after the barrier: 11 %).
-#if LLMQ_TWO_BARRIERS
-        // The a-rows half of this stage was read in the previous step (fb of this step is in registers): once
-        // every wave is here it may be refilled, half a step before the b-rows half.
+        // The write of M0 for a copy sits in front of the matrix instruction the copy follows.  The CU's one
+        // address unit takes 16 cycles per copy instruction and the four waves issue theirs at the same time; a
+        // dense burst backs up into the waves' instruction issue and stalls the matrix instructions behind it (with
+        // all copies behind the second barrier: one per instruction over rows 5 and 6 was 4 % slower over six large
+        // shapes than spread over rows 5..7, all sixteen right after the barrier 11 %).
+        // First barrier: the a-rows half of this stage was read during the previous step; once every wave's reads
+        // have returned and all waves are here it may be refilled.
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         __syncthreads();
         constexpr int Q_SLOTS = 4 * NJ, SPREAD = ITERS - 4, SLOTS = 3 * NJ;
-#else
-        constexpr int SPREAD = COPIES - 4, SLOTS = 3 * NJ;
-#endif
         static_assert(SPREAD <= SLOTS, "not every copy of a K-step has a place in the schedule");
         static_for<0, NF>([&](auto i_tag) {
             constexpr int i = decltype(i_tag)::value;
             static_for<0, NJ>([&](auto j_tag) {
                 constexpr int j = decltype(j_tag)::value;
                 constexpr int p = (i - 5) * NJ + j;  // slot in rows 5..7
-#if LLMQ_TWO_BARRIERS
                 constexpr int pq = i * NJ + j;  // slot in rows 0..3
                 constexpr bool Q_HERE = i < 4 && ((pq + 1) * ITERS_Q / Q_SLOTS > pq * ITERS_Q / Q_SLOTS);
                 constexpr bool P_HERE = i >= 5 && ((p + 1) * SPREAD / SLOTS > p * SPREAD / SLOTS);
                 constexpr bool COPY_HERE = Q_HERE || P_HERE;
                 constexpr int COPY_C = Q_HERE ? ITERS + pq * ITERS_Q / Q_SLOTS : P_HERE ? 4 + p * SPREAD / SLOTS : 0;
-#else
-                constexpr bool COPY_HERE = i >= 5 && ((p + 1) * SPREAD / SLOTS > p * SPREAD / SLOTS);
-                constexpr int COPY_C = COPY_HERE ? 4 + p * SPREAD / SLOTS : 0;
-#endif
                 uint32_t tok = 0;
                 if constexpr (COPY_HERE) tok = set_m0(std::integral_constant<int, COPY_C>{}, refill);
                 if constexpr (FIRST) mfma_first(acc[i][j], fa[i % 4], fb[FP][j]);
