@@ -149,6 +149,20 @@ def run_linear_fwd_bwd(K, O, BT, C, OC, x, w, dy, seed, backward=True, reuse_inp
     assert np.array_equal(host_bits(g_tp), gc.T), "gradient transpose"
     check_gemm(O, dinp, np.ascontiguousarray(wc.T), gc, dw_s, dg_s, seed + 1, "dgrad dx")
     check_gemm(O, dweight, np.ascontiguousarray(xc.T), np.ascontiguousarray(gc.T), dx_s, dg_s, seed + 2, "wgrad dw")
+    # The same weight gradient with the quantized output gradient read where it lies (matmul mode TT: dout.quant
+    # [BT, OC] as the K-major second operand, no transposed copy), wherever that mode serves the shape
+    if OC % 256 == 0 and BT % 256 == 0 and (C % 256 == 0 or C % 224 == 0):
+        dw_tt = torch.full((OC, C), float("nan"), dtype=torch.bfloat16, device="cuda")
+        K.matmul(dw_tt, a_tp, dout.quant, None, inp.scale, dout.scale, C, OC, BT, b_kmajor=True)
+        torch.cuda.synchronize()
+        check_gemm(O, dw_tt, np.ascontiguousarray(xc.T), np.ascontiguousarray(gc.T), dx_s, dg_s, seed + 2, "wgrad dw, mode TT")
+        if C % 256 == 0:
+            old_tt = dw_tt.float().cpu().numpy()
+            K.matmul(dw_tt, a_tp, dout.quant, None, inp.scale, dout.scale, C, OC, BT, accumulate=True, b_kmajor=True)
+            torch.cuda.synchronize()
+            check_gemm(O, dw_tt, np.ascontiguousarray(xc.T), np.ascontiguousarray(gc.T), dx_s, dg_s, seed + 2,
+                       "wgrad dw +=, mode TT", c_old=old_tt)
+        del dw_tt
     # accumulate into an existing gradient (second micro-step of gradient accumulation)
     old = dweight.float().cpu().numpy()
     K.matmul(dweight, a_tp, g_tp, None, inp.scale, dout.scale, C, OC, BT, accumulate=True,

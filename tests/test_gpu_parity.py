@@ -667,6 +667,11 @@ def test_gemm_second_operand_in_k_major_layout(K, O, mnk):
         finally:
             set_variant((0, 0))
         assert torch.equal(c_tn.view(torch.int16), c_tt.view(torch.int16)), e5m2
+        for _ in range(8):                                  # repeated launches: the same bits every time
+            again = torch.full((N, M), float("nan"), dtype=torch.bfloat16, device="cuda")
+            K.matmul(again, dev_u8(ar), dev_u8(np.ascontiguousarray(br.T)), None, dev_scalar(0.37), dev_scalar(1.0 / 448), M, N, Kd,
+                     b_e5m2=e5m2, b_kmajor=True)
+            assert torch.equal(again.view(torch.int16), c_tt.view(torch.int16)), e5m2
 
 
 def test_gemm_k_major_operand_rejects_what_it_cannot_serve(K):
