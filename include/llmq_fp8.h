@@ -140,8 +140,8 @@ int llmq_gemm_tn_e4m3_bf16(uint16_t* c, const uint8_t* a, const uint8_t* b, cons
  *                                    operand of the weight gradient, so that no transposed copy of it is needed)
  * The reference's FP8 path takes TN only (it materialises the transposes, src/models/llama_model.cpp:309-339) and
  * modes NT / NN (a stored [K, M]) are not provided here either.  TT: N and K multiples of 256, M a multiple of 256
- * (without accumulation also of 224); other shapes return LLMQ_ERR_INVALID_ARGUMENT and the caller takes the
- * transposing route.  b_format: 0 = e4m3, 1 = e5m2.  Results are bit-identical to mode TN on the transposed copy.
+ * (without accumulation also of 224), K * N below 2 GiB; other shapes return LLMQ_ERR_INVALID_ARGUMENT and the caller
+ * takes the transposing route.  b_format: 0 = e4m3, 1 = e5m2.  Results are bit-identical to mode TN on the transposed copy.
  */
 #define LLMQ_MODE_TT 0
 #define LLMQ_MODE_TN 1

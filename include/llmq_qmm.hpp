@@ -33,7 +33,7 @@ struct QmmRunState {
     // the larger cost while C, the matmul's row count, stays below about 10^4.
     static bool direct_grad_layout_applies(int B, int T, int C, int OC, ETensorDType dweight_dtype, bool accumulate) {
         const long BT = (long)B * T;
-        return dweight_dtype == ETensorDType::BF16 && OC % 256 == 0 && BT % 256 == 0 &&
+        return dweight_dtype == ETensorDType::BF16 && OC % 256 == 0 && BT % 256 == 0 && BT * OC < (1L << 31) &&
                (C % 256 == 0 || (C % 224 == 0 && !accumulate)) && C <= 8192;
     }
     std::vector<std::byte*> Live;

@@ -1598,6 +1598,10 @@ static int gemm_dispatch_b_kmajor(GemmArgs g, hipStream_t stream) {
     LLMQ_REQUIRE(g.N % 256 == 0 && g.K % 256 == 0 && (g.M % 256 == 0 || m224) && cus % xcds == 0,
                  "matmul: the K-major second operand (mode TT) needs N %% 256 == 0, K %% 256 == 0 and M %% 256 == 0 (without "
                  "accumulation also M %% 224 == 0); got M, N, K = %d, %d, %d", g.M, g.N, g.K);
+    // the copies of the K-major operand address it as "tile base + 32-bit lane offset", and that offset walks the
+    // whole K extent of the operand (K * N bytes)
+    LLMQ_REQUIRE((int64_t)g.K * g.N < ((int64_t)1 << 31), "matmul: the K-major second operand must be smaller than 2 GiB "
+                 "(K * N = %lld bytes)", (long long)((int64_t)g.K * g.N));
     const int tiles = (g.N / 256) * (m224 ? g.M / 224 : g.M / 256);
     const int grid = tiles < cus ? (tiles + xcds - 1) / xcds * xcds : cus;
     const bool cached_out = ((int64_t)g.M + g.N) * g.K + (int64_t)g.N * g.M * 2 <= ((int64_t)224 << 20);

@@ -682,6 +682,12 @@ def test_gemm_k_major_operand_rejects_what_it_cannot_serve(K):
         K.matmul(c, a, b, None, None, None, 256, 256, 384, b_kmajor=True)      # K % 256 != 0
     with pytest.raises(ValueError, match="bf16 output"):
         K.matmul(c.float(), a, b, None, None, None, 256, 256, 384, b_kmajor=True)
+    # a K-major operand of 2 GiB or more is refused before anything is launched (32-bit lane offsets walk it);
+    # called through the C ABI with the sizes alone, no such tensor is allocated
+    from llmq_amd import capi
+    rc = capi.lib.llmq_gemm_e4m3_bf16_mode(c.data_ptr(), a.data_ptr(), b.data_ptr(), None, None, None, None, 0,
+                                           256, 65536, 32768, 0, 0, 0, None)
+    assert rc == capi.LLMQ_ERR_INVALID_ARGUMENT and b"2 GiB" in capi.lib.llmq_last_error()
 
 
 def test_gemm_rejects_unaligned_k(K):
