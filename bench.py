@@ -358,8 +358,10 @@ def main():
         g5 = torch.empty((BT, UP), dtype=torch.float8_e5m2, device=dev)
         swiglu["quantize to e5m2 [8192 x 37888] (3 B/el)"] = gbs(
             lambda: K.quantize_with_abs_max(g5, sw_sc, t["dy_up"], stats["dy_up"][0:1]), 3 * BT * UP)
-        e5 = gbs(lambda: K.matmul(out["dx"], q["w_up_t"], g5, None, stats["w_up"][1:2], sw_sc, C, BT, UP, workspace=ws), 1)
-        swiglu["matmul e4m3 x e5m2, gate_up dgrad shape"] = {"TFLOPs": 2.0 * C * BT * UP / e5["mean_us"] / 1e6, "mean_us": e5["mean_us"]}
+        e5_us = min(gbs(lambda: K.matmul(out["dx"], q["w_up_t"], g5, None, stats["w_up"][1:2], sw_sc, C, BT, UP, workspace=ws), 1)["mean_us"]
+                    for _ in range(3))
+        swiglu["matmul e4m3 x e5m2, gate_up dgrad shape"] = {"TFLOPs": 2.0 * C * BT * UP / e5_us / 1e6, "us": e5_us,
+                                                             "timing": "best of 3 x 5 launches"}
         del g5
         swiglu["fused_residual_rmsnorm_forward+abs_max (8 B/el)"] = gbs(
             lambda: K.fused_residual_rmsnorm_forward(r_out, r_norm, r_rms, r_in, r_att, r_w, sw_am, 1e-6), 8 * BT * C, iters=10)
