@@ -249,6 +249,10 @@ inline void quantize_with_abs_max_and_transpose(Tensor& out, Tensor& out_tp, flo
 
 // ---- matmul (reference: src/kernels/kernels.h:72-78, 88-90, 96-98) --------------------------------------
 // Row-major a[M,K], b[N,K] -> row-major c[N,M] = (b . a^T) * (*scale_a * *scale_b) (+ bias[M]) (+ c).
+// Mode TN: any M, N >= 1 and K a multiple of 16 (16-byte aligned fp8 rows).  bf16 output also takes mode TT (b stored
+// [K, N]: e.g. the output gradient dY[B*T, OC] of the weight gradient without its transposed copy) when N and K are
+// multiples of 256 and M of 256 (without accumulation also of 224).  Anything else throws std::invalid_argument
+// before a kernel is launched.
 inline void matmul(__hip_bfloat16* c, const __hip_fp8_e4m3* a, const __hip_fp8_e4m3* b, const __hip_bfloat16* bias,
                    const float* scale_a, const float* scale_b, llmqBlasHandle_t, std::byte* workspace,
                    std::size_t workspace_size, int M, int N, int K, EMMTranspose mode, bool accumulate,
