@@ -641,6 +641,15 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     }
     if (my_tiles <= 0) return;  // uniform for the whole workgroup, before any barrier
     auto decode = [&](int logical, int& n_blk, int& m_blk) { decode_tile256<BLKM>(g, logical, n_blk, m_blk); };
+    // The output factor sa * sb is read here, once, before the copy stream starts.  Read in the epilogue it would be
+    // two global loads per tile, and the wait the compiler puts behind each of them (it counts only the loads it
+    // knows about, so it waits for "all": vmcnt(0)) would also drain the copies of the next tile's first two K-steps
+    // that are in flight at that point.
+    float out_scale = 1.f;
+    if constexpr (!SEG) {
+        if (g.sa) out_scale = *g.sa;
+        if (g.sb) out_scale = out_scale * *g.sb;
+    }
 
     // copies: lane -> (row tid/8 of a 32-row slab, physical 16-byte chunk tid%8); every address is a
     // wave-uniform base plus a 32-bit lane offset
@@ -993,14 +1002,12 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         int n_blk, m_blk;
         decode(logical, n_blk, m_blk);
         logical += tile_stride;
-        float scale = 1.f;
+        const float scale = out_scale;
         int ldc = BLK;
         OutT* c = reinterpret_cast<OutT*>(g.partial + ((int64_t)xcd * g.part_per_xcd + slot) * (BLK * BLK));
         if constexpr (SEG) {
             n_blk = m_blk = 0;  // tile-local coordinates in this slot's partial tile
         } else {
-            if (g.sa) scale = *g.sa;
-            if (g.sb) scale = scale * *g.sb;
             ldc = g.M;
             c = reinterpret_cast<OutT*>(g.c);
         }
