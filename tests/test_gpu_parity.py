@@ -618,6 +618,48 @@ def test_gemm_general_shapes(K, O, mnk):
         gemm_check(c5.cpu().numpy(), exact5, sumabs5, 0.25, False)
 
 
+def _swept_shapes():
+    """Seeded shapes around the edges of the dispatch's lattice: M on or just off multiples of 128 / 192 / 224 / 256, N
+    with every kind of remainder, K any multiple of 16 (one K-step, odd and even step counts, not a multiple of 128)."""
+    rng = np.random.default_rng(20260)
+    shapes = []
+    for _ in range(28):
+        base_m = int(rng.choice([128, 192, 224, 256, 384, 448, 512, 640, 768]))
+        M = max(1, base_m + int(rng.choice([0, 0, 0, 0, -8, 8, -1, 1, 16])))
+        N = int(rng.choice([1, 17, 64, 127, 128, 129, 200, 255, 256, 257, 300, 384, 511, 512, 520, 640, 777]))
+        Kd = 16 * int(rng.choice([1, 2, 5, 8, 9, 16, 17, 24, 32, 40, 48, 56, 64]))
+        shapes.append((M, N, Kd))
+    return shapes
+
+
+@pytest.mark.parametrize("mnk", _swept_shapes())
+def test_gemm_swept_shapes_exact_and_inside_their_rows(K, O, mnk):
+    """Integer operands -> bit exact against the oracle, for whatever mix of tiled and general-shape launches the
+    dispatch picks; the output sits between guard rows that must come back untouched (a kernel that wrote past its
+    part of c, e.g. the tiled part into the remainder rows' neighbours, would show here)."""
+    M, N, Kd = mnk
+    a, _ = O.fill_int_e4m3(M * Kd, 909, 0)
+    b, _ = O.fill_int_e4m3(N * Kd, 909, 1)
+    a, b = a.reshape(M, Kd), b.reshape(N, Kd)
+    s = float(np.sqrt(np.float32(4.0 / Kd)))
+    _, biasv = O.fill_int_e4m3(M, 909, 2)
+    bias = O.f32_to_bf16(biasv.astype(np.float32))
+    pad = 8                                              # 8 rows of M bf16 / fp32 values: the interior stays 16-byte aligned
+    for out_f32, use_bias in ((False, False), (False, True), (True, True)):
+        dt = torch.float32 if out_f32 else torch.bfloat16
+        guard = -7.0 if out_f32 else -1.5
+        big = torch.full((N + 2 * pad, M), guard, dtype=dt, device="cuda")
+        c = big[pad:pad + N]
+        assert c.data_ptr() % 16 == 0                  # only the base of c has to be aligned; an odd M gives unaligned rows
+        mm(K, c, dev_u8(a), dev_u8(b), dev_bf16(bias) if use_bias else None, dev_scalar(s), dev_scalar(s), M, N, Kd,
+           workspace=workspace())
+        torch.cuda.synchronize()
+        want = O.gemm_tn(a, b, sa=s, sb=s, bias=bias if use_bias else None, out_f32=out_f32, mt=False)
+        got = c.cpu().numpy() if out_f32 else host_bits(c)
+        assert np.array_equal(got, want), (out_f32, use_bias)
+        assert bool((big[:pad] == guard).all()) and bool((big[pad + N:] == guard).all()), "guard rows were written"
+
+
 @pytest.mark.parametrize("mnk", [(256, 256, 256), (512, 768, 512), (448, 512, 768), (1024, 2048, 1024), (2304, 512, 2816),
                                  (3584, 4096, 512)])
 def test_gemm_second_operand_in_k_major_layout(K, O, mnk):
