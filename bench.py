@@ -23,8 +23,9 @@ One JSON line is printed:
 Extra fields: roofline.mfma_only_ceiling_TFLOPs (register-only matrix-instruction loops: what the chip sustains
 under its power limit), roofline.traffic (hardware-counter bytes per GEMM launch, from profiles/), hip_graph_replay
 (the same step replayed from a HIP graph), fused_quantize_transpose_step (the step with the single-read
-quantize + transposed-copy extension), direct_gradient_layout_step (that step with the gate+up weight gradient
-reading the output gradient in its stored layout, matmul mode TT, instead of a transposed copy), vendor_gemm (torch._scaled_mm, i.e. hipBLASLt, on the six GEMM shapes,
+quantize + transposed-copy extension), direct_gradient_layout_step (the step with the backward matmuls reading
+weights, activations and output gradients in their stored layouts, matmul modes NN / NT / TT, instead of transposed
+copies), vendor_gemm (torch._scaled_mm, i.e. hipBLASLt, on the six GEMM shapes,
 alternating with this library's GEMM: context for the roofline fraction, not part of the path).
 """
 import argparse
@@ -118,8 +119,9 @@ def main():
         timed("abs_max", 2 * n, lambda: K.abs_max(stats[name][0:1], t[name]))
         timed("quantize", 3 * n, lambda: K.quantize_with_abs_max(q[name], stats[name][1:2], t[name], stats[name][0:1]))
 
-    def gemm(c, a, b, sa, sb, M, N, Kd, b_kmajor=False):
-        timed("gemm", 2.0 * M * N * Kd, lambda: K.matmul(c, a, b, None, sa, sb, M, N, Kd, workspace=ws, b_kmajor=b_kmajor))
+    def gemm(c, a, b, sa, sb, M, N, Kd, b_kmajor=False, a_kmajor=False):
+        timed("gemm", 2.0 * M * N * Kd, lambda: K.matmul(c, a, b, None, sa, sb, M, N, Kd, workspace=ws, b_kmajor=b_kmajor,
+                                                         a_kmajor=a_kmajor))
         if record[0] == 1:
             timers["gemm"][-1] += ("M%d_N%d_K%d" % (M, N, Kd),)
 
@@ -183,25 +185,23 @@ def main():
         gemm(out["dw_up"], q["x_t"], q["dy_up_t"], stats["x"][1:2], stats["dy_up"][1:2], C, UP, BT)
 
     def step_direct():
-        """step_fused with the gate+up weight gradient reading the quantized output gradient dY[BT, UP] where it
-        lies (matmul mode TT, K-major second operand): no transposed copy of the step's largest tensor.  The down
-        projection's weight gradient keeps the copy: there the copy (29 M elements) costs less than the mode's
-        slower K loop does on that GEMM."""
-        timed("abs_max", 0, lambda: K.abs_max(stats["w_up"][0:1], t["w_up"]))
-        both("w_up", q["w_up_t"])
-        timed("abs_max", 0, lambda: K.abs_max(stats["w_down"][0:1], t["w_down"]))
-        both("w_down", q["w_down_t"])
+        """The step as backward_qmm issues it with DirectGradLayout: the matmuls read their operands where they lie
+        (matmul modes NN / NT / TT) wherever that is cheaper than a transposed copy.  Weights: no transposed copies (both
+        dgrads in mode NN).  Down projection: the weight gradient reads h and dY in place (mode NT; h is quantized
+        again, as the reference's path without a retained quantized input does, but not transposed).  Gate+up: the weight
+        gradient reads dY[8192, 37888] in place (mode TT) and keeps the quantize+transpose of the small x."""
+        absmax_and_quantize("w_up")
+        absmax_and_quantize("w_down")
         absmax_and_quantize("x")
         gemm(out["y_up"], q["w_up"], q["x"], stats["w_up"][1:2], stats["x"][1:2], UP, BT, C)
         absmax_and_quantize("h")
         gemm(out["y_down"], q["w_down"], q["h"], stats["w_down"][1:2], stats["h"][1:2], C, BT, FFN)
-        timed("abs_max", 0, lambda: K.abs_max(stats["dy_down"][0:1], t["dy_down"]))
-        both("dy_down", q["dy_down_t"])
-        gemm(out["dh"], q["w_down_t"], q["dy_down"], stats["w_down"][1:2], stats["dy_down"][1:2], FFN, BT, C)
-        qtr(q["h_t"], "h")
-        gemm(out["dw_down"], q["h_t"], q["dy_down_t"], stats["h"][1:2], stats["dy_down"][1:2], FFN, C, BT)
+        absmax_and_quantize("dy_down")
+        gemm(out["dh"], q["w_down"], q["dy_down"], stats["w_down"][1:2], stats["dy_down"][1:2], FFN, BT, C, a_kmajor=True)
+        timed("quantize", 3 * t["h"].numel(), lambda: K.quantize_with_abs_max(q["h"], stats["h"][1:2], t["h"], stats["h"][0:1]))
+        gemm(out["dw_down"], q["h"], q["dy_down"], stats["h"][1:2], stats["dy_down"][1:2], FFN, C, BT, a_kmajor=True, b_kmajor=True)
         absmax_and_quantize("dy_up")
-        gemm(out["dx"], q["w_up_t"], q["dy_up"], stats["w_up"][1:2], stats["dy_up"][1:2], C, BT, UP)
+        gemm(out["dx"], q["w_up"], q["dy_up"], stats["w_up"][1:2], stats["dy_up"][1:2], C, BT, UP, a_kmajor=True)
         qtr(q["x_t"], "x")
         gemm(out["dw_up"], q["x_t"], q["dy_up"], stats["x"][1:2], stats["dy_up"][1:2], C, UP, BT, b_kmajor=True)
 
@@ -263,11 +263,13 @@ def main():
             torch.cuda.synchronize()
             return (time.perf_counter() - f0) * 1e3 / args.steps
         step_fused()
-        want_dw = out["dw_up"].clone()
+        want = [out[k].clone() for k in ("dh", "dw_down", "dx", "dw_up")]
         step_direct()
         torch.cuda.synchronize()
-        direct_identical = bool(torch.equal(out["dw_up"], want_dw))
-        del want_dw
+        # bit for bit, except where the materialised route cuts its last round of tiles into K segments (dw_down):
+        # other partial sums, same tolerance
+        direct_identical = {k: bool(torch.equal(out[k], w)) for k, w in zip(("dh", "dw_down", "dx", "dw_up"), want)}
+        del want
         rounds = [(ms_of(step_fused), ms_of(step_direct)) for _ in range(3)]
         fused_ms = sorted(r[0] for r in rounds)[1]
         direct_ms = sorted(r[1] for r in rounds)[1]
@@ -551,9 +553,10 @@ def main():
             "note": "extension: single-read quantize + transposed copy for weights and output gradients"},
         "direct_gradient_layout_step": None if direct_ms is None else {
             "ms_per_step": direct_ms, "value": gemm_flop / (direct_ms * 1e-3) / 1e12,
-            "dw_identical_to_materialised_route": direct_identical,
-            "note": "extension: fused_quantize_transpose_step without the transposed copy of dY[8192, 37888]; the "
-                    "gate+up weight gradient reads dY in its stored layout (matmul mode TT)"},
+            "gradients_identical_to_materialised_route": direct_identical,
+            "note": "extension: the backward matmuls read their operands in their stored layouts (modes NN for both dgrads, "
+                    "NT for the down weight gradient, TT for the gate+up weight gradient): no transposed copies of the "
+                    "weights, of h or of the output gradients"},
         "vendor_gemm": vendor,
         "secondary_gemm_shapes": secondary,
         "producers": swiglu,

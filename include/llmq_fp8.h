@@ -137,11 +137,14 @@ int llmq_gemm_tn_e4m3_bf16(uint16_t* c, const uint8_t* a, const uint8_t* b, cons
  * TT = 0, TN = 1, NT = 2, NN = 3; in its column-major reading, src/kernels/matmul.cpp:66-67).  With row-major storage:
  *   TN  a[M, K], b[N, K]            (both K contiguous: llmq_gemm_tn_e4m3_bf16 / llmq_gemm_tn_e4m3_e5m2_bf16)
  *   TT  a[M, K], b[K, N]            (b K-major: the output gradient dY[BT, OC] in its stored layout as the second
- *                                    operand of the weight gradient, so that no transposed copy of it is needed)
- * The reference's FP8 path takes TN only (it materialises the transposes, src/models/llama_model.cpp:309-339) and
- * modes NT / NN (a stored [K, M]) are not provided here either.  TT: N and K multiples of 256, M a multiple of 256
- * (without accumulation also of 224), K * N below 2 GiB; other shapes return LLMQ_ERR_INVALID_ARGUMENT and the caller
- * takes the transposing route.  b_format: 0 = e4m3, 1 = e5m2.  Results are bit-identical to mode TN on the transposed copy.
+ *                                    operand of the weight gradient)
+ *   NN  a[K, M], b[N, K]            (a K-major: the weight W[OC, C] in its stored layout as the first operand of the dgrad)
+ *   NT  a[K, M], b[K, N]            (both K-major: activation X[BT, C] and gradient dY[BT, OC] of the weight gradient)
+ * so that the transposed copies the reference's FP8 path materialises (src/models/llama_model.cpp:309-339; its own
+ * kernels take TN only) are not needed.  The K-major modes serve M, N and K multiples of 256 (TT without
+ * accumulation also M a multiple of 224) and K-major operands below 2 GiB; NN and NT do not accumulate into c.  Other
+ * shapes return LLMQ_ERR_INVALID_ARGUMENT before anything is launched and the caller takes the transposing route.
+ * b_format: 0 = e4m3, 1 = e5m2.  Results are bit-identical to mode TN on the transposed copies.
  */
 #define LLMQ_MODE_TT 0
 #define LLMQ_MODE_TN 1

@@ -137,11 +137,15 @@ inline void require_tn(EMMTranspose mode) {
     if (mode != EMMTranspose::TN)
         throw std::invalid_argument("matmul: FP8 operands are only supported in TN layout (both K-contiguous)");
 }
-// bf16 output: TN, and TT (b stored [K, N]; restricted shapes, see llmq_gemm_e4m3_bf16_mode)
+// bf16 output: TN, and the K-major modes TT / NN / NT (restricted shapes, see llmq_gemm_e4m3_bf16_mode)
 inline int mode_code(EMMTranspose mode) {
-    if (mode == EMMTranspose::TN) return LLMQ_MODE_TN;
-    if (mode == EMMTranspose::TT) return LLMQ_MODE_TT;
-    throw std::invalid_argument("matmul: FP8 operands are supported in modes TN and TT only");
+    switch (mode) {
+        case EMMTranspose::TN: return LLMQ_MODE_TN;
+        case EMMTranspose::TT: return LLMQ_MODE_TT;
+        case EMMTranspose::NT: return LLMQ_MODE_NT;
+        case EMMTranspose::NN: return LLMQ_MODE_NN;
+    }
+    throw std::invalid_argument("matmul: unknown operand mode");
 }
 template <class... T> [[noreturn]] void unsupported(const char* func, const T&... t) {
     std::string msg = std::string(func) + ": unsupported dtypes. Got [";
@@ -249,10 +253,11 @@ inline void quantize_with_abs_max_and_transpose(Tensor& out, Tensor& out_tp, flo
 
 // ---- matmul (reference: src/kernels/kernels.h:72-78, 88-90, 96-98) --------------------------------------
 // Row-major a[M,K], b[N,K] -> row-major c[N,M] = (b . a^T) * (*scale_a * *scale_b) (+ bias[M]) (+ c).
-// Mode TN: any M, N >= 1 and K a multiple of 16 (16-byte aligned fp8 rows).  bf16 output also takes mode TT (b stored
-// [K, N]: e.g. the output gradient dY[B*T, OC] of the weight gradient without its transposed copy) when N and K are
-// multiples of 256 and M of 256 (without accumulation also of 224).  Anything else throws std::invalid_argument
-// before a kernel is launched.
+// Mode TN: any M, N >= 1 and K a multiple of 16 (16-byte aligned fp8 rows).  bf16 output also takes the K-major modes:
+// TT (b stored [K, N]: e.g. the output gradient dY[B*T, OC] of the weight gradient without its transposed copy), NN
+// (a stored [K, M]: the weight W[OC, C] of the dgrad) and NT (both), when M, N and K are multiples of 256 (mode TT
+// without accumulation also M of 224); NN and NT do not accumulate into c.  Anything else throws
+// std::invalid_argument before a kernel is launched.
 inline void matmul(__hip_bfloat16* c, const __hip_fp8_e4m3* a, const __hip_fp8_e4m3* b, const __hip_bfloat16* bias,
                    const float* scale_a, const float* scale_b, llmqBlasHandle_t, std::byte* workspace,
                    std::size_t workspace_size, int M, int N, int K, EMMTranspose mode, bool accumulate,

@@ -8,6 +8,13 @@
 
 #include "llmq_kernels.hpp"
 
+// What backward_qmm does about the transposed copies of its matmul operands (QmmRunState::DirectGradLayout).
+enum class EQmmWgrad { Copies, GradInPlace, BothInPlace };   // reference sequence; mode TT; mode NT
+struct QmmDirectPlan {
+    bool DgradInPlace = false;   // dgrad reads weight[OC, C] as the K-major first operand (mode NN): no weight_tp
+    EQmmWgrad Wgrad = EQmmWgrad::Copies;
+};
+
 // LIFO bump allocator over one device arena: temp_alloc / temp_free are host pointer arithmetic only,
 // so the sequence stays legal under stream capture.  Blocks are rounded up to 4096 bytes.
 struct QmmRunState {
@@ -24,17 +31,31 @@ struct QmmRunState {
     // Extension: quantize the output gradient and produce its transpose from one read of dout.Value (saves one
     // read and one launch per layer; the transposed gradient then lives on the stack during the dgrad as well).
     bool FuseGradTranspose = false;
-    // Extension: the weight-gradient matmul reads the quantized output gradient in its stored layout [B*T, OC]
-    // (matmul mode TT) instead of a transposed copy, wherever direct_grad_layout_applies() says the shape allows
-    // it and the copy costs more than the mode's slower K loop; elsewhere backward_qmm behaves as without the flag.
+    // Extension: backward_qmm hands the matmuls their operands where they lie (matmul modes NN / TT / NT) instead of
+    // transposed copies, wherever direct_layout_plan() finds the shapes served and the copy dearer than the mode's
+    // slower K loop; elsewhere it behaves as without the flag.
     bool DirectGradLayout = false;
-    // Mode TT serves whole 256-wide tiles and bf16 output.  Measured on Qwen2.5-7B shapes at 8192 tokens: the K-major
-    // operand slows the matmul by 4-6 %, the transposed copy costs 2 * B*T * OC bytes of HBM traffic; the copy is
-    // the larger cost while C, the matmul's row count, stays below about 10^4.
-    static bool direct_grad_layout_applies(int B, int T, int C, int OC, ETensorDType dweight_dtype, bool accumulate) {
-        const long BT = (long)B * T;
-        return dweight_dtype == ETensorDType::BF16 && OC % 256 == 0 && BT % 256 == 0 && BT * OC < (1L << 31) &&
-               (C % 256 == 0 || (C % 224 == 0 && !accumulate)) && C <= 8192;
+    using EWgrad = EQmmWgrad;
+    using DirectPlan = QmmDirectPlan;
+    // The K-major modes serve whole 256-wide tiles, bf16 output and operands below 2 GiB; modes NN / NT do not
+    // accumulate.  Measured on the Qwen2.5-7B MLP at 8192 tokens (one box, alternating): mode NN costs 2-3 % of the
+    // matmul and saves the weight's transposed copy (dgrad 439 -> 423 us and 788 -> 764 us); a K-major second operand
+    // costs 6 %, both operands K-major 9-11 %, against transposed copies of 2 bytes per element: reading the gradient
+    // in place pays while the matmul's row count C stays below about 10^4, reading the activation in place as well
+    // while OC does.
+    static DirectPlan direct_layout_plan(int B, int T, int C, int OC, ETensorDType dinp_dtype, ETensorDType dweight_dtype,
+                                         bool accumulate) {
+        const long BT = (long)B * T, lim = 1L << 31;
+        const bool tiles = C % 256 == 0 && OC % 256 == 0 && BT % 256 == 0;
+        DirectPlan p;
+        // mode NN: 2-3 % of a matmul of 2 * BT * C * OC flop against a copy of 2 * C * OC bytes: the copy is the larger
+        // cost up to about 2 * 10^4 tokens
+        p.DgradInPlace = tiles && dinp_dtype == ETensorDType::BF16 && (long)C * OC < lim && BT <= 16384;
+        if (dweight_dtype == ETensorDType::BF16 && OC % 256 == 0 && BT % 256 == 0 && BT * OC < lim) {
+            if (tiles && !accumulate && BT * C < lim && OC <= 8192) p.Wgrad = EWgrad::BothInPlace;
+            else if ((C % 256 == 0 || (C % 224 == 0 && !accumulate)) && C <= 8192) p.Wgrad = EWgrad::GradInPlace;
+        }
+        return p;
     }
     std::vector<std::byte*> Live;
 
@@ -56,10 +77,12 @@ struct QmmRunState {
     }
     // Bytes of stack backward_qmm needs for one layer (the dry run of llama_run_state.cpp:362-390).
     static std::size_t backward_temp_bytes(int B, int T, int C, int OC, bool fuse_grad_transpose = false,
-                                           bool direct_grad = false) {
+                                           DirectPlan plan = DirectPlan{}) {
         auto up = [](std::size_t b) { return (b + 4095) / 4096 * 4096; };
-        const std::size_t wt = up((std::size_t)C * OC), at = up((std::size_t)C * B * T), gt = up((std::size_t)OC * B * T);
-        if (direct_grad) return wt > at ? wt : at;
+        const bool copies = plan.Wgrad == EWgrad::Copies;
+        const std::size_t wt = plan.DgradInPlace ? 0 : up((std::size_t)C * OC);
+        const std::size_t at = plan.Wgrad == EWgrad::BothInPlace ? 0 : up((std::size_t)C * B * T);
+        const std::size_t gt = copies ? up((std::size_t)OC * B * T) : 0;
         if (fuse_grad_transpose) return gt + (wt > at ? wt : at);
         return wt > at + gt ? wt : at + gt;
     }
@@ -86,10 +109,12 @@ inline void backward_qmm(Tensor& dinp, Tensor& dweight, Tensor dbias, Quantizabl
                          int C, int OC, bool reuse_inp, hipStream_t stream) {
     if (weight.DType != ETensorDType::FP8_E4M3)
         throw std::invalid_argument("backward_qmm: this build implements the FP8 (e4m3 weight) branch only");
-    const bool direct_grad = rs.DirectGradLayout &&
-                             QmmRunState::direct_grad_layout_applies(B, T, C, OC, dweight.DType, accumulate_gradient);
+    const QmmRunState::DirectPlan plan =
+        rs.DirectGradLayout ? QmmRunState::direct_layout_plan(B, T, C, OC, dinp.DType, dweight.DType, accumulate_gradient)
+                            : QmmRunState::DirectPlan{};
+    const bool copies = plan.Wgrad == QmmRunState::EWgrad::Copies;
     Tensor grad_tp{};
-    if (rs.FuseGradTranspose && !direct_grad) {
+    if (rs.FuseGradTranspose && copies) {
         grad_tp = rs.temp_alloc(dout.Quant.DType, {OC, (long)B * T});
         quantize_with_abs_max_and_transpose(dout.Quant, grad_tp, dout.Quant.scale(), dout.Value, dout.Quant.abs_max(),
                                             B * T, OC, rs.DeviceProp, stream);
@@ -99,15 +124,31 @@ inline void backward_qmm(Tensor& dinp, Tensor& dweight, Tensor dbias, Quantizabl
     }
 
     auto& inp_q = inp.Quant;
-    Tensor weight_tp = rs.temp_alloc(inp_q.DType, {C, OC});
-    transpose(weight_tp, weight, OC, C, stream);
     Tensor no_bias{};
-    matmul(dinp, weight_tp, dout.Quant, no_bias, weight.scale(), dout.Quant.scale(), rs.BlasHandle, rs.Workspace, C,
-           B * T, OC, EMMTranspose::TN, false, stream, rs.MatmulBackend);
-    rs.temp_free(weight_tp);
+    if (plan.DgradInPlace) {
+        // weight[OC, C] in its stored layout is the K-major first operand (mode NN): no transposed copy
+        matmul(dinp, weight, dout.Quant, no_bias, weight.scale(), dout.Quant.scale(), rs.BlasHandle, rs.Workspace, C, B * T,
+               OC, EMMTranspose::NN, false, stream, rs.MatmulBackend);
+    } else {
+        Tensor weight_tp = rs.temp_alloc(inp_q.DType, {C, OC});
+        transpose(weight_tp, weight, OC, C, stream);
+        matmul(dinp, weight_tp, dout.Quant, no_bias, weight.scale(), dout.Quant.scale(), rs.BlasHandle, rs.Workspace, C,
+               B * T, OC, EMMTranspose::TN, false, stream, rs.MatmulBackend);
+        rs.temp_free(weight_tp);
+    }
 
+    if (plan.Wgrad == QmmRunState::EWgrad::BothInPlace) {
+        // activation [B*T, C] and gradient [B*T, OC] in their stored layouts are the two K-major operands (mode NT)
+        if (!reuse_inp)
+            quantize_with_abs_max(inp_q, inp_q.scale(), inp.Value, inp_q.abs_max(), (long)B * T * C, rs.DeviceProp, stream);
+        matmul(dweight, inp_q, dout.Quant, no_bias, inp_q.scale(), dout.Quant.scale(), rs.BlasHandle, rs.Workspace, C, OC,
+               B * T, EMMTranspose::NT, false, stream, rs.MatmulBackend);
+        if (!dbias.empty())
+            backward_bias(dbias, dout.Quant, inp_q.scale(), dout.Quant.scale(), bias_buffer, B, T, OC, rs.DeviceProp, stream);
+        return;
+    }
     Tensor activation_tp = rs.temp_alloc(inp_q.DType, {C, (long)B * T});
-    if (!rs.FuseGradTranspose && !direct_grad) grad_tp = rs.temp_alloc(dout.Quant.DType, {OC, (long)B * T});
+    if (!rs.FuseGradTranspose && copies) grad_tp = rs.temp_alloc(dout.Quant.DType, {OC, (long)B * T});
     if (reuse_inp) {
         transpose(activation_tp, inp_q, B * T, C, stream);
     } else {
@@ -115,8 +156,8 @@ inline void backward_qmm(Tensor& dinp, Tensor& dweight, Tensor dbias, Quantizabl
         quantize_and_transpose_with_abs_max(activation_tp, activation_tp.scale(), inp.Value, inp.Quant.abs_max(),
                                             B * T, C, rs.DeviceProp, stream);
     }
-    if (direct_grad) {
-        // the quantized gradient in its stored layout [B*T, OC] is the K-major second operand (mode TT): no transposed copy
+    if (!copies) {
+        // the quantized gradient in its stored layout [B*T, OC] is the K-major second operand (mode TT)
         matmul(dweight, activation_tp, dout.Quant, no_bias, inp_q.scale(), dout.Quant.scale(), rs.BlasHandle, rs.Workspace, C,
                OC, B * T, EMMTranspose::TT, accumulate_gradient, stream, rs.MatmulBackend);
     } else {
@@ -127,7 +168,7 @@ inline void backward_qmm(Tensor& dinp, Tensor& dweight, Tensor dbias, Quantizabl
     if (!dbias.empty()) {
         backward_bias(dbias, dout.Quant, inp_q.scale(), dout.Quant.scale(), bias_buffer, B, T, OC, rs.DeviceProp, stream);
     }
-    if (direct_grad) {
+    if (!copies) {
         rs.temp_free(activation_tp);
     } else if (rs.FuseGradTranspose) {
         rs.temp_free(activation_tp);

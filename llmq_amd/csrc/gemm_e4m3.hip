@@ -598,10 +598,21 @@ __device__ __forceinline__ int frag_swizzle(int row) {
 // the 8 bytes of column i, i.e. 8 consecutive k of one n; four of them fill a fragment (32 k per lane, in the
 // same k order as the other operand's two 16-byte reads).  The swizzle spreads the 8 rows of one read, and the
 // two lane groups that share an LDS pass, over all banks.
-template <typename OutT, int B_FMT, bool SEG, int NJ = 8, bool STREAM_OUT = true, bool ODDK = false, bool KMB = false>
+//
+// KMA: the a operand is stored K-major, row-major [K, M] (modes NN and NT: the weight W[OC, C] as the first operand of
+// the dgrad, the activation X[BT, C] as that of the wgrad, without their transposed copies).  Copies and fragment reads
+// are those of KMB with the operands' roles exchanged.  What does not carry over is the row permutation that gives
+// a lane 8 adjacent columns of c (it is made by the copy addressing of a K-contiguous a; a transposing read hands 16
+// adjacent columns to 16 adjacent lanes): a lane then owns columns 16 j + l16, and the epilogue goes through LDS --
+// scale, bias and the rounding to bf16 where the accumulators are, 16 rows x 128 columns of bf16 per wave and
+// fragment row into a private 4 KiB piece of LDS, read back as 16 bytes per lane and row.  bf16 output without
+// accumulation (the old values of c would have to be fetched in the scattered layout).
+template <typename OutT, int B_FMT, bool SEG, int NJ = 8, bool STREAM_OUT = true, bool ODDK = false, bool KMB = false,
+          bool KMA = false>
 __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     static_assert(!(SEG && ODDK), "K segments are whole pairs of K-steps");
-    static_assert(!(KMB && (SEG || ODDK)), "the K-major operand mode is built for whole tiles and even K-step counts");
+    static_assert(!((KMB || KMA) && (SEG || ODDK)), "the K-major operand modes are built for whole tiles and even K-step counts");
+    static_assert(!KMA || (NJ == 8 && std::is_same_v<OutT, uint16_t>), "the K-major first operand is built for 256-wide tiles and bf16 output");
     constexpr int BLK = 256, T = 256, WT = 128, NF = 8;
     constexpr int WTM = 16 * NJ, BLKM = 2 * WTM;  // columns (first-operand rows) per wave and per tile
     constexpr int P_BYTES = BLK * kBK, STAGE = 2 * P_BYTES;
@@ -610,7 +621,8 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     static_assert(NJ == 8 || ((NJ == 7 || NJ == 6) && !SEG && std::is_same_v<OutT, uint16_t>), "unsupported tile width");
     typedef float v4f __attribute__((ext_vector_type(4)));
 
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * STAGE];
+    constexpr int EPI_STAGE = 16 * WTM * 2;  // KMA: one fragment row of a wave's outputs as bf16
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * STAGE + (KMA ? 4 * EPI_STAGE : 0)];
 
     const int tid = threadIdx.x;
     const int lane = tid % 64;
@@ -681,7 +693,10 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         const int l = ld_row % 16;
         return ld_row < 16 ? frag_step(2 * it) * l : frag_row(2 * it + 1) - frag_row(2 * it) + frag_step(2 * it + 1) * l;
     };
-    const uint32_t q_lane = (uint32_t)slab_lane_rows(0) * (uint32_t)g.K + (uint32_t)ld_chunk * 16u;
+    const uint32_t q_lane = KMA ? (uint32_t)kb_row * (uint32_t)g.M + (uint32_t)kb_chunk * 16u
+                                : (uint32_t)slab_lane_rows(0) * (uint32_t)g.K + (uint32_t)ld_chunk * 16u;
+    const uint32_t q_lane_hi = (uint32_t)kb_row * (uint32_t)g.M + (uint32_t)(kb_chunk ^ 8) * 16u;  // KMA, slabs 2, 3, 6, 7
+    const uint32_t q_step = KMA ? (uint32_t)kBK * (uint32_t)g.M : (uint32_t)kBK;
     const uint32_t q_lane_3 = (uint32_t)slab_lane_rows(NJ == 7 ? 3 : 0) * (uint32_t)g.K + (uint32_t)ld_chunk * 16u;
     const uint32_t q_lane_6 = (uint32_t)slab_lane_rows(NJ == 7 ? 6 : 0) * (uint32_t)g.K + (uint32_t)ld_chunk * 16u;
     // The copy stream runs two K-steps ahead of the matrix instructions and has its own position: tile number
@@ -693,11 +708,12 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     const uint8_t* p_base[ITERS];
     const uint8_t* q_base[ITERS_Q];
     uint32_t vp = p_lane, vp_hi = p_lane_hi, vq = q_lane, vq3 = q_lane_3, vq6 = q_lane_6;
+    [[maybe_unused]] uint32_t vq_hi = q_lane_hi;
     auto tile_bases = [&](int logical) {
         int nb, mb;
         decode(logical, nb, mb);
         const uint8_t* pb = KMB ? g.b + (int64_t)k_first * g.N + nb : g.b + (int64_t)nb * g.K + k_first;
-        const uint8_t* qb = g.a + (int64_t)mb * g.K + k_first;
+        const uint8_t* qb = KMA ? g.a + (int64_t)k_first * g.M + mb : g.a + (int64_t)mb * g.K + k_first;
         // pinned in scalar registers here, once per tile (otherwise the compiler sinks the additions to the
         // copies and repeats them in every K-step)
 #pragma unroll
@@ -707,7 +723,7 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         }
 #pragma unroll
         for (int it = 0; it < ITERS_Q; ++it) {
-            q_base[it] = qb + (int64_t)frag_row(2 * it) * g.K;
+            q_base[it] = KMA ? qb + (int64_t)(16 * it) * g.M : qb + (int64_t)frag_row(2 * it) * g.K;
             asm volatile("" : "+s"(q_base[it]));
         }
     };
@@ -718,7 +734,8 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         copy_k0 += kBK;
         vp += p_step;
         if constexpr (KMB) vp_hi += p_step;
-        vq += kBK;
+        vq += q_step;
+        if constexpr (KMA) vq_hi += q_step;
         if constexpr (NJ == 7) {
             vq3 += kBK;
             vq6 += kBK;
@@ -727,7 +744,12 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
             copy_k0 = 0;
             vp = p_lane;
             if constexpr (KMB) vp_hi = p_lane_hi;
-            vq -= (uint32_t)k_total;
+            if constexpr (KMA) {
+                vq = q_lane;
+                vq_hi = q_lane_hi;
+            } else {
+                vq -= (uint32_t)k_total;
+            }
             if constexpr (NJ == 7) {
                 vq3 -= (uint32_t)k_total;
                 vq6 -= (uint32_t)k_total;
@@ -765,7 +787,7 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         } else {
             const int it = c - ITERS;  // slab `it` covers LDS rows 32 it .. 32 it + 31: fragments 2 it and 2 it + 1
             src = q_base[it];
-            lane_ofs = (NJ == 7 && it == 3) ? vq3 : (NJ == 7 && it == 6) ? vq6 : vq;
+            lane_ofs = KMA ? (((it >> 1) & 1) ? vq_hi : vq) : (NJ == 7 && it == 3) ? vq3 : (NJ == 7 && it == 6) ? vq6 : vq;
         }
     };
     auto issue_copy = [&](int c, uint32_t tok) {
@@ -812,6 +834,24 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
             return read_frag(stage + p_frag + i * 16 * kBK);
         }
     };
+    // a fragment j (columns 16 j .. 16 j + 15 of the wave's 128 columns of c) from the stage at `stage`: the same two
+    // ways, with the wave's column half wm in the place of its row half wn
+    const uint32_t ka_base = (uint32_t)((32 * kg + l16 / 2) * 256 + (l16 & 1) * 8) + (uint32_t)(((8 * wm) ^ ((kg & 1) << 3)) * 16) +
+                             (uint32_t)((l16 / 2) * 16);
+    typedef __attribute__((address_space(3))) v2i_lds* lds_v2i_a;
+    auto read_frag_a = [&](const uint8_t* stage, int j) -> v8i {
+        if constexpr (KMA) {
+            const uint8_t* p = stage + P_BYTES + (opaque((int)ka_base) ^ (16 * j));
+            const v2i_lds r0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_a)(p));
+            const v2i_lds r1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_a)(p + 2048));
+            const v2i_lds r2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_a)(p + 4096));
+            const v2i_lds r3 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_a)(p + 6144));
+            const v8i f = {r0[0], r0[1], r1[0], r1[1], r2[0], r2[1], r3[0], r3[1]};
+            return f;
+        } else {
+            return read_frag(stage + q_frag + j * 16 * kBK);
+        }
+    };
 
     // The matrix instruction as an asm statement with the accumulator tied in place in the accumulation
     // registers: with all 256 of them holding the wave tile there is no spare for the register allocator's
@@ -846,7 +886,7 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) fa[i] = read_frag_b(lds, i);
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) fb[0][j] = read_frag(lds + q_frag + j * 16 * kBK);
+    for (int j = 0; j < NJ; ++j) fb[0][j] = read_frag_a(lds, j);
 
     // One K-step of parity PAR (LDS stage PAR, fb half PAR): rows i = 0..7 of first-operand fragments
     // against all 8 second-operand fragments.  fa rotates through 4 slots (fragment i+4 is read once row i
@@ -908,7 +948,7 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
                 if constexpr (COPY_HERE) issue_copy(COPY_C, tok);
                 if constexpr (i >= 5 && (j == 2 || j == 5)) {  // rows 5..7: fragments 2..7 of the next step
                     constexpr int f = 2 * (i - 4) + (j == 5 ? 1 : 0);
-                    if constexpr (f < NJ) fb[1 - FP][f] = read_frag(nxt + q_frag + f * 16 * kBK);
+                    if constexpr (f < NJ) fb[1 - FP][f] = read_frag_a(nxt, f);
                 }
             });
             if constexpr (i == 4) {
@@ -931,22 +971,49 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
                 __syncthreads();
                 // copies 0..3, each with one of the four LDS reads of the next step's first two second-operand
                 // fragments between the write of M0 and the copy
-                const uint8_t* r0 = nxt + q_frag;
-                const uint8_t* r1 = nxt + q_frag + 16 * kBK;
-                uint32_t tok = set_m0(std::integral_constant<int, 0>{}, refill);
-                const v4i lo0 = *reinterpret_cast<const v4i*>(r0 + c0);
-                issue_copy(0, tok);
-                tok = set_m0(std::integral_constant<int, 1>{}, refill);
-                const v4i hi0 = *reinterpret_cast<const v4i*>(r0 + c1);
-                issue_copy(1, tok);
-                tok = set_m0(std::integral_constant<int, 2>{}, refill);
-                const v4i lo1 = *reinterpret_cast<const v4i*>(r1 + c0);
-                issue_copy(2, tok);
-                tok = set_m0(std::integral_constant<int, 3>{}, refill);
-                const v4i hi1 = *reinterpret_cast<const v4i*>(r1 + c1);
-                issue_copy(3, tok);
-                fb[1 - FP][0] = __builtin_shufflevector(lo0, hi0, 0, 1, 2, 3, 4, 5, 6, 7);
-                fb[1 - FP][1] = __builtin_shufflevector(lo1, hi1, 0, 1, 2, 3, 4, 5, 6, 7);
+                if constexpr (KMA) {
+                    // the eight transposing reads of the next step's first two a fragments, two between each write of M0
+                    // and its copy
+                    const uint8_t* pa0 = nxt + P_BYTES + opaque((int)ka_base);
+                    const uint8_t* pa1 = nxt + P_BYTES + (opaque((int)ka_base) ^ 16);
+                    uint32_t tok = set_m0(std::integral_constant<int, 0>{}, refill);
+                    const v2i_lds a00 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_a)(pa0));
+                    const v2i_lds a01 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_a)(pa0 + 2048));
+                    issue_copy(0, tok);
+                    tok = set_m0(std::integral_constant<int, 1>{}, refill);
+                    const v2i_lds a02 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_a)(pa0 + 4096));
+                    const v2i_lds a03 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_a)(pa0 + 6144));
+                    issue_copy(1, tok);
+                    tok = set_m0(std::integral_constant<int, 2>{}, refill);
+                    const v2i_lds a10 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_a)(pa1));
+                    const v2i_lds a11 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_a)(pa1 + 2048));
+                    issue_copy(2, tok);
+                    tok = set_m0(std::integral_constant<int, 3>{}, refill);
+                    const v2i_lds a12 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_a)(pa1 + 4096));
+                    const v2i_lds a13 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_a)(pa1 + 6144));
+                    issue_copy(3, tok);
+                    const v8i f0 = {a00[0], a00[1], a01[0], a01[1], a02[0], a02[1], a03[0], a03[1]};
+                    const v8i f1 = {a10[0], a10[1], a11[0], a11[1], a12[0], a12[1], a13[0], a13[1]};
+                    fb[1 - FP][0] = f0;
+                    fb[1 - FP][1] = f1;
+                } else {
+                    const uint8_t* r0 = nxt + q_frag;
+                    const uint8_t* r1 = nxt + q_frag + 16 * kBK;
+                    uint32_t tok = set_m0(std::integral_constant<int, 0>{}, refill);
+                    const v4i lo0 = *reinterpret_cast<const v4i*>(r0 + c0);
+                    issue_copy(0, tok);
+                    tok = set_m0(std::integral_constant<int, 1>{}, refill);
+                    const v4i hi0 = *reinterpret_cast<const v4i*>(r0 + c1);
+                    issue_copy(1, tok);
+                    tok = set_m0(std::integral_constant<int, 2>{}, refill);
+                    const v4i lo1 = *reinterpret_cast<const v4i*>(r1 + c0);
+                    issue_copy(2, tok);
+                    tok = set_m0(std::integral_constant<int, 3>{}, refill);
+                    const v4i hi1 = *reinterpret_cast<const v4i*>(r1 + c1);
+                    issue_copy(3, tok);
+                    fb[1 - FP][0] = __builtin_shufflevector(lo0, hi0, 0, 1, 2, 3, 4, 5, 6, 7);
+                    fb[1 - FP][1] = __builtin_shufflevector(lo1, hi1, 0, 1, 2, 3, 4, 5, 6, 7);
+                }
             }
             if constexpr (i < 4) fa[i % 4] = read_frag_b(cur, i + 4);
             else fa[i % 4] = read_frag_b(nxt, i - 4);
@@ -1022,7 +1089,48 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
             constexpr bool BIAS = decltype(bias_tag)::value;
             constexpr bool ACC = decltype(acc_tag)::value;
             typedef float v4fl __attribute__((ext_vector_type(4)));
-            if constexpr (NJ < 8) {
+            if constexpr (KMA) {
+                // acc[i][j][r] is c row 16 i + 4 ekg + r, column 16 j + el16 of the wave tile.  Per fragment row i the
+                // wave writes its 16 x 128 outputs as bf16 into its own piece of LDS ([16 rows][256 bytes], the 32-byte
+                // pieces of a row xor-ed with the row quad so that the four row quads of a write land on different
+                // banks) and reads them back as 16 bytes per lane: row 4 q + lane / 16, columns 8 (lane % 16) ..+7.
+                // One wave's LDS operations are carried out in order, so no barrier is needed around the exchange.
+                uint8_t* es = lds + 2 * STAGE + wave * EPI_STAGE;
+                float bias_c[NJ];
+                if constexpr (BIAS) {
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j) bias_c[j] = load_bias(g.bias, g.bias_is_bf16, m_blk + wm * WTM + 16 * j + el16);
+                }
+                const uint32_t wr_ofs = (uint32_t)(4 * ekg) * 256u + ((uint32_t)(el16 * 2) ^ (uint32_t)(ekg * 32));
+                const uint32_t rd_ofs = (uint32_t)(e_lane / 16) * 256u + (uint32_t)(e_lane % 16) * 16u;
+                const uint32_t out_bytes = ((uint32_t)(e_lane / 16) * (uint32_t)ldc + (uint32_t)(m_blk + wm * WTM + 8 * (e_lane % 16))) * 2u;
+#pragma unroll
+                for (int i = 0; i < NF; ++i) {
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j) {
+#pragma unroll
+                        for (int r = 0; r < 4; r += 2) {
+                            float v0 = acc[i][j][r] * scale, v1 = acc[i][j][r + 1] * scale;
+                            if constexpr (BIAS) {
+                                v0 = v0 + bias_c[j];
+                                v1 = v1 + bias_c[j];
+                            }
+                            const f32x2_t pr = {v0, v1};
+                            const uint32_t pk = __builtin_bit_cast(uint32_t, __builtin_convertvector(pr, bf16x2_t));
+                            uint8_t* w = es + (wr_ofs ^ (uint32_t)(32 * j)) + r * 256;   // column 16 j: byte 32 j of the row
+                            *reinterpret_cast<uint16_t*>(w) = (uint16_t)pk;
+                            *reinterpret_cast<uint16_t*>(w + 256) = (uint16_t)(pk >> 16);
+                        }
+                    }
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const v4i packed = *reinterpret_cast<const v4i*>(es + q * 1024 + (rd_ofs ^ (uint32_t)(32 * q)));
+                        LLMQ_GLOBAL char* row_ptr = scalar_ptr((LLMQ_GLOBAL char*)(c + (int64_t)(row0 + 16 * i + 4 * q) * ldc));
+                        if constexpr (STREAM_OUT) __builtin_nontemporal_store(packed, (LLMQ_GLOBAL v4i*)(row_ptr + out_bytes));
+                        else *(LLMQ_GLOBAL v4i*)(row_ptr + out_bytes) = packed;
+                    }
+                }
+            } else if constexpr (NJ < 8) {
                 static_assert(NJ == 8 || !ACC, "the narrow tiles do not accumulate");
                 float bias_n[NJ];
                 if constexpr (BIAS) {
@@ -1123,7 +1231,7 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         constexpr std::false_type no{};
         if constexpr (SEG) {
             rows(no, no);
-        } else if constexpr (NJ != 8) {
+        } else if constexpr (NJ != 8 || KMA) {
             if (g.bias) rows(yes, no);
             else rows(no, no);
             pending_stores = true;
@@ -1591,9 +1699,12 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
     return launch_pipe<128, 128, 2, 2, OutT, B_FMT>(g, splits, 0, stream);
 }
 
-// b stored K-major, [K, N] row-major (the reference's mode TT): the four-wave kernel's KMB instances, whole tiles only.
-template <int B_FMT>
-static int gemm_dispatch_b_kmajor(GemmArgs g, hipStream_t stream) {
+// Operands stored K-major (the reference's modes TT: b [K, N]; NN: a [K, M]; NT: both): the four-wave kernel's KMB / KMA
+// instances, whole tiles only.
+template <int B_FMT, bool KMA, bool KMB>
+static int gemm_dispatch_kmajor(GemmArgs g, hipStream_t stream) {
+    static_assert(KMA || KMB, "mode TN goes through gemm_dispatch");
+    const char* mode = KMA ? (KMB ? "NT" : "NN") : "TT";
     LLMQ_REQUIRE(g.M > 0 && g.N > 0 && g.K > 0, "matmul: M, N, K must be positive (got %d, %d, %d)", g.M, g.N, g.K);
     const int cus = cu_count(), xcds = xcd_count();
     g.xcds = xcds;
@@ -1601,26 +1712,34 @@ static int gemm_dispatch_b_kmajor(GemmArgs g, hipStream_t stream) {
     LLMQ_REQUIRE(g.a && g.b && g.c, "matmul: null operand pointer");
     LLMQ_REQUIRE(aligned16(g.a) && aligned16(g.b) && aligned16(g.c) && aligned16(g.bias),
                  "matmul: all pointers must be 16-byte aligned");
-    const bool m224 = g.M % 256 != 0 && g.M % 224 == 0 && !g.accumulate;
+    const bool m224 = !KMA && g.M % 256 != 0 && g.M % 224 == 0 && !g.accumulate;
     LLMQ_REQUIRE(g.N % 256 == 0 && g.K % 256 == 0 && (g.M % 256 == 0 || m224) && cus % xcds == 0,
-                 "matmul: the K-major second operand (mode TT) needs N %% 256 == 0, K %% 256 == 0 and M %% 256 == 0 (without "
-                 "accumulation also M %% 224 == 0); got M, N, K = %d, %d, %d", g.M, g.N, g.K);
-    // the copies of the K-major operand address it as "tile base + 32-bit lane offset", and that offset walks the
-    // whole K extent of the operand (K * N bytes)
-    LLMQ_REQUIRE((int64_t)g.K * g.N < ((int64_t)1 << 31), "matmul: the K-major second operand must be smaller than 2 GiB "
+                 "matmul: a K-major operand (mode %s) needs N %% 256 == 0, K %% 256 == 0 and M %% 256 == 0 (mode TT without "
+                 "accumulation also M %% 224 == 0); got M, N, K = %d, %d, %d", mode, g.M, g.N, g.K);
+    LLMQ_REQUIRE(!KMA || !g.accumulate, "matmul: mode %s (first operand K-major) does not accumulate into c", mode);
+    // the copies of a K-major operand address it as "tile base + 32-bit lane offset", and that offset walks the
+    // whole K extent of the operand
+    LLMQ_REQUIRE(!KMB || (int64_t)g.K * g.N < ((int64_t)1 << 31), "matmul: the K-major second operand must be smaller than 2 GiB "
                  "(K * N = %lld bytes)", (long long)((int64_t)g.K * g.N));
+    LLMQ_REQUIRE(!KMA || (int64_t)g.K * g.M < ((int64_t)1 << 31), "matmul: the K-major first operand must be smaller than 2 GiB "
+                 "(K * M = %lld bytes)", (long long)((int64_t)g.K * g.M));
     const int tiles = (g.N / 256) * (m224 ? g.M / 224 : g.M / 256);
     const int grid = tiles < cus ? (tiles + xcds - 1) / xcds * xcds : cus;
     const bool cached_out = ((int64_t)g.M + g.N) * g.K + (int64_t)g.N * g.M * 2 <= ((int64_t)224 << 20);
-    if (m224)
-        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, B_FMT, false, 7, true, false, true>), dim3((unsigned)grid), dim3(256),
-                           0, stream, g);
-    else if (cached_out)
-        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, B_FMT, false, 8, false, false, true>), dim3((unsigned)grid), dim3(256),
-                           0, stream, g);
+    if constexpr (!KMA) {
+        if (m224) {
+            hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, B_FMT, false, 7, true, false, true>), dim3((unsigned)grid),
+                               dim3(256), 0, stream, g);
+            LLMQ_HIP_TRY(hipGetLastError());
+            return LLMQ_OK;
+        }
+    }
+    if (cached_out)
+        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, B_FMT, false, 8, false, false, KMB, KMA>), dim3((unsigned)grid),
+                           dim3(256), 0, stream, g);
     else
-        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, B_FMT, false, 8, true, false, true>), dim3((unsigned)grid), dim3(256),
-                           0, stream, g);
+        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, B_FMT, false, 8, true, false, KMB, KMA>), dim3((unsigned)grid),
+                           dim3(256), 0, stream, g);
     LLMQ_HIP_TRY(hipGetLastError());
     return LLMQ_OK;
 }
@@ -1638,8 +1757,10 @@ extern "C" int llmq_gemm_e4m3_bf16_mode(uint16_t* c, const uint8_t* a, const uin
     if (mode == LLMQ_MODE_TN)
         return b_format ? gemm_dispatch<uint16_t, 1>(g, workspace_or_null, workspace_bytes, st)
                         : gemm_dispatch<uint16_t, 0>(g, workspace_or_null, workspace_bytes, st);
-    LLMQ_REQUIRE(mode == LLMQ_MODE_TT, "matmul: FP8 operands are served in modes TN and TT (got mode %d)", mode);
-    return b_format ? gemm_dispatch_b_kmajor<1>(g, st) : gemm_dispatch_b_kmajor<0>(g, st);
+    if (mode == LLMQ_MODE_TT) return b_format ? gemm_dispatch_kmajor<1, false, true>(g, st) : gemm_dispatch_kmajor<0, false, true>(g, st);
+    if (mode == LLMQ_MODE_NN) return b_format ? gemm_dispatch_kmajor<1, true, false>(g, st) : gemm_dispatch_kmajor<0, true, false>(g, st);
+    LLMQ_REQUIRE(mode == LLMQ_MODE_NT, "matmul: unknown operand mode %d (TT = 0, TN = 1, NT = 2, NN = 3)", mode);
+    return b_format ? gemm_dispatch_kmajor<1, true, true>(g, st) : gemm_dispatch_kmajor<0, true, true>(g, st);
 }
 
 extern "C" int llmq_gemm_tn_e4m3_bf16(uint16_t* c, const uint8_t* a, const uint8_t* b, const uint16_t* bias_or_null,

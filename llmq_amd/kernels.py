@@ -113,7 +113,7 @@ def transpose(dst, src, stream=0):
 
 
 def matmul(c, a, b, bias, scale_a, scale_b, M, N, K, accumulate=False, stream=0, workspace=None, b_e5m2=False, _lib=None,
-           b_kmajor=False):
+           b_kmajor=False, a_kmajor=False):
     """TN matmul in the convention of the reference's kernels.h: row-major a[M,K], b[N,K] (e4m3) give
     row-major c[N,M] = (b @ a.T) * scale_a * scale_b (+ bias[M]) (+ c).  c: bf16 or fp32.
     workspace: optional device byte tensor (the reference passes a 32 MiB one); it enables the
@@ -121,11 +121,12 @@ def matmul(c, a, b, bias, scale_a, scale_b, M, N, K, accumulate=False, stream=0,
     dtype option): a float8_e5m2 tensor, or uint8 with b_e5m2=True.  _lib: tests pass the test-aid build of
     the same entry points (capi.testaid()) to force a kernel variant; everyone else leaves it alone."""
     L = _lib or capi.lib
-    if b_kmajor:
-        # the reference's mode TT: b stored [K, N] row-major (e.g. the output gradient dY[BT, OC] as the second
-        # operand of the weight gradient, without its transposed copy); bf16 output, whole 256-tiles only
+    if b_kmajor or a_kmajor:
+        # the reference's modes TT (b stored [K, N] row-major, e.g. the output gradient dY[BT, OC] as the second operand
+        # of the weight gradient without its transposed copy), NN (a stored [K, M], e.g. the weight W[OC, C] as the
+        # first operand of the dgrad) and NT (both); bf16 output, whole 256-tiles only
         if c.dtype != torch.bfloat16:
-            raise ValueError("matmul: the K-major second operand is served with bf16 output only")
+            raise ValueError("matmul: K-major operands are served with bf16 output only")
         pa = _dev(a, "a", (torch.float8_e4m3fn, torch.uint8))
         pb = _dev(b, "b", (torch.float8_e4m3fn, torch.float8_e5m2, torch.uint8))
         if a.numel() != M * K or b.numel() != N * K or c.numel() != N * M:
@@ -133,7 +134,8 @@ def matmul(c, a, b, bias, scale_a, scale_b, M, N, K, accumulate=False, stream=0,
         pbias = _dev(bias, "bias", (torch.bfloat16,), optional=True)
         capi.check(capi.lib.llmq_gemm_e4m3_bf16_mode(
             _dev(c, "c", (torch.bfloat16,)), pa, pb, pbias, _dev(scale_a, "scale_a", (torch.float32,), optional=True),
-            _dev(scale_b, "scale_b", (torch.float32,), optional=True), None, 0, M, N, K, 0,
+            _dev(scale_b, "scale_b", (torch.float32,), optional=True), None, 0, M, N, K,
+            (2 if b_kmajor else 3) if a_kmajor else 0,      # EMMTranspose: TT = 0, TN = 1, NT = 2, NN = 3
             int(bool(b_e5m2) or b.dtype == torch.float8_e5m2), int(accumulate), _stream(stream)))
         return
     pws, ws_bytes = None, 0

@@ -64,7 +64,7 @@ int main(int argc, char** argv) {
     const int BT = argc > 1 ? std::atoi(argv[1]) : 1024, C = argc > 2 ? std::atoi(argv[2]) : 896, OC = argc > 3 ? std::atoi(argv[3]) : 1152;
     const bool reuse_inp = argc > 4 && std::atoi(argv[4]) != 0;
     const bool fuse = argc > 5 && std::atoi(argv[5]) != 0;   // gradient quantize + transpose from one read
-    // 1: bf16 weight gradient; 2: also ask for the gradient's stored layout as the wgrad's K-major operand
+    // 1: bf16 weight gradient; 2: also ask for operands in their stored layouts (matmul modes NN / TT / NT)
     const int dw_mode = argc > 6 ? std::atoi(argv[6]) : 0;
     const bool dw_bf16 = dw_mode >= 1, direct = dw_mode == 2;
     const int B = 1, T = BT;
@@ -74,9 +74,13 @@ int main(int argc, char** argv) {
     QmmRunState rs; HIP_OK(hipGetDeviceProperties(&rs.DeviceProp, 0));
     rs.FuseGradTranspose = fuse;
     rs.DirectGradLayout = direct;
-    const bool direct_applies = direct && QmmRunState::direct_grad_layout_applies(B, T, C, OC, dw_bf16 ? ETensorDType::BF16 : ETensorDType::FP32, false);
-    std::printf("direct gradient layout applies: %d\n", (int)direct_applies);
-    rs.Capacity = QmmRunState::backward_temp_bytes(B, T, C, OC, fuse, direct_applies);
+    const QmmRunState::DirectPlan plan =
+        direct ? QmmRunState::direct_layout_plan(B, T, C, OC, ETensorDType::BF16, dw_bf16 ? ETensorDType::BF16 : ETensorDType::FP32, false)
+               : QmmRunState::DirectPlan{};
+    std::printf("stored-layout plan: dgrad in place %d, wgrad %s\n", (int)plan.DgradInPlace,
+                plan.Wgrad == QmmRunState::EWgrad::Copies ? "copies" : plan.Wgrad == QmmRunState::EWgrad::GradInPlace ? "gradient in place (TT)"
+                                                                                                                    : "both in place (NT)");
+    rs.Capacity = QmmRunState::backward_temp_bytes(B, T, C, OC, fuse, plan);
     rs.Arena = dalloc<std::byte>(rs.Capacity);
 
     std::vector<uint16_t> hx((std::size_t)BT * C), hw((std::size_t)OC * C), hdy((std::size_t)BT * OC);
@@ -114,7 +118,7 @@ int main(int argc, char** argv) {
     orc_fill_normal_bf16(hdb0.data(), hdb0.size(), 7, 4, 0.f, 1e-2f);
     Tensor dbias = make(ETensorDType::BF16, dalloc<uint16_t>(OC), {OC});
     HIP_OK(hipMemcpy(dbias.Data, hdb0.data(), (std::size_t)OC * 2, hipMemcpyHostToDevice));
-    const int bias_scratch = get_bias_backward_scratch_size(ETensorDType::BF16, OC, rs.DeviceProp);
+    const int bias_scratch = get_bias_backward_scratch_size(ETensorDType::FP8_E4M3, OC, rs.DeviceProp);   // dtype of the gradient it sums
     Tensor bias_buffer = make(ETensorDType::FP32, dalloc<float>((std::size_t)bias_scratch / 4), {bias_scratch / 4});
     backward_qmm(dinp, dweight, dbias, dout, inp, weight, bias_buffer, false, rs, B, T, C, OC, reuse_inp, stream);
     HIP_OK(hipStreamSynchronize(stream));
@@ -240,9 +244,9 @@ int main(int argc, char** argv) {
     catch (const std::invalid_argument&) { threw = true; }
     EXPECT(threw, "matmul with K %% 16 != 0 (operand rows not 16-byte aligned) must throw std::invalid_argument");
     threw = false;
-    try { matmul(out, weight, inp.Quant, no_bias, nullptr, nullptr, nullptr, workspace, OC, BT, C, EMMTranspose::NN, false, stream); }
+    try { matmul(out, weight, inp.Quant, no_bias, nullptr, nullptr, nullptr, workspace, OC, BT, C, EMMTranspose::NN, true, stream); }
     catch (const std::invalid_argument&) { threw = true; }
-    EXPECT(threw, "non-TN FP8 matmul must throw std::invalid_argument");
+    EXPECT(threw, "FP8 matmul in mode NN with accumulation (not served) must throw std::invalid_argument");
     threw = false;
     try { quantize_with_abs_max(out, nullptr, inp.Value, stats, 8, rs.DeviceProp, stream); }
     catch (const std::invalid_argument&) { threw = true; }

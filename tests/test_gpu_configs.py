@@ -149,8 +149,20 @@ def run_linear_fwd_bwd(K, O, BT, C, OC, x, w, dy, seed, backward=True, reuse_inp
     assert np.array_equal(host_bits(g_tp), gc.T), "gradient transpose"
     check_gemm(O, dinp, np.ascontiguousarray(wc.T), gc, dw_s, dg_s, seed + 1, "dgrad dx")
     check_gemm(O, dweight, np.ascontiguousarray(xc.T), np.ascontiguousarray(gc.T), dx_s, dg_s, seed + 2, "wgrad dw")
-    # The same weight gradient with the quantized output gradient read where it lies (matmul mode TT: dout.quant
-    # [BT, OC] as the K-major second operand, no transposed copy), wherever that mode serves the shape
+    # The same gradients with operands read where they lie, wherever the K-major modes serve the shape: dgrad with the
+    # weight [OC, C] as the K-major first operand (mode NN), wgrad with activation [BT, C] and gradient [BT, OC] both in
+    # place (mode NT) ...
+    if OC % 256 == 0 and BT % 256 == 0 and C % 256 == 0:
+        dx_nn = torch.full((BT, C), float("nan"), dtype=torch.bfloat16, device="cuda")
+        K.matmul(dx_nn, wq.quant, dout.quant, None, wq.scale, dout.scale, C, BT, OC, a_kmajor=True)
+        dw_nt = torch.full((OC, C), float("nan"), dtype=torch.bfloat16, device="cuda")
+        K.matmul(dw_nt, inp.quant, dout.quant, None, inp.scale, dout.scale, C, OC, BT, a_kmajor=True, b_kmajor=True)
+        torch.cuda.synchronize()
+        check_gemm(O, dx_nn, np.ascontiguousarray(wc.T), gc, dw_s, dg_s, seed + 1, "dgrad dx, mode NN")
+        check_gemm(O, dw_nt, np.ascontiguousarray(xc.T), np.ascontiguousarray(gc.T), dx_s, dg_s, seed + 2, "wgrad dw, mode NT")
+        del dx_nn, dw_nt
+    # ... and with the quantized output gradient alone read in place (matmul mode TT: dout.quant [BT, OC] as the
+    # K-major second operand)
     if OC % 256 == 0 and BT % 256 == 0 and (C % 256 == 0 or C % 224 == 0):
         dw_tt = torch.full((OC, C), float("nan"), dtype=torch.bfloat16, device="cuda")
         K.matmul(dw_tt, a_tp, dout.quant, None, inp.scale, dout.scale, C, OC, BT, b_kmajor=True)

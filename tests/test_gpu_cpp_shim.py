@@ -13,12 +13,13 @@ BIN = os.path.join(HERE, "cpp", "build", "qmm_harness")
 @pytest.mark.parametrize("args", [("1024", "896", "1152", "0"), ("2048", "896", "896", "1"), ("512", "4864", "896", "0"),
                                   ("4096", "1536", "1792", "0"), ("1024", "896", "1152", "0", "1"),
                                   ("2048", "1152", "896", "1", "1"),
-                                  # bf16 weight gradient; then the same layers with the gradient read in its stored
-                                  # layout (matmul mode TT): 256-tiles, 224-wide tiles (C = 896), and a shape the
-                                  # mode does not serve (OC = 1152 = 4.5 * 256), which must take the copying path
+                                  # bf16 weight gradient; then the same layers with operands read in their stored
+                                  # layouts: dgrad NN + wgrad NT (all dimensions on 256-tiles, OC <= 8192), dgrad NN +
+                                  # wgrad TT (OC = 9216), wgrad TT on 224-wide tiles with the copying dgrad (C = 896),
+                                  # a shape no K-major mode serves (OC = 1152), NT with the quantized input reused
                                   ("1024", "1024", "1536", "0", "0", "1"), ("1024", "1024", "1536", "0", "0", "2"),
-                                  ("2048", "896", "768", "1", "0", "2"), ("1024", "896", "1152", "0", "1", "2"),
-                                  ("512", "1536", "512", "0", "1", "2")])
+                                  ("1024", "768", "9216", "0", "0", "2"), ("2048", "896", "768", "1", "0", "2"),
+                                  ("1024", "896", "1152", "0", "1", "2"), ("512", "1536", "512", "1", "1", "2")])
 def test_qmm_harness(args):
     assert os.path.exists(BIN), "build it with `make -C tests/cpp` (done by __graft_entry__.build())"
     r = subprocess.run([BIN, *args], capture_output=True, text=True, timeout=150)

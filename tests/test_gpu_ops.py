@@ -65,7 +65,7 @@ def test_matmul_torch_convention(P, O):
     extra = bias.float().cpu().numpy().astype(np.float64)[None, :] + old.float().cpu().numpy().astype(np.float64)
     gemm_check(c.float().cpu().numpy(), exact, sumabs, scale, True, extra=extra)
     with pytest.raises(ValueError):
-        P.matmul(c, ad, bd, None, None, None, 0, ws, P.MODE_NN, False)       # FP8 is TN-only in the kernel layer
+        P.matmul(c, ad, bd, None, None, None, 0, ws, P.MODE_NN, False)       # mode NN wants b as [K, N]: shapes do not match
     with pytest.raises(ValueError):
         P.matmul(c, ad, bd[:, :256].contiguous(), None, None, None, 0, ws, P.MODE_NT, False)
 
@@ -92,6 +92,29 @@ def test_matmul_mode_tt_reads_the_first_operand_in_k_major_storage(P, O):
         P.matmul(torch.empty((M, N), device="cuda"), at, bd, None, None, None, 0, ws, P.MODE_TT, False)
     with pytest.raises(ValueError):                                            # a is [K, M]: handing over [M, K] mismatches c
         P.matmul(c, ad, bd, None, None, None, 0, ws, P.MODE_TT, False)
+
+
+@pytest.mark.parametrize("mode", ["NN", "TN"])
+def test_matmul_modes_with_b_in_k_major_storage(P, O, mode):
+    """Torch-sense modes NN (c = a @ b, b stored [K, N]) and TN (c = a^T @ b, a stored [K, M] as well): the kernel layer's
+    modes NN and NT after the operand swap of the binding (src/binding/kernel_binding.cpp:403-431)."""
+    M, N, Kd = 512, 256, 768
+    rng = np.random.default_rng(15)
+    a = rng.integers(0, 0x7E, (M, Kd)).astype(np.uint8) | (rng.integers(0, 2, (M, Kd)).astype(np.uint8) << 7)
+    b = rng.integers(0, 0x7E, (N, Kd)).astype(np.uint8)
+    dev = lambda x: torch.from_numpy(np.ascontiguousarray(x)).cuda().view(torch.float8_e4m3fn)
+    ad = dev(a) if mode == "NN" else dev(a.T)            # [M, K] or [K, M]
+    bd = dev(b.T)                                        # [K, N]
+    sa, sb = torch.tensor([0.25], device="cuda"), torch.tensor([0.125], device="cuda")
+    bias = torch.randn(N, device="cuda", dtype=torch.bfloat16)
+    ws = torch.empty(32 << 20, dtype=torch.uint8, device="cuda")
+    c = torch.full((M, N), float("nan"), device="cuda", dtype=torch.bfloat16)
+    P.matmul(c, ad, bd, bias, sa, sb, 0, ws, P.MODE_NN if mode == "NN" else P.MODE_TN, False)
+    exact, sumabs = O.gemm_exact(b, a)
+    extra = bias.float().cpu().numpy().astype(np.float64)[None, :]
+    gemm_check(c.float().cpu().numpy(), exact, sumabs, np.float32(0.25 * 0.125), True, extra=extra)
+    with pytest.raises(ValueError):                      # these two modes do not accumulate
+        P.matmul(c, ad, bd, None, sa, sb, 0, ws, P.MODE_NN if mode == "NN" else P.MODE_TN, True)
 
 
 def test_backward_bias_through_ops(P):

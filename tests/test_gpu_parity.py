@@ -660,32 +660,38 @@ def test_gemm_swept_shapes_exact_and_inside_their_rows(K, O, mnk):
         assert bool((big[:pad] == guard).all()) and bool((big[pad + N:] == guard).all()), "guard rows were written"
 
 
+@pytest.mark.parametrize("mode", ["TT", "NN", "NT"])
 @pytest.mark.parametrize("mnk", [(256, 256, 256), (512, 768, 512), (448, 512, 768), (1024, 2048, 1024), (2304, 512, 2816),
                                  (3584, 4096, 512)])
-def test_gemm_second_operand_in_k_major_layout(K, O, mnk):
-    """Mode TT of the reference's matmul signature (src/kernels/kernels.h:22, matmul.cpp:66-67): b stored [K, N]
-    row-major, read through transposing LDS reads instead of a materialised transpose (what backward_qmm does with
-    the output gradient, src/models/llama_model.cpp:331-333).  Integer operands -> bit exact against the oracle,
-    with bias and accumulation; random codes (e5m2 included) within the tolerance of the exact product and
-    bit-identical to mode TN on the transposed copy when that runs on the same kernel family (same sums in the same
-    order; the 8-wave kernel's other matrix instruction groups K differently)."""
+def test_gemm_operands_in_k_major_layout(K, O, mnk, mode):
+    """Modes TT / NN / NT of the reference's matmul signature (src/kernels/kernels.h:22, matmul.cpp:66-67): b stored
+    [K, N] and / or a stored [K, M] row-major, read through transposing LDS reads instead of a materialised transpose
+    (what backward_qmm does with the output gradient, the weight and the activation,
+    src/models/llama_model.cpp:309-339).  Integer operands -> bit exact against the oracle, with bias and (mode TT)
+    accumulation; random codes (e5m2 included) within the tolerance of the exact product, bit-identical to mode TN on
+    the transposed copies when that runs on the same kernel family (same sums in the same order), and the same bits on
+    every one of 8 repeated launches."""
     M, N, Kd = mnk
+    a_km, b_km = mode[0] == "N", mode[1] == "T"
+    if a_km and M % 256:
+        pytest.skip("a K-major first operand is served on 256-wide tiles only")
+    lay_a = (lambda x: np.ascontiguousarray(x.T)) if a_km else (lambda x: x)      # [K, M]: what the caller holds
+    lay_b = (lambda x: np.ascontiguousarray(x.T)) if b_km else (lambda x: x)      # [K, N]
     a, _ = O.fill_int_e4m3(M * Kd, 606, 0)
     b, _ = O.fill_int_e4m3(N * Kd, 606, 1)
     a, b = a.reshape(M, Kd), b.reshape(N, Kd)
-    bt = np.ascontiguousarray(b.T)                      # [K, N]: what the caller holds
     s = float(np.sqrt(np.float32(4.0 / Kd)))
     _, biasv = O.fill_int_e4m3(M, 606, 2)
     _, oldv = O.fill_int_e4m3(N * M, 606, 3)
     bias = O.f32_to_bf16(biasv.astype(np.float32))
     old = O.f32_to_bf16(oldv.astype(np.float32)).reshape(N, M)
     mt = M % 64 == 0
-    cases = [(False, False), (True, False)] + ([(True, True)] if M % 256 == 0 else [])
+    cases = [(False, False), (True, False)] + ([(True, True)] if M % 256 == 0 and not a_km else [])
     for use_bias, use_old in cases:
         want = O.gemm_tn(a, b, sa=s, sb=s, bias=bias if use_bias else None, c_old=old if use_old else None, mt=mt)
         c = dev_bf16(old).reshape(N, M).clone() if use_old else torch.full((N, M), float("nan"), dtype=torch.bfloat16, device="cuda")
-        K.matmul(c, dev_u8(a), dev_u8(bt), dev_bf16(bias) if use_bias else None, dev_scalar(s), dev_scalar(s), M, N, Kd,
-                 accumulate=use_old, b_kmajor=True)
+        K.matmul(c, dev_u8(lay_a(a)), dev_u8(lay_b(b)), dev_bf16(bias) if use_bias else None, dev_scalar(s), dev_scalar(s), M, N, Kd,
+                 accumulate=use_old, a_kmajor=a_km, b_kmajor=b_km)
         assert np.array_equal(host_bits(c), want), (use_bias, use_old)
     rng = np.random.default_rng(M + Kd)
     for e5m2 in (False, True):
@@ -697,23 +703,23 @@ def test_gemm_second_operand_in_k_major_layout(K, O, mnk):
             br &= 0xBF
         else:
             br[(br & 0x7F) == 0x7F] ^= 1
+        da, db = dev_u8(lay_a(ar)), dev_u8(lay_b(br))
         c_tn = torch.empty((N, M), dtype=torch.bfloat16, device="cuda")
-        c_tt = torch.empty((N, M), dtype=torch.bfloat16, device="cuda")
-        K.matmul(c_tt, dev_u8(ar), dev_u8(np.ascontiguousarray(br.T)), None, dev_scalar(0.37), dev_scalar(1.0 / 448), M, N, Kd,
-                 b_e5m2=e5m2, b_kmajor=True)
+        c_km = torch.empty((N, M), dtype=torch.bfloat16, device="cuda")
+        K.matmul(c_km, da, db, None, dev_scalar(0.37), dev_scalar(1.0 / 448), M, N, Kd, b_e5m2=e5m2, a_kmajor=a_km, b_kmajor=b_km)
         exact, sumabs = O.gemm_exact(ar, br, b_e5m2=e5m2)
-        gemm_check(c_tt.float().cpu().numpy(), exact, sumabs, np.float32(np.float32(0.37) * np.float32(1.0 / 448)), True)
+        gemm_check(c_km.float().cpu().numpy(), exact, sumabs, np.float32(np.float32(0.37) * np.float32(1.0 / 448)), True)
         set_variant((4, 0) if M % 256 else (3, 1))       # mode TN on the same kernel family: the same sums in the same order
         try:
             mm(K, c_tn, dev_u8(ar), dev_u8(br), None, dev_scalar(0.37), dev_scalar(1.0 / 448), M, N, Kd, b_e5m2=e5m2)
         finally:
             set_variant((0, 0))
-        assert torch.equal(c_tn.view(torch.int16), c_tt.view(torch.int16)), e5m2
+        assert torch.equal(c_tn.view(torch.int16), c_km.view(torch.int16)), e5m2
         for _ in range(8):                                  # repeated launches: the same bits every time
             again = torch.full((N, M), float("nan"), dtype=torch.bfloat16, device="cuda")
-            K.matmul(again, dev_u8(ar), dev_u8(np.ascontiguousarray(br.T)), None, dev_scalar(0.37), dev_scalar(1.0 / 448), M, N, Kd,
-                     b_e5m2=e5m2, b_kmajor=True)
-            assert torch.equal(again.view(torch.int16), c_tt.view(torch.int16)), e5m2
+            K.matmul(again, da, db, None, dev_scalar(0.37), dev_scalar(1.0 / 448), M, N, Kd, b_e5m2=e5m2, a_kmajor=a_km,
+                     b_kmajor=b_km)
+            assert torch.equal(again.view(torch.int16), c_km.view(torch.int16)), e5m2
 
 
 def test_gemm_k_major_operand_rejects_what_it_cannot_serve(K):
@@ -722,6 +728,9 @@ def test_gemm_k_major_operand_rejects_what_it_cannot_serve(K):
     c = torch.zeros((256, 256), dtype=torch.bfloat16, device="cuda")
     with pytest.raises(ValueError, match="mode TT"):
         K.matmul(c, a, b, None, None, None, 256, 256, 384, b_kmajor=True)      # K % 256 != 0
+    with pytest.raises(ValueError, match="does not accumulate"):
+        K.matmul(c, torch.zeros((512, 256), dtype=torch.uint8, device="cuda"), torch.zeros((256, 512), dtype=torch.uint8, device="cuda"),
+                 None, None, None, 256, 256, 512, accumulate=True, a_kmajor=True)
     with pytest.raises(ValueError, match="bf16 output"):
         K.matmul(c.float(), a, b, None, None, None, 256, 256, 384, b_kmajor=True)
     # a K-major operand of 2 GiB or more is refused before anything is launched (32-bit lane offsets walk it);
