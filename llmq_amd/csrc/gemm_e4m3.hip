@@ -1,31 +1,35 @@
-// e4m3 x e4m3 TN GEMM for gfx950 (CDNA4) with fp32 accumulation and a scaled bf16 / fp32 epilogue.
+// e4m3 x e4m3 (or x e5m2) GEMM for gfx950 (CDNA4) with fp32 accumulation and a scaled bf16 / fp32 epilogue.
 //
 // Interface semantics follow the reference's matmul for FP8 operands (src/kernels/matmul.cpp:47-153,
 // 216-220; hand-written variant src/kernels/gemm_mma.cu:258-284): row-major a[M,K], b[N,K] (both K
-// contiguous) produce row-major c[N,M],
+// contiguous, mode TN) produce row-major c[N,M],
 //     c[n,m] = round( (sum_k b[n,k] a[m,k]) * (sa*sb) + bias[m] + (accumulate ? c[n,m] : 0) ).
+// For bf16 output the operands may also be stored K-major (a as [K,M], b as [K,N]: the reference's modes NN, TT, NT).
 //
-// Kernel design (nothing here is derived from the reference's mma.sync kernel).  Two kernels share the
-// tiling, the LDS layout and the copy scheme; each has its own description further down:
-//   * gemm_tn_e4m3_w4_kernel: 256 x 256 tile, 4 waves of 128 x 128, v_mfma_f32_16x16x128_f8f6f4,
-//     persistent; the default whenever M, N are multiples of 256 and K is a multiple of 256;
+// Kernel design (nothing here is derived from the reference's mma.sync kernel).  Three kernels; the two tiled ones
+// share the tiling, the LDS layout and the copy scheme; each has its own description further down:
+//   * gemm_tn_e4m3_w4_kernel: 256 x 256 (or 256 x 224 / 192) tile, 4 waves of 128 x 128, v_mfma_f32_16x16x128_f8f6f4,
+//     persistent; the default whenever M, N fit those tiles and K is a multiple of 128 from 256 up; also the K-major
+//     operand modes and the K segments of a cut last round;
 //   * gemm_tn_e4m3_pipe_kernel: 256 x 256 tile with 8 waves of 128 x 64 or 128 x 128 tile with 4 waves
-//     of 64 x 64, v_mfma_f32_32x32x64_f8f6f4; every other shape, and the split-K path.
-// Common to both:
+//     of 64 x 64, v_mfma_f32_32x32x64_f8f6f4; the other shapes on the 128 lattice, and the split-K path;
+//   * gemm_tn_e4m3_edge_kernel: 64 x 64 tile with predicated loads and stores: shapes off the lattice (any M, N; K a
+//     multiple of 16) and the last N % tile rows of the others.
+// Common to the tiled kernels:
 //   * one workgroup computes a tile of c, K is walked in steps of 128 bytes;
 //   * both operand tiles are staged in LDS, double buffered, by 16-byte-per-lane direct-to-LDS loads
 //     (no VGPR staging);
-//   * LDS rows are 128 bytes (one K-step) and the eight 16-byte chunks of a row are XOR-swizzled
-//     with (row >> 1) & 7, which makes the 128-bit fragment reads of 16 consecutive rows hit all 64
-//     banks exactly once; the swizzle is applied on the global side (each lane picks its source chunk)
-//     because direct-to-LDS loads land linearly (lane i -> base + 16 i);
+//   * LDS rows are 128 bytes (one K-step) and the eight 16-byte chunks of a row are XOR-swizzled with a function of
+//     the row that makes the 128-bit fragment reads conflict-free for the kernel's lane -> row mapping ((row >> 1) & 7
+//     for the 32x32x64 fragments, frag_swizzle() for the 16x16x128 ones); the swizzle is applied on the global side
+//     (each lane picks its source chunk) because direct-to-LDS loads land linearly (lane i -> base + 16 i);
 //   * both operands of the matrix instruction use the same lane->K mapping, so any consistent mapping
 //     is correct;
 //   * rows of the a-tile (the m / column index of c) are permuted on their way into LDS so that the
 //     accumulators a lane holds for one c row are consecutive columns: the epilogue stores packed
 //     groups and neighbouring lanes cover a contiguous row segment;
-//   * the linear workgroup id is remapped so that each of the 8 XCDs (workgroups are dealt to XCDs
-//     round-robin) works on a contiguous range of tiles, walked in column-major groups of `group`
+//   * the linear workgroup id is remapped so that each XCD (workgroups are dealt to the XCDs round-robin; their
+//     number is a launch argument) works on a contiguous range of tiles, walked in column-major groups of `group`
 //     tile-rows for L2 reuse of both operands.
 // The 8-wave kernel's K loop is an explicit software pipeline over half-steps (K = 64, one matrix
 // instruction deep).  Within a half-step the matrix instructions run row by row (b-rows fragment i
