@@ -291,6 +291,67 @@ def test_hip_graph_replay_matches_eager(K, O):
                                b.view(torch.uint8) if b.dtype != torch.uint8 else b), "replay for seed %d differs" % seed
 
 
+@pytest.mark.parametrize("wgrad", ["NT", "TT"])
+def test_hip_graph_replay_of_the_stored_layout_backward(K, O, wgrad):
+    """The backward of a layer with its matmuls in the K-major operand modes (dgrad NN on the weight as stored,
+    weight gradient NT on activation and gradient as stored, or TT on the gradient as stored), recorded into a HIP
+    graph: every replay, with new inputs and eager work in between, must reproduce the eager result bit for bit, and
+    the eager result must equal the transposing route's."""
+    BT, C, OC = 1024, 768, 512
+    x = torch.empty((BT, C), dtype=torch.bfloat16, device="cuda")
+    w = torch.empty((OC, C), dtype=torch.bfloat16, device="cuda")
+    dy = torch.empty((BT, OC), dtype=torch.bfloat16, device="cuda")
+    inp, wq, dout = QT(x), QT(w), QT(dy)
+    dinp = torch.empty((BT, C), dtype=torch.bfloat16, device="cuda")
+    dweight = torch.empty((OC, C), dtype=torch.bfloat16, device="cuda")
+    act_tp = torch.empty((C, BT), dtype=F8, device="cuda")
+    ref_dinp, ref_dweight = torch.empty_like(dinp), torch.empty_like(dweight)
+    workspace()
+
+    def fill(seed):
+        x.copy_(dev_bf16(O.fill_normal_bf16(BT * C, seed, 1).reshape(BT, C)))
+        w.copy_(dev_bf16(O.fill_normal_bf16(OC * C, seed, 2, 0.0, 0.02).reshape(OC, C)))
+        dy.copy_(dev_bf16(O.fill_normal_bf16(BT * OC, seed, 3, 0.0, 1e-3).reshape(BT, OC)))
+
+    def sequence():
+        for qt in (inp, wq, dout):
+            K.abs_max(qt.abs_max, qt.value)
+            K.quantize_with_abs_max(qt.quant, qt.scale, qt.value, qt.abs_max)
+        K.matmul(dinp, wq.quant, dout.quant, None, wq.scale, dout.scale, C, BT, OC, a_kmajor=True)
+        if wgrad == "NT":
+            K.matmul(dweight, inp.quant, dout.quant, None, inp.scale, dout.scale, C, OC, BT, a_kmajor=True, b_kmajor=True)
+        else:
+            K.quantize_and_transpose_with_abs_max(act_tp, None, inp.value, inp.abs_max)
+            K.matmul(dweight, act_tp, dout.quant, None, inp.scale, dout.scale, C, OC, BT, b_kmajor=True)
+
+    fill(60)
+    sequence()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        sequence()
+        with torch.cuda.graph(graph, stream=side):
+            sequence()
+    torch.cuda.current_stream().wait_stream(side)
+    for seed in (61, 62, 63):
+        fill(seed)
+        sequence()
+        torch.cuda.synchronize()
+        want = [dinp.clone(), dweight.clone()]
+        backward_qmm(K, ref_dinp, ref_dweight, dout, inp, wq.quant, wq.scale, BT, C, OC, reuse_inp=False)
+        torch.cuda.synchronize()
+        # 768 x 512 outputs: both routes run whole 256-tiles of the four-wave kernel over the same K order
+        assert torch.equal(ref_dinp.view(torch.int16), dinp.view(torch.int16)), "dgrad differs from the transposing route"
+        assert torch.equal(ref_dweight.view(torch.int16), dweight.view(torch.int16)), "wgrad differs from the transposing route"
+        dinp.fill_(float("nan"))
+        dweight.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(want[0].view(torch.int16), dinp.view(torch.int16)), "replay for seed %d differs" % seed
+        assert torch.equal(want[1].view(torch.int16), dweight.view(torch.int16)), "replay for seed %d differs" % seed
+
+
 def test_backward_with_e5m2_gradients(K, O):
     """The e5m2 gradient dtype (`--gradient-dtype=e5m2` in the reference): dY is quantized to e5m2 with the
     same 448-based scale (src/kernels/quant.cu:79, 130-132), transposed as bytes, and multiplied as the b
