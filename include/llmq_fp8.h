@@ -124,9 +124,11 @@ int llmq_transpose_u8(uint8_t* dst, const uint8_t* src, int rows, int cols, void
  *           cudaStream_t, EMatmulBackend)  src/kernels/kernels.h:88-90, src/kernels/matmul.cpp:216-220,
  *           and gemm_mma_tn(...) src/kernels/gemm_mma.cu:279-284.
  * workspace: device scratch like the reference's matmul workspace (32 MiB in src/training/model.cpp:69),
- * or NULL with size 0.  It is only used when the output has too few tiles to fill the chip: K is
- * then split, fp32 partial results (N*M*4 bytes per split) go to the workspace and are added in a
- * fixed order, so results are deterministic.  Calls that share a workspace must be stream ordered.
+ * or NULL with size 0.  It is used in two cases, both deterministic (fp32 partial results go to the workspace and are
+ * added in a fixed order by a second kernel): an output with too few tiles to fill the chip has K split over more
+ * workgroups (N*M*4 bytes per split), and a large output whose last round of 256 x 256 tiles would leave most of the
+ * chip idle has the tiles of that round cut into K segments (256 KiB per segment).  What does not fit the workspace is
+ * not split.  Calls that share a workspace must be stream ordered.
  */
 int llmq_gemm_tn_e4m3_bf16(uint16_t* c, const uint8_t* a, const uint8_t* b, const uint16_t* bias_or_null,
                            const float* sa_or_null, const float* sb_or_null, void* workspace_or_null,
@@ -144,7 +146,9 @@ int llmq_gemm_tn_e4m3_bf16(uint16_t* c, const uint8_t* a, const uint8_t* b, cons
  * kernels take TN only) are not needed.  The K-major modes serve M, N and K multiples of 256 (TT without
  * accumulation also M a multiple of 224) and K-major operands below 2 GiB; NN and NT do not accumulate into c.  Other
  * shapes return LLMQ_ERR_INVALID_ARGUMENT before anything is launched and the caller takes the transposing route.
- * b_format: 0 = e4m3, 1 = e5m2.  Results are bit-identical to mode TN on the transposed copies.
+ * b_format: 0 = e4m3, 1 = e5m2.  The workspace serves the cut of the last round of tiles as in mode TN (the K-major
+ * modes have no split-K for few-tile outputs).  Results are bit-identical to mode TN on the transposed copies whenever
+ * both run the same plan (256 x 256 tiles of the same kernel family, the same cut).
  */
 #define LLMQ_MODE_TT 0
 #define LLMQ_MODE_TN 1

@@ -35,25 +35,34 @@ struct QmmRunState {
     // transposed copies, wherever direct_layout_plan() finds the shapes served and the copy dearer than the mode's
     // slower K loop; elsewhere it behaves as without the flag.
     bool DirectGradLayout = false;
+    // With DirectGradLayout: take every stored-layout mode the shapes allow, whatever it costs in time (the transposed
+    // copies then never occupy the stack: backward_temp_bytes() shrinks accordingly).
+    bool DirectGradLayoutWhereverServed = false;
     using EWgrad = EQmmWgrad;
     using DirectPlan = QmmDirectPlan;
     // The K-major modes serve whole 256-wide tiles, bf16 output and operands below 2 GiB; modes NN / NT do not
-    // accumulate.  Measured on the Qwen2.5-7B MLP at 8192 tokens (one box, alternating): mode NN costs 2-3 % of the
-    // matmul and saves the weight's transposed copy (dgrad 439 -> 423 us and 788 -> 764 us); a K-major second operand
-    // costs 6 %, both operands K-major 9-11 %, against transposed copies of 2 bytes per element: reading the gradient
-    // in place pays while the matmul's row count C stays below about 10^4, reading the activation in place as well
-    // while OC does.
+    // accumulate.  Which of them pay was measured on MLP layers of Qwen2.5-7B (C = 3584, FFN 18944), 1.5B (1536, 8960)
+    // and a 2048 / 8192 layer at 4096 to 16384 tokens, every matmul with the 32 MiB workspace, against mode TN plus the
+    // byte transposes it needs (2 bytes moved per element copied):
+    //  * weight gradient: a K-major second operand costs 3-6 % of the matmul, both operands K-major 2-10 %; the copies
+    //    cost more on every layer measured (7B at 8192 tokens: 442 -> 389 us in mode NT, 862 -> 778 us in mode TT with
+    //    the activation's copy; 1.5B at 16384 tokens: 207 -> 181 us and 422 -> 340 us).  NT where the activation is the
+    //    larger copy (OC <= 8192), else TT while the matmul stays small enough (C <= 8192).
+    //  * dgrad in mode NN saves only the weight's copy (26 and 45 us on the 7B layers, 7-11 us on the 1.5B ones) and has
+    //    one tile plan (256 x 256, bf16 staged through LDS) where mode TN picks 224- or 192-wide tiles or a small-output
+    //    plan: level with TN per tile on the 7B down projection from 8192 tokens on (439 -> 415 us, 760 -> 750 us for
+    //    gate+up), 13-16 % slower at 4096 tokens, 20-48 % slower on the 1.5B and 2048-wide layers (short K, few tiles).
+    //    Taken for weights of 48 M elements and more at 8192 to 16384 tokens.
     static DirectPlan direct_layout_plan(int B, int T, int C, int OC, ETensorDType dinp_dtype, ETensorDType dweight_dtype,
-                                         bool accumulate) {
+                                         bool accumulate, bool wherever_served = false) {
         const long BT = (long)B * T, lim = 1L << 31;
         const bool tiles = C % 256 == 0 && OC % 256 == 0 && BT % 256 == 0;
         DirectPlan p;
-        // mode NN: 2-3 % of a matmul of 2 * BT * C * OC flop against a copy of 2 * C * OC bytes: the copy is the larger
-        // cost up to about 2 * 10^4 tokens
-        p.DgradInPlace = tiles && dinp_dtype == ETensorDType::BF16 && (long)C * OC < lim && BT <= 16384;
+        p.DgradInPlace = tiles && dinp_dtype == ETensorDType::BF16 && (long)C * OC < lim &&
+                         (wherever_served || ((long)C * OC >= (48L << 20) && BT >= 8192 && BT <= 16384));
         if (dweight_dtype == ETensorDType::BF16 && OC % 256 == 0 && BT % 256 == 0 && BT * OC < lim) {
-            if (tiles && !accumulate && BT * C < lim && OC <= 8192) p.Wgrad = EWgrad::BothInPlace;
-            else if ((C % 256 == 0 || (C % 224 == 0 && !accumulate)) && C <= 8192) p.Wgrad = EWgrad::GradInPlace;
+            if (tiles && !accumulate && BT * C < lim && (wherever_served || OC <= 8192)) p.Wgrad = EWgrad::BothInPlace;
+            else if ((C % 256 == 0 || (C % 224 == 0 && !accumulate)) && (wherever_served || C <= 8192)) p.Wgrad = EWgrad::GradInPlace;
         }
         return p;
     }
@@ -110,7 +119,8 @@ inline void backward_qmm(Tensor& dinp, Tensor& dweight, Tensor dbias, Quantizabl
     if (weight.DType != ETensorDType::FP8_E4M3)
         throw std::invalid_argument("backward_qmm: this build implements the FP8 (e4m3 weight) branch only");
     const QmmRunState::DirectPlan plan =
-        rs.DirectGradLayout ? QmmRunState::direct_layout_plan(B, T, C, OC, dinp.DType, dweight.DType, accumulate_gradient)
+        rs.DirectGradLayout ? QmmRunState::direct_layout_plan(B, T, C, OC, dinp.DType, dweight.DType, accumulate_gradient,
+                                                              rs.DirectGradLayoutWhereverServed)
                             : QmmRunState::DirectPlan{};
     const bool copies = plan.Wgrad == QmmRunState::EWgrad::Copies;
     Tensor grad_tp{};

@@ -80,7 +80,7 @@ _testaid = None
 
 
 def testaid():
-    """The test-aid library (tests and bench.py only; never needed by a user of the path): the four matmul
+    """The test-aid library (tests and bench.py only; never needed by a user of the path): the matmul
     entry points from a build of the GEMM file whose kernel selection can be forced
     (llmq_debug_set_gemm_variant / llmq_debug_set_gemm_persist), and the measurement aids llmq_debug_copy_u8 and llmq_debug_stream_u8
     (plain copy, read-only and write-only kernels) and llmq_debug_mfma_ceiling (register-only matrix-instruction loop)."""
@@ -91,7 +91,7 @@ def testaid():
         t = C.CDLL(TESTAID_PATH)
         t.llmq_last_error.restype = C.c_char_p
         for name in ("llmq_gemm_tn_e4m3_bf16", "llmq_gemm_tn_e4m3_f32", "llmq_gemm_tn_e4m3_e5m2_bf16",
-                     "llmq_gemm_tn_e4m3_e5m2_f32"):
+                     "llmq_gemm_tn_e4m3_e5m2_f32", "llmq_gemm_e4m3_bf16_mode"):
             getattr(t, name).argtypes = getattr(lib, name).argtypes
             getattr(t, name).restype = _int
         t.llmq_debug_set_gemm_variant.argtypes = [_int, _int]

@@ -615,8 +615,9 @@ template <typename OutT, int B_FMT, bool SEG, int NJ = 8, bool STREAM_OUT = true
           bool KMA = false>
 __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     static_assert(!(SEG && ODDK), "K segments are whole pairs of K-steps");
-    static_assert(!((KMB || KMA) && (SEG || ODDK)), "the K-major operand modes are built for whole tiles and even K-step counts");
-    static_assert(!KMA || (NJ == 8 && std::is_same_v<OutT, uint16_t>), "the K-major first operand is built for 256-wide tiles and bf16 output");
+    static_assert(!((KMB || KMA) && ODDK), "the K-major operand modes are built for even K-step counts");
+    static_assert(!KMA || (NJ == 8 && (SEG || std::is_same_v<OutT, uint16_t>)),
+                  "the K-major first operand is built for 256-wide tiles and bf16 output (fp32 only as K segments)");
     constexpr int BLK = 256, T = 256, WT = 128, NF = 8;
     constexpr int WTM = 16 * NJ, BLKM = 2 * WTM;  // columns (first-operand rows) per wave and per tile
     constexpr int P_BYTES = BLK * kBK, STAGE = 2 * P_BYTES;
@@ -1093,7 +1094,20 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
             constexpr bool BIAS = decltype(bias_tag)::value;
             constexpr bool ACC = decltype(acc_tag)::value;
             typedef float v4fl __attribute__((ext_vector_type(4)));
-            if constexpr (KMA) {
+            if constexpr (KMA && SEG) {
+                // acc[i][j][r] is row 16 i + 4 ekg + r, column 16 j + el16 of the wave tile: the raw accumulators go to
+                // the partial tile one by one (16 lanes fill 64 bytes of a row; the tile stays in the caches until
+                // the reduction kernel reads it)
+                LLMQ_GLOBAL float* pc = (LLMQ_GLOBAL float*)c + (row0 + 4 * ekg) * BLK + wm * WTM + el16;
+#pragma unroll
+                for (int i = 0; i < NF; ++i) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+#pragma unroll
+                        for (int j = 0; j < NJ; ++j) pc[(16 * i + r) * BLK + 16 * j] = acc[i][j][r];
+                    }
+                }
+            } else if constexpr (KMA) {
                 // acc[i][j][r] is c row 16 i + 4 ekg + r, column 16 j + el16 of the wave tile.  Per fragment row i the
                 // wave writes its 16 x 128 outputs as bf16 into its own piece of LDS ([16 rows][256 bytes], the 32-byte
                 // pieces of a row xor-ed with the row quad so that the four row quads of a write land on different
@@ -1706,7 +1720,7 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
 // Operands stored K-major (the reference's modes TT: b [K, N]; NN: a [K, M]; NT: both): the four-wave kernel's KMB / KMA
 // instances, whole tiles only.
 template <int B_FMT, bool KMA, bool KMB>
-static int gemm_dispatch_kmajor(GemmArgs g, hipStream_t stream) {
+static int gemm_dispatch_kmajor(GemmArgs g, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     static_assert(KMA || KMB, "mode TN goes through gemm_dispatch");
     const char* mode = KMA ? (KMB ? "NT" : "NN") : "TT";
     LLMQ_REQUIRE(g.M > 0 && g.N > 0 && g.K > 0, "matmul: M, N, K must be positive (got %d, %d, %d)", g.M, g.N, g.K);
@@ -1714,8 +1728,9 @@ static int gemm_dispatch_kmajor(GemmArgs g, hipStream_t stream) {
     g.xcds = xcds;
     g.group = 8;
     LLMQ_REQUIRE(g.a && g.b && g.c, "matmul: null operand pointer");
-    LLMQ_REQUIRE(aligned16(g.a) && aligned16(g.b) && aligned16(g.c) && aligned16(g.bias),
+    LLMQ_REQUIRE(aligned16(g.a) && aligned16(g.b) && aligned16(g.c) && aligned16(g.bias) && aligned16(workspace),
                  "matmul: all pointers must be 16-byte aligned");
+    LLMQ_REQUIRE(workspace != nullptr || workspace_bytes == 0, "matmul: workspace size given without a workspace");
     const bool m224 = !KMA && g.M % 256 != 0 && g.M % 224 == 0 && !g.accumulate;
     LLMQ_REQUIRE(g.N % 256 == 0 && g.K % 256 == 0 && (g.M % 256 == 0 || m224) && cus % xcds == 0,
                  "matmul: a K-major operand (mode %s) needs N %% 256 == 0, K %% 256 == 0 and M %% 256 == 0 (mode TT without "
@@ -1728,23 +1743,41 @@ static int gemm_dispatch_kmajor(GemmArgs g, hipStream_t stream) {
     LLMQ_REQUIRE(!KMA || (int64_t)g.K * g.M < ((int64_t)1 << 31), "matmul: the K-major first operand must be smaller than 2 GiB "
                  "(K * M = %lld bytes)", (long long)((int64_t)g.K * g.M));
     const int tiles = (g.N / 256) * (m224 ? g.M / 224 : g.M / 256);
-    const int grid = tiles < cus ? (tiles + xcds - 1) / xcds * xcds : cus;
     const bool cached_out = ((int64_t)g.M + g.N) * g.K + (int64_t)g.N * g.M * 2 <= ((int64_t)224 << 20);
     if constexpr (!KMA) {
         if (m224) {
+            const int grid = tiles < cus ? (tiles + xcds - 1) / xcds * xcds : cus;
             hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, B_FMT, false, 7, true, false, true>), dim3((unsigned)grid),
                                dim3(256), 0, stream, g);
             LLMQ_HIP_TRY(hipGetLastError());
             return LLMQ_OK;
         }
     }
+    // the last, partial round of tiles cut into K segments as in mode TN (needs the caller's workspace)
+    const int force_tile = g_gemm_tile, force_splits = g_gemm_splits;
+    const W4Plan plan = plan_w4(tiles, cus, xcds, g.M, g.N, g.K, force_tile == 3 ? force_splits : 0, workspace ? workspace_bytes : 0);
+    LLMQ_REQUIRE(force_tile != 3 || force_splits <= 1 || plan.rem_split == force_splits,
+                 "matmul: cannot cut the last round into %d segments (K = %d, workspace %zu bytes)", force_splits, g.K,
+                 workspace_bytes);
+    g.rem_split = plan.rem_split;
+    g.k_len = plan.k_len;
+    g.part_per_xcd = plan.part_per_xcd;
+    g.partial = reinterpret_cast<float*>(workspace);
     if (cached_out)
-        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, B_FMT, false, 8, false, false, KMB, KMA>), dim3((unsigned)grid),
+        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, B_FMT, false, 8, false, false, KMB, KMA>), dim3((unsigned)plan.grid),
                            dim3(256), 0, stream, g);
     else
-        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, B_FMT, false, 8, true, false, KMB, KMA>), dim3((unsigned)grid),
+        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, B_FMT, false, 8, true, false, KMB, KMA>), dim3((unsigned)plan.grid),
                            dim3(256), 0, stream, g);
     LLMQ_HIP_TRY(hipGetLastError());
+    if (plan.rem_split > 1) {
+        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<float, B_FMT, true, 8, true, false, KMB, KMA>), dim3((unsigned)plan.grid),
+                           dim3(256), 0, stream, g);
+        LLMQ_HIP_TRY(hipGetLastError());
+        hipLaunchKernelGGL((w4_segment_reduce_kernel<uint16_t>), dim3((unsigned)(xcds * plan.rem_max * 32)), dim3(256), 0, stream,
+                           g, plan.grid / xcds, plan.rem_max);
+        LLMQ_HIP_TRY(hipGetLastError());
+    }
     return LLMQ_OK;
 }
 
@@ -1761,10 +1794,10 @@ extern "C" int llmq_gemm_e4m3_bf16_mode(uint16_t* c, const uint8_t* a, const uin
     if (mode == LLMQ_MODE_TN)
         return b_format ? gemm_dispatch<uint16_t, 1>(g, workspace_or_null, workspace_bytes, st)
                         : gemm_dispatch<uint16_t, 0>(g, workspace_or_null, workspace_bytes, st);
-    if (mode == LLMQ_MODE_TT) return b_format ? gemm_dispatch_kmajor<1, false, true>(g, st) : gemm_dispatch_kmajor<0, false, true>(g, st);
-    if (mode == LLMQ_MODE_NN) return b_format ? gemm_dispatch_kmajor<1, true, false>(g, st) : gemm_dispatch_kmajor<0, true, false>(g, st);
+    if (mode == LLMQ_MODE_TT) return b_format ? gemm_dispatch_kmajor<1, false, true>(g, workspace_or_null, workspace_bytes, st) : gemm_dispatch_kmajor<0, false, true>(g, workspace_or_null, workspace_bytes, st);
+    if (mode == LLMQ_MODE_NN) return b_format ? gemm_dispatch_kmajor<1, true, false>(g, workspace_or_null, workspace_bytes, st) : gemm_dispatch_kmajor<0, true, false>(g, workspace_or_null, workspace_bytes, st);
     LLMQ_REQUIRE(mode == LLMQ_MODE_NT, "matmul: unknown operand mode %d (TT = 0, TN = 1, NT = 2, NN = 3)", mode);
-    return b_format ? gemm_dispatch_kmajor<1, true, true>(g, st) : gemm_dispatch_kmajor<0, true, true>(g, st);
+    return b_format ? gemm_dispatch_kmajor<1, true, true>(g, workspace_or_null, workspace_bytes, st) : gemm_dispatch_kmajor<0, true, true>(g, workspace_or_null, workspace_bytes, st);
 }
 
 extern "C" int llmq_gemm_tn_e4m3_bf16(uint16_t* c, const uint8_t* a, const uint8_t* b, const uint16_t* bias_or_null,

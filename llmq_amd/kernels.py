@@ -117,10 +117,15 @@ def matmul(c, a, b, bias, scale_a, scale_b, M, N, K, accumulate=False, stream=0,
     """TN matmul in the convention of the reference's kernels.h: row-major a[M,K], b[N,K] (e4m3) give
     row-major c[N,M] = (b @ a.T) * scale_a * scale_b (+ bias[M]) (+ c).  c: bf16 or fp32.
     workspace: optional device byte tensor (the reference passes a 32 MiB one); it enables the
-    split-K path for outputs with too few tiles to fill the chip.  b may hold e5m2 codes (the gradient
+    split-K path for outputs with too few tiles to fill the chip and the cut of a last, partial round of tiles into
+    K segments (all operand modes).  b may hold e5m2 codes (the gradient
     dtype option): a float8_e5m2 tensor, or uint8 with b_e5m2=True.  _lib: tests pass the test-aid build of
     the same entry points (capi.testaid()) to force a kernel variant; everyone else leaves it alone."""
     L = _lib or capi.lib
+    pws, ws_bytes = None, 0
+    if workspace is not None:
+        pws = _dev(workspace, "workspace", (torch.uint8, torch.int8, torch.float32))
+        ws_bytes = workspace.numel() * workspace.element_size()
     if b_kmajor or a_kmajor:
         # the reference's modes TT (b stored [K, N] row-major, e.g. the output gradient dY[BT, OC] as the second operand
         # of the weight gradient without its transposed copy), NN (a stored [K, M], e.g. the weight W[OC, C] as the
@@ -132,16 +137,12 @@ def matmul(c, a, b, bias, scale_a, scale_b, M, N, K, accumulate=False, stream=0,
         if a.numel() != M * K or b.numel() != N * K or c.numel() != N * M:
             raise ValueError("operand sizes do not match M, N, K")
         pbias = _dev(bias, "bias", (torch.bfloat16,), optional=True)
-        capi.check(capi.lib.llmq_gemm_e4m3_bf16_mode(
+        capi.check(L.llmq_gemm_e4m3_bf16_mode(
             _dev(c, "c", (torch.bfloat16,)), pa, pb, pbias, _dev(scale_a, "scale_a", (torch.float32,), optional=True),
-            _dev(scale_b, "scale_b", (torch.float32,), optional=True), None, 0, M, N, K,
+            _dev(scale_b, "scale_b", (torch.float32,), optional=True), pws, ws_bytes, M, N, K,
             (2 if b_kmajor else 3) if a_kmajor else 0,      # EMMTranspose: TT = 0, TN = 1, NT = 2, NN = 3
-            int(bool(b_e5m2) or b.dtype == torch.float8_e5m2), int(accumulate), _stream(stream)))
+            int(bool(b_e5m2) or b.dtype == torch.float8_e5m2), int(accumulate), _stream(stream)), L)
         return
-    pws, ws_bytes = None, 0
-    if workspace is not None:
-        pws = _dev(workspace, "workspace", (torch.uint8, torch.int8, torch.float32))
-        ws_bytes = workspace.numel() * workspace.element_size()
     pa = _dev(a, "a", (torch.float8_e4m3fn, torch.uint8))   # e5m2 is supported for b only (kernels.h:92-94)
     pb = _dev(b, "b", (torch.float8_e4m3fn, torch.float8_e5m2, torch.uint8))
     b_e5m2 = bool(b_e5m2) or b.dtype == torch.float8_e5m2

@@ -64,18 +64,21 @@ int main(int argc, char** argv) {
     const int BT = argc > 1 ? std::atoi(argv[1]) : 1024, C = argc > 2 ? std::atoi(argv[2]) : 896, OC = argc > 3 ? std::atoi(argv[3]) : 1152;
     const bool reuse_inp = argc > 4 && std::atoi(argv[4]) != 0;
     const bool fuse = argc > 5 && std::atoi(argv[5]) != 0;   // gradient quantize + transpose from one read
-    // 1: bf16 weight gradient; 2: also ask for operands in their stored layouts (matmul modes NN / TT / NT)
+    // 1: bf16 weight gradient; 2: also ask for operands in their stored layouts (matmul modes NN / TT / NT) where the
+    // plan expects them to pay; 3: wherever the shapes are served
     const int dw_mode = argc > 6 ? std::atoi(argv[6]) : 0;
-    const bool dw_bf16 = dw_mode >= 1, direct = dw_mode == 2;
+    const bool dw_bf16 = dw_mode >= 1, direct = dw_mode >= 2, wherever = dw_mode == 3;
     const int B = 1, T = BT;
-    std::printf("qmm_harness BT=%d C=%d OC=%d reuse_inp=%d fuse=%d dweight=%s direct_grad_layout=%d\n", BT, C, OC, (int)reuse_inp,
-                (int)fuse, dw_bf16 ? "bf16" : "fp32", (int)direct);
+    std::printf("qmm_harness BT=%d C=%d OC=%d reuse_inp=%d fuse=%d dweight=%s direct_grad_layout=%d wherever_served=%d\n", BT, C, OC,
+                (int)reuse_inp, (int)fuse, dw_bf16 ? "bf16" : "fp32", (int)direct, (int)wherever);
     hipStream_t stream; HIP_OK(hipStreamCreate(&stream));
     QmmRunState rs; HIP_OK(hipGetDeviceProperties(&rs.DeviceProp, 0));
     rs.FuseGradTranspose = fuse;
     rs.DirectGradLayout = direct;
+    rs.DirectGradLayoutWhereverServed = wherever;
     const QmmRunState::DirectPlan plan =
-        direct ? QmmRunState::direct_layout_plan(B, T, C, OC, ETensorDType::BF16, dw_bf16 ? ETensorDType::BF16 : ETensorDType::FP32, false)
+        direct ? QmmRunState::direct_layout_plan(B, T, C, OC, ETensorDType::BF16, dw_bf16 ? ETensorDType::BF16 : ETensorDType::FP32, false,
+                                                 wherever)
                : QmmRunState::DirectPlan{};
     std::printf("stored-layout plan: dgrad in place %d, wgrad %s\n", (int)plan.DgradInPlace,
                 plan.Wgrad == QmmRunState::EWgrad::Copies ? "copies" : plan.Wgrad == QmmRunState::EWgrad::GradInPlace ? "gradient in place (TT)"

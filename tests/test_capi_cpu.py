@@ -137,3 +137,15 @@ def test_reference_python_ops_register_without_a_gpu():
     assert ops.MODE_NT == 2 and ops.create_cublas_handle() == 0
     with pytest.raises(ValueError):                      # host tensors are rejected before any launch
         ops.abs_max(torch.zeros(1), torch.zeros(8, dtype=torch.bfloat16))
+
+
+def test_stored_layout_plan_and_stack_of_backward_qmm():
+    """Host logic of the C++ glue (tests/cpp/plan_check.cpp): which backward matmuls read their operands where
+    they lie (QmmRunState::direct_layout_plan) on layers of the Qwen2.5 sizes, and the stack backward_qmm then needs."""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp", "build", "plan_check")
+    assert os.path.exists(exe), "build it with `make -C tests/cpp` (done by __graft_entry__.build())"
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=60)
+    print(r.stdout[-2000:], r.stderr[-1000:])
+    assert r.returncode == 0 and "RESULT: PASS" in r.stdout

@@ -13,15 +13,30 @@ BIN = os.path.join(HERE, "cpp", "build", "qmm_harness")
 @pytest.mark.parametrize("args", [("1024", "896", "1152", "0"), ("2048", "896", "896", "1"), ("512", "4864", "896", "0"),
                                   ("4096", "1536", "1792", "0"), ("1024", "896", "1152", "0", "1"),
                                   ("2048", "1152", "896", "1", "1"),
-                                  # bf16 weight gradient; then the same layers with operands read in their stored
-                                  # layouts: dgrad NN + wgrad NT (all dimensions on 256-tiles, OC <= 8192), dgrad NN +
-                                  # wgrad TT (OC = 9216), wgrad TT on 224-wide tiles with the copying dgrad (C = 896),
-                                  # a shape no K-major mode serves (OC = 1152), NT with the quantized input reused
+                                  # bf16 weight gradient; then layers with operands read in their stored layouts, "2"
+                                  # where the plan expects a gain, "3" wherever the shapes are served: wgrad NT with
+                                  # the copying dgrad; dgrad NN + wgrad NT; wgrad TT (OC = 9216) with the copying dgrad;
+                                  # the same layer with NN + NT; wgrad TT on 224-wide tiles (C = 896); a shape no
+                                  # K-major mode serves (OC = 1152); NN + NT with the quantized input reused
                                   ("1024", "1024", "1536", "0", "0", "1"), ("1024", "1024", "1536", "0", "0", "2"),
-                                  ("1024", "768", "9216", "0", "0", "2"), ("2048", "896", "768", "1", "0", "2"),
-                                  ("1024", "896", "1152", "0", "1", "2"), ("512", "1536", "512", "1", "1", "2")])
+                                  ("1024", "1024", "1536", "0", "0", "3"), ("1024", "768", "9216", "0", "0", "2"),
+                                  ("1024", "768", "9216", "0", "0", "3"), ("2048", "896", "768", "1", "0", "2"),
+                                  ("1024", "896", "1152", "0", "1", "2"), ("512", "1536", "512", "1", "1", "3")])
 def test_qmm_harness(args):
     assert os.path.exists(BIN), "build it with `make -C tests/cpp` (done by __graft_entry__.build())"
     r = subprocess.run([BIN, *args], capture_output=True, text=True, timeout=150)
     print(r.stdout[-3000:], r.stderr[-2000:])
     assert r.returncode == 0 and "RESULT: PASS" in r.stdout
+    plan = PLANS.get(args)
+    if plan is not None:
+        assert "stored-layout plan: " + plan in r.stdout
+
+
+# what QmmRunState::direct_layout_plan must have chosen for the stored-layout cases above
+PLANS = {("1024", "1024", "1536", "0", "0", "2"): "dgrad in place 0, wgrad both in place (NT)",
+         ("1024", "1024", "1536", "0", "0", "3"): "dgrad in place 1, wgrad both in place (NT)",
+         ("1024", "768", "9216", "0", "0", "2"): "dgrad in place 0, wgrad gradient in place (TT)",
+         ("1024", "768", "9216", "0", "0", "3"): "dgrad in place 1, wgrad both in place (NT)",
+         ("2048", "896", "768", "1", "0", "2"): "dgrad in place 0, wgrad gradient in place (TT)",
+         ("1024", "896", "1152", "0", "1", "2"): "dgrad in place 0, wgrad copies",
+         ("512", "1536", "512", "1", "1", "3"): "dgrad in place 1, wgrad both in place (NT)"}

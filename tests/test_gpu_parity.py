@@ -722,6 +722,80 @@ def test_gemm_operands_in_k_major_layout(K, O, mnk, mode):
             assert torch.equal(again.view(torch.int16), c_km.view(torch.int16)), e5m2
 
 
+@pytest.mark.parametrize("mode", ["TT", "NN", "NT"])
+@pytest.mark.parametrize("cut", [0, 2, 4])
+@pytest.mark.parametrize("mnk", [(4352, 4352, 1024), (4608, 4096, 512), (4352, 4096, 1536), (8192, 4864, 512)])
+def test_gemm_k_major_last_round_cut(K, O, mnk, mode, cut):
+    """K-major operands with a workspace: the tiles left over after the full rounds are cut into K segments (a
+    second launch of the same operand mode writing raw fp32 tiles, summed in a fixed order by the reduction kernel),
+    as in mode TN.  cut = 2, 4: forced; 0: whatever the plan decides with the workspace given.  Integer operands ->
+    bit exact against the oracle, with bias and (mode TT) accumulation; random codes bit-identical to mode TN under
+    the same plan, and on repeated launches."""
+    M, N, Kd = mnk
+    variant = (3, cut)          # mode TN on the four-wave kernel as well: the same sums in the same order
+    skip_unsupported(variant, M, N, Kd)
+    a_km, b_km = mode[0] == "N", mode[1] == "T"
+    lay_a = (lambda x: np.ascontiguousarray(x.T)) if a_km else (lambda x: x)
+    lay_b = (lambda x: np.ascontiguousarray(x.T)) if b_km else (lambda x: x)
+    a, _ = O.fill_int_e4m3(M * Kd, 818, 0)
+    b, _ = O.fill_int_e4m3(N * Kd, 818, 1)
+    a, b = a.reshape(M, Kd), b.reshape(N, Kd)
+    s = float(np.sqrt(np.float32(4.0 / Kd)))
+    _, biasv = O.fill_int_e4m3(M, 818, 2)
+    _, oldv = O.fill_int_e4m3(N * M, 818, 3)
+    bias = O.f32_to_bf16(biasv.astype(np.float32))
+    old = O.f32_to_bf16(oldv.astype(np.float32)).reshape(N, M)
+    rng = np.random.default_rng(M + N + Kd)
+    ar = rng.integers(0, 256, (M, Kd)).astype(np.uint8)
+    br = rng.integers(0, 256, (N, Kd)).astype(np.uint8)
+    ar[(ar & 0x7F) == 0x7F] ^= 1
+    br[(br & 0x7F) == 0x7F] ^= 1
+    set_variant(variant)
+    try:
+        for use_bias, use_old in [(False, False), (True, False)] + ([] if a_km else [(True, True)]):
+            want = O.gemm_tn(a, b, sa=s, sb=s, bias=bias if use_bias else None, c_old=old if use_old else None, mt=True)
+            c = dev_bf16(old).reshape(N, M).clone() if use_old else torch.full((N, M), float("nan"), dtype=torch.bfloat16, device="cuda")
+            mm(K, c, dev_u8(lay_a(a)), dev_u8(lay_b(b)), dev_bf16(bias) if use_bias else None, dev_scalar(s), dev_scalar(s), M, N, Kd,
+               accumulate=use_old, a_kmajor=a_km, b_kmajor=b_km, workspace=workspace())
+            assert np.array_equal(host_bits(c), want), (use_bias, use_old)
+        c_tn = torch.empty((N, M), dtype=torch.bfloat16, device="cuda")
+        mm(K, c_tn, dev_u8(ar), dev_u8(br), None, dev_scalar(0.37), dev_scalar(1.0 / 448), M, N, Kd, workspace=workspace())
+        da, db = dev_u8(lay_a(ar)), dev_u8(lay_b(br))
+        for _ in range(4):
+            c_km = torch.full((N, M), float("nan"), dtype=torch.bfloat16, device="cuda")
+            mm(K, c_km, da, db, None, dev_scalar(0.37), dev_scalar(1.0 / 448), M, N, Kd, a_kmajor=a_km, b_kmajor=b_km,
+               workspace=workspace())
+            assert torch.equal(c_tn.view(torch.int16), c_km.view(torch.int16))
+    finally:
+        set_variant((0, 0))
+
+
+@pytest.mark.parametrize("mode", ["TT", "NN", "NT"])
+def test_gemm_k_major_automatic_cut_on_a_weight_gradient_shape(K, mode):
+    """18944 x 3584 x 8192 (the down projection's weight gradient of the headline layer): with a workspace the plan
+    cuts the one or two last-round tiles per XCD into K segments in every operand mode; the K-major modes must give
+    the bits of mode TN on the transposed copies (same plan, same sums in the same order), launch after launch."""
+    M, N, Kd = 18944, 3584, 8192
+    g = torch.Generator(device="cuda").manual_seed(5)
+    a = torch.randint(0, 0x7E, (M, Kd), dtype=torch.uint8, device="cuda", generator=g) | (torch.randint(0, 2, (M, Kd), dtype=torch.uint8, device="cuda", generator=g) << 7)
+    b = torch.randint(0, 0x7E, (N, Kd), dtype=torch.uint8, device="cuda", generator=g) | (torch.randint(0, 2, (N, Kd), dtype=torch.uint8, device="cuda", generator=g) << 7)
+    a_km, b_km = mode[0] == "N", mode[1] == "T"
+    da = a.t().contiguous() if a_km else a
+    db = b.t().contiguous() if b_km else b
+    sa = dev_scalar(2.0 ** -6)
+    c_tn = torch.empty((N, M), dtype=torch.bfloat16, device="cuda")
+    K.matmul(c_tn, a, b, None, sa, None, M, N, Kd, workspace=workspace())
+    c_whole = torch.empty((N, M), dtype=torch.bfloat16, device="cuda")
+    K.matmul(c_whole, da, db, None, sa, None, M, N, Kd, a_kmajor=a_km, b_kmajor=b_km)
+    for _ in range(4):
+        c_km = torch.full((N, M), float("nan"), dtype=torch.bfloat16, device="cuda")
+        K.matmul(c_km, da, db, None, sa, None, M, N, Kd, a_kmajor=a_km, b_kmajor=b_km, workspace=workspace())
+        assert torch.equal(c_tn.view(torch.int16), c_km.view(torch.int16))
+    # the cut changes the order of the sums in the cut tiles only: a few outputs differ from the uncut launch by an ulp
+    differing = (c_whole.view(torch.int16) != c_tn.view(torch.int16)).float().mean().item()
+    assert 0 < differing < 0.02, differing
+
+
 def test_gemm_k_major_operand_rejects_what_it_cannot_serve(K):
     a = torch.zeros((256, 384), dtype=torch.uint8, device="cuda")
     b = torch.zeros((384, 256), dtype=torch.uint8, device="cuda")
