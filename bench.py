@@ -378,6 +378,24 @@ def main():
         del g5
         swiglu["fused_residual_rmsnorm_forward+abs_max (8 B/el)"] = gbs(
             lambda: K.fused_residual_rmsnorm_forward(r_out, r_norm, r_rms, r_in, r_att, r_w, sw_am, 1e-6), 8 * BT * C, iters=10)
+        # the fp32 overloads of the same producers (an fp32 model in front of FP8 matmuls): twice the bytes per element
+        f_y = torch.randn((1, BT // 2, 2 * FFN), device=dev)
+        f_h, f_dh, f_dy = torch.empty((1, BT // 2, FFN), device=dev), torch.randn((1, BT // 2, FFN), device=dev), torch.empty_like(f_y)
+        n32 = (BT // 2) * FFN
+        swiglu["fp32 swiglu_forward+abs_max [4096 x 18944] (12 B/el)"] = gbs(lambda: K.swiglu_forward(f_h, f_y, sw_am), 12 * n32)
+        swiglu["fp32 swiglu_backward+abs_max [4096 x 18944] (20 B/el)"] = gbs(lambda: K.swiglu_backward(f_dy, f_dh, f_y, sw_am), 20 * n32)
+        del f_y, f_h, f_dh, f_dy
+        f_in, f_att = torch.randn((1, BT, C), device=dev), torch.randn((1, BT, C), device=dev)
+        f_out, f_norm, f_w, f_dw = torch.empty_like(f_in), torch.empty_like(f_in), torch.ones(C, device=dev), torch.zeros(C, device=dev)
+        swiglu["fp32 fused_residual_rmsnorm_forward+abs_max (16 B/el)"] = gbs(
+            lambda: K.fused_residual_rmsnorm_forward(f_out, f_norm, r_rms, f_in, f_att, f_w, sw_am, 1e-6), 16 * BT * C, iters=10)
+        swiglu["fp32 rmsnorm_backward+abs_max (16 B/el)"] = gbs(
+            lambda: K.rmsnorm_backward(f_out, f_dw, r_scr, f_att, f_norm, f_in, f_w, r_rstd, sw_am), 16 * BT * C, iters=10)
+        f_tab = K.precompute_freqs_cis(128, 2048, 1e6, dtype=torch.float32).to(dev)
+        f_qkv = torch.randn((BT // 2048, 2048, 4608), device=dev)
+        swiglu["fp32 rope_forward+abs_max in place [8192 x 4608] (q, k heads 8 B/el, v heads 4)"] = gbs(
+            lambda: K.rope_forward(f_qkv, f_qkv, f_tab, sw_am, 28, 4), BT * 128 * (32 * 8 + 4 * 4), iters=10)
+        del f_in, f_att, f_out, f_norm, f_qkv
     # The HBM-bound kernels on their own, cold: 5 warm-up and 20 timed launches each, one pair of events per
     # launch, rotating through three distinct 310 MB tensors (930 MB, well beyond the 256 MB last-level cache,
     # so every launch reads from HBM); median and best launch.  The in-step figures above include what the

@@ -321,6 +321,34 @@ int llmq_rope_backward_bf16(uint16_t* dinp, const uint16_t* dout, const uint16_t
 int llmq_precompute_freqs_cis_f16(uint16_t* freqs_cis_host, int dim, int end, float theta);
 
 /*
+ * fp32 overloads of the producers above (a model kept in fp32 whose matmuls run in FP8): the same arithmetic without the
+ * roundings to bf16, fp32 tensors throughout; abs_max_or_null as above, bit-identical to llmq_abs_max_f32 of the tensor
+ * written.  C must be a multiple of 4 (RMSNorm: at most 8192), head_dim a multiple of 8; the rope table is fp32
+ * [T, head_dim] of (cos, sin) pairs.  In fp32 RMSNorm the normalised value s * x is the fp32 product itself.
+ * Replace the float overloads: swiglu_forward / swiglu_backward  src/kernels/kernels.h:157,164 (src/kernels/swiglu.cu:
+ *           304-346,374-401; tested by src/testing/test-swiglu.cu:83-156), rope_forward / rope_backward and
+ *           precompute_freqs_cis  kernels.h:110,112,115 (src/kernels/rope.cu:15-40,129-163; src/testing/test-rope.cu:88-183,
+ *           303-345), rmsnorm_forward  kernels.h:45, rmsnorm_backward  kernels.h:50-51, fused_residual_rmsnorm_forward
+ *           kernels.h:57-58 (src/kernels/rmsnorm.cu:183-227,447-470).
+ */
+int llmq_swiglu_forward_f32(float* out, const float* inp, float* abs_max_or_null, int B, int T, int C, void* stream);
+int llmq_swiglu_backward_f32(float* dinp, const float* dout, const float* inp, float* abs_max_or_null, int B, int T, int C,
+                             void* stream);
+int llmq_rope_forward_f32(float* out, const float* inp, const float* freqs_cis_f32, float* abs_max_or_null, int B, int T,
+                          int Nq, int Nkv, int head_dim, void* stream);
+int llmq_rope_backward_f32(float* dinp, const float* dout, const float* freqs_cis_f32, float* abs_max_or_null, int B, int T,
+                           int Nq, int Nkv, int head_dim, void* stream);
+int llmq_precompute_freqs_cis_f32(float* freqs_cis_host, int dim, int end, float theta);
+int llmq_rmsnorm_forward_f32(float* out, float* rms_or_null, const float* inp, const float* weight, float* abs_max_or_null,
+                             float epsilon, int B, int T, int C, void* stream);
+int llmq_fused_residual_rmsnorm_forward_f32(float* residual, float* normed, float* rrms, const float* inp1, const float* inp2,
+                                            const float* weight, float* abs_max_or_null, float epsilon, int N, int C,
+                                            void* stream);
+int llmq_rmsnorm_backward_f32(float* dinp, float* dweight, void* scratch, size_t scratch_bytes, const float* dresidual,
+                              const float* dout, const float* inp, const float* weight, const float* rstd,
+                              float* abs_max_or_null, int B, int T, int C, void* stream);
+
+/*
  * AdamW update of bf16 parameters from bf16 gradients, moments in fp32 or bf16 (m_dtype / v_dtype: 0 = fp32, 1 = bf16;
  * supported pairs (m, v): (0, 0), (1, 0), (1, 1)), per element:
  *     grad = *grad_scale * g;  m = fma(beta1, m, fma(-beta1, grad, grad));  v = fma(beta2, v, fma(-beta2, grad^2, grad^2))

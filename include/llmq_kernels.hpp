@@ -378,12 +378,18 @@ inline void backward_bias(Tensor& dbias, const Tensor& dout, const float* scale_
 }
 
 // ---- swiglu (reference: src/kernels/kernels.h:155-165, src/kernels/swiglu.cu) --------------------------------
-// inp[B, T, 2C] rows are [up | gate]; bf16 only (the fp32 overloads of the reference belong to its fp32 models).
+// inp[B, T, 2C] rows are [up | gate]; bf16 tensors, or fp32 throughout (the quantizing variant: bf16 input only, as in
+// the reference).
 inline void swiglu_forward(__hip_bfloat16* out, const __hip_bfloat16* inp, float* abs_max_ptr, int B, int T, int C,
                            hipStream_t stream) {
     llmq_detail::check(llmq_swiglu_forward_bf16(llmq_detail::u16(out), llmq_detail::u16(inp), abs_max_ptr, B, T, C, stream));
 }
+inline void swiglu_forward(float* out, const float* inp, float* abs_max_ptr, int B, int T, int C, hipStream_t stream) {
+    llmq_detail::check(llmq_swiglu_forward_f32(out, inp, abs_max_ptr, B, T, C, stream));
+}
 inline void swiglu_forward(Tensor& out, const Tensor& inp, float* abs_max_ptr, int B, int T, int C, hipStream_t stream) {
+    if (out.DType == ETensorDType::FP32 && inp.DType == ETensorDType::FP32)
+        return swiglu_forward(out.get<float>(), inp.get<float>(), abs_max_ptr, B, T, C, stream);
     if (out.DType != ETensorDType::BF16 || inp.DType != ETensorDType::BF16) llmq_detail::unsupported(__func__, out, inp);
     swiglu_forward(out.get<__hip_bfloat16>(), inp.get<__hip_bfloat16>(), abs_max_ptr, B, T, C, stream);
 }
@@ -402,8 +408,14 @@ inline void swiglu_backward(__hip_bfloat16* dinp, const __hip_bfloat16* dout, co
     llmq_detail::check(llmq_swiglu_backward_bf16(llmq_detail::u16(dinp), llmq_detail::u16(dout), llmq_detail::u16(inp),
                                                  abs_max, B, T, C, stream));
 }
+inline void swiglu_backward(float* dinp, const float* dout, const float* inp, float* abs_max, int B, int T, int C,
+                            hipStream_t stream) {
+    llmq_detail::check(llmq_swiglu_backward_f32(dinp, dout, inp, abs_max, B, T, C, stream));
+}
 inline void swiglu_backward(Tensor& dinp, const Tensor& dout, const Tensor& inp, float* abs_max, int B, int T, int C,
                             hipStream_t stream) {
+    if (dinp.DType == ETensorDType::FP32 && dout.DType == ETensorDType::FP32 && inp.DType == ETensorDType::FP32)
+        return swiglu_backward(dinp.get<float>(), dout.get<float>(), inp.get<float>(), abs_max, B, T, C, stream);
     if (dinp.DType != ETensorDType::BF16 || dout.DType != ETensorDType::BF16 || inp.DType != ETensorDType::BF16)
         llmq_detail::unsupported(__func__, dinp, dout, inp);
     swiglu_backward(dinp.get<__hip_bfloat16>(), dout.get<__hip_bfloat16>(), inp.get<__hip_bfloat16>(), abs_max, B, T, C,
@@ -416,8 +428,16 @@ inline void rmsnorm_forward(__hip_bfloat16* out, float* rms, const __hip_bfloat1
     llmq_detail::check(llmq_rmsnorm_forward_bf16(llmq_detail::u16(out), rms, llmq_detail::u16(inp), llmq_detail::u16(weight),
                                                  abs_max_ptr, epsilon, B, T, C, stream));
 }
+inline void rmsnorm_forward(float* out, float* rms, const float* inp, const float* weight, float* abs_max_ptr, float epsilon,
+                            int B, int T, int C, hipStream_t stream) {
+    llmq_detail::check(llmq_rmsnorm_forward_f32(out, rms, inp, weight, abs_max_ptr, epsilon, B, T, C, stream));
+}
 inline void rmsnorm_forward(Tensor& out, Tensor& rms, const Tensor& inp, const Tensor& weight, float* abs_max_ptr,
                             float epsilon, int B, int T, int C, hipStream_t stream) {
+    if (out.DType == ETensorDType::FP32 && inp.DType == ETensorDType::FP32 && weight.DType == ETensorDType::FP32 &&
+        rms.DType == ETensorDType::FP32)
+        return rmsnorm_forward(out.get<float>(), rms.get<float>(), inp.get<float>(), weight.get<float>(), abs_max_ptr, epsilon,
+                               B, T, C, stream);
     if (out.DType != ETensorDType::BF16 || inp.DType != ETensorDType::BF16 || weight.DType != ETensorDType::BF16 ||
         rms.DType != ETensorDType::FP32)
         llmq_detail::unsupported(__func__, out, rms, inp, weight);
@@ -432,9 +452,19 @@ inline void fused_residual_rmsnorm_forward(__hip_bfloat16* residual, __hip_bfloa
                                                                 llmq_detail::u16(inp1), llmq_detail::u16(inp2),
                                                                 llmq_detail::u16(weight), abs_max_ptr, epsilon, N, C, stream));
 }
+inline void fused_residual_rmsnorm_forward(float* residual, float* normed, float* rrms, const float* inp1, const float* inp2,
+                                           const float* weight, float* abs_max_ptr, float epsilon, int N, int C,
+                                           hipStream_t stream) {
+    llmq_detail::check(llmq_fused_residual_rmsnorm_forward_f32(residual, normed, rrms, inp1, inp2, weight, abs_max_ptr, epsilon,
+                                                               N, C, stream));
+}
 inline void fused_residual_rmsnorm_forward(Tensor& residual, Tensor& normed, Tensor& rrms, const Tensor& inp1,
                                            const Tensor& inp2, const Tensor& weight, float* abs_max_ptr, float epsilon,
                                            int N, int C, hipStream_t stream) {
+    if (residual.DType == ETensorDType::FP32 && normed.DType == ETensorDType::FP32 && inp1.DType == ETensorDType::FP32 &&
+        inp2.DType == ETensorDType::FP32 && weight.DType == ETensorDType::FP32 && rrms.DType == ETensorDType::FP32)
+        return fused_residual_rmsnorm_forward(residual.get<float>(), normed.get<float>(), rrms.get<float>(), inp1.get<float>(),
+                                              inp2.get<float>(), weight.get<float>(), abs_max_ptr, epsilon, N, C, stream);
     if (residual.DType != ETensorDType::BF16 || normed.DType != ETensorDType::BF16 || inp1.DType != ETensorDType::BF16 ||
         inp2.DType != ETensorDType::BF16 || weight.DType != ETensorDType::BF16 || rrms.DType != ETensorDType::FP32)
         llmq_detail::unsupported(__func__, residual, normed, rrms, inp1, inp2, weight);
@@ -454,9 +484,25 @@ inline void rmsnorm_backward(__hip_bfloat16* dinp, __hip_bfloat16* dweight, std:
                                                   llmq_detail::u16(dresidual), llmq_detail::u16(dout), llmq_detail::u16(inp),
                                                   llmq_detail::u16(weight), rstd, abs_max_ptr, B, T, C, stream));
 }
+inline void rmsnorm_backward(float* dinp, float* dweight, std::byte* scratch, const float* dresidual, const float* dout,
+                             const float* inp, const float* weight, const float* rstd, float* abs_max_ptr, int B, int T, int C,
+                             const hipDeviceProp_t& dp, hipStream_t stream) {
+    llmq_detail::check(llmq_rmsnorm_backward_f32(dinp, dweight, scratch, (std::size_t)get_rmsnorm_backward_scratch_size(C, dp),
+                                                 dresidual, dout, inp, weight, rstd, abs_max_ptr, B, T, C, stream));
+}
 inline void rmsnorm_backward(Tensor& dinp, Tensor& dweight, Tensor& scratch, const Tensor& dresidual, const Tensor& dout,
                              const Tensor& inp, const Tensor& weight, const Tensor& rstd, float* abs_max_ptr, int B, int T,
                              int C, const hipDeviceProp_t& dp, hipStream_t stream) {
+    if (dinp.DType == ETensorDType::FP32 && dweight.DType == ETensorDType::FP32 && dresidual.DType == ETensorDType::FP32 &&
+        dout.DType == ETensorDType::FP32 && inp.DType == ETensorDType::FP32 && weight.DType == ETensorDType::FP32 &&
+        rstd.DType == ETensorDType::FP32) {
+        if (scratch.bytes() < (std::size_t)get_rmsnorm_backward_scratch_size(C, dp))
+            throw std::invalid_argument("rmsnorm_backward: scratch buffer too small");
+        llmq_detail::check(llmq_rmsnorm_backward_f32(dinp.get<float>(), dweight.get<float>(), scratch.Data, scratch.bytes(),
+                                                     dresidual.get<float>(), dout.get<float>(), inp.get<float>(),
+                                                     weight.get<float>(), rstd.get<float>(), abs_max_ptr, B, T, C, stream));
+        return;
+    }
     if (dinp.DType != ETensorDType::BF16 || dweight.DType != ETensorDType::BF16 || dresidual.DType != ETensorDType::BF16 ||
         dout.DType != ETensorDType::BF16 || inp.DType != ETensorDType::BF16 || weight.DType != ETensorDType::BF16 ||
         rstd.DType != ETensorDType::FP32)
@@ -487,6 +533,37 @@ inline void rope_backward(__hip_bfloat16* dinp, const __hip_bfloat16* dout, cons
     llmq_detail::check(llmq_rope_backward_bf16(llmq_detail::u16(dinp), llmq_detail::u16(dout),
                                                reinterpret_cast<const std::uint16_t*>(freqs_cis), abs_max_ptr, B, T, Nq, Nkv,
                                                head_dim, stream));
+}
+
+inline void precompute_freqs_cis(float* freqs_cis, int dim, int end, float theta) {
+    llmq_detail::check(llmq_precompute_freqs_cis_f32(freqs_cis, dim, end, theta));
+}
+inline void rope_forward(float* out, const float* in, const float* freqs_cis, float* abs_max_ptr, int B, int T, int Nq, int Nkv,
+                         int head_dim, hipStream_t stream) {
+    llmq_detail::check(llmq_rope_forward_f32(out, in, freqs_cis, abs_max_ptr, B, T, Nq, Nkv, head_dim, stream));
+}
+inline void rope_backward(float* dinp, const float* dout, const float* freqs_cis, float* abs_max_ptr, int B, int T, int Nq,
+                          int Nkv, int head_dim, hipStream_t stream) {
+    llmq_detail::check(llmq_rope_backward_f32(dinp, dout, freqs_cis, abs_max_ptr, B, T, Nq, Nkv, head_dim, stream));
+}
+inline void rope_forward(Tensor& out, const Tensor& in, const Tensor& freqs_cis, float* abs_max_ptr, int B, int T, int Nq,
+                         int Nkv, int head_dim, hipStream_t stream) {
+    if (out.DType == ETensorDType::FP32 && in.DType == ETensorDType::FP32 && freqs_cis.DType == ETensorDType::FP32)
+        return rope_forward(out.get<float>(), in.get<float>(), freqs_cis.get<float>(), abs_max_ptr, B, T, Nq, Nkv, head_dim, stream);
+    if (out.DType != ETensorDType::BF16 || in.DType != ETensorDType::BF16 || freqs_cis.DType != ETensorDType::FP16)
+        llmq_detail::unsupported(__func__, out, in, freqs_cis);
+    rope_forward(out.get<__hip_bfloat16>(), in.get<__hip_bfloat16>(), freqs_cis.get<__half>(), abs_max_ptr, B, T, Nq, Nkv,
+                 head_dim, stream);
+}
+inline void rope_backward(Tensor& dinp, const Tensor& dout, const Tensor& freqs_cis, float* abs_max_ptr, int B, int T, int Nq,
+                          int Nkv, int head_dim, hipStream_t stream) {
+    if (dinp.DType == ETensorDType::FP32 && dout.DType == ETensorDType::FP32 && freqs_cis.DType == ETensorDType::FP32)
+        return rope_backward(dinp.get<float>(), dout.get<float>(), freqs_cis.get<float>(), abs_max_ptr, B, T, Nq, Nkv, head_dim,
+                             stream);
+    if (dinp.DType != ETensorDType::BF16 || dout.DType != ETensorDType::BF16 || freqs_cis.DType != ETensorDType::FP16)
+        llmq_detail::unsupported(__func__, dinp, dout, freqs_cis);
+    rope_backward(dinp.get<__hip_bfloat16>(), dout.get<__hip_bfloat16>(), freqs_cis.get<__half>(), abs_max_ptr, B, T, Nq, Nkv,
+                  head_dim, stream);
 }
 
 // ---- adamw (reference: src/kernels/kernels.h:225-235, src/kernels/adamw.cu) ----------------------------------------

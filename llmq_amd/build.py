@@ -20,7 +20,7 @@ LIB = os.path.join(HERE, "lib", "libllmq_fp8.so")
 TESTAID_LIB = os.path.join(HERE, "lib", "libllmq_fp8_testaid.so")
 
 SOURCES = ["runtime.hip", "absmax.hip", "quantize.hip", "transpose.hip", "gemm_e4m3.hip", "bias.hip", "swiglu.hip",
-           "rmsnorm.hip", "rope.hip", "adamw.hip"]
+           "rmsnorm.hip", "rope.hip", "adamw.hip", "producers_f32.hip"]
 # (source, object name, extra flags)
 TESTAID_UNITS = [("gemm_e4m3.hip", "gemm_e4m3_hooks.o", ["-DLLMQ_TEST_HOOKS"]), ("calibrate.hip", "calibrate.o", []),
                  ("runtime.hip", "runtime.o", [])]

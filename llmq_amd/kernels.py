@@ -196,6 +196,17 @@ def backward_bias(dbias, dout, scale_a, scale_b, dbias_buffer, stream=0):
                                                 BT, OC, _stream(stream)))
 
 
+_PRODUCER_DTYPES = (torch.bfloat16, torch.float32)
+
+
+def _producer_entry(name, t):
+    """The C entry point of producer `name` for tensors of t's dtype (bf16, or the fp32 overload) and that dtype as
+    the one every tensor of the call must have."""
+    if t.dtype not in _PRODUCER_DTYPES:
+        raise ValueError("%s: tensors must be bfloat16 or float32 (got %s)" % (name, t.dtype))
+    return getattr(capi.lib, "llmq_%s_%s" % (name, "f32" if t.dtype == torch.float32 else "bf16")), (t.dtype,)
+
+
 def _swiglu_dims(inp, other, name):
     """inp: [B, T, 2C]; other: [B, T, C] (reference: src/binding/kernel_binding.cpp:289-322)."""
     if inp.dim() != 3 or other.dim() != 3:
@@ -206,13 +217,14 @@ def _swiglu_dims(inp, other, name):
 
 
 def swiglu_forward(out, inp, abs_max, stream=0):
-    """out[B,T,C] = up * gate * sigmoid(gate) for inp[B,T,2C] = [up | gate] (bf16); abs_max (fp32 device scalar
-    or None) receives max |out|."""
+    """out[B,T,C] = up * gate * sigmoid(gate) for inp[B,T,2C] = [up | gate] (bf16, or fp32 throughout); abs_max (fp32
+    device scalar or None) receives max |out|."""
     B, T, Cc = _swiglu_dims(inp, out, "out")
-    o = _dev(out, "out", (torch.bfloat16,))
-    i = _dev(inp, "inp", (torch.bfloat16,))
+    fn, dt = _producer_entry("swiglu_forward", inp)
+    o = _dev(out, "out", dt)
+    i = _dev(inp, "inp", dt)
     a = _dev(abs_max, "abs_max", (torch.float32,), optional=True)
-    capi.check(capi.lib.llmq_swiglu_forward_bf16(o, i, a, B, T, Cc, _stream(stream)))
+    capi.check(fn(o, i, a, B, T, Cc, _stream(stream)))
 
 
 def swiglu_forward_quant(out, scale, inp, abs_max, stream=0):
@@ -231,27 +243,30 @@ def swiglu_backward(dinp, dout, inp, abs_max, stream=0):
     B, T, Cc = _swiglu_dims(inp, dout, "dout")
     if dinp.shape != inp.shape:
         raise ValueError("dinp must have the shape of inp")
-    d = _dev(dinp, "dinp", (torch.bfloat16,))
-    g = _dev(dout, "dout", (torch.bfloat16,))
-    i = _dev(inp, "inp", (torch.bfloat16,))
+    fn, dt = _producer_entry("swiglu_backward", inp)
+    d = _dev(dinp, "dinp", dt)
+    g = _dev(dout, "dout", dt)
+    i = _dev(inp, "inp", dt)
     a = _dev(abs_max, "abs_max", (torch.float32,), optional=True)
-    capi.check(capi.lib.llmq_swiglu_backward_bf16(d, g, i, a, B, T, Cc, _stream(stream)))
+    capi.check(fn(d, g, i, a, B, T, Cc, _stream(stream)))
 
 
 def rmsnorm_forward(out, rms, inp, weight, abs_max, epsilon, stream=0):
     """out[B,T,C] = bf16(bf16(inp / rms(inp)) * weight), rms[B,T] = 1/sqrt(mean(inp^2) + epsilon); abs_max (fp32
-    device scalar or None) receives max |out| (reference: src/binding/kernel_binding.cpp:130-143)."""
+    device scalar or None) receives max |out| (reference: src/binding/kernel_binding.cpp:130-143).  fp32 tensors
+    throughout take the fp32 overload (no intermediate rounding)."""
     if inp.dim() != 3 or out.shape != inp.shape or weight.dim() != 1 or weight.shape[0] != inp.shape[2]:
         raise ValueError("inp and out must be [B, T, C] and weight [C]")
     if rms is not None and (rms.dim() != 2 or rms.shape[0] != inp.shape[0] or rms.shape[1] != inp.shape[1]):
         raise ValueError("rms must be [B, T]")
-    o = _dev(out, "out", (torch.bfloat16,))
+    fn, dt = _producer_entry("rmsnorm_forward", inp)
+    o = _dev(out, "out", dt)
     r = _dev(rms, "rms", (torch.float32,), optional=True)
-    i = _dev(inp, "inp", (torch.bfloat16,))
-    w = _dev(weight, "weight", (torch.bfloat16,))
+    i = _dev(inp, "inp", dt)
+    w = _dev(weight, "weight", dt)
     a = _dev(abs_max, "abs_max", (torch.float32,), optional=True)
     B, T, Cc = (int(v) for v in inp.shape)
-    capi.check(capi.lib.llmq_rmsnorm_forward_bf16(o, r, i, w, a, float(epsilon), B, T, Cc, _stream(stream)))
+    capi.check(fn(o, r, i, w, a, float(epsilon), B, T, Cc, _stream(stream)))
 
 
 def fused_residual_rmsnorm_forward(residual, normed, rrms, inp1, inp2, weight, abs_max, epsilon, stream=0):
@@ -262,13 +277,13 @@ def fused_residual_rmsnorm_forward(residual, normed, rrms, inp1, inp2, weight, a
         raise ValueError("inp1, inp2, residual and normed must be [B, T, C] and weight [C]")
     if rrms.dim() != 2 or rrms.shape[0] != inp1.shape[0] or rrms.shape[1] != inp1.shape[1]:
         raise ValueError("rrms must be [B, T]")
-    ptrs = [_dev(t, n, (torch.bfloat16,)) for t, n in ((residual, "residual"), (normed, "normed"))]
+    fn, dt = _producer_entry("fused_residual_rmsnorm_forward", inp1)
+    ptrs = [_dev(t, n, dt) for t, n in ((residual, "residual"), (normed, "normed"))]
     r = _dev(rrms, "rrms", (torch.float32,))
-    ins = [_dev(t, n, (torch.bfloat16,)) for t, n in ((inp1, "inp1"), (inp2, "inp2"), (weight, "weight"))]
+    ins = [_dev(t, n, dt) for t, n in ((inp1, "inp1"), (inp2, "inp2"), (weight, "weight"))]
     a = _dev(abs_max, "abs_max", (torch.float32,), optional=True)
     N, Cc = int(inp1.shape[0] * inp1.shape[1]), int(inp1.shape[2])
-    capi.check(capi.lib.llmq_fused_residual_rmsnorm_forward_bf16(ptrs[0], ptrs[1], r, ins[0], ins[1], ins[2], a,
-                                                                 float(epsilon), N, Cc, _stream(stream)))
+    capi.check(fn(ptrs[0], ptrs[1], r, ins[0], ins[1], ins[2], a, float(epsilon), N, Cc, _stream(stream)))
 
 
 def get_rmsnorm_backward_scratch_size(C):
@@ -286,45 +301,51 @@ def rmsnorm_backward(dinp, dweight, scratch, dresidual, dout, inp, weight, rstd,
         raise ValueError("dinp, dresidual, dout and inp must be [B, T, C], weight and dweight [C]")
     if rstd.dim() != 2 or rstd.shape[0] != inp.shape[0] or rstd.shape[1] != inp.shape[1]:
         raise ValueError("rstd must be [B, T]")
-    bf = (torch.bfloat16,)
+    fn, bf = _producer_entry("rmsnorm_backward", inp)
     p = [_dev(t, n, bf) for t, n in ((dinp, "dinp"), (dweight, "dweight"))]
     sc = _dev(scratch, "scratch")
     q = [_dev(t, n, bf) for t, n in ((dresidual, "dresidual"), (dout, "dout"), (inp, "inp"), (weight, "weight"))]
     r = _dev(rstd, "rstd", (torch.float32,))
     a = _dev(abs_max, "abs_max", (torch.float32,), optional=True)
     B, T, Cc = (int(v) for v in inp.shape)
-    capi.check(capi.lib.llmq_rmsnorm_backward_bf16(p[0], p[1], sc, scratch.numel() * scratch.element_size(), q[0], q[1],
-                                                   q[2], q[3], r, a, B, T, Cc, _stream(stream)))
+    capi.check(fn(p[0], p[1], sc, scratch.numel() * scratch.element_size(), q[0], q[1], q[2], q[3], r, a, B, T, Cc,
+                  _stream(stream)))
 
 
-def _rope(fn, out, inp, freqs_cis, abs_max, Nq, Nkv, stream):
-    """Tensors [B, T, (Nq + 2 Nkv) * HD] bf16 (reference: src/binding/kernel_binding.cpp:193-223); freqs_cis [T, HD] fp16."""
+def _rope(name, out, inp, freqs_cis, abs_max, Nq, Nkv, stream):
+    """Tensors [B, T, (Nq + 2 Nkv) * HD] bf16 with freqs_cis [T, HD] fp16, or fp32 with an fp32 table (reference:
+    src/binding/kernel_binding.cpp:193-223)."""
     if inp.dim() != 3 or out.shape != inp.shape or freqs_cis.dim() != 2 or freqs_cis.shape[0] < inp.shape[1]:
         raise ValueError("inp and out must be [B, T, C] and freqs_cis [>= T, HD]")
     HD = int(freqs_cis.shape[1])
     if HD == 0 or inp.shape[2] != (Nq + 2 * Nkv) * HD:
         raise ValueError("C must equal (Nq + 2 Nkv) * head_dim")
-    o = _dev(out, "out", (torch.bfloat16,))
-    i = _dev(inp, "inp", (torch.bfloat16,))
-    f = _dev(freqs_cis, "freqs_cis", (torch.float16,))
+    fn, dt = _producer_entry(name, inp)
+    o = _dev(out, "out", dt)
+    i = _dev(inp, "inp", dt)
+    f = _dev(freqs_cis, "freqs_cis", (torch.float32 if inp.dtype == torch.float32 else torch.float16,))
     a = _dev(abs_max, "abs_max", (torch.float32,), optional=True)
     capi.check(fn(o, i, f, a, int(inp.shape[0]), int(inp.shape[1]), int(Nq), int(Nkv), HD, _stream(stream)))
 
 
 def rope_forward(out, inp, freqs_cis, abs_max, Nq, Nkv, stream=0):
     """Rotary embedding of the query and key heads of the fused QKV tensor (out may be inp); abs_max receives max |out|."""
-    _rope(capi.lib.llmq_rope_forward_bf16, out, inp, freqs_cis, abs_max, Nq, Nkv, stream)
+    _rope("rope_forward", out, inp, freqs_cis, abs_max, Nq, Nkv, stream)
 
 
 def rope_backward(dinp, dout, freqs_cis, abs_max, Nq, Nkv, stream=0):
     """Gradient of rope_forward: the rotation by the negative angle."""
-    _rope(capi.lib.llmq_rope_backward_bf16, dinp, dout, freqs_cis, abs_max, Nq, Nkv, stream)
+    _rope("rope_backward", dinp, dout, freqs_cis, abs_max, Nq, Nkv, stream)
 
 
-def precompute_freqs_cis(dim, end, theta):
-    """Host tensor [end, dim] fp16 of (cos, sin) pairs (reference: precompute_freqs_cis, src/kernels/rope.cu:15-40)."""
-    tab = torch.empty((end, dim), dtype=torch.float16)
-    capi.check(capi.lib.llmq_precompute_freqs_cis_f16(tab.data_ptr(), int(dim), int(end), float(theta)))
+def precompute_freqs_cis(dim, end, theta, dtype=torch.float16):
+    """Host tensor [end, dim] of (cos, sin) pairs, fp16 (for bf16 tensors) or fp32 (reference: precompute_freqs_cis,
+    src/kernels/rope.cu:15-40)."""
+    if dtype not in (torch.float16, torch.float32):
+        raise ValueError("precompute_freqs_cis: the table is float16 or float32")
+    tab = torch.empty((end, dim), dtype=dtype)
+    fn = capi.lib.llmq_precompute_freqs_cis_f32 if dtype == torch.float32 else capi.lib.llmq_precompute_freqs_cis_f16
+    capi.check(fn(tab.data_ptr(), int(dim), int(end), float(theta)))
     return tab
 
 

@@ -376,34 +376,56 @@ void orc_backward_bias_bf16(uint16_t* dbias, const void* dout, int fmt, const fl
 }
 
 /*
- * SwiGLU forward / backward on bf16 tensors (kernel: src/kernels/swiglu.cu:20-23,25-65,244-300; CPU
+ * Element access of the producer functions below: a tensor is bf16 bits (is_f32 == 0) or fp32 (is_f32 != 0); values
+ * are taken to double (exact for both) and results are rounded once: double -> float (-> bf16).
+ */
+static inline double ld_elem(const void* p, int64_t i, int is_f32) {
+    return is_f32 ? (double)((const float*)p)[i] : (double)orc_bf16_to_f32(((const uint16_t*)p)[i]);
+}
+static inline void st_elem(void* p, int64_t i, double v, int is_f32) {
+    if (is_f32) ((float*)p)[i] = (float)v;
+    else ((uint16_t*)p)[i] = orc_f32_to_bf16((float)v);
+}
+static inline void copy_elem(void* dst, const void* src, int64_t i, int is_f32) {
+    if (is_f32) ((float*)dst)[i] = ((const float*)src)[i];
+    else ((uint16_t*)dst)[i] = ((const uint16_t*)src)[i];
+}
+
+/*
+ * SwiGLU forward / backward on bf16 or fp32 tensors (kernel: src/kernels/swiglu.cu:20-23,25-65,244-300; CPU
  * baselines of the reference's own tests: src/testing/test-swiglu.cu:28-72).  inp rows are [up(C) | gate(C)]:
  *     s = 1 / (1 + exp(-gate));  out = up * gate * s;  dup = dout * gate * s;
  *     dgate = dout * up * s * (1 + gate * (1 - s)).
  * The reference's device code uses expf and an approximate reciprocal whose bits are not specified, and its
- * tests accept 3e-2 absolute error; the oracle therefore evaluates the formulas in double and rounds once
- * (double -> float -> bf16), i.e. it gives the correctly rounded result a device implementation is measured
- * against.  exact_* (optional, may be NULL) receive the double values.
+ * tests accept 3e-2 absolute error (bf16) / 1e-6 and 1e-5 (fp32); the oracle therefore evaluates the formulas in
+ * double and rounds once (double -> float [-> bf16]), i.e. it gives the correctly rounded result a device
+ * implementation is measured against.  exact_* (optional, may be NULL) receive the double values.
  */
-void orc_swiglu_forward_bf16(uint16_t* out, double* exact_out, const uint16_t* inp, int64_t BT, int C) {
+static void swiglu_forward_any(void* out, double* exact_out, const void* inp, int64_t BT, int C, int is_f32) {
     for (int64_t r = 0; r < BT; ++r) {
         for (int c = 0; c < C; ++c) {
-            const double up = (double)orc_bf16_to_f32(inp[r * 2 * C + c]);
-            const double gate = (double)orc_bf16_to_f32(inp[r * 2 * C + C + c]);
+            const double up = ld_elem(inp, r * 2 * C + c, is_f32);
+            const double gate = ld_elem(inp, r * 2 * C + C + c, is_f32);
             const double v = up * gate * (1.0 / (1.0 + exp(-gate)));
             if (exact_out) exact_out[r * C + c] = v;
-            out[r * C + c] = orc_f32_to_bf16((float)v);
+            st_elem(out, r * C + c, v, is_f32);
         }
     }
 }
+void orc_swiglu_forward_bf16(uint16_t* out, double* exact_out, const uint16_t* inp, int64_t BT, int C) {
+    swiglu_forward_any(out, exact_out, inp, BT, C, 0);
+}
+void orc_swiglu_forward_f32(float* out, double* exact_out, const float* inp, int64_t BT, int C) {
+    swiglu_forward_any(out, exact_out, inp, BT, C, 1);
+}
 
-void orc_swiglu_backward_bf16(uint16_t* dinp, double* exact_dinp, const uint16_t* dout, const uint16_t* inp,
-                              int64_t BT, int C) {
+static void swiglu_backward_any(void* dinp, double* exact_dinp, const void* dout, const void* inp, int64_t BT, int C,
+                                int is_f32) {
     for (int64_t r = 0; r < BT; ++r) {
         for (int c = 0; c < C; ++c) {
-            const double up = (double)orc_bf16_to_f32(inp[r * 2 * C + c]);
-            const double gate = (double)orc_bf16_to_f32(inp[r * 2 * C + C + c]);
-            const double d = (double)orc_bf16_to_f32(dout[r * C + c]);
+            const double up = ld_elem(inp, r * 2 * C + c, is_f32);
+            const double gate = ld_elem(inp, r * 2 * C + C + c, is_f32);
+            const double d = ld_elem(dout, r * C + c, is_f32);
             const double s = 1.0 / (1.0 + exp(-gate));
             const double d1 = d * gate * s;
             const double d2 = d * up * s * (1.0 + gate * (1.0 - s));
@@ -411,101 +433,125 @@ void orc_swiglu_backward_bf16(uint16_t* dinp, double* exact_dinp, const uint16_t
                 exact_dinp[r * 2 * C + c] = d1;
                 exact_dinp[r * 2 * C + C + c] = d2;
             }
-            dinp[r * 2 * C + c] = orc_f32_to_bf16((float)d1);
-            dinp[r * 2 * C + C + c] = orc_f32_to_bf16((float)d2);
+            st_elem(dinp, r * 2 * C + c, d1, is_f32);
+            st_elem(dinp, r * 2 * C + C + c, d2, is_f32);
         }
     }
+}
+void orc_swiglu_backward_bf16(uint16_t* dinp, double* exact_dinp, const uint16_t* dout, const uint16_t* inp,
+                              int64_t BT, int C) {
+    swiglu_backward_any(dinp, exact_dinp, dout, inp, BT, C, 0);
+}
+void orc_swiglu_backward_f32(float* dinp, double* exact_dinp, const float* dout, const float* inp, int64_t BT, int C) {
+    swiglu_backward_any(dinp, exact_dinp, dout, inp, BT, C, 1);
 }
 
 /*
  * RMSNorm forward, plain (inp2 == NULL) or with the residual add in front (src/kernels/rmsnorm.cu:17-86,
- * 88-164): res = inp1 or bf16((float)inp1 + (float)inp2) [stored to residual]; s = 1/sqrt(mean(res^2) + eps);
- * out = bf16((float)bf16(s * res) * (float)weight) -- the reference rounds the normalised value to bf16 before
- * the scale (rmsnorm.cu:68-71).  The reference's s comes from an fp32 sum in a launch-dependent order and
- * the approximate rsqrt; the oracle takes the sum, mean and inverse root in double and rounds s once to
- * fp32, the value any such implementation approximates.  exact_out (optional) receives s_double * res *
- * weight without the intermediate rounding.
+ * 88-164), tensors of type X = bf16 or fp32: res = inp1 or X((float)inp1 + (float)inp2) [stored to residual];
+ * s = 1/sqrt(mean(res^2) + eps); out = X((float)X(s * res) * (float)weight) -- the reference rounds the normalised
+ * value to X before the scale (rmsnorm.cu:68-71; for fp32 that is the fp32 product itself).  The reference's s
+ * comes from an fp32 sum in a launch-dependent order and the approximate rsqrt; the oracle takes the sum, mean and
+ * inverse root in double and rounds s once to fp32, the value any such implementation approximates.  exact_out
+ * (optional) receives s_double * res * weight without the intermediate rounding.
  */
-void orc_rmsnorm_forward_bf16(uint16_t* residual, uint16_t* normed, float* rrms, double* exact_out,
-                              const uint16_t* inp1, const uint16_t* inp2, const uint16_t* weight, float eps,
-                              int64_t N, int C) {
-    uint16_t* row = (uint16_t*)malloc((size_t)(C > 0 ? C : 1) * sizeof(uint16_t));
+static void rmsnorm_forward_any(void* residual, void* normed, float* rrms, double* exact_out, const void* inp1,
+                                const void* inp2, const void* weight, float eps, int64_t N, int C, int is_f32) {
+    float* row = (float*)malloc((size_t)(C > 0 ? C : 1) * sizeof(float));
     for (int64_t r = 0; r < N; ++r) {
         double acc = 0.0;
         for (int c = 0; c < C; ++c) {
-            uint16_t v = inp1[r * C + c];
+            float v = (float)ld_elem(inp1, r * C + c, is_f32);
             if (inp2) {
-                volatile float sum = orc_bf16_to_f32(v) + orc_bf16_to_f32(inp2[r * C + c]);
-                v = orc_f32_to_bf16(sum);
-                if (residual) residual[r * C + c] = v;
+                volatile float sum = v + (float)ld_elem(inp2, r * C + c, is_f32);
+                v = is_f32 ? sum : orc_bf16_to_f32(orc_f32_to_bf16(sum));
+                if (residual) st_elem(residual, r * C + c, (double)v, is_f32);
             }
             row[c] = v;
-            const double x = (double)orc_bf16_to_f32(v);
-            acc += x * x;
+            acc += (double)v * (double)v;
         }
         const double sd = 1.0 / sqrt(acc / (double)C + (double)eps);
         const float s = (float)sd;
         if (rrms) rrms[r] = s;
         for (int c = 0; c < C; ++c) {
-            const float x = orc_bf16_to_f32(row[c]), w = orc_bf16_to_f32(weight[c]);
+            const float x = row[c], w = (float)ld_elem(weight, c, is_f32);
             volatile float n = s * x;
-            const float nb = orc_bf16_to_f32(orc_f32_to_bf16(n));
+            const float nb = is_f32 ? n : orc_bf16_to_f32(orc_f32_to_bf16(n));
             volatile float prod = nb * w;
-            normed[r * C + c] = orc_f32_to_bf16(prod);
+            st_elem(normed, r * C + c, (double)prod, is_f32);
             if (exact_out) exact_out[r * C + c] = sd * (double)x * (double)w;
         }
     }
     free(row);
 }
+void orc_rmsnorm_forward_bf16(uint16_t* residual, uint16_t* normed, float* rrms, double* exact_out,
+                              const uint16_t* inp1, const uint16_t* inp2, const uint16_t* weight, float eps,
+                              int64_t N, int C) {
+    rmsnorm_forward_any(residual, normed, rrms, exact_out, inp1, inp2, weight, eps, N, C, 0);
+}
+void orc_rmsnorm_forward_f32(float* residual, float* normed, float* rrms, double* exact_out, const float* inp1,
+                             const float* inp2, const float* weight, float eps, int64_t N, int C) {
+    rmsnorm_forward_any(residual, normed, rrms, exact_out, inp1, inp2, weight, eps, N, C, 1);
+}
 
 /*
- * RMSNorm backward (src/kernels/rmsnorm.cu:229-440): with r = rstd[bt], g_c = weight[c] * dout[bt,c],
- * k = (sum_c g_c * inp[bt,c]) / C * r:
- *     dinp[bt,c] = bf16(dresidual[bt,c] + (g_c - inp[bt,c] * r * k) * r)
- *     dweight[c] = bf16(dweight[c] + sum_bt inp[bt,c] * r * dout[bt,c])
- * evaluated in double and rounded once (double -> float -> bf16); the reference's fp32 sums have a launch-
+ * RMSNorm backward (src/kernels/rmsnorm.cu:229-440), tensors of type X = bf16 or fp32: with r = rstd[bt],
+ * g_c = weight[c] * dout[bt,c], k = (sum_c g_c * inp[bt,c]) / C * r:
+ *     dinp[bt,c] = X(dresidual[bt,c] + (g_c - inp[bt,c] * r * k) * r)
+ *     dweight[c] = X(dweight[c] + sum_bt inp[bt,c] * r * dout[bt,c])
+ * evaluated in double and rounded once (double -> float [-> bf16]); the reference's fp32 sums have a launch-
  * dependent order.  exact_* receive the double values, mag_* the sums of the absolute values of the terms
  * (the scale of the fp32 evaluation error, for tolerances); all four are optional.
  */
-void orc_rmsnorm_backward_bf16(uint16_t* dinp, uint16_t* dweight, double* exact_dinp, double* mag_dinp,
-                               double* exact_dw, double* mag_dw, const uint16_t* dresidual, const uint16_t* dout,
-                               const uint16_t* inp, const uint16_t* weight, const float* rstd, int64_t N, int C) {
+static void rmsnorm_backward_any(void* dinp, void* dweight, double* exact_dinp, double* mag_dinp, double* exact_dw,
+                                 double* mag_dw, const void* dresidual, const void* dout, const void* inp,
+                                 const void* weight, const float* rstd, int64_t N, int C, int is_f32) {
     double* dw = (double*)calloc((size_t)(C > 0 ? C : 1), sizeof(double));
     double* dwa = (double*)calloc((size_t)(C > 0 ? C : 1), sizeof(double));
     for (int64_t bt = 0; bt < N; ++bt) {
         const double r = (double)rstd[bt];
         double dot = 0.0;
         for (int c = 0; c < C; ++c)
-            dot += (double)orc_bf16_to_f32(weight[c]) * (double)orc_bf16_to_f32(dout[bt * C + c]) *
-                   (double)orc_bf16_to_f32(inp[bt * C + c]);
+            dot += ld_elem(weight, c, is_f32) * ld_elem(dout, bt * C + c, is_f32) * ld_elem(inp, bt * C + c, is_f32);
         const double k = dot / (double)C * r;
         for (int c = 0; c < C; ++c) {
-            const double x = (double)orc_bf16_to_f32(inp[bt * C + c]), d = (double)orc_bf16_to_f32(dout[bt * C + c]);
-            const double g = (double)orc_bf16_to_f32(weight[c]) * d, old = (double)orc_bf16_to_f32(dresidual[bt * C + c]);
+            const double x = ld_elem(inp, bt * C + c, is_f32), d = ld_elem(dout, bt * C + c, is_f32);
+            const double g = ld_elem(weight, c, is_f32) * d, old = ld_elem(dresidual, bt * C + c, is_f32);
             const double v = old + (g - x * r * k) * r;
             dw[c] += x * r * d;
             dwa[c] += fabs(x * r * d);
             if (exact_dinp) exact_dinp[bt * C + c] = v;
             if (mag_dinp) mag_dinp[bt * C + c] = fabs(old) + (fabs(g) + fabs(x * r * k)) * fabs(r);
-            dinp[bt * C + c] = orc_f32_to_bf16((float)v);
+            st_elem(dinp, bt * C + c, v, is_f32);
         }
     }
     for (int c = 0; c < C; ++c) {
-        const double old = (double)orc_bf16_to_f32(dweight[c]);
+        const double old = ld_elem(dweight, c, is_f32);
         if (exact_dw) exact_dw[c] = old + dw[c];
         if (mag_dw) mag_dw[c] = fabs(old) + dwa[c];
-        dweight[c] = orc_f32_to_bf16((float)(old + dw[c]));
+        st_elem(dweight, c, old + dw[c], is_f32);
     }
     free(dw);
     free(dwa);
 }
+void orc_rmsnorm_backward_bf16(uint16_t* dinp, uint16_t* dweight, double* exact_dinp, double* mag_dinp,
+                               double* exact_dw, double* mag_dw, const uint16_t* dresidual, const uint16_t* dout,
+                               const uint16_t* inp, const uint16_t* weight, const float* rstd, int64_t N, int C) {
+    rmsnorm_backward_any(dinp, dweight, exact_dinp, mag_dinp, exact_dw, mag_dw, dresidual, dout, inp, weight, rstd, N, C, 0);
+}
+void orc_rmsnorm_backward_f32(float* dinp, float* dweight, double* exact_dinp, double* mag_dinp, double* exact_dw,
+                              double* mag_dw, const float* dresidual, const float* dout, const float* inp,
+                              const float* weight, const float* rstd, int64_t N, int C) {
+    rmsnorm_backward_any(dinp, dweight, exact_dinp, mag_dinp, exact_dw, mag_dw, dresidual, dout, inp, weight, rstd, N, C, 1);
+}
 
 /*
- * Rotary embedding on [BT][N = Nq + 2 Nkv][HD] bf16 with an fp16 table [T][HD] of (cos, sin) pairs
- * (src/kernels/rope.cu:42-127): query and key heads rotate (x[d], x[d + HD/2]) by the angle of (t, d), the
- * backward by the negative angle; value heads pass through.  Evaluated in double (products of bf16 and fp16
- * values are exact there) and rounded once.  t = bt % T.  exact / mag (optional): the double value and
- * |real*cos| + |imag*sin| (resp. |real*sin| + |imag*cos|), the scale of an fp32 evaluation's error.
+ * Rotary embedding on [BT][N = Nq + 2 Nkv][HD] with a table [T][HD] of (cos, sin) pairs (src/kernels/rope.cu:42-127):
+ * bf16 tensors with an fp16 table, or fp32 tensors with an fp32 table.  Query and key heads rotate
+ * (x[d], x[d + HD/2]) by the angle of (t, d), the backward by the negative angle; value heads pass through.
+ * Evaluated in double (products of bf16 and fp16 values are exact there) and rounded once.  t = bt % T.
+ * exact / mag (optional): the double value and |real*cos| + |imag*sin| (resp. |real*sin| + |imag*cos|), the scale of
+ * an fp32 evaluation's error.
  */
 static double f16_to_double(uint16_t h) {
     const int sign = h >> 15, e = (h >> 10) & 31, m = h & 1023;
@@ -516,32 +562,44 @@ static double f16_to_double(uint16_t h) {
     return sign ? -v : v;
 }
 
-void orc_rope_bf16(uint16_t* out, double* exact, double* mag, const uint16_t* inp, const uint16_t* freqs_f16,
-                   int64_t BT, int T, int Nq, int Nkv, int HD, int backward) {
+static void rope_any(void* out, double* exact, double* mag, const void* inp, const void* freqs, int64_t BT, int T,
+                     int Nq, int Nkv, int HD, int backward, int is_f32) {
     const int N = Nq + 2 * Nkv, half = HD / 2;
     for (int64_t bt = 0; bt < BT; ++bt) {
         const int t = (int)(bt % T);
         for (int h = 0; h < N; ++h) {
             const int64_t base = (bt * N + h) * HD;
             for (int d = 0; d < half; ++d) {
-                const double re = (double)orc_bf16_to_f32(inp[base + d]), im = (double)orc_bf16_to_f32(inp[base + half + d]);
+                const double re = ld_elem(inp, base + d, is_f32), im = ld_elem(inp, base + half + d, is_f32);
                 double o_re = re, o_im = im, m_re = fabs(re), m_im = fabs(im);
                 if (h < Nq + Nkv) {
-                    const double c = f16_to_double(freqs_f16[(int64_t)t * HD + 2 * d]);
-                    double sn = f16_to_double(freqs_f16[(int64_t)t * HD + 2 * d + 1]);
+                    const int64_t fi = (int64_t)t * HD + 2 * d;
+                    const double c = is_f32 ? (double)((const float*)freqs)[fi] : f16_to_double(((const uint16_t*)freqs)[fi]);
+                    double sn = is_f32 ? (double)((const float*)freqs)[fi + 1] : f16_to_double(((const uint16_t*)freqs)[fi + 1]);
                     if (backward) sn = -sn;
                     o_re = re * c - im * sn;
                     o_im = re * sn + im * c;
                     m_re = fabs(re * c) + fabs(im * sn);
                     m_im = fabs(re * sn) + fabs(im * c);
+                    st_elem(out, base + d, o_re, is_f32);
+                    st_elem(out, base + half + d, o_im, is_f32);
+                } else {
+                    copy_elem(out, inp, base + d, is_f32);
+                    copy_elem(out, inp, base + half + d, is_f32);
                 }
-                out[base + d] = h < Nq + Nkv ? orc_f32_to_bf16((float)o_re) : inp[base + d];
-                out[base + half + d] = h < Nq + Nkv ? orc_f32_to_bf16((float)o_im) : inp[base + half + d];
                 if (exact) { exact[base + d] = o_re; exact[base + half + d] = o_im; }
                 if (mag) { mag[base + d] = m_re; mag[base + half + d] = m_im; }
             }
         }
     }
+}
+void orc_rope_bf16(uint16_t* out, double* exact, double* mag, const uint16_t* inp, const uint16_t* freqs_f16,
+                   int64_t BT, int T, int Nq, int Nkv, int HD, int backward) {
+    rope_any(out, exact, mag, inp, freqs_f16, BT, T, Nq, Nkv, HD, backward, 0);
+}
+void orc_rope_f32(float* out, double* exact, double* mag, const float* inp, const float* freqs_f32, int64_t BT, int T,
+                  int Nq, int Nkv, int HD, int backward) {
+    rope_any(out, exact, mag, inp, freqs_f32, BT, T, Nq, Nkv, HD, backward, 1);
 }
 
 /*

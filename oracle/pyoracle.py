@@ -111,6 +111,16 @@ def lib():
     L.orc_rmsnorm_backward_bf16.argtypes = [u16p, u16p, f64p, f64p, f64p, f64p, u16p, u16p, u16p, u16p, f32p, C.c_int64, C.c_int]
     L.orc_rope_bf16.restype = None
     L.orc_rope_bf16.argtypes = [u16p, f64p, f64p, u16p, u16p, C.c_int64, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
+    L.orc_swiglu_forward_f32.restype = None
+    L.orc_swiglu_forward_f32.argtypes = [f32p, f64p, f32p, C.c_int64, C.c_int]
+    L.orc_swiglu_backward_f32.restype = None
+    L.orc_swiglu_backward_f32.argtypes = [f32p, f64p, f32p, f32p, C.c_int64, C.c_int]
+    L.orc_rmsnorm_forward_f32.restype = None
+    L.orc_rmsnorm_forward_f32.argtypes = [f32p, f32p, f32p, f64p, f32p, f32p, f32p, C.c_float, C.c_int64, C.c_int]
+    L.orc_rmsnorm_backward_f32.restype = None
+    L.orc_rmsnorm_backward_f32.argtypes = [f32p, f32p, f64p, f64p, f64p, f64p, f32p, f32p, f32p, f32p, f32p, C.c_int64, C.c_int]
+    L.orc_rope_f32.restype = None
+    L.orc_rope_f32.argtypes = [f32p, f64p, f64p, f32p, f32p, C.c_int64, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
     L.orc_squirrel_noise_5.restype = C.c_uint32
     L.orc_squirrel_noise_5.argtypes = [C.c_uint32, C.c_uint32]
     L.orc_stochastic_round_bf16.restype = C.c_uint16
@@ -312,78 +322,89 @@ def quantize_f32(x, absmax, fmt="e4m3"):
     return out, sc[0]
 
 
+def _elem(arr):
+    """(numpy dtype, ctypes element type, suffix of the oracle function) of a producer tensor: bf16 bits or fp32."""
+    if np.asarray(arr).dtype == np.float32:
+        return np.float32, C.c_float, "f32"
+    return np.uint16, C.c_uint16, "bf16"
+
+
 def swiglu_forward(inp):
-    """inp: uint16 bf16 bits [BT, 2C] (rows [up | gate]) -> (out bits uint16 [BT, C], exact float64 [BT, C])."""
-    inp = np.ascontiguousarray(inp, dtype=np.uint16)
+    """inp: uint16 bf16 bits or float32 [BT, 2C] (rows [up | gate]) -> (out of the same type [BT, C], exact float64)."""
+    dt, ct, sfx = _elem(inp)
+    inp = np.ascontiguousarray(inp, dtype=dt)
     BT, C2 = inp.shape
-    out = np.empty((BT, C2 // 2), dtype=np.uint16)
+    out = np.empty((BT, C2 // 2), dtype=dt)
     exact = np.empty((BT, C2 // 2), dtype=np.float64)
-    lib().orc_swiglu_forward_bf16(_p(out, C.c_uint16), _p(exact, C.c_double), _p(inp, C.c_uint16), BT, C2 // 2)
+    getattr(lib(), "orc_swiglu_forward_" + sfx)(_p(out, ct), _p(exact, C.c_double), _p(inp, ct), BT, C2 // 2)
     return out, exact
 
 
 def swiglu_backward(dout, inp):
-    """dout: bf16 bits [BT, C], inp: [BT, 2C] -> (dinp bits uint16 [BT, 2C] = [dup | dgate], exact float64)."""
-    inp = np.ascontiguousarray(inp, dtype=np.uint16)
-    dout = np.ascontiguousarray(dout, dtype=np.uint16)
+    """dout: [BT, C], inp: [BT, 2C] (bf16 bits or float32) -> (dinp of the same type [BT, 2C] = [dup | dgate], exact)."""
+    dt, ct, sfx = _elem(inp)
+    inp = np.ascontiguousarray(inp, dtype=dt)
+    dout = np.ascontiguousarray(dout, dtype=dt)
     BT, C2 = inp.shape
-    dinp = np.empty((BT, C2), dtype=np.uint16)
+    dinp = np.empty((BT, C2), dtype=dt)
     exact = np.empty((BT, C2), dtype=np.float64)
-    lib().orc_swiglu_backward_bf16(_p(dinp, C.c_uint16), _p(exact, C.c_double), _p(dout, C.c_uint16),
-                                   _p(inp, C.c_uint16), BT, C2 // 2)
+    getattr(lib(), "orc_swiglu_backward_" + sfx)(_p(dinp, ct), _p(exact, C.c_double), _p(dout, ct), _p(inp, ct), BT, C2 // 2)
     return dinp, exact
 
 
 def rmsnorm_forward(inp1, weight, eps, inp2=None):
-    """inp1 (and inp2): bf16 bits [N, C]; weight: bf16 bits [C].  Returns (normed bits [N, C], rrms float32 [N],
-    exact float64 [N, C], residual bits [N, C] or None)."""
-    inp1 = np.ascontiguousarray(inp1, dtype=np.uint16)
-    weight = np.ascontiguousarray(weight, dtype=np.uint16)
+    """inp1 (and inp2): bf16 bits or float32 [N, C]; weight: [C] of the same type.  Returns (normed [N, C], rrms
+    float32 [N], exact float64 [N, C], residual [N, C] or None)."""
+    dt, ct, sfx = _elem(inp1)
+    inp1 = np.ascontiguousarray(inp1, dtype=dt)
+    weight = np.ascontiguousarray(weight, dtype=dt)
     N, Cc = inp1.shape
-    normed = np.empty((N, Cc), dtype=np.uint16)
+    normed = np.empty((N, Cc), dtype=dt)
     rrms = np.empty(N, dtype=np.float32)
     exact = np.empty((N, Cc), dtype=np.float64)
     res = None
     p2 = None
     if inp2 is not None:
-        inp2 = np.ascontiguousarray(inp2, dtype=np.uint16)
-        res = np.empty((N, Cc), dtype=np.uint16)
-        p2 = _p(inp2, C.c_uint16)
-    lib().orc_rmsnorm_forward_bf16(_p(res, C.c_uint16) if res is not None else None, _p(normed, C.c_uint16),
-                                   _p(rrms, C.c_float), _p(exact, C.c_double), _p(inp1, C.c_uint16), p2,
-                                   _p(weight, C.c_uint16), C.c_float(eps), N, Cc)
+        inp2 = np.ascontiguousarray(inp2, dtype=dt)
+        res = np.empty((N, Cc), dtype=dt)
+        p2 = _p(inp2, ct)
+    getattr(lib(), "orc_rmsnorm_forward_" + sfx)(_p(res, ct) if res is not None else None, _p(normed, ct),
+                                                 _p(rrms, C.c_float), _p(exact, C.c_double), _p(inp1, ct), p2,
+                                                 _p(weight, ct), C.c_float(eps), N, Cc)
     return normed, rrms, exact, res
 
 
 def rmsnorm_backward(dresidual, dweight, dout, inp, weight, rstd):
-    """bf16 bits: dresidual, dout, inp [N, C]; dweight (old value), weight [C]; rstd float32 [N].
-    Returns dict(dinp, dweight (bits), exact_dinp, mag_dinp, exact_dw, mag_dw (float64))."""
-    inp = np.ascontiguousarray(inp, dtype=np.uint16)
+    """bf16 bits or float32: dresidual, dout, inp [N, C]; dweight (old value), weight [C]; rstd float32 [N].
+    Returns dict(dinp, dweight (same type), exact_dinp, mag_dinp, exact_dw, mag_dw (float64))."""
+    dt, ct, sfx = _elem(inp)
+    inp = np.ascontiguousarray(inp, dtype=dt)
     N, Cc = inp.shape
-    dres = np.ascontiguousarray(dresidual, dtype=np.uint16)
-    dout = np.ascontiguousarray(dout, dtype=np.uint16)
-    weight = np.ascontiguousarray(weight, dtype=np.uint16)
+    dres = np.ascontiguousarray(dresidual, dtype=dt)
+    dout = np.ascontiguousarray(dout, dtype=dt)
+    weight = np.ascontiguousarray(weight, dtype=dt)
     rstd = np.ascontiguousarray(rstd, dtype=np.float32)
-    dinp = np.empty((N, Cc), dtype=np.uint16)
-    dw = np.array(dweight, dtype=np.uint16, copy=True)
+    dinp = np.empty((N, Cc), dtype=dt)
+    dw = np.array(dweight, dtype=dt, copy=True)
     ed, md = np.empty((N, Cc)), np.empty((N, Cc))
     ew, mw = np.empty(Cc), np.empty(Cc)
-    lib().orc_rmsnorm_backward_bf16(_p(dinp, C.c_uint16), _p(dw, C.c_uint16), _p(ed, C.c_double), _p(md, C.c_double),
-                                    _p(ew, C.c_double), _p(mw, C.c_double), _p(dres, C.c_uint16), _p(dout, C.c_uint16),
-                                    _p(inp, C.c_uint16), _p(weight, C.c_uint16), _p(rstd, C.c_float), N, Cc)
+    getattr(lib(), "orc_rmsnorm_backward_" + sfx)(_p(dinp, ct), _p(dw, ct), _p(ed, C.c_double), _p(md, C.c_double),
+                                                  _p(ew, C.c_double), _p(mw, C.c_double), _p(dres, ct), _p(dout, ct),
+                                                  _p(inp, ct), _p(weight, ct), _p(rstd, C.c_float), N, Cc)
     return dict(dinp=dinp, dweight=dw, exact_dinp=ed, mag_dinp=md, exact_dw=ew, mag_dw=mw)
 
 
-def rope(inp, freqs_f16, T, Nq, Nkv, backward=False):
-    """inp: bf16 bits [BT, Nq + 2 Nkv, HD]; freqs_f16: fp16 bits [T, HD] of (cos, sin) pairs.
-    Returns (out bits, exact float64, magnitude float64), all shaped like inp."""
-    inp = np.ascontiguousarray(inp, dtype=np.uint16)
-    freqs = np.ascontiguousarray(freqs_f16, dtype=np.uint16)
+def rope(inp, freqs, T, Nq, Nkv, backward=False):
+    """inp: bf16 bits with an fp16-bits table, or float32 with a float32 table; inp [BT, Nq + 2 Nkv, HD], table [T, HD]
+    of (cos, sin) pairs.  Returns (out of inp's type, exact float64, magnitude float64), all shaped like inp."""
+    dt, ct, sfx = _elem(inp)
+    inp = np.ascontiguousarray(inp, dtype=dt)
+    freqs = np.ascontiguousarray(freqs, dtype=dt)
     BT, N, HD = inp.shape
     out = np.empty_like(inp)
     exact, mag = np.empty(inp.shape), np.empty(inp.shape)
-    lib().orc_rope_bf16(_p(out, C.c_uint16), _p(exact, C.c_double), _p(mag, C.c_double), _p(inp, C.c_uint16),
-                        _p(freqs, C.c_uint16), BT, T, Nq, Nkv, HD, 1 if backward else 0)
+    getattr(lib(), "orc_rope_" + sfx)(_p(out, ct), _p(exact, C.c_double), _p(mag, C.c_double), _p(inp, ct), _p(freqs, ct),
+                                      BT, T, Nq, Nkv, HD, 1 if backward else 0)
     return out, exact, mag
 
 

@@ -21,6 +21,8 @@ void orc_gemm_tn_e4m3_exact_sampled(double* exact, double* sumabs, const uint8_t
                                     const int32_t* idx_n, const int32_t* idx_m, int64_t count);
 void orc_fill_normal_bf16(uint16_t* out, int64_t n, uint64_t seed, uint64_t stream, float mean, float std);
 void orc_swiglu_forward_bf16(uint16_t* out, double* exact_out, const uint16_t* inp, int64_t BT, int C);
+void orc_swiglu_forward_f32(float* out, double* exact_out, const float* inp, int64_t BT, int C);
+float orc_abs_max_f32(const float* in, int64_t n);
 void orc_backward_bias_bf16(uint16_t* dbias, const void* dout, int fmt, const float* sa, const float* sb, int64_t BT, int OC, double* colsum, double* colabs);
 }
 
@@ -211,6 +213,27 @@ int main(int argc, char** argv) {
         EXPECT(std::memcmp(&st[1], &sq, 4) == 0 && std::memcmp(&st[3], &sq, 4) == 0, "swiglu quantization scales differ");
         EXPECT(std::memcmp(q1.data(), qo.data(), n) == 0, "quantized activation differs from the oracle");
         EXPECT(std::memcmp(q1.data(), q2.data(), n) == 0, "swiglu_forward_quant differs from swiglu_forward + quantize");
+        {   // the fp32 overload through the same Tensor entry (an fp32 model in front of FP8 matmuls): the same input as fp32
+            std::vector<float> hin((std::size_t)BT * OC), hout(n);
+            for (std::size_t i = 0; i < hin.size(); ++i) hin[i] = orc_bf16_to_f32(hy[i]) * 1.0009765625f;
+            Tensor in32 = make(ETensorDType::FP32, dalloc<float>(hin.size()), {BT, OC});
+            Tensor out32 = make(ETensorDType::FP32, dalloc<float>(n), {BT, D});
+            HIP_OK(hipMemcpy(in32.Data, hin.data(), hin.size() * 4, hipMemcpyHostToDevice));
+            swiglu_forward(out32, in32, hstat, B, T, D, stream);
+            HIP_OK(hipStreamSynchronize(stream));
+            float am32;
+            HIP_OK(hipMemcpy(hout.data(), out32.Data, n * 4, hipMemcpyDeviceToHost));
+            HIP_OK(hipMemcpy(&am32, hstat, 4, hipMemcpyDeviceToHost));
+            std::vector<float> want32(n);
+            orc_swiglu_forward_f32(want32.data(), exact.data(), hin.data(), BT, D);
+            double worst32 = 0;
+            for (std::size_t i = 0; i < n; ++i)
+                worst32 = std::fmax(worst32, std::fabs((double)hout[i] - exact[i]) / (std::ldexp(std::fabs(exact[i]), -23) + 1e-37));
+            std::printf("%-10s [%d x %d]: worst error / (one fp32 ulp) %.3f\n", "swiglu f32", BT, D, worst32);
+            EXPECT(worst32 <= 4.0, "fp32 swiglu_forward is more than four fp32 ulp from the oracle");
+            const float aa32 = orc_abs_max_f32(hout.data(), n);
+            EXPECT(std::memcmp(&am32, &aa32, 4) == 0, "fp32 swiglu abs-max differs from the abs-max of its output");
+        }
         bool sw_threw = false;
         try { swiglu_forward(act, out, nullptr, B, T, D + 4, stream); }
         catch (const std::invalid_argument&) { sw_threw = true; }

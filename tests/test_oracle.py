@@ -588,6 +588,79 @@ def test_rope_vs_complex_multiplication(O):
     assert np.allclose(back[:, qk, half:], zz[:, qk].imag, rtol=1e-14, atol=1e-300)
 
 
+# ----------------------------------------------------------------------------- fp32 producer variants
+def test_fp32_producer_oracles_reduce_to_the_pinned_bf16_ones_and_match_torch(O):
+    """The fp32 variants share the formula code of the bf16 ones (pinned above): on bf16-representable inputs their
+    double values must be identical and their outputs the fp32 rounding of those; on general fp32 inputs SwiGLU and
+    RMSNorm agree with torch float64 (silu, autograd, mean / rsqrt) and rope with complex multiplication."""
+    BT, Cc = 7, 24
+    inp_b = O.fill_normal_bf16(BT * 2 * Cc, 61, 0, 0.0, 2.0).reshape(BT, 2 * Cc)
+    dout_b = O.fill_normal_bf16(BT * Cc, 61, 1).reshape(BT, Cc)
+    inp_f, dout_f = O.bf16_to_f32(inp_b), O.bf16_to_f32(dout_b)
+    for fn_args_b, fn_args_f in (((O.swiglu_forward, (inp_b,)), (O.swiglu_forward, (inp_f,))),
+                                 ((O.swiglu_backward, (dout_b, inp_b)), (O.swiglu_backward, (dout_f, inp_f)))):
+        _, ex_b = fn_args_b[0](*fn_args_b[1])
+        out_f, ex_f = fn_args_f[0](*fn_args_f[1])
+        assert out_f.dtype == np.float32 and np.array_equal(ex_b, ex_f) and np.array_equal(out_f, ex_f.astype(np.float32))
+    # general fp32 inputs against torch float64
+    rng = np.random.default_rng(5)
+    x = rng.normal(0, 2, (BT, 2 * Cc)).astype(np.float32)
+    d = rng.normal(0, 1, (BT, Cc)).astype(np.float32)
+    xt = torch.from_numpy(x.astype(np.float64)).requires_grad_(True)
+    a, b = torch.tensor_split(xt, 2, dim=-1)
+    y = torch.nn.functional.silu(b) * a
+    y.backward(torch.from_numpy(d.astype(np.float64)))
+    out, ex = O.swiglu_forward(x)
+    assert np.allclose(ex, y.detach().numpy(), rtol=1e-13, atol=1e-300) and np.array_equal(out, y.detach().numpy().astype(np.float32))
+    dinp, dex = O.swiglu_backward(d, x)
+    assert np.allclose(dex, xt.grad.numpy(), rtol=1e-12, atol=1e-14) and np.array_equal(dinp, xt.grad.numpy().astype(np.float32))
+
+    # rmsnorm forward: fp32 chain fl(fl(s x) w), residual one fp32 add
+    N, eps = 5, 1e-6
+    x1, x2 = rng.normal(0, 1.5, (N, Cc)).astype(np.float32), rng.normal(0, 0.7, (N, Cc)).astype(np.float32)
+    w = rng.normal(1, 0.3, Cc).astype(np.float32)
+    for fused in (False, True):
+        normed, rrms, exact, res = O.rmsnorm_forward(x1, w, eps, x2 if fused else None)
+        r = (x1 + x2).astype(np.float32) if fused else x1
+        if fused:
+            assert np.array_equal(res, r)
+        rd = torch.from_numpy(r.astype(np.float64))
+        r_rms = 1.0 / torch.sqrt((rd ** 2).mean(dim=-1, keepdim=True) + float(np.float32(eps)))
+        assert np.allclose(exact, (rd * r_rms * torch.from_numpy(w.astype(np.float64))).numpy(), rtol=1e-13, atol=0)
+        assert np.array_equal(rrms, r_rms.squeeze(-1).float().numpy())
+        assert np.array_equal(normed, ((rrms[:, None] * r).astype(np.float32) * w[None, :]).astype(np.float32))
+    # rmsnorm backward: the explicit formulas of the reference's test in float64 with the same fp32 rstd
+    dres, dw0 = rng.normal(0, 0.5, (N, Cc)).astype(np.float32), rng.normal(0, 2, Cc).astype(np.float32)
+    dd = rng.normal(0, 0.8, (N, Cc)).astype(np.float32)
+    rstd = (1.0 / np.sqrt((x1.astype(np.float64) ** 2).mean(axis=1))).astype(np.float32)
+    got = O.rmsnorm_backward(dres, dw0, dd, x1, w, rstd)
+    t64 = lambda v: torch.from_numpy(v.astype(np.float64))
+    rr = t64(rstd).unsqueeze(-1)
+    normed_t = t64(x1) * rr
+    dy_w = t64(dd) * t64(w)
+    dinp_t = rr * (dy_w - normed_t * (dy_w * normed_t).sum(dim=-1, keepdim=True) / Cc)
+    assert np.allclose(got["exact_dinp"], (t64(dres) + dinp_t).numpy(), rtol=1e-12, atol=1e-14)
+    assert np.allclose(got["exact_dw"], (t64(dw0) + (t64(dd) * t64(x1) * rr).sum(dim=0)).numpy(), rtol=1e-12, atol=1e-14)
+    assert np.array_equal(got["dinp"], got["exact_dinp"].astype(np.float32)) and np.array_equal(got["dweight"], got["exact_dw"].astype(np.float32))
+
+    # rope: complex multiplication with an fp32 table; value heads copied
+    B, T, Nq, Nkv, HD = 2, 5, 3, 2, 16
+    Nh, half = Nq + 2 * Nkv, HD // 2
+    xr = rng.normal(0, 1, (B * T, Nh, HD)).astype(np.float32)
+    tab = _rope_table(T, HD).astype(np.float32) + np.float32(1e-4) * rng.normal(0, 1, (T, HD)).astype(np.float32)
+    for backward in (False, True):
+        out, exact, _ = O.rope(xr, tab, T, Nq, Nkv, backward=backward)
+        z = xr[..., :half].astype(np.float64) + 1j * xr[..., half:].astype(np.float64)
+        rot = tab[:, 0::2].astype(np.float64) + 1j * tab[:, 1::2].astype(np.float64)
+        rot_bt = np.tile(np.conj(rot) if backward else rot, (B, 1))[:, None, :]
+        want = z * rot_bt
+        qk = slice(0, Nq + Nkv)
+        assert np.allclose(exact[:, qk, :half], want[:, qk].real, rtol=1e-14, atol=1e-300)
+        assert np.allclose(exact[:, qk, half:], want[:, qk].imag, rtol=1e-14, atol=1e-300)
+        assert np.array_equal(out[:, Nq + Nkv:], xr[:, Nq + Nkv:]) and out.dtype == np.float32
+        assert np.array_equal(out[:, qk], np.concatenate([want[:, qk].real, want[:, qk].imag], -1).astype(np.float32))
+
+
 # ------------------------------------------------------------------------------------------- adamw
 def test_squirrel_noise_properties(O):
     """No known-answer vectors exist in the reference tree; what the construction guarantees is checked: for a
