@@ -40,6 +40,9 @@
  *   rope               numpy complex128 multiplication by (cos + i sin) of numpy's fp16 decoding, norm
  *                      preservation, backward(forward(x)) = x (cos^2 + sin^2), value heads untouched; the
  *                      host table against numpy float64 cos / sin within fp16 rounding
+ *   fp32 producers     the swiglu / rmsnorm / rope functions are one formula code for bf16 and fp32 elements (ld_elem /
+ *                      st_elem); the fp32 variants are additionally checked to give the bf16 variants' double values on
+ *                      bf16-representable inputs and to agree with torch float64 / numpy complex128 on general fp32 inputs
  *   adamw              torch float64 evaluation of the reference's own test formulas
  *                      (scripts/test_kernels.py:695-727) for fp32 moments (exact fp32 outputs) and within the
  *                      stochastic rounding's one-ulp spread for bf16 ones; stochastic rounding: both
