@@ -383,6 +383,18 @@ int llmq_adamw_update_bf16_fp8m(uint16_t* params, const uint16_t* grads, uint8_t
                                 float weight_decay, const float* grad_scale, float* abs_max_or_null, unsigned int seed,
                                 void* stream);
 
+/*
+ * The same update on fp32 parameters, gradients and moments: nothing is narrower than fp32, so there is no stochastic
+ * rounding (seed is accepted for the reference's signature and unused); num_parameters must be a multiple of 4.
+ * abs_max_or_null as above (merged, not reset).  Bit exact against the formulas above evaluated operation by operation.
+ * Replaces: adamw_update(float* params, const float* grads, float* m, float* v, size_t num_parameters, float learning_rate,
+ *           float beta1, float beta2, int t, float eps, float weight_decay, const float* grad_scale, float* abs_max,
+ *           unsigned int seed, cudaStream_t)  src/kernels/kernels.h:221-223, src/kernels/adamw.cu:159-163.
+ */
+int llmq_adamw_update_f32(float* params, const float* grads, float* m, float* v, int64_t num_parameters, float learning_rate,
+                          float beta1, float beta2, int t, float eps, float weight_decay, const float* grad_scale,
+                          float* abs_max_or_null, unsigned int seed, void* stream);
+
 #if defined(__GNUC__)
 #pragma GCC visibility pop
 #endif

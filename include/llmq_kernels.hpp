@@ -567,8 +567,14 @@ inline void rope_backward(Tensor& dinp, const Tensor& dout, const Tensor& freqs_
 }
 
 // ---- adamw (reference: src/kernels/kernels.h:225-235, src/kernels/adamw.cu) ----------------------------------------
-// bf16 parameters and gradients; moments fp32/fp32, bf16/fp32, bf16/bf16 or e4m3 (block scales)/bf16.  abs_max is
-// merged, not reset.
+// bf16 parameters and gradients; moments fp32/fp32, bf16/fp32, bf16/bf16 or e4m3 (block scales)/bf16; or everything
+// fp32 (no stochastic rounding).  abs_max is merged, not reset.
+inline void adamw_update(float* params, const float* grads, float* m, float* v, std::size_t num_parameters, float learning_rate,
+                         float beta1, float beta2, int t, float eps, float weight_decay, const float* grad_scale, float* abs_max,
+                         unsigned int seed, hipStream_t stream) {
+    llmq_detail::check(llmq_adamw_update_f32(params, grads, m, v, (std::int64_t)num_parameters, learning_rate, beta1, beta2, t, eps,
+                                             weight_decay, grad_scale, abs_max, seed, stream));
+}
 inline void adamw_update(__hip_bfloat16* params, const __hip_bfloat16* grads, float* m, float* v, std::size_t num_parameters,
                          float learning_rate, float beta1, float beta2, int t, float eps, float weight_decay,
                          const float* grad_scale, float* abs_max, unsigned int seed, hipStream_t stream) {

@@ -27,7 +27,7 @@ EXPORTS = [
     "llmq_adamw_update_bf16", "llmq_adamw_update_bf16_fp8m",
     "llmq_swiglu_forward_f32", "llmq_swiglu_backward_f32", "llmq_rope_forward_f32", "llmq_rope_backward_f32",
     "llmq_precompute_freqs_cis_f32", "llmq_rmsnorm_forward_f32", "llmq_fused_residual_rmsnorm_forward_f32",
-    "llmq_rmsnorm_backward_f32",
+    "llmq_rmsnorm_backward_f32", "llmq_adamw_update_f32",
 ]
 
 if not os.path.exists(LIB_PATH):
@@ -76,6 +76,8 @@ for _name in ("swiglu_forward", "swiglu_backward", "rope_forward", "rope_backwar
               "fused_residual_rmsnorm_forward", "rmsnorm_backward"):
     getattr(lib, "llmq_%s_f32" % _name).argtypes = getattr(lib, "llmq_%s_bf16" % _name).argtypes
 lib.llmq_precompute_freqs_cis_f32.argtypes = lib.llmq_precompute_freqs_cis_f16.argtypes
+lib.llmq_adamw_update_f32.argtypes = [_vp, _vp, _vp, _vp, _i64, C.c_float, C.c_float, C.c_float, _int, C.c_float, C.c_float, _vp,
+                                      _vp, C.c_uint, _vp]
 for _name in EXPORTS[3:]:
     getattr(lib, _name).restype = _int
 lib.llmq_backward_bias_scratch_bytes.restype = _i64

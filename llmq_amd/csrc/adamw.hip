@@ -150,6 +150,47 @@ __global__ __launch_bounds__(THREADS) void adamw_kernel(uint4* __restrict__ para
     }
 }
 
+// fp32 parameters, gradients and moments (the reference's all-float overload, src/kernels/adamw.cu:159-163): the same
+// formulas; nothing is narrower than fp32, so nothing is stochastically rounded and the seed is unused.  A lane takes 4
+// consecutive parameters (16-byte accesses); 28 bytes per parameter.
+template <bool ABSMAX, int THREADS>
+__global__ __launch_bounds__(THREADS) void adamw_f32_kernel(uint4* __restrict__ params, const uint4* __restrict__ grads,
+                                                            uint4* __restrict__ m_mem, uint4* __restrict__ v_mem, int64_t nvec,
+                                                            AdamArgs a, const float* __restrict__ grad_scale,
+                                                            unsigned* __restrict__ absmax_out) {
+    const int64_t vec = (int64_t)blockIdx.x * THREADS + threadIdx.x;
+    uint32_t fold = 0x7F800000u;  // +Inf pattern - |x| pattern, minimised: NaNs wrap to huge values and are ignored
+    if (vec < nvec) {
+        const float gs = *grad_scale;
+        const uint4 pw = load_nt(&params[vec]), gw = load_nt(&grads[vec]), mw = load_nt(&m_mem[vec]), vw = load_nt(&v_mem[vec]);
+        const uint32_t pws[4] = {pw.x, pw.y, pw.z, pw.w}, gws[4] = {gw.x, gw.y, gw.z, gw.w}, mws[4] = {mw.x, mw.y, mw.z, mw.w},
+                       vws[4] = {vw.x, vw.y, vw.z, vw.w};
+        uint32_t p_out[4], m_out[4], v_out[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float p_old = __uint_as_float(pws[e]);
+            const float grad = gs * __uint_as_float(gws[e]);
+            const float m_new = __builtin_fmaf(a.beta1, __uint_as_float(mws[e]), __builtin_fmaf(-a.beta1, grad, grad));
+            const float g2 = grad * grad;
+            const float v_new = __builtin_fmaf(a.beta2, __uint_as_float(vws[e]), __builtin_fmaf(-a.beta2, g2, g2));
+            const float m_hat = m_new * a.c1, v_hat = v_new * a.c2;
+            const float quot = __fdiv_rn(m_hat, sqrt_rn(v_hat) + a.eps);
+            const float p_new = __builtin_fmaf(-a.lr, __builtin_fmaf(a.wd, p_old, quot), p_old);
+            p_out[e] = __float_as_uint(p_new);
+            m_out[e] = __float_as_uint(m_new);
+            v_out[e] = __float_as_uint(v_new);
+            if constexpr (ABSMAX) {
+                const uint32_t y = 0x7F800000u - (p_out[e] & 0x7FFFFFFFu);
+                fold = y < fold ? y : fold;
+            }
+        }
+        store_nt(&params[vec], make_uint4(p_out[0], p_out[1], p_out[2], p_out[3]));
+        store_nt(&m_mem[vec], make_uint4(m_out[0], m_out[1], m_out[2], m_out[3]));
+        store_nt(&v_mem[vec], make_uint4(v_out[0], v_out[1], v_out[2], v_out[3]));
+    }
+    if constexpr (ABSMAX) block_min_to_atomic_max(absmax_out, fold, 0x7F800000u, 0);
+}
+
 // fp32 -> e4m3 code with the reference's stochastic rounding (squirrel_noise.cuh:58-75): outside [2^-6, 448] in
 // magnitude plain round-to-nearest; inside, the 20 bits below e4m3's three mantissa bits are filled with ones
 // (the conversion then rounds away from zero) when they exceed the 20-bit threshold, else cleared.
@@ -279,6 +320,35 @@ extern "C" int llmq_adamw_update_bf16(uint16_t* params, const uint16_t* grads, v
     else if (v_dtype == 0) LLMQ_ADAM(true, false);
     else LLMQ_ADAM(true, true);
 #undef LLMQ_ADAM
+    LLMQ_HIP_TRY(hipGetLastError());
+    return LLMQ_OK;
+}
+
+// fp32 parameters, gradients and moments.  `seed` is accepted for the reference's signature and unused.
+extern "C" int llmq_adamw_update_f32(float* params, const float* grads, float* m, float* v, int64_t num_parameters,
+                                     float learning_rate, float beta1, float beta2, int t, float eps, float weight_decay,
+                                     const float* grad_scale, float* abs_max_or_null, unsigned int seed, void* stream_) {
+    using namespace llmq;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    LLMQ_REQUIRE(num_parameters >= 0, "adamw_update: negative parameter count %lld", (long long)num_parameters);
+    LLMQ_REQUIRE(num_parameters % 4 == 0, "adamw_update: num_parameters must be divisible by 4 for fp32 tensors (got %lld)",
+                 (long long)num_parameters);
+    LLMQ_REQUIRE(grad_scale != nullptr, "adamw_update: grad_scale pointer is null");
+    if (num_parameters == 0) return LLMQ_OK;
+    LLMQ_REQUIRE(params && grads && m && v, "adamw_update: null tensor pointer");
+    LLMQ_REQUIRE(aligned16(params) && aligned16(grads) && aligned16(m) && aligned16(v),
+                 "adamw_update: tensors must be 16-byte aligned");
+    const float c1 = 1.0f / (1.0f - powf(beta1, (float)t)), c2 = 1.0f / (1.0f - powf(beta2, (float)t));
+    const AdamArgs a{learning_rate, beta1, beta2, c1, c2, eps, weight_decay, seed};
+    const int64_t nvec = num_parameters / 4;
+    LLMQ_REQUIRE((nvec + 255) / 256 <= 0x7FFFFFFF, "adamw_update: tensor too large");
+    auto launch = [&](auto kernel, int threads) {
+        hipLaunchKernelGGL(kernel, dim3((unsigned)((nvec + threads - 1) / threads)), dim3(threads), 0, stream,
+                           reinterpret_cast<uint4*>(params), reinterpret_cast<const uint4*>(grads), reinterpret_cast<uint4*>(m),
+                           reinterpret_cast<uint4*>(v), nvec, a, grad_scale, reinterpret_cast<unsigned*>(abs_max_or_null));
+    };
+    if (abs_max_or_null) launch(adamw_f32_kernel<true, 1024>, 1024);
+    else launch(adamw_f32_kernel<false, 256>, 256);
     LLMQ_HIP_TRY(hipGetLastError());
     return LLMQ_OK;
 }

@@ -353,8 +353,8 @@ def adamw_update(params, grads, m, v, learning_rate, beta1, beta2, t, eps, weigh
                  abs_max=None, seed=0, stream=0):
     """In-place AdamW step on bf16 params with stochastic rounding (reference:
     src/binding/kernel_binding.cpp:536-551).  Moments: fp32 / fp32, bf16 / fp32, bf16 / bf16, or an e4m3 first
-    moment (float8_e4m3fn or uint8 codes) with m_scales, one fp32 scale per 128 elements, and a bf16 second moment.
-    grad_scale: fp32 device scalar.  abs_max, if given, is merged with max |new params| (not reset)."""
+    moment (float8_e4m3fn or uint8 codes) with m_scales, one fp32 scale per 128 elements, and a bf16 second moment; or
+    fp32 params, grads and moments (no stochastic rounding).  grad_scale: fp32 device scalar.  abs_max, if given, is merged with max |new params| (not reset)."""
     if m_scales is not None or m.dtype in (torch.float8_e4m3fn, torch.uint8):
         n = params.numel()
         if m_scales is None or any(x.numel() != n for x in (grads, m, v)) or m_scales.numel() < (n + 127) // 128:
@@ -369,6 +369,13 @@ def adamw_update(params, grads, m, v, learning_rate, beta1, beta2, t, eps, weigh
     n = params.numel()
     if any(x.numel() != n for x in (grads, m, v)):
         raise ValueError("adamw_update: shape mismatch")
+    if params.dtype == torch.float32:       # the all-fp32 overload: nothing to round stochastically, seed unused
+        f32 = (torch.float32,)
+        capi.check(capi.lib.llmq_adamw_update_f32(
+            _dev(params, "params", f32), _dev(grads, "grads", f32), _dev(m, "m", f32), _dev(v, "v", f32), n, float(learning_rate),
+            float(beta1), float(beta2), int(t), float(eps), float(weight_decay), _dev(grad_scale, "grad_scale", f32),
+            _dev(abs_max, "abs_max", f32, optional=True), int(seed) & 0xFFFFFFFF, _stream(stream)))
+        return
     p = _dev(params, "params", (torch.bfloat16,))
     g = _dev(grads, "grads", (torch.bfloat16,))
     pm = _dev(m, "m", (torch.float32, torch.bfloat16))

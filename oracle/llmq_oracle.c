@@ -670,6 +670,30 @@ float orc_adamw_update_bf16(uint16_t* params, const uint16_t* grads, void* m_mem
  * below the three mantissa bits e4m3 keeps) are compared with a 20-bit threshold: above it they are filled with
  * ones (the conversion then rounds away from zero), else cleared (the value is an e4m3 number already).
  */
+/* The all-fp32 overload (src/kernels/adamw.cu:159-163): the same formulas, nothing narrower than fp32 and therefore no
+ * stochastic rounding; the parameter line with the same contraction.  Returns max |new parameter| (NaNs skipped). */
+float orc_adamw_update_f32(float* params, const float* grads, float* m_mem, float* v_mem, int64_t n, float lr, float beta1,
+                           float beta2, int t, float eps, float wd, float grad_scale) {
+    const float c1 = 1.0f / (1.0f - powf(beta1, (float)t)), c2 = 1.0f / (1.0f - powf(beta2, (float)t));
+    float amax = 0.f;
+    for (int64_t i = 0; i < n; ++i) {
+        const float p_old = params[i];
+        volatile float grad = grad_scale * grads[i];
+        const float m_new = fmaf(beta1, m_mem[i], fmaf(-beta1, grad, grad));
+        volatile float g2 = grad * grad;
+        const float v_new = fmaf(beta2, v_mem[i], fmaf(-beta2, g2, g2));
+        volatile float m_hat = m_new * c1, v_hat = v_new * c2;
+        volatile float den = sqrtf(v_hat) + eps;
+        volatile float quot = m_hat / den;
+        params[i] = fmaf(-lr, fmaf(wd, p_old, quot), p_old);
+        m_mem[i] = m_new;
+        v_mem[i] = v_new;
+        const float pa = fabsf(params[i]);
+        if (pa > amax) amax = pa;
+    }
+    return amax;
+}
+
 uint8_t orc_stochastic_round_e4m3(float x, uint32_t random) {
     const float ax = fabsf(x);
     if (ax > 448.f || ax < 0.015625f) return orc_e4m3_encode(x);

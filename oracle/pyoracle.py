@@ -128,6 +128,9 @@ def lib():
     L.orc_adamw_update_bf16.restype = C.c_float
     L.orc_adamw_update_bf16.argtypes = [u16p, u16p, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int64, C.c_float, C.c_float,
                                         C.c_float, C.c_int, C.c_float, C.c_float, C.c_float, C.c_uint32]
+    L.orc_adamw_update_f32.restype = C.c_float
+    L.orc_adamw_update_f32.argtypes = [f32p, f32p, f32p, f32p, C.c_int64, C.c_float, C.c_float, C.c_float, C.c_int, C.c_float,
+                                       C.c_float, C.c_float]
     L.orc_adamw_update_bf16_fp8m.restype = C.c_float
     L.orc_adamw_update_bf16_fp8m.argtypes = [u16p, u16p, C.POINTER(C.c_uint8), C.POINTER(C.c_float), u16p, C.c_int64, C.c_float,
                                              C.c_float, C.c_float, C.c_int, C.c_float, C.c_float, C.c_float, C.c_uint32]
@@ -409,8 +412,14 @@ def rope(inp, freqs, T, Nq, Nkv, backward=False):
 
 
 def adamw_update(params, grads, m, v, lr, beta1, beta2, t, eps, wd, grad_scale, seed):
-    """params, grads: bf16 bits; m, v: float32 arrays (fp32 moments) or uint16 bf16 bits.  Returns new
-    (params, m, v, abs-max of the new params); inputs are not modified."""
+    """params, grads: bf16 bits; m, v: float32 arrays (fp32 moments) or uint16 bf16 bits -- or everything float32 (the
+    all-fp32 overload).  Returns new (params, m, v, abs-max of the new params); inputs are not modified."""
+    if np.asarray(params).dtype == np.float32:      # the all-fp32 overload: no stochastic rounding, seed unused
+        p, g = np.array(params, dtype=np.float32, copy=True), np.ascontiguousarray(grads, dtype=np.float32)
+        mm, vv = np.array(m, dtype=np.float32, copy=True), np.array(v, dtype=np.float32, copy=True)
+        am = lib().orc_adamw_update_f32(_p(p, C.c_float), _p(g, C.c_float), _p(mm, C.c_float), _p(vv, C.c_float), p.size, lr, beta1,
+                                        beta2, t, eps, wd, grad_scale)
+        return p, mm, vv, np.float32(am)
     p = np.array(params, dtype=np.uint16, copy=True)
     g = np.ascontiguousarray(grads, dtype=np.uint16)
     mm, vv = np.array(m, copy=True), np.array(v, copy=True)

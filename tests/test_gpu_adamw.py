@@ -174,3 +174,36 @@ def test_adamw_golden_known_answers(K):
     assert np.array_equal(host_bits(dp), g["fp8_p_out"]) and np.array_equal(host_bits(dv), g["fp8_v_out"])
     assert np.array_equal(ds.cpu().numpy().view(np.uint32), g["fp8_scales_out"].view(np.uint32))
     assert np.array_equal(dm.cpu().numpy(), g["fp8_m_out"])
+
+
+@pytest.mark.parametrize("n", [4, 1020, 8192 + 4, 1 << 20])
+def test_adamw_fp32_parameters_bit_exact(K, O, n):
+    """The all-fp32 overload (src/kernels/kernels.h:221-223): nothing is rounded stochastically, every operation is a
+    correctly rounded fp32 one -> parameters, moments and abs-max equal the oracle's bit for bit, whatever the seed;
+    the abs-max is merged into the slot; the reference's own check (rtol 1e-2 / atol 5e-3 against the float64
+    formulas, scripts/test_kernels.py:695-727) holds as well."""
+    rng = np.random.default_rng(n)
+    params, grads = (rng.standard_normal(n) * 0.05).astype(np.float32), (rng.standard_normal(n) * 2e-3).astype(np.float32)
+    m, v = (rng.standard_normal(n) * 1e-3).astype(np.float32), (rng.random(n) * 1e-5 + 1e-8).astype(np.float32)
+    lr, b1, b2, t, eps, wd, gsv = 3e-4, 0.9, 0.95, 7, 1e-8, 0.1, 0.625
+    want_p, want_m, want_v, want_am = O.adamw_update(params, grads, m, v, lr, b1, b2, t, eps, wd, gsv, 0)
+    gs = torch.tensor([gsv], dtype=torch.float32, device="cuda")
+    for seed in (0, 12345):
+        dp, dg, dm, dv = (torch.from_numpy(a.copy()).cuda() for a in (params, grads, m, v))
+        am = torch.zeros(1, dtype=torch.float32, device="cuda")
+        K.adamw_update(dp, dg, dm, dv, lr, b1, b2, t, eps, wd, gs, None, am, seed)
+        for got, want in ((dp, want_p), (dm, want_m), (dv, want_v)):
+            assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+        assert am.cpu().numpy().view(np.uint32)[0] == np.float32(want_am).view(np.uint32)
+    big = torch.full((1,), 1e6, dtype=torch.float32, device="cuda")
+    dp, dg, dm, dv = (torch.from_numpy(a.copy()).cuda() for a in (params, grads, m, v))
+    K.adamw_update(dp, dg, dm, dv, lr, b1, b2, t, eps, wd, gs, None, big, 0)
+    assert big.item() == 1e6                                                      # merged, not reset
+    g64, p64 = grads.astype(np.float64) * gsv, params.astype(np.float64)
+    m_new = b1 * m.astype(np.float64) + (1 - b1) * g64
+    v_new = b2 * v.astype(np.float64) + (1 - b2) * g64 ** 2
+    p_new = p64 * (1 - lr * wd) - lr * (m_new / (1 - b1 ** t)) / (np.sqrt(v_new / (1 - b2 ** t)) + eps)
+    assert np.allclose(want_p, p_new, rtol=1e-2, atol=5e-3) and np.allclose(want_p, p_new, rtol=1e-5, atol=1e-9)
+    with pytest.raises(ValueError, match="divisible by 4"):
+        f = lambda: torch.zeros(6, dtype=torch.float32, device="cuda")
+        K.adamw_update(f(), f(), f(), f(), lr, b1, b2, t, eps, wd, gs, None, None, 0)

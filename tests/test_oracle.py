@@ -588,6 +588,34 @@ def test_rope_vs_complex_multiplication(O):
     assert np.allclose(back[:, qk, half:], zz[:, qk].imag, rtol=1e-14, atol=1e-300)
 
 
+def test_adamw_fp32_parameters_vs_torch_formulas(O):
+    """The all-fp32 overload: the reference's test formulas (scripts/test_kernels.py:695-727) in float64; every output is
+    an fp32 evaluation of them (no stochastic rounding), so it agrees to a few fp32 ulp of the terms, and the abs-max is
+    that of the new parameters."""
+    n = 4096
+    rng = np.random.default_rng(3)
+    params, grads = rng.standard_normal(n).astype(np.float32), rng.standard_normal(n).astype(np.float32)
+    m0 = (rng.standard_normal(n) * 0.1).astype(np.float32)
+    v0 = (rng.random(n) * 0.01 + 1e-8).astype(np.float32)
+    lr, b1, b2, t, eps, wd, gs = 1e-3, 0.9, 0.999, 3, 1e-8, 0.1, 0.75
+    p1, m1, v1, am = O.adamw_update(params, grads, m0, v0, lr, b1, b2, t, eps, wd, gs, 42)
+    f = lambda x: np.float64(np.float32(x))
+    g, p, m, v = grads.astype(np.float64) * f(gs), params.astype(np.float64), m0.astype(np.float64), v0.astype(np.float64)
+    m_new = f(b1) * m + (1 - f(b1)) * g
+    v_new = f(b2) * v + (1 - f(b2)) * g ** 2
+    c1, c2 = np.float64(np.float32(1.0) / (np.float32(1.0) - np.float32(b1) ** np.float32(t))), np.float64(np.float32(1.0) / (np.float32(1.0) - np.float32(b2) ** np.float32(t)))
+    quot = (m_new * c1) / (np.sqrt(v_new * c2) + f(eps))
+    p_new = p - f(lr) * (quot + f(wd) * p)
+    assert p1.dtype == np.float32 and m1.dtype == np.float32 and v1.dtype == np.float32
+    assert np.all(np.abs(m1 - m_new) <= 2.0 ** -22 * (np.abs(m) + np.abs(g)))
+    assert np.all(np.abs(v1 - v_new) <= 2.0 ** -22 * (np.abs(v) + g ** 2))
+    assert np.all(np.abs(p1 - p_new) <= 2.0 ** -22 * (np.abs(p) + f(lr) * np.abs(quot)) + f(lr) * np.abs(quot) * 2.0 ** -20)
+    assert am == np.abs(p1).max()
+    # the seed plays no role
+    p2, _, _, _ = O.adamw_update(params, grads, m0, v0, lr, b1, b2, t, eps, wd, gs, 7)
+    assert np.array_equal(p1, p2)
+
+
 # ----------------------------------------------------------------------------- fp32 producer variants
 def test_fp32_producer_oracles_reduce_to_the_pinned_bf16_ones_and_match_torch(O):
     """The fp32 variants share the formula code of the bf16 ones (pinned above): on bf16-representable inputs their
