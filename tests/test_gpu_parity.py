@@ -796,6 +796,33 @@ def test_gemm_k_major_automatic_cut_on_a_weight_gradient_shape(K, mode):
     assert 0 < differing < 0.02, differing
 
 
+@pytest.mark.parametrize("mode", ["TT", "NN"])
+def test_gemm_k_major_operand_near_the_size_limit(K, mode):
+    """A K-major operand of 1.88 GB (the lane offsets of its copies are 32-bit and walk the whole operand; 2 GiB is the
+    documented limit): the result must equal mode TN on the transposed copy bit for bit, including the tiles whose
+    operand bytes lie at the far end."""
+    big, small, Kd = 57344, 256, 32768
+    M, N = (small, big) if mode == "TT" else (big, small)
+    g = torch.Generator(device="cuda").manual_seed(11)
+    codes = lambda r, c: torch.randint(0, 0x7E, (r, c), dtype=torch.uint8, device="cuda", generator=g)
+    a, b = codes(M, Kd), codes(N, Kd)
+    sa = dev_scalar(2.0 ** -9)
+    c_tn = torch.empty((N, M), dtype=torch.bfloat16, device="cuda")
+    K.matmul(c_tn, a, b, None, sa, None, M, N, Kd)
+    if mode == "TT":
+        b_km = b.t().contiguous()
+        del b
+        c_km = torch.full((N, M), float("nan"), dtype=torch.bfloat16, device="cuda")
+        K.matmul(c_km, a, b_km, None, sa, None, M, N, Kd, b_kmajor=True)
+    else:
+        a_km = a.t().contiguous()
+        del a
+        c_km = torch.full((N, M), float("nan"), dtype=torch.bfloat16, device="cuda")
+        K.matmul(c_km, a_km, b, None, sa, None, M, N, Kd, a_kmajor=True)
+    assert torch.equal(c_tn.view(torch.int16), c_km.view(torch.int16))
+    assert bool(torch.isfinite(c_km.float()).all()) and float(c_km.float().abs().max()) > 0
+
+
 def test_gemm_k_major_operand_rejects_what_it_cannot_serve(K):
     a = torch.zeros((256, 384), dtype=torch.uint8, device="cuda")
     b = torch.zeros((384, 256), dtype=torch.uint8, device="cuda")
