@@ -44,7 +44,8 @@ struct QmmRunState {
     // accumulate.  Which of them pay was measured on MLP layers of Qwen2.5-7B (C = 3584, FFN 18944), 1.5B (1536, 8960)
     // and a 2048 / 8192 layer at 4096 to 16384 tokens, every matmul with the 32 MiB workspace, against mode TN plus the
     // byte transposes it needs (2 bytes moved per element copied):
-    //  * weight gradient: a K-major second operand costs 3-6 % of the matmul, both operands K-major 2-10 %; the copies
+    //  * weight gradient: on the 7B layers a K-major second operand costs 3-4 % of the matmul and both operands K-major
+    //    2-9 % (up to 20 % on the 1.5B layers, whose small outputs mode TN serves with plans of its own); the copies
     //    cost more on every layer measured (7B at 8192 tokens: 442 -> 389 us in mode NT, 862 -> 778 us in mode TT with
     //    the activation's copy; 1.5B at 16384 tokens: 207 -> 181 us and 422 -> 340 us).  NT where the activation is the
     //    larger copy (OC <= 8192), else TT while the matmul stays small enough (C <= 8192).
