@@ -450,6 +450,25 @@ def main():
             "plain write-only kernel, same protocol (1 B/el)": cold_run(lambda i: capi.check(capi.testaid().llmq_debug_stream_u8(
                 qt_dsts[i].data_ptr(), None, n_h, 1, torch.cuda.current_stream().cuda_stream)), n_h),
         }
+        # Independent of this repository's kernels: what the vendor's own routines sustain under the same protocol
+        # (same tensors, same rotation, same event pairs) -- a device-to-device copy (torch's copy_, i.e. the HIP
+        # runtime's copy path) and two full reductions over the bf16 tensor (torch's amax and its infinity norm, which
+        # is an abs-max).  They bound what "a read stream" and "a 1:1 stream" reach on this chip from outside.
+        v_am = [torch.zeros((), dtype=torch.bfloat16, device=dev) for _ in srcs]
+        v_u8 = [x_.view(torch.uint8).view(-1) for x_ in q_srcs]
+        v_t8 = [x_.view(torch.uint8).view(-1) for x_ in qt_dsts]
+        v_bf = [x_.view(-1) for x_ in srcs]
+        v_dst = [torch.empty(n_h, dtype=torch.bfloat16, device=dev) for _ in srcs]
+        cold["vendor"] = {
+            "what": "torch / HIP runtime routines under the same protocol: copy_ between two 155 MB byte tensors and between "
+                    "two 310 MB bf16 tensors, torch.amax and torch.linalg.vector_norm(inf) over a 310 MB bf16 tensor",
+            "copy_ 155 MB bytes (2 B/el)": cold_run(lambda i: v_t8[i].copy_(v_u8[(i + 1) % 3]), 2 * n_h),
+            "copy_ 310 MB bf16 (4 B/el)": cold_run(lambda i: v_dst[i].copy_(v_bf[i]), 4 * n_h),
+            "amax over bf16 (2 B/el)": cold_run(lambda i: torch.amax(v_bf[i], 0, out=v_am[i]), 2 * n_h),
+            "vector_norm(inf) over bf16 = abs-max (2 B/el)": cold_run(
+                lambda i: torch.linalg.vector_norm(v_bf[i], float("inf"), out=v_am[i]), 2 * n_h),
+        }
+        del v_dst
         K.abs_max(stats["h"][0:1], t["h"])   # restore what the step left in the buffers used above
         K.quantize_with_abs_max(q["h"], stats["h"][1:2], t["h"], stats["h"][0:1])
         qtr(q["h_t"], "h")
@@ -494,6 +513,9 @@ def main():
                 tf = 2.0 * M_ * N_ * K_ / best / 1e6
                 secondary["%s %s (%d, %d, %d)" % (lname, kind, M_, N_, K_)] = {
                     "us": best, "TFLOPs": tf, "frac_fp8_peak": tf / FP8_PEAK_TFLOPS}
+    secondary_steps = None
+    if not args.no_graph:
+        secondary_steps = secondary_path_steps(K, torch, dev, ws)
     step_ms = (t1 - t0) * 1e3 / args.steps
 
     # What the matrix cores sustain with no memory traffic at all: a register-only MFMA loop on random
@@ -577,6 +599,7 @@ def main():
                     "weights, of h or of the output gradients"},
         "vendor_gemm": vendor,
         "secondary_gemm_shapes": secondary,
+        "secondary_steps": secondary_steps,
         "producers": swiglu,
         "library": capi.version(),
     }
@@ -587,6 +610,128 @@ def main():
         # part of this CPU leg, outside every timed region)
         result["gemm_error"] = gemm_error_report(error_samples, np)
     print(json.dumps(result))
+
+
+def secondary_path_steps(K, torch, dev, ws, iters=20):
+    """The whole path (not the matmul alone) on the layers of BASELINE.json's small configurations, where launches and
+    the extra passes weigh most: the Qwen2.5-0.5B block (qkv, o_proj, gate+up, down; 8192 tokens; bf16 dX, fp32 dW as
+    configuration 3 asks) and the Qwen2.5-1.5B MLP (gate+up, down; 16384 tokens).  Per linear and step, the reference's
+    sequence (src/models/llama_model.cpp:25-47, 309-339 and the weight quantization of llama_weights.cpp:207-223):
+    weight abs-max + quantize; forward: abs-max + quantize of x, matmul; backward: abs-max + quantize of dY, transpose
+    of W, dgrad matmul, quantize+transpose of x, transpose of dY, wgrad matmul.  Timed eagerly and replayed from a HIP
+    graph, next to the matmuls alone (the three matmul launches per linear and nothing else) and to the sequence with the single-read quantize + transposed copy for W and dY."""
+    f8, bf = torch.float8_e4m3fn, torch.bfloat16
+    gen = torch.Generator(device=dev).manual_seed(9)
+    models = {
+        "qwen2.5-0.5B block, 8192 tokens": (8192, [("qkv", 896, 1152), ("o_proj", 896, 896), ("gate_up", 896, 9728),
+                                                    ("down", 4864, 896)], torch.float32),
+        "qwen2.5-1.5B mlp, 16384 tokens": (16384, [("gate_up", 1536, 17920), ("down", 8960, 1536)], bf),
+    }
+    report = {"what": "full path steps (every abs-max / quantize / transpose launch and the three matmuls per linear, "
+                      "per-step weight quantization included), %d steps each after 3 warm-ups: eager, replayed from a HIP "
+                      "graph, the matmuls alone, and the sequence with the single-read quantize + transposed copy for "
+                      "weights and output gradients; launches = stream operations per step" % iters}
+
+    def ms_of(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        f0 = time.perf_counter()
+        for _ in range(iters):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - f0) * 1e3 / iters
+
+    for mname, (bt, linears, dw_dtype) in models.items():
+        L = []
+        for lname, cin, oc in linears:
+            d = {"cin": cin, "oc": oc}
+            d["x"] = torch.randn((bt, cin), device=dev, generator=gen).to(bf)
+            d["w"] = (torch.randn((oc, cin), device=dev, generator=gen) * 0.02).to(bf)
+            d["dy"] = (torch.randn((bt, oc), device=dev, generator=gen) * 1e-3).to(bf)
+            for k_, shp in (("xq", (bt, cin)), ("xq_t", (cin, bt)), ("wq", (oc, cin)), ("wq_t", (cin, oc)), ("dyq", (bt, oc)),
+                            ("dyq_t", (oc, bt))):
+                d[k_] = torch.empty(shp, dtype=f8, device=dev)
+            d["st"] = {k_: torch.zeros(2, device=dev) for k_ in ("x", "w", "dy")}
+            d["y"] = torch.empty((bt, oc), dtype=bf, device=dev)
+            d["dx"] = torch.empty((bt, cin), dtype=bf, device=dev)
+            d["dw"] = torch.empty((oc, cin), dtype=dw_dtype, device=dev)
+            L.append(d)
+        launches = [0]
+
+        def aq(d, name, src, dst):
+            K.abs_max(d["st"][name][0:1], src)
+            K.quantize_with_abs_max(dst, d["st"][name][1:2], src, d["st"][name][0:1])
+            launches[0] += 2
+
+        def mm(c, a, b, sa, sb, M, N, Kd):
+            K.matmul(c, a, b, None, sa, sb, M, N, Kd, workspace=ws)
+            launches[0] += 1
+
+        def matmuls(d, bt=bt):
+            s_ = d["st"]
+            mm(d["y"], d["wq"], d["xq"], s_["w"][1:2], s_["x"][1:2], d["oc"], bt, d["cin"])
+            mm(d["dx"], d["wq_t"], d["dyq"], s_["w"][1:2], s_["dy"][1:2], d["cin"], bt, d["oc"])
+            mm(d["dw"], d["xq_t"], d["dyq_t"], s_["x"][1:2], s_["dy"][1:2], d["cin"], d["oc"], bt)
+
+        def step(fused):
+            for d in L:
+                s_ = d["st"]
+                if fused:
+                    K.abs_max(s_["w"][0:1], d["w"])
+                    K.quantize_with_abs_max_and_transpose(d["wq"], d["wq_t"], s_["w"][1:2], d["w"], s_["w"][0:1])
+                    launches[0] += 2
+                else:
+                    aq(d, "w", d["w"], d["wq"])
+                aq(d, "x", d["x"], d["xq"])
+                mm(d["y"], d["wq"], d["xq"], s_["w"][1:2], s_["x"][1:2], d["oc"], bt, d["cin"])
+            for d in reversed(L):
+                s_ = d["st"]
+                if fused:
+                    K.abs_max(s_["dy"][0:1], d["dy"])
+                    K.quantize_with_abs_max_and_transpose(d["dyq"], d["dyq_t"], s_["dy"][1:2], d["dy"], s_["dy"][0:1])
+                    launches[0] += 2
+                else:
+                    aq(d, "dy", d["dy"], d["dyq"])
+                    K.transpose(d["wq_t"], d["wq"])
+                    launches[0] += 1
+                mm(d["dx"], d["wq_t"], d["dyq"], s_["w"][1:2], s_["dy"][1:2], d["cin"], bt, d["oc"])
+                K.quantize_and_transpose_with_abs_max(d["xq_t"], None, d["x"], s_["x"][0:1])
+                launches[0] += 1
+                if not fused:
+                    K.transpose(d["dyq_t"], d["dyq"])
+                    launches[0] += 1
+                mm(d["dw"], d["xq_t"], d["dyq_t"], s_["x"][1:2], s_["dy"][1:2], d["cin"], d["oc"], bt)
+
+        def count(fn):
+            launches[0] = 0
+            fn()
+            return launches[0]
+
+        flop = sum(6.0 * bt * d["cin"] * d["oc"] for d in L)
+        n_ref, n_fused = count(lambda: step(False)), count(lambda: step(True))
+        eager = ms_of(lambda: step(False))
+        fused = ms_of(lambda: step(True))
+        only = ms_of(lambda: [matmuls(d) for d in L])
+        graphs = {}
+        for label, fz in (("reference sequence", False), ("single-read quantize + transposed copy", True)):
+            g_ = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g_):
+                step(fz)
+            graphs[label] = ms_of(g_.replay)
+            del g_
+        report[mname] = {
+            "gemm_flop_per_step": flop,
+            "reference sequence": {"launches": n_ref, "eager_ms": eager, "hip_graph_ms": graphs["reference sequence"],
+                                   "TFLOPs_eager": flop / eager / 1e9, "TFLOPs_hip_graph": flop / graphs["reference sequence"] / 1e9},
+            "single-read quantize + transposed copy": {
+                "launches": n_fused, "eager_ms": fused, "hip_graph_ms": graphs["single-read quantize + transposed copy"],
+                "TFLOPs_hip_graph": flop / graphs["single-read quantize + transposed copy"] / 1e9},
+            "matmuls_alone_ms": only, "TFLOPs_matmuls_alone": flop / only / 1e9,
+            "non_matmul_share_of_eager_step": 1.0 - only / eager,
+        }
+        del L
+    return report
 
 
 def measured_traffic():

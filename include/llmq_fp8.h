@@ -41,11 +41,17 @@ const char* llmq_target_arch(void);
 
 /*
  * *out = max_i |in[i]| as fp32 (NaNs ignored, |+-Inf| wins, result >= +0; 0 for n == 0).
- * The slot is reset first, then reduced into, all on `stream`.
+ * One kernel launch on `stream`: whatever the slot held before is overwritten (no clearing needed, none done).
+ * The workgroups meet in one of LLMQ_ABS_MAX_ARRIVAL_AREAS arrival areas built into the device code, selected by
+ * ((uintptr_t)out / 4) % LLMQ_ABS_MAX_ARRIVAL_AREAS.  Calls on one stream, or ordered by events, may share an area.
+ * Calls that can run at the same time on one GPU (different streams, nothing ordering them) must use result slots
+ * that map to different areas -- any two slots less than 256 bytes apart do -- or they race on the arrival counter
+ * (the reference's memset + atomic-max form has no such limit; its abs-max calls all sit on the one compute stream).
  * Replaces: abs_max(float*, const nv_bfloat16*, long, const cudaDeviceProp&, cudaStream_t)
  *           src/kernels/kernels.h:247, src/kernels/quant.cu:107-109 (kernel :11-28).
  * n may be any non-negative count (the reference requires n % 8 == 0).
  */
+#define LLMQ_ABS_MAX_ARRIVAL_AREAS 64
 int llmq_abs_max_bf16(float* out, const uint16_t* in, int64_t n, void* stream);
 
 /* fp32 input variant.  Replaces abs_max(float*, const float*, long, ...) src/kernels/kernels.h:246,
@@ -210,7 +216,9 @@ int llmq_backward_bias_bf16(uint16_t* dbias, const void* dout, int dout_format, 
  * GPU, held until the process ends); the call allocates and frees nothing.  A shape whose band sums
  * (llmq_backward_bias_scratch_bytes) exceed that size is refused with LLMQ_ERR_INVALID_ARGUMENT.  All calls on one
  * GPU share the array: calls that overlap there (different streams, no ordering between them) race; the array
- * needs no clearing between calls (every call overwrites what it reads).
+ * needs no clearing between calls (every call overwrites what it reads).  The first call on a device looks up the
+ * array's device address (a host-side query under a mutex, not a stream operation): make one ordinary call per device
+ * before capturing this entry point into a HIP graph; every later call enqueues its two kernels and nothing else.
  */
 #define LLMQ_BACKWARD_BIAS_STATIC_SCRATCH_BYTES ((size_t)16 << 20)
 int llmq_backward_bias_bf16_static_scratch(uint16_t* dbias, const void* dout, int dout_format, const float* sa_or_null,
@@ -360,8 +368,8 @@ int llmq_rmsnorm_backward_f32(float* dinp, float* dweight, void* scratch, size_t
  * Replaces: adamw_update(nv_bfloat16* params, const nv_bfloat16* grads, {float|nv_bfloat16}* m, {float|nv_bfloat16}* v,
  *           size_t num_parameters, float learning_rate, float beta1, float beta2, int t, float eps, float weight_decay,
  *           const float* grad_scale, float* abs_max, unsigned int seed, cudaStream_t)
- *           src/kernels/kernels.h:225-235, src/kernels/adamw.cu:18-195.  Not provided: fp32 parameters
- *           (kernels.h:221); the e4m3 first moment is llmq_adamw_update_bf16_fp8m below.
+ *           src/kernels/kernels.h:225-235, src/kernels/adamw.cu:18-195.  The e4m3 first moment is
+ *           llmq_adamw_update_bf16_fp8m and fp32 parameters (kernels.h:221) are llmq_adamw_update_f32, both below.
  */
 int llmq_adamw_update_bf16(uint16_t* params, const uint16_t* grads, void* m, int m_dtype, void* v, int v_dtype,
                            int64_t num_parameters, float learning_rate, float beta1, float beta2, int t, float eps,

@@ -6,8 +6,8 @@
 //     nv_bfloat16 -> __hip_bfloat16        __nv_fp8_e4m3 -> __hip_fp8_e4m3     __nv_fp8_e5m2 -> __hip_fp8_e5m2
 //     cudaStream_t -> hipStream_t          cudaDeviceProp -> hipDeviceProp_t   cublasLtHandle_t -> llmqBlasHandle_t
 // The device-property and handle arguments are accepted and ignored.  The matmul workspace is passed
-// through: the gfx950 GEMM uses it for split-K partial sums when the output has too few tiles to fill
-// the chip, and works without one.  Errors surface as the reference's exception types:
+// through: the gfx950 GEMM keeps raw fp32 partial tiles there when it splits K (outputs with too few tiles to fill the
+// chip) and when it cuts a last, partial round of tiles into K segments (all operand modes); it works without one.  Errors surface as the reference's exception types:
 // std::invalid_argument for shape / dtype / argument errors, std::runtime_error for runtime failures.
 #ifndef LLMQ_KERNELS_HPP
 #define LLMQ_KERNELS_HPP

@@ -48,6 +48,13 @@ def _compile(unit):
     return obj, out
 
 
+def _hazard_scan(_unit=None):
+    """The GEMM file compiled to assembly text and scanned for the two hazards its inline-asm copies could meet
+    (asm_check.py); runs beside the object compiles.  A violation raises and nothing is linked."""
+    from llmq_amd import asm_check
+    return asm_check.check_source(HIPCC, FLAGS, os.path.join(CSRC, "gemm_e4m3.hip"), os.path.join(OBJ, "gemm_e4m3.hazard_scan.s"))
+
+
 def _link(lib, objs):
     subprocess.check_call([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,-Bsymbolic",
                            "-Wl,--version-script=" + os.path.join(CSRC, "exports.map"), "-o", lib] + objs)
@@ -59,7 +66,11 @@ def build(verbose=True):
     units = [(s, s.replace(".hip", ".o"), []) for s in SOURCES]
     extra_units = [u for u in TESTAID_UNITS if u[1] not in {n for _, n, _ in units}]
     with ThreadPoolExecutor(max_workers=8) as ex:
+        scan = ex.submit(_hazard_scan)
         results = dict(zip([u[1] for u in units + extra_units], ex.map(_compile, units + extra_units)))
+        kernels, copies = scan.result()   # raises on a hazard: nothing is linked
+    if verbose:
+        print("hazard scan of the four-wave GEMM: %d kernel instances, %d copies, clean" % (kernels, copies))
     for obj, out in results.values():
         if verbose and out.strip():
             print(out)

@@ -582,8 +582,9 @@ __device__ __forceinline__ int frag_swizzle(int row) {
 // distance of 4 rows; the workgroup barrier sits after row 4, where every read of the current stage has
 // been issued (and awaited) and the copies for step s+2 may overwrite it.
 // The workgroup is persistent (one per compute unit, walking its XCD's tile list) and the stream of
-// K-steps and copies runs across tile boundaries.  Needs K to be a multiple of 256: the LDS stage and the
-// fb half of a step are then compile-time functions of the step's parity.
+// K-steps and copies runs across tile boundaries.  With an even number of K-steps per tile the LDS stage and the fb
+// half of a step are compile-time functions of the step's parity; the ODDK instances (below) carry the stage as a
+// run-time value.
 //
 // NJ < 8 narrows the tile along m to 2 * 16 * NJ columns (NJ second-operand fragments per wave instead of 8): a
 // shape whose 256-wide tiles fill the last round of the chip badly can have a tile count that divides evenly

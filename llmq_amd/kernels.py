@@ -112,16 +112,15 @@ def transpose(dst, src, stream=0):
     capi.check(capi.lib.llmq_transpose_u8(d, s, src.shape[0], src.shape[1], _stream(stream)))
 
 
-def matmul(c, a, b, bias, scale_a, scale_b, M, N, K, accumulate=False, stream=0, workspace=None, b_e5m2=False, _lib=None,
+def matmul(c, a, b, bias, scale_a, scale_b, M, N, K, accumulate=False, stream=0, workspace=None, b_e5m2=False,
            b_kmajor=False, a_kmajor=False):
     """TN matmul in the convention of the reference's kernels.h: row-major a[M,K], b[N,K] (e4m3) give
     row-major c[N,M] = (b @ a.T) * scale_a * scale_b (+ bias[M]) (+ c).  c: bf16 or fp32.
     workspace: optional device byte tensor (the reference passes a 32 MiB one); it enables the
     split-K path for outputs with too few tiles to fill the chip and the cut of a last, partial round of tiles into
     K segments (all operand modes).  b may hold e5m2 codes (the gradient
-    dtype option): a float8_e5m2 tensor, or uint8 with b_e5m2=True.  _lib: tests pass the test-aid build of
-    the same entry points (capi.testaid()) to force a kernel variant; everyone else leaves it alone."""
-    L = _lib or capi.lib
+    dtype option): a float8_e5m2 tensor, or uint8 with b_e5m2=True."""
+    L = capi.lib
     pws, ws_bytes = None, 0
     if workspace is not None:
         pws = _dev(workspace, "workspace", (torch.uint8, torch.int8, torch.float32))
@@ -137,6 +136,8 @@ def matmul(c, a, b, bias, scale_a, scale_b, M, N, K, accumulate=False, stream=0,
         if a.numel() != M * K or b.numel() != N * K or c.numel() != N * M:
             raise ValueError("operand sizes do not match M, N, K")
         pbias = _dev(bias, "bias", (torch.bfloat16,), optional=True)
+        if bias is not None and bias.numel() != M:
+            raise ValueError("bias must have M elements")
         capi.check(L.llmq_gemm_e4m3_bf16_mode(
             _dev(c, "c", (torch.bfloat16,)), pa, pb, pbias, _dev(scale_a, "scale_a", (torch.float32,), optional=True),
             _dev(scale_b, "scale_b", (torch.float32,), optional=True), pws, ws_bytes, M, N, K,

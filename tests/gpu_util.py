@@ -1,9 +1,27 @@
 """Helpers shared by the GPU parity tests: host<->device moves of raw bit patterns and the GEMM
 tolerance of the path (stated once, here)."""
+import contextlib
 import os
 
 import numpy as np
 import torch
+
+
+@contextlib.contextmanager
+def gemm_library(lib):
+    """Runs llmq_amd.kernels on `lib` instead of the product library for the duration of the block (None: no change).
+    The parity tests pass the test-aid build of the GEMM entry points (capi.testaid()), whose kernel selection can be
+    forced; the product wrapper itself has no such switch."""
+    from llmq_amd import capi
+    if lib is None:
+        yield
+        return
+    saved = capi.lib
+    capi.lib = lib
+    try:
+        yield
+    finally:
+        capi.lib = saved
 
 
 def dev_bf16(bits):

@@ -1,55 +1,42 @@
-"""The four-wave GEMM issues its global->LDS copies from inline-asm statements.  The compiler does not know that
-such a statement is a memory instruction that reads scalar registers, so its hazard recognizer does not keep the
-5 wait states the hardware needs between a vector instruction writing a scalar register (v_readlane reloading a
-spilled scalar, v_readfirstlane) and a memory instruction reading it, nor is it asked to keep the one wait state
-between a write of M0 and the copy that takes its LDS destination from M0.  The kernel is written so that neither
-happens (no scalar of the copy stream is spilled; a matrix instruction or an LDS read sits between the write of
-M0 and the copy); this test compiles the file to assembly and checks both distances for every copy (a stale
-scalar means a wrong address: wrong data or a memory fault)."""
+"""The hazard scan of the four-wave GEMM's generated code (llmq_amd/asm_check.py), run on its own: the scanner's
+parsing on hand-written snippets, and the scan of the product source compiled to assembly (the library build runs
+the same scan and refuses to link on a violation)."""
 import os
-import re
-import subprocess
 
-ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+import pytest
+
+from llmq_amd import asm_check
 
 
-def instructions(body):
-    out = []
-    for line in body.split("\n"):
-        l = line.strip()
-        if l and not l.startswith(";") and not l.startswith(".") and not l.endswith(":"):
-            out.append(l)
-    return out
+def _kernel(body):
+    return "_Z4demow4_kernelv:\n" + body + "\n.end_amdhsa_kernel\n"
+
+
+def test_scanner_parses_scalar_destinations():
+    d = asm_check.scalar_destinations
+    assert d("v_readlane_b32 s10, v3, 0") == {"s10"}
+    assert d("v_readfirstlane_b32 s7, v1") == {"s7"}
+    assert d("v_cmp_lt_u32_e64 s[10:11], v1, v2") == {"s10", "s11"}
+    assert "vcc" in d("v_cmp_eq_u32_e32 vcc, v1, v2")
+    assert "vcc" in d("v_cmp_eq_u32 v1, v2")
+    assert d("v_add_u32 v1, v2, v3") == set()
+
+
+def test_scanner_flags_each_hazard():
+    filler = "\n".join("v_mov_b32 v1, v2" for _ in range(6))
+    ok = _kernel("s_add_i32 m0, s3, 16\nv_mov_b32 v1, v2\n" + filler + "\nglobal_load_lds_dwordx4 v5, s[10:11]")
+    asm_check.check_text(ok, min_kernels=1, min_copies=1)
+    with pytest.raises(AssertionError, match="M0 written right in front"):
+        asm_check.check_text(_kernel(filler + "\ns_add_i32 m0, s3, 16\nglobal_load_lds_dwordx4 v5, s[10:11]"), 1, 1)
+    with pytest.raises(AssertionError, match="wait states"):
+        asm_check.check_text(_kernel(filler + "\nv_readlane_b32 s11, v9, 3\nv_mov_b32 v1, v2\nglobal_load_lds_dwordx4 v5, s[10:11]"), 1, 1)
+    with pytest.raises(AssertionError, match="wait states"):   # a lane mask written as a register pair
+        asm_check.check_text(_kernel(filler + "\nv_cmp_lt_u32_e64 s[10:11], v1, v2\nv_mov_b32 v1, v2\nglobal_load_lds_dwordx4 v5, s[10:11]"), 1, 1)
+    # five wait states (an s_nop counts its argument + 1) are enough
+    asm_check.check_text(_kernel(filler + "\nv_readlane_b32 s11, v9, 3\ns_nop 4\nglobal_load_lds_dwordx4 v5, s[10:11]"), 1, 1)
 
 
 def test_lds_copies_keep_their_distance_from_scalar_writes(tmp_path):
     from llmq_amd import build as B
-    asm = tmp_path / "gemm.s"
-    cmd = [B.HIPCC] + [f for f in B.FLAGS if not f.startswith("-W")] + [
-        "--cuda-device-only", "-S", os.path.join(B.CSRC, "gemm_e4m3.hip"), "-o", str(asm)]
-    subprocess.run(cmd, check=True, capture_output=True)
-    text = asm.read_text()
-    kernels = re.findall(r"^(_Z\S*w4_kernel\S*):[^\n]*\n(.*?)\.end_amdhsa_kernel", text, re.S | re.M)
-    assert len(kernels) >= 10
-    copies = 0
-    for name, body in kernels:
-        ins = instructions(body)
-        for i, l in enumerate(ins):
-            if not l.startswith("global_load_lds"):
-                continue
-            copies += 1
-            m = re.search(r"s\[(\d+):(\d+)\]", l)
-            regs = {"s%d" % r for r in range(int(m.group(1)), int(m.group(2)) + 1)} | {"m0"}
-            assert not re.match(r"s_\w+ m0,", ins[i - 1]), "%s: M0 written right in front of '%s'" % (name, l)
-            wait, j = 0, i - 1
-            while j >= 0 and wait < 5:
-                p = ins[j]
-                if p.startswith("s_nop"):
-                    wait += int(p.split()[1]) + 1
-                else:
-                    if p.startswith(("v_readlane", "v_readfirstlane", "v_cmp")):
-                        assert p.split()[1].rstrip(",") not in regs, "%s: '%s' only %d wait states before '%s'" % (
-                            name, p, wait, l)
-                    wait += 1
-                j -= 1
-    assert copies >= 1000
+    kernels, copies = asm_check.check_source(B.HIPCC, B.FLAGS, os.path.join(B.CSRC, "gemm_e4m3.hip"), str(tmp_path / "gemm.s"))
+    assert kernels >= 10 and copies >= 1000

@@ -18,7 +18,7 @@ import numpy as np
 import pytest
 import torch
 
-from gpu_util import ACC_TERM
+from gpu_util import ACC_TERM, gemm_library
 
 pytestmark = pytest.mark.gpu
 
@@ -45,7 +45,8 @@ def gemm_f32(variant, a, b):
     try:
         M, N = a.shape[0], b.shape[0]
         c = torch.full((N, M), float("nan"), dtype=torch.float32, device="cuda")
-        K.matmul(c, torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda(), None, None, None, M, N, a.shape[1], _lib=lib)
+        with gemm_library(lib):
+            K.matmul(c, torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda(), None, None, None, M, N, a.shape[1])
         torch.cuda.synchronize()
         return c.cpu().numpy().astype(np.float64)
     finally:

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 import torch
 
-from gpu_util import dev_bf16, dev_scalar, dev_u8, gemm_check, host_bits, report_gemm_error
+from gpu_util import dev_bf16, dev_scalar, dev_u8, gemm_check, gemm_library, host_bits, report_gemm_error
 
 pytestmark = pytest.mark.gpu
 
@@ -68,6 +68,55 @@ def test_abs_max_f32(K):
     out = torch.zeros(1, device="cuda")
     K.abs_max(out, x)
     assert out.item() == torch.nan_to_num(x, nan=0.0).abs().max().item()
+
+
+def test_abs_max_single_launch_arrival_area_is_reusable(K):
+    """abs_max is one launch: the workgroups meet in an arrival area of the device code that the last of them
+    leaves ready for the next call.  A run of calls of different sizes into ONE result slot (one area: many
+    workgroups, few, one, many again) must each give the exact maximum, whatever the slot and the area held before."""
+    g = torch.Generator(device="cuda").manual_seed(21)
+    out = torch.full((1,), float("nan"), device="cuda")
+    big = torch.randn(40 * 1000 * 1000 + 24, device="cuda", generator=g).to(torch.bfloat16)
+    for rep in range(3):
+        for n in (big.numel(), 3 * 1000 * 1000 + 5, 65536, 64, 65537, 9 * 65536, big.numel() - 8):
+            x = big[:n] * float(1 + rep)
+            K.abs_max(out, x)
+            assert out.item() == x.float().abs().max().item(), (rep, n)
+    # the maximum hidden in every workgroup's share in turn (a workgroup covers 65536 elements)
+    x = torch.zeros(20 * 65536, dtype=torch.bfloat16, device="cuda")
+    for blk in range(20):
+        x.zero_()
+        x[blk * 65536 + 4321] = -3.0
+        K.abs_max(out, x)
+        assert out.item() == 3.0, blk
+
+
+def test_abs_max_beyond_the_workgroup_cap(K):
+    """More elements than 8192 workgroups cover in one trip (1 GiB of bf16): the grid is capped and loops."""
+    n = 8192 * 65536 + 3 * 65536 + 40
+    x = torch.zeros(n, dtype=torch.bfloat16, device="cuda")
+    out = torch.zeros(1, device="cuda")
+    for pos, v in ((5, 1.5), (8192 * 65536 + 77, -2.5), (n - 1, 7.0)):
+        x[pos] = v
+        K.abs_max(out, x)
+        assert out.item() == abs(v)
+    del x
+
+
+def test_abs_max_neighbouring_slots_on_two_streams(K):
+    """Result slots 4 bytes apart (the [abs_max, ...] tables of the reference's run state) map to different arrival
+    areas, so their calls may overlap in time: two streams, no ordering between them, 40 rounds."""
+    g = torch.Generator(device="cuda").manual_seed(22)
+    xs = [torch.randn(6 * 1000 * 1000, device="cuda", generator=g).to(torch.bfloat16) * s for s in (1.0, 3.0)]
+    want = [x.float().abs().max().item() for x in xs]
+    table = torch.zeros(2, device="cuda")
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    torch.cuda.synchronize()
+    for rnd in range(40):
+        for i, st in enumerate(streams):
+            K.abs_max(table[i:i + 1], xs[i], stream=st.cuda_stream)
+    torch.cuda.synchronize()
+    assert table.tolist() == want
 
 
 # ----------------------------------------------------------------------------------------- quantize
@@ -217,7 +266,8 @@ def set_variant(v):
 
 def mm(K, *args, **kw):
     """K.matmul on whichever library set_variant selected."""
-    return K.matmul(*args, _lib=_FORCED["lib"], **kw)
+    with gemm_library(_FORCED["lib"]):
+        return K.matmul(*args, **kw)
 
 
 # (tile selector, K splits[, persistent walk]); for the four-wave kernel (tile 3) the second number cuts the
@@ -796,6 +846,43 @@ def test_gemm_k_major_automatic_cut_on_a_weight_gradient_shape(K, mode):
     assert 0 < differing < 0.02, differing
 
 
+def test_product_library_cuts_the_last_round_into_k_segments(K):
+    """The K-segment instance of the four-wave kernel, reached on the product library through the automatic plan (no
+    forced variant): 18944 x 3584 x 8192 leaves one or two tiles per XCD for the last round, and with a workspace the
+    plan cuts them.  Proof that the segment launch ran: it is the only kernel that writes the workspace, so the
+    workspace (filled with a pattern no partial sum has) must afterwards hold 12 S partial tiles of 256 KiB (XCDs 0-3
+    have two last-round tiles, XCDs 4-7 one; S segments each), S >= 2, in the places the plan reserves per XCD.
+    Integer-valued operands: every sum is exact in fp32 in any order, so the cut result must equal the uncut one and
+    the int64 product bit for bit."""
+    M, N, Kd = 18944, 3584, 8192
+    g = torch.Generator(device="cuda").manual_seed(77)
+    ints = torch.tensor([0x00, 0x38, 0x40, 0x44, 0x48, 0xB8, 0xC0, 0xC4], dtype=torch.uint8, device="cuda")   # 0, 1, 2, 3, 4, -1, -2, -3
+    vals = torch.tensor([0, 1, 2, 3, 4, -1, -2, -3], dtype=torch.float64)
+    ia = torch.randint(0, 8, (M, Kd), device="cuda", generator=g)
+    ib = torch.randint(0, 8, (N, Kd), device="cuda", generator=g)
+    a, b = ints[ia], ints[ib]
+    ws = torch.full((32 << 20,), 0xFF, dtype=torch.uint8, device="cuda")
+    c_cut = torch.full((N, M), float("nan"), dtype=torch.float32, device="cuda")
+    K.matmul(c_cut, a, b, None, None, None, M, N, Kd, workspace=ws)
+    c_whole = torch.full((N, M), float("nan"), dtype=torch.float32, device="cuda")
+    K.matmul(c_whole, a, b, None, None, None, M, N, Kd)
+    torch.cuda.synchronize()
+    touched = (ws.view(128, 256 * 1024) != 0xFF).any(dim=1).cpu().numpy()
+    n_touched = int(touched.sum())
+    assert n_touched >= 24 and n_touched % 12 == 0, n_touched        # 12 tiles x S segments, S >= 2
+    S = n_touched // 12
+    expect = np.zeros(128, dtype=bool)
+    for xcd in range(8):
+        rem = 2 if xcd < 4 else 1
+        expect[xcd * 2 * S: xcd * 2 * S + rem * S] = True            # part_per_xcd = rem_max * S = 2 S
+    assert np.array_equal(touched, expect), (S, np.flatnonzero(touched))
+    assert torch.equal(c_cut, c_whole)
+    # the last-round tiles and a sample of the others against the int64 product
+    rows = np.r_[0:8, 1700:1708, N - 256:N - 248, N - 8:N]
+    want = (vals[ib[rows].cpu()] @ vals[ia.cpu()].T).numpy()
+    assert np.array_equal(c_cut[rows].cpu().numpy().astype(np.float64), want)
+
+
 @pytest.mark.parametrize("mode", ["TT", "NN"])
 def test_gemm_k_major_operand_near_the_size_limit(K, mode):
     """A K-major operand of 1.88 GB (the lane offsets of its copies are 32-bit and walk the whole operand; 2 GiB is the
@@ -834,6 +921,11 @@ def test_gemm_k_major_operand_rejects_what_it_cannot_serve(K):
                  None, None, None, 256, 256, 512, accumulate=True, a_kmajor=True)
     with pytest.raises(ValueError, match="bf16 output"):
         K.matmul(c.float(), a, b, None, None, None, 256, 256, 384, b_kmajor=True)
+    # a bias that is too short would be read out of bounds by the epilogue: refused by the wrapper in every operand mode
+    short_bias = torch.zeros(128, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ValueError, match="bias must have M elements"):
+        K.matmul(c, torch.zeros((256, 256), dtype=torch.uint8, device="cuda"), torch.zeros((256, 256), dtype=torch.uint8, device="cuda"),
+                 short_bias, None, None, 256, 256, 256, b_kmajor=True)
     # a K-major operand of 2 GiB or more is refused before anything is launched (32-bit lane offsets walk it);
     # called through the C ABI with the sizes alone, no such tensor is allocated
     from llmq_amd import capi
@@ -946,6 +1038,15 @@ def test_config1_forward_pipeline(K, O):
     scale = np.float32(dw * dx)
     max_abs, fro = gemm_check(got, ex, sabs, scale, True)
     report_gemm_error("config1", "forward y", BT, OC, C, max_abs, fro, "%d sampled outputs incl. boundary rows/columns" % idx_n.size)
+    # Every one of the 4096 x 4864 outputs: the exact product as a float64 matrix product of the decoded codes (every
+    # e4m3 product and every partial sum of 896 of them fits 53 bits, so the library routine returns the exact sums
+    # in any order), tied to the oracle's exact sums on the sampled coordinates above.
+    xf, wf = O.e4m3_decode(xq_o).astype(np.float64), O.e4m3_decode(wq_o).astype(np.float64)
+    ex_all, sabs_all = xf @ wf.T, np.abs(xf) @ np.abs(wf).T
+    assert np.array_equal(ex_all[idx_n, idx_m], ex) and np.array_equal(sabs_all[idx_n, idx_m], sabs)
+    max_abs_all, fro_all = gemm_check(y.float().cpu().numpy(), ex_all, sabs_all, scale, True)
+    report_gemm_error("config1", "forward y (all outputs)", BT, OC, C, max_abs_all, fro_all, "all %d outputs" % (BT * OC))
+    del xf, wf, ex_all, sabs_all
     # closeness to the unquantised product, as a sanity check of the whole path (fp8 noise ~ 3-4 %)
     ref = (O.bf16_to_f32(x)[idx_n[:2000]].astype(np.float64) * O.bf16_to_f32(w)[idx_m[:2000]].astype(np.float64)).sum(1)
     rel = np.linalg.norm(got[:2000] - ref) / np.linalg.norm(ref)

@@ -59,3 +59,36 @@ def test_static_scratch_rejects_oversized_shape():
     rc = capi.lib.llmq_backward_bias_bf16_static_scratch(p, p, 0, None, None, BT, OC, None)
     assert rc == capi.LLMQ_ERR_INVALID_ARGUMENT
     assert b"built-in scratch" in capi.lib.llmq_last_error()
+
+
+def test_static_scratch_entry_replays_from_a_hip_graph():
+    """After one ordinary call on the device (the first call looks up the built-in array's address, a host-side
+    query), the entry point is two kernel launches and nothing else: captured into a HIP graph and replayed three
+    times with eager work in between, every replay must equal the eager result bit for bit."""
+    from llmq_amd import capi
+    BT, OC, fmt = 4096, 2304, 0
+    g = torch.Generator(device="cuda").manual_seed(5)
+    codes = torch.randint(0, 256, (BT, OC), device="cuda", dtype=torch.uint8, generator=g)
+    dout = torch.where((codes & 0x7F) == 0x7F, codes ^ 0x40, codes)          # no NaN codes
+    sa, sb = torch.tensor([0.5], device="cuda"), torch.tensor([0.25], device="cuda")
+    start = torch.randn(OC, device="cuda", generator=g).to(torch.bfloat16)
+
+    def call(dbias):
+        capi.check(capi.lib.llmq_backward_bias_bf16_static_scratch(dbias.data_ptr(), dout.data_ptr(), fmt, sa.data_ptr(),
+                                                                   sb.data_ptr(), BT, OC, torch.cuda.current_stream().cuda_stream))
+
+    want = start.clone()
+    call(want)                                   # the eager call every capture must be preceded by
+    torch.cuda.synchronize()
+    got = start.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(got)
+    for _ in range(3):
+        got.copy_(start)
+        other = start.clone()
+        call(other)                              # eager use of the same array between the replays
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+        assert torch.equal(other.view(torch.int16), want.view(torch.int16))
