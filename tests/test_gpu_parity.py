@@ -82,17 +82,17 @@ def test_abs_max_single_launch_arrival_area_is_reusable(K):
             x = big[:n] * float(1 + rep)
             K.abs_max(out, x)
             assert out.item() == x.float().abs().max().item(), (rep, n)
-    # the maximum hidden in every workgroup's share in turn (a workgroup covers 65536 elements)
-    x = torch.zeros(20 * 65536, dtype=torch.bfloat16, device="cuda")
-    for blk in range(20):
+    # the maximum hidden in every workgroup's chunk in turn (a chunk is 16384 elements)
+    x = torch.zeros(40 * 16384 + 8, dtype=torch.bfloat16, device="cuda")
+    for blk in range(41):
         x.zero_()
-        x[blk * 65536 + 4321] = -3.0
+        x[min(blk * 16384 + 4321, x.numel() - 1)] = -3.0
         K.abs_max(out, x)
         assert out.item() == 3.0, blk
 
 
 def test_abs_max_beyond_the_workgroup_cap(K):
-    """More elements than 8192 workgroups cover in one trip (1 GiB of bf16): the grid is capped and loops."""
+    """A tensor of more than 1 GiB: every workgroup of the capped grid walks many chunks, 64-bit element offsets."""
     n = 8192 * 65536 + 3 * 65536 + 40
     x = torch.zeros(n, dtype=torch.bfloat16, device="cuda")
     out = torch.zeros(1, device="cuda")
