@@ -92,7 +92,7 @@ _testaid = None
 def testaid():
     """The test-aid library (tests and bench.py only; never needed by a user of the path): the matmul
     entry points from a build of the GEMM file whose kernel selection can be forced
-    (llmq_debug_set_gemm_variant / llmq_debug_set_gemm_persist), and the measurement aids llmq_debug_copy_u8 and llmq_debug_stream_u8
+    (llmq_debug_set_gemm_variant / llmq_debug_set_gemm_persist / llmq_debug_set_gemm_fuse), and the measurement aids llmq_debug_copy_u8 and llmq_debug_stream_u8
     (plain copy, read-only and write-only kernels) and llmq_debug_mfma_ceiling (register-only matrix-instruction loop)."""
     global _testaid
     if _testaid is None:
@@ -108,6 +108,8 @@ def testaid():
         t.llmq_debug_set_gemm_variant.restype = None
         t.llmq_debug_set_gemm_persist.argtypes = [_int]
         t.llmq_debug_set_gemm_persist.restype = None
+        t.llmq_debug_set_gemm_fuse.argtypes = [_int]
+        t.llmq_debug_set_gemm_fuse.restype = None
         t.llmq_debug_copy_u8.argtypes = [_vp, _vp, _i64, _vp]
         t.llmq_debug_copy_u8.restype = _int
         t.llmq_debug_stream_u8.argtypes = [_vp, _vp, _i64, _int, _vp]

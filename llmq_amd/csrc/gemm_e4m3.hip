@@ -613,9 +613,11 @@ __device__ __forceinline__ int frag_swizzle(int row) {
 // fragment row into a private 4 KiB piece of LDS, read back as 16 bytes per lane and row.  bf16 output without
 // accumulation (the old values of c would have to be fetched in the scattered layout).
 template <typename OutT, int B_FMT, bool SEG, int NJ = 8, bool STREAM_OUT = true, bool ODDK = false, bool KMB = false,
-          bool KMA = false>
+          bool KMA = false, bool FUSE_EPI = false>
 __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     static_assert(!(SEG && ODDK), "K segments are whole pairs of K-steps");
+    static_assert(!FUSE_EPI || (NJ == 8 && !SEG && !KMA && std::is_same_v<OutT, uint16_t>),
+                  "the epilogue under the last K-step is written for full-width bf16 tiles of K-contiguous a");
     static_assert(!((KMB || KMA) && ODDK), "the K-major operand modes are built for even K-step counts");
     static_assert(!KMA || (NJ == 8 && (SEG || std::is_same_v<OutT, uint16_t>)),
                   "the K-major first operand is built for 256-wide tiles and bf16 output (fp32 only as K segments)");
@@ -910,6 +912,57 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     // released at the start of the step and the landing barrier moves to row 6 (copies have 7 to 14 rows): 1-4 % slower,
     // the 32 extra live registers push address registers into scratch around the tile epilogue.  Shorter copy windows
     // (rows 0..2 for the a-rows half, rows 5..6 or row 5 for the b-rows half): 0.3-1 % slower.
+    // FUSE_EPI: the epilogue of a tile runs under matrix instructions -- fragment rows 0..3 under the tile's own last
+    // K-step, rows 4..7 under the first K-step of the workgroup's next tile.  Done after the K loop, the epilogue is
+    // 1.5 to 2.4 us per tile in which the matrix cores idle (measured by leaving it out: 37888 x 8192 x 3584 702 ->
+    // 649 us, 17920 x 16384 x 1536 316 -> 268 us).  Two resources bound how it can be hidden:
+    //   * the wave's instruction issue: a slice (below) is 10 vector instructions, a matrix instruction occupies its
+    //     pipe for 32 cycles -- one slice per matrix instruction (all eight rows under one K-step) was measured to
+    //     stretch that K-step by as much as 60 % of what was saved; two slices per three matrix instructions fit;
+    //   * the compute unit's one address unit: 16 cycles per copy or store instruction of a wave, four waves, so the
+    //     16 copies of a K-step take half of its 2048 cycles and at most 16 of a tile's 32 stores per wave fit
+    //     beside them (with 28 stores in one K-step: +1.3 us per tile; with 16: within the noise of none).
+    // Fragment row q of a tile is final once its eight matrix instructions of the last K-step have been issued, and
+    // stays intact until the next tile's first K-step reaches row q.  A slice takes four accumulators of one c row (two
+    // pairs of adjacent columns): accumulation register -> vector register, times the output factor, packed rounding
+    // to bf16; every second slice completes the lane's 16 bytes of a c row and stores them.  The 32 slices of rows 0..3
+    // follow the matrix instructions 8 + 3k/2 (k = 0..31) of the last K-step, those of rows 4..7 the matrix
+    // instructions 3k/2 of the next first K-step (each row before the step overwrites it); after a workgroup's last
+    // tile rows 4..7 are written out on their own.  The slices are asm statements so that they stay where they are
+    // written: the compiler would otherwise gather the read-outs behind the matrix instruction that wrote the
+    // register (too close for the hardware, which needs the instruction's passes to finish first, and the values would
+    // then occupy registers through the whole step).
+    [[maybe_unused]] uint32_t epi_lane = 0;   // this tile: byte offset of the lane's 16 bytes within "its" c row (4 ekg rows down)
+    [[maybe_unused]] int epi_row0 = 0;        // this tile: first c row of the wave tile
+    [[maybe_unused]] uint32_t prev_lane = 0;  // the same two for the previous tile of this workgroup (rows 4..7 still to write)
+    [[maybe_unused]] int prev_row0 = 0;
+    [[maybe_unused]] uint32_t epi_pk[4];
+    [[maybe_unused]] auto scaled_pair = [&](float x0, float x1) -> uint32_t {
+        uint32_t out, tmp;
+        asm volatile(
+            "v_accvgpr_read_b32 %0, %2\n\t"
+            "v_accvgpr_read_b32 %1, %3\n\t"
+            "v_mul_f32 %0, %4, %0\n\t"
+            "v_mul_f32 %1, %4, %1\n\t"
+            "v_cvt_pk_bf16_f32 %0, %0, %1"
+            : "=&v"(out), "=&v"(tmp)
+            : "a"(x0), "a"(x1), "s"(out_scale));
+        return out;
+    };
+    // slice sl (0..7) of fragment row i: c row r = sl / 2 of the row's four, column half h = sl % 2
+    [[maybe_unused]] auto epi_slice = [&](auto i_tag, auto s_tag, int row0, uint32_t lane_bytes) {
+        constexpr int i = decltype(i_tag)::value, sl = decltype(s_tag)::value;
+        constexpr int r = sl / 2, h = sl % 2;
+        epi_pk[2 * h] = scaled_pair(acc[i][4 * h][r], acc[i][4 * h + 1][r]);
+        epi_pk[2 * h + 1] = scaled_pair(acc[i][4 * h + 2][r], acc[i][4 * h + 3][r]);
+        if constexpr (h == 1) {
+            const v4i packed = {(int)epi_pk[0], (int)epi_pk[1], (int)epi_pk[2], (int)epi_pk[3]};
+            LLMQ_GLOBAL char* row_ptr =
+                scalar_ptr((LLMQ_GLOBAL char*)(reinterpret_cast<uint16_t*>(g.c) + (int64_t)(row0 + 16 * i + r) * g.M));
+            if constexpr (STREAM_OUT) __builtin_nontemporal_store(packed, (LLMQ_GLOBAL v4i*)(row_ptr + lane_bytes));
+            else *(LLMQ_GLOBAL v4i*)(row_ptr + lane_bytes) = packed;
+        }
+    };
     bool pending_stores = false;  // an epilogue without accumulation has just issued its stores
     [[maybe_unused]] int stage_rt = 0;  // ODDK: byte offset of the LDS stage of the current K-step
     // par_tag: LDS stage of the step; fp_tag: the half of fb that holds its second-operand fragments (the same
@@ -917,10 +970,28 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     // kYoung: copies of this step that are in flight at the step's second barrier and need not have landed (they
     // refill the a-rows half of the stage this step computes from)
     constexpr int kYoung = ITERS_Q;
-    auto k_step = [&](auto par_tag, auto fp_tag, auto first_tag) {
+    // Slice schedule of FUSE_EPI: slice k (0..31: fragment row k / 8 of a group of four, slice k % 8 of it) follows
+    // the matrix instruction number 3k/2 of its window; slice_of(m) is the slice behind instruction m of the window
+    // (-1: none) and stores_through(m) the number of stores issued with the slices up to instruction m.
+    constexpr auto slice_of = [](int m) {
+        for (int k = 0; k < 32; ++k)
+            if (3 * k / 2 == m) return k;
+        return -1;
+    };
+    constexpr auto stores_through = [](int m) {
+        int n = 0;
+        for (int k = 1; k < 32; k += 2)
+            if (3 * k / 2 <= m) ++n;
+        return n;
+    };
+    // last_tag: the tile's last K-step (FUSE_EPI: carries the slices of rows 0..3, window from instruction 8 on);
+    // prev_tag: a first K-step that carries the slices of rows 4..7 of the workgroup's previous tile (FUSE_EPI).
+    auto k_step = [&](auto par_tag, auto fp_tag, auto first_tag, auto last_tag, auto prev_tag) {
         constexpr int PAR = decltype(par_tag)::value;
         constexpr int FP = decltype(fp_tag)::value;
         constexpr bool FIRST = decltype(first_tag)::value;
+        constexpr bool LAST = FUSE_EPI && decltype(last_tag)::value;
+        constexpr bool PREV = FUSE_EPI && FIRST && decltype(prev_tag)::value;
         // the stage this step computes from and then releases to the copies; with ODDK a run-time value
         const uint8_t* cur = lds + (ODDK ? stage_rt : PAR * STAGE);
         const uint8_t* nxt = lds + (ODDK ? STAGE - stage_rt : (1 - PAR) * STAGE);
@@ -956,12 +1027,32 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
                     constexpr int f = 2 * (i - 4) + (j == 5 ? 1 : 0);
                     if constexpr (f < NJ) fb[1 - FP][f] = read_frag_a(nxt, f);
                 }
+                if constexpr (LAST && i >= 1) {
+                    constexpr int k = slice_of(8 * i + j - 8);
+                    if constexpr (k >= 0)
+                        epi_slice(std::integral_constant<int, k / 8>{}, std::integral_constant<int, k % 8>{}, epi_row0, epi_lane);
+                }
+                if constexpr (PREV) {
+                    constexpr int k = slice_of(8 * i + j);
+                    if constexpr (k >= 0)
+                        epi_slice(std::integral_constant<int, 4 + k / 8>{}, std::integral_constant<int, k % 8>{}, prev_row0, prev_lane);
+                }
             });
             if constexpr (i == 4) {
                 // every read of the current stage has been issued (the last one after row 3); once they
                 // have returned and all waves are here the stage may be overwritten, and the next stage
                 // (copied one step ago) is complete
-                if constexpr (FIRST) {
+                if constexpr (LAST) {
+                    // the stores of this step's slices so far (instructions 8..39 of the step) sit behind every copy this
+                    // barrier is about
+                    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kYoung + stores_through(31)) : "memory");
+                } else if constexpr (PREV) {
+                    // likewise (instructions 0..39); the last copy this barrier is about went out with the last matrix
+                    // instruction of the previous tile, behind all of that step's stores
+                    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kYoung + stores_through(39)) : "memory");
+                } else if constexpr (FIRST && FUSE_EPI) {
+                    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kYoung) : "memory");
+                } else if constexpr (FIRST) {
                     // Behind the copies this barrier is about (the tile's second K-step, issued before the
                     // previous tile's epilogue) sit that epilogue's stores; the counter retires in issue
                     // order, so allowing as many outstanding operations as there were stores is enough.
@@ -1036,25 +1127,42 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     const int KT = k_total / kBK;  // even, or odd and at least 3 with ODDK
     int logical = xcd_first + slot;
     for (int t = 0; t < my_tiles; ++t) {
-        if constexpr (!ODDK) {
-            k_step(P0, P0, Y);
-            k_step(P1, P1, NO);
+        if constexpr (FUSE_EPI) {  // where this tile's outputs go: needed by its last K-step
+            int n_blk, m_blk;
+            decode(logical, n_blk, m_blk);
+            logical += tile_stride;
+            const int e_lane = opaque(threadIdx.x) % 64;
+            epi_lane = ((uint32_t)(4 * (e_lane / 16)) * (uint32_t)g.M + (uint32_t)(m_blk + wm * WTM + 8 * (e_lane % 16))) * 2u;
+            epi_row0 = n_blk + wn * WT;
+        }
+        if constexpr (!ODDK && FUSE_EPI) {
+            if (t == 0) k_step(P0, P0, Y, NO, NO);
+            else k_step(P0, P0, Y, NO, Y);
+            for (int kt = 1; kt + 1 < KT; kt += 2) {
+                k_step(P1, P1, NO, NO, NO);
+                k_step(P0, P0, NO, NO, NO);
+            }
+            k_step(P1, P1, NO, Y, NO);
+        } else if constexpr (!ODDK) {
+            k_step(P0, P0, Y, NO, NO);
+            k_step(P1, P1, NO, NO, NO);
             for (int kt = 2; kt < KT; kt += 2) {
-                k_step(P0, P0, NO);
-                k_step(P1, P1, NO);
+                k_step(P0, P0, NO, NO, NO);
+                k_step(P1, P1, NO, NO, NO);
             }
         } else {
             // An odd number of K-steps: the LDS stage of a tile's first step alternates from tile to tile, so the
             // stage is a run-time value here (stage_rt, toggled by every step; the tags only name the fb half).  The
             // last step leaves the next tile's first second-operand fragments in fb half 1; they are moved to half
             // 0, where every tile starts.
-            k_step(P0, P0, Y);
-            k_step(P1, P1, NO);
+            if (FUSE_EPI && t > 0) k_step(P0, P0, Y, NO, Y);
+            else k_step(P0, P0, Y, NO, NO);
+            k_step(P1, P1, NO, NO, NO);
             for (int kt = 3; kt < KT; kt += 2) {
-                k_step(P0, P0, NO);
-                k_step(P1, P1, NO);
+                k_step(P0, P0, NO, NO, NO);
+                k_step(P1, P1, NO, NO, NO);
             }
-            k_step(P0, P0, NO);
+            k_step(P0, P0, NO, Y, NO);
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
             for (int j = 0; j < NJ; ++j) fb[0][j] = fb[1][j];
@@ -1062,6 +1170,19 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         // the compiler does not know the statements above are matrix instructions: give the last ones time
         // to retire before their results are read (generously: four times the instruction's 32 cycles)
         asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+        if constexpr (FUSE_EPI) {
+            // rows 0..3 went out under the last K-step; rows 4..7 go out under the next tile's first K-step, or here
+            // after the workgroup's last tile
+            prev_lane = epi_lane;
+            prev_row0 = epi_row0;
+            if (t + 1 == my_tiles) {
+                static_for<0, 32>([&](auto k_tag) {
+                    constexpr int k = decltype(k_tag)::value;
+                    epi_slice(std::integral_constant<int, 4 + k / 8>{}, std::integral_constant<int, k % 8>{}, prev_row0, prev_lane);
+                });
+            }
+            continue;
+        }
 
         // Epilogue.  acc[i][j][r] is c row 16 i + 4 kg + r of the wave tile and, thanks to the a-tile row
         // permutation, column NJ l16 + j: a lane owns NJ adjacent columns of each of its 32 rows (8: one 16-byte
@@ -1411,10 +1532,12 @@ static int launch_pipe(const GemmArgs& g, int splits, int persistent_grid, hipSt
 // they are constants and the dispatch below is a function of its arguments alone.  tile: 1 = 256 x 256 tile with
 // 8 waves, 2 = 128 x 128 tile with 4 waves, 3 = four-wave kernel, 4 / 5 = its 224- / 192-wide tiles.  splits:
 // forced number of K splits (needs a workspace).  persist: -1 = automatic, 0 = never, 1 = whenever possible.
+// fuse: -1 = automatic, 0 = the four-wave kernel's epilogue always after the K loop, 1 = under the last K-step wherever
+// that instance exists (full-width bf16 tiles without bias and accumulation).
 #ifdef LLMQ_TEST_HOOKS
-static std::atomic<int> g_gemm_tile{0}, g_gemm_splits{0}, g_gemm_persist{-1};
+static std::atomic<int> g_gemm_tile{0}, g_gemm_splits{0}, g_gemm_persist{-1}, g_gemm_fuse{-1};
 #else
-constexpr int g_gemm_tile = 0, g_gemm_splits = 0, g_gemm_persist = -1;
+constexpr int g_gemm_tile = 0, g_gemm_splits = 0, g_gemm_persist = -1, g_gemm_fuse = -1;
 #endif
 
 // Launch plan of the four-wave kernel.  A persistent grid of `grid` workgroups (grid / 8 per XCD) walks
@@ -1524,14 +1647,14 @@ static SmallPlan plan_small(int M, int N, int K, int cus, bool ok256, bool ok224
 
 // One launch of the four-wave kernel's main variant (no K segments); odd_k selects the instance for an odd number of
 // K-steps.
-template <typename OutT, int B_FMT, int NJ, bool STREAM_OUT>
+template <typename OutT, int B_FMT, int NJ, bool STREAM_OUT, bool FUSE_EPI = false>
 static void launch_w4(bool odd_k, int grid, const GemmArgs& g, hipStream_t stream) {
     if (odd_k)
-        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<OutT, B_FMT, false, NJ, STREAM_OUT, true>), dim3((unsigned)grid), dim3(256), 0,
-                           stream, g);
+        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<OutT, B_FMT, false, NJ, STREAM_OUT, true, false, false, FUSE_EPI>),
+                           dim3((unsigned)grid), dim3(256), 0, stream, g);
     else
-        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<OutT, B_FMT, false, NJ, STREAM_OUT, false>), dim3((unsigned)grid), dim3(256), 0,
-                           stream, g);
+        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<OutT, B_FMT, false, NJ, STREAM_OUT, false, false, false, FUSE_EPI>),
+                           dim3((unsigned)grid), dim3(256), 0, stream, g);
 }
 
 template <typename OutT, int B_FMT>
@@ -1698,8 +1821,16 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
         const bool cached_out = std::is_same_v<OutT, uint16_t> &&
                                 ((int64_t)g.M + g.N) * g.K + (int64_t)g.N * g.M * 2 <= ((int64_t)224 << 20);
         if constexpr (std::is_same_v<OutT, uint16_t>) {
-            if (cached_out) launch_w4<uint16_t, B_FMT, 8, false>(odd_k, plan.grid, g, stream);
-            else launch_w4<uint16_t, B_FMT, 8, true>(odd_k, plan.grid, g, stream);
+            const int force_fuse = g_gemm_fuse;
+            const bool fuse = force_fuse != 0 && g.bias == nullptr && !g.accumulate;
+            if (fuse) {
+                if (cached_out) launch_w4<uint16_t, B_FMT, 8, false, true>(odd_k, plan.grid, g, stream);
+                else launch_w4<uint16_t, B_FMT, 8, true, true>(odd_k, plan.grid, g, stream);
+            } else if (cached_out) {
+                launch_w4<uint16_t, B_FMT, 8, false>(odd_k, plan.grid, g, stream);
+            } else {
+                launch_w4<uint16_t, B_FMT, 8, true>(odd_k, plan.grid, g, stream);
+            }
         } else {
             launch_w4<OutT, B_FMT, 8, true>(odd_k, plan.grid, g, stream);
         }
@@ -1839,4 +1970,5 @@ extern "C" __attribute__((visibility("default"))) void llmq_debug_set_gemm_varia
     llmq::g_gemm_splits = splits;
 }
 extern "C" __attribute__((visibility("default"))) void llmq_debug_set_gemm_persist(int v) { llmq::g_gemm_persist = v; }
+extern "C" __attribute__((visibility("default"))) void llmq_debug_set_gemm_fuse(int v) { llmq::g_gemm_fuse = v; }
 #endif

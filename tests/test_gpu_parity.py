@@ -846,6 +846,47 @@ def test_gemm_k_major_automatic_cut_on_a_weight_gradient_shape(K, mode):
     assert 0 < differing < 0.02, differing
 
 
+FUSED_EPILOGUE_SHAPES = [(256, 256, 256), (256, 256, 384), (512, 768, 896), (4352, 4352, 512), (4352, 4096, 1024), (4608, 4096, 256),
+                         (8192, 4608, 1536), (4352, 4352, 640), (9728, 8192, 896), (18944, 3584, 8192)]
+
+
+@pytest.mark.parametrize("mnk", FUSED_EPILOGUE_SHAPES)
+def test_gemm_epilogue_under_matrix_instructions_matches_epilogue_after_the_loop(K, O, mnk):
+    """The four-wave kernel writes full-width bf16 tiles (no bias, no accumulation) out under matrix instructions: rows
+    0..3 under the tile's last K-step, rows 4..7 under the next tile's first K-step, the last tile's on their own.  Same
+    arithmetic in the same order as the epilogue after the K loop, so the two instances must agree bit for bit: one tile
+    and many per workgroup, two K-steps per tile (the last step follows the first directly), odd K-step counts, a cut
+    last round; repeated launches; and integer-valued operands against the exact product."""
+    from llmq_amd import capi
+    M, N, Kd = mnk
+    t = capi.testaid()
+    g = torch.Generator(device="cuda").manual_seed(M + N + Kd)
+    a = torch.randint(0, 0x7E, (M, Kd), dtype=torch.uint8, device="cuda", generator=g) | (torch.randint(0, 2, (M, Kd), dtype=torch.uint8, device="cuda", generator=g) << 7)
+    b = torch.randint(0, 0x7E, (N, Kd), dtype=torch.uint8, device="cuda", generator=g) | (torch.randint(0, 2, (N, Kd), dtype=torch.uint8, device="cuda", generator=g) << 7)
+    sa = dev_scalar(2.0 ** -7 * 1.37)
+    try:
+        with gemm_library(t):
+            t.llmq_debug_set_gemm_fuse(0)
+            c0 = torch.full((N, M), float("nan"), dtype=torch.bfloat16, device="cuda")
+            K.matmul(c0, a, b, None, sa, None, M, N, Kd, workspace=workspace())
+            t.llmq_debug_set_gemm_fuse(1)
+            for _ in range(3):
+                c1 = torch.full((N, M), float("nan"), dtype=torch.bfloat16, device="cuda")
+                K.matmul(c1, a, b, None, sa, None, M, N, Kd, workspace=workspace())
+                assert torch.equal(c0.view(torch.int16), c1.view(torch.int16))
+            if M * N * Kd <= 4352 * 4352 * 1024:
+                ai, _ = O.fill_int_e4m3(M * Kd, 7 + M, 0)
+                bi, _ = O.fill_int_e4m3(N * Kd, 7 + N, 1)
+                ai, bi = ai.reshape(M, Kd), bi.reshape(N, Kd)
+                s = float(np.sqrt(np.float32(4.0 / Kd)))
+                want = O.gemm_tn(ai, bi, sa=s, sb=s, mt=True)
+                c2 = torch.full((N, M), float("nan"), dtype=torch.bfloat16, device="cuda")
+                K.matmul(c2, dev_u8(ai), dev_u8(bi), None, dev_scalar(s), dev_scalar(s), M, N, Kd, workspace=workspace())
+                assert np.array_equal(host_bits(c2), want)
+    finally:
+        t.llmq_debug_set_gemm_fuse(-1)
+
+
 def test_product_library_cuts_the_last_round_into_k_segments(K):
     """The K-segment instance of the four-wave kernel, reached on the product library through the automatic plan (no
     forced variant): 18944 x 3584 x 8192 leaves one or two tiles per XCD for the last round, and with a workspace the
