@@ -137,7 +137,7 @@ inline void require_tn(EMMTranspose mode) {
     if (mode != EMMTranspose::TN)
         throw std::invalid_argument("matmul: FP8 operands are only supported in TN layout (both K-contiguous)");
 }
-// bf16 output: TN, and the K-major modes TT / NN / NT (restricted shapes, see llmq_gemm_e4m3_bf16_mode)
+// TN, and the K-major modes TT / NN / NT (restricted shapes, see llmq_gemm_e4m3_bf16_mode)
 inline int mode_code(EMMTranspose mode) {
     switch (mode) {
         case EMMTranspose::TN: return LLMQ_MODE_TN;
@@ -253,10 +253,10 @@ inline void quantize_with_abs_max_and_transpose(Tensor& out, Tensor& out_tp, flo
 
 // ---- matmul (reference: src/kernels/kernels.h:72-78, 88-90, 96-98) --------------------------------------
 // Row-major a[M,K], b[N,K] -> row-major c[N,M] = (b . a^T) * (*scale_a * *scale_b) (+ bias[M]) (+ c).
-// Mode TN: any M, N >= 1 and K a multiple of 16 (16-byte aligned fp8 rows).  bf16 output also takes the K-major modes:
-// TT (b stored [K, N]: e.g. the output gradient dY[B*T, OC] of the weight gradient without its transposed copy), NN
-// (a stored [K, M]: the weight W[OC, C] of the dgrad) and NT (both), when M, N and K are multiples of 256 (mode TT
-// without accumulation also M of 224); NN and NT do not accumulate into c.  Anything else throws
+// Mode TN: any M, N >= 1 and K a multiple of 16 (16-byte aligned fp8 rows).  The K-major modes -- TT (b stored [K, N]:
+// e.g. the output gradient dY[B*T, OC] of the weight gradient without its transposed copy), NN (a stored [K, M]: the
+// weight W[OC, C] of the dgrad) and NT (both) -- serve M, N and K multiples of 256 (mode TT with bf16 output and without
+// accumulation also M of 224), bf16 and fp32 output, with bias and accumulation.  Anything else throws
 // std::invalid_argument before a kernel is launched.
 inline void matmul(__hip_bfloat16* c, const __hip_fp8_e4m3* a, const __hip_fp8_e4m3* b, const __hip_bfloat16* bias,
                    const float* scale_a, const float* scale_b, llmqBlasHandle_t, std::byte* workspace,
@@ -270,17 +270,15 @@ inline void matmul(float* c, const __hip_fp8_e4m3* a, const __hip_fp8_e4m3* b, c
                    const float* scale_b, llmqBlasHandle_t, std::byte* workspace, std::size_t workspace_size, int M,
                    int N, int K, EMMTranspose mode, bool accumulate, hipStream_t stream,
                    EMatmulBackend = EMatmulBackend::Custom) {
-    llmq_detail::require_tn(mode);
-    llmq_detail::check(llmq_gemm_tn_e4m3_f32(c, llmq_detail::u8(a), llmq_detail::u8(b), bias, 0, scale_a, scale_b,
-                                             workspace, workspace_size, M, N, K, accumulate, stream));
+    llmq_detail::check(llmq_gemm_e4m3_f32_mode(c, llmq_detail::u8(a), llmq_detail::u8(b), bias, 0, scale_a, scale_b, workspace,
+                                               workspace_size, M, N, K, llmq_detail::mode_code(mode), 0, accumulate, stream));
 }
 inline void matmul(float* c, const __hip_fp8_e4m3* a, const __hip_fp8_e4m3* b, const __hip_bfloat16* bias,
                    const float* scale_a, const float* scale_b, llmqBlasHandle_t, std::byte* workspace,
                    std::size_t workspace_size, int M, int N, int K, EMMTranspose mode, bool accumulate,
                    hipStream_t stream, EMatmulBackend = EMatmulBackend::Custom) {
-    llmq_detail::require_tn(mode);
-    llmq_detail::check(llmq_gemm_tn_e4m3_f32(c, llmq_detail::u8(a), llmq_detail::u8(b), bias, 1, scale_a, scale_b,
-                                             workspace, workspace_size, M, N, K, accumulate, stream));
+    llmq_detail::check(llmq_gemm_e4m3_f32_mode(c, llmq_detail::u8(a), llmq_detail::u8(b), bias, 1, scale_a, scale_b, workspace,
+                                               workspace_size, M, N, K, llmq_detail::mode_code(mode), 0, accumulate, stream));
 }
 // e4m3 x e5m2 (gradient dtype option; reference: src/kernels/kernels.h:80-82, 92-94)
 inline void matmul(__hip_bfloat16* c, const __hip_fp8_e4m3* a, const __hip_fp8_e5m2* b, const __hip_bfloat16* bias,
@@ -295,9 +293,8 @@ inline void matmul(float* c, const __hip_fp8_e4m3* a, const __hip_fp8_e5m2* b, c
                    const float* scale_a, const float* scale_b, llmqBlasHandle_t, std::byte* workspace,
                    std::size_t workspace_size, int M, int N, int K, EMMTranspose mode, bool accumulate,
                    hipStream_t stream, EMatmulBackend = EMatmulBackend::Custom) {
-    llmq_detail::require_tn(mode);
-    llmq_detail::check(llmq_gemm_tn_e4m3_e5m2_f32(c, llmq_detail::u8(a), llmq_detail::u8(b), bias, 1, scale_a, scale_b,
-                                                  workspace, workspace_size, M, N, K, accumulate, stream));
+    llmq_detail::check(llmq_gemm_e4m3_f32_mode(c, llmq_detail::u8(a), llmq_detail::u8(b), bias, 1, scale_a, scale_b, workspace,
+                                               workspace_size, M, N, K, llmq_detail::mode_code(mode), 1, accumulate, stream));
 }
 inline void matmul(Tensor& c, const Tensor& a, const Tensor& b, const Tensor& bias, const float* scale_a,
                    const float* scale_b, llmqBlasHandle_t handle, Tensor& workspace, int M, int N, int K,

@@ -40,8 +40,9 @@ struct QmmRunState {
     bool DirectGradLayoutWhereverServed = false;
     using EWgrad = EQmmWgrad;
     using DirectPlan = QmmDirectPlan;
-    // The K-major modes serve whole 256-wide tiles, bf16 output and operands below 2 GiB; modes NN / NT do not
-    // accumulate.  Which of them pay was measured on MLP layers of Qwen2.5-7B (C = 3584, FFN 18944), 1.5B (1536, 8960)
+    // The K-major modes serve whole 256-wide tiles and operands below 2 GiB (bf16 and fp32 output, with accumulation;
+    // a K-major first operand with fp32 output or accumulation takes a slower, fp32-staged epilogue).  Which of them pay
+    // was measured on MLP layers of Qwen2.5-7B (C = 3584, FFN 18944), 1.5B (1536, 8960)
     // and a 2048 / 8192 layer at 4096 to 16384 tokens, every matmul with the 32 MiB workspace, against mode TN plus the
     // byte transposes it needs (2 bytes moved per element copied):
     //  * weight gradient: on the 7B layers a K-major second operand costs 3-4 % of the matmul and both operands K-major
@@ -61,9 +62,10 @@ struct QmmRunState {
         DirectPlan p;
         p.DgradInPlace = tiles && dinp_dtype == ETensorDType::BF16 && (long)C * OC < lim &&
                          (wherever_served || ((long)C * OC >= (48L << 20) && BT >= 8192 && BT <= 16384));
-        if (dweight_dtype == ETensorDType::BF16 && OC % 256 == 0 && BT % 256 == 0 && BT * OC < lim) {
-            if (tiles && !accumulate && BT * C < lim && (wherever_served || OC <= 8192)) p.Wgrad = EWgrad::BothInPlace;
-            else if ((C % 256 == 0 || (C % 224 == 0 && !accumulate)) && (wherever_served || C <= 8192)) p.Wgrad = EWgrad::GradInPlace;
+        const bool bf16_dw = dweight_dtype == ETensorDType::BF16;
+        if ((bf16_dw || dweight_dtype == ETensorDType::FP32) && OC % 256 == 0 && BT % 256 == 0 && BT * OC < lim) {
+            if (tiles && BT * C < lim && (wherever_served || OC <= 8192)) p.Wgrad = EWgrad::BothInPlace;
+            else if ((C % 256 == 0 || (C % 224 == 0 && bf16_dw && !accumulate)) && (wherever_served || C <= 8192)) p.Wgrad = EWgrad::GradInPlace;
         }
         return p;
     }
@@ -153,7 +155,7 @@ inline void backward_qmm(Tensor& dinp, Tensor& dweight, Tensor dbias, Quantizabl
         if (!reuse_inp)
             quantize_with_abs_max(inp_q, inp_q.scale(), inp.Value, inp_q.abs_max(), (long)B * T * C, rs.DeviceProp, stream);
         matmul(dweight, inp_q, dout.Quant, no_bias, inp_q.scale(), dout.Quant.scale(), rs.BlasHandle, rs.Workspace, C, OC,
-               B * T, EMMTranspose::NT, false, stream, rs.MatmulBackend);
+               B * T, EMMTranspose::NT, accumulate_gradient, stream, rs.MatmulBackend);
         if (!dbias.empty())
             backward_bias(dbias, dout.Quant, inp_q.scale(), dout.Quant.scale(), bias_buffer, B, T, OC, rs.DeviceProp, stream);
         return;

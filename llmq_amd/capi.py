@@ -18,7 +18,7 @@ EXPORTS = [
     "llmq_last_error", "llmq_version", "llmq_target_arch",
     "llmq_abs_max_bf16", "llmq_abs_max_f32",
     "llmq_quantize_e4m3_bf16", "llmq_quantize_e5m2_bf16", "llmq_quantize_transpose_e4m3_bf16", "llmq_quantize_transpose_e4m3_f32",
-    "llmq_transpose_u8", "llmq_gemm_tn_e4m3_bf16", "llmq_gemm_e4m3_bf16_mode", "llmq_gemm_tn_e4m3_f32", "llmq_gemm_tn_e4m3_e5m2_bf16", "llmq_gemm_tn_e4m3_e5m2_f32",
+    "llmq_transpose_u8", "llmq_gemm_tn_e4m3_bf16", "llmq_gemm_e4m3_bf16_mode", "llmq_gemm_e4m3_f32_mode", "llmq_gemm_tn_e4m3_f32", "llmq_gemm_tn_e4m3_e5m2_bf16", "llmq_gemm_tn_e4m3_e5m2_f32",
     "llmq_backward_bias_bf16", "llmq_backward_bias_scratch_bytes", "llmq_backward_bias_bf16_static_scratch", "llmq_quantize_both_bf16", "llmq_quantize_e4m3_f32", "llmq_quantize_e5m2_f32",
     "llmq_swiglu_forward_bf16", "llmq_swiglu_forward_quant_bf16", "llmq_swiglu_backward_bf16",
     "llmq_rmsnorm_forward_bf16", "llmq_fused_residual_rmsnorm_forward_bf16",
@@ -51,6 +51,7 @@ lib.llmq_quantize_both_bf16.argtypes = [_vp, _vp, _vp, _vp, _vp, _int, _int, _in
 lib.llmq_transpose_u8.argtypes = [_vp, _vp, _int, _int, _vp]
 lib.llmq_gemm_tn_e4m3_bf16.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, C.c_size_t, _int, _int, _int, _int, _vp]
 lib.llmq_gemm_e4m3_bf16_mode.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, C.c_size_t, _int, _int, _int, _int, _int, _int, _vp]
+lib.llmq_gemm_e4m3_f32_mode.argtypes = [_vp, _vp, _vp, _vp, _int, _vp, _vp, _vp, C.c_size_t, _int, _int, _int, _int, _int, _int, _vp]
 lib.llmq_gemm_tn_e4m3_f32.argtypes = [_vp, _vp, _vp, _vp, _int, _vp, _vp, _vp, C.c_size_t, _int, _int, _int, _int, _vp]
 lib.llmq_gemm_tn_e4m3_e5m2_bf16.argtypes = lib.llmq_gemm_tn_e4m3_bf16.argtypes
 lib.llmq_gemm_tn_e4m3_e5m2_f32.argtypes = lib.llmq_gemm_tn_e4m3_f32.argtypes
@@ -101,7 +102,7 @@ def testaid():
         t = C.CDLL(TESTAID_PATH)
         t.llmq_last_error.restype = C.c_char_p
         for name in ("llmq_gemm_tn_e4m3_bf16", "llmq_gemm_tn_e4m3_f32", "llmq_gemm_tn_e4m3_e5m2_bf16",
-                     "llmq_gemm_tn_e4m3_e5m2_f32", "llmq_gemm_e4m3_bf16_mode"):
+                     "llmq_gemm_tn_e4m3_e5m2_f32", "llmq_gemm_e4m3_bf16_mode", "llmq_gemm_e4m3_f32_mode"):
             getattr(t, name).argtypes = getattr(lib, name).argtypes
             getattr(t, name).restype = _int
         t.llmq_debug_set_gemm_variant.argtypes = [_int, _int]

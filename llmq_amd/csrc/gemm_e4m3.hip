@@ -613,14 +613,15 @@ __device__ __forceinline__ int frag_swizzle(int row) {
 // fragment row into a private 4 KiB piece of LDS, read back as 16 bytes per lane and row.  bf16 output without
 // accumulation (the old values of c would have to be fetched in the scattered layout).
 template <typename OutT, int B_FMT, bool SEG, int NJ = 8, bool STREAM_OUT = true, bool ODDK = false, bool KMB = false,
-          bool KMA = false, bool FUSE_EPI = false>
+          bool KMA = false, bool FUSE_EPI = false, bool STAGE32 = false>
 __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     static_assert(!(SEG && ODDK), "K segments are whole pairs of K-steps");
+    static_assert(!STAGE32 || (KMA && !SEG && NJ == 8), "the fp32-staged epilogue belongs to the K-major first operand");
     static_assert(!FUSE_EPI || (NJ == 8 && !SEG && !KMA && std::is_same_v<OutT, uint16_t>),
                   "the epilogue under the last K-step is written for full-width bf16 tiles of K-contiguous a");
     static_assert(!((KMB || KMA) && ODDK), "the K-major operand modes are built for even K-step counts");
-    static_assert(!KMA || (NJ == 8 && (SEG || std::is_same_v<OutT, uint16_t>)),
-                  "the K-major first operand is built for 256-wide tiles and bf16 output (fp32 only as K segments)");
+    static_assert(!KMA || (NJ == 8 && (SEG || STAGE32 || std::is_same_v<OutT, uint16_t>)),
+                  "the K-major first operand is built for 256-wide tiles; fp32 output as K segments or through the fp32-staged epilogue");
     constexpr int BLK = 256, T = 256, WT = 128, NF = 8;
     constexpr int WTM = 16 * NJ, BLKM = 2 * WTM;  // columns (first-operand rows) per wave and per tile
     constexpr int P_BYTES = BLK * kBK, STAGE = 2 * P_BYTES;
@@ -630,7 +631,9 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     typedef float v4f __attribute__((ext_vector_type(4)));
 
     constexpr int EPI_STAGE = 16 * WTM * 2;  // KMA: one fragment row of a wave's outputs as bf16
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * STAGE + (KMA ? 4 * EPI_STAGE : 0)];
+    constexpr int EPI32_ROW = 4 * WTM + 32;  // STAGE32: half a fragment row (8 c rows) of raw accumulators, rows padded by 32 bytes
+    constexpr int EPI32_STAGE = 8 * EPI32_ROW;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * STAGE + (KMA ? 4 * (STAGE32 ? EPI32_STAGE : EPI_STAGE) : 0)];
 
     const int tid = threadIdx.x;
     const int lane = tid % 64;
@@ -1229,6 +1232,64 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
                         for (int j = 0; j < NJ; ++j) pc[(16 * i + r) * BLK + 16 * j] = acc[i][j][r];
                     }
                 }
+            } else if constexpr (KMA && STAGE32) {
+                // The general epilogue of the K-major first operand: fp32 or bf16 output, bias, accumulation.  acc[i][j][r] is
+                // c row 16 i + 4 ekg + r, column 16 j + el16 of the wave tile; the old values of c and the bias belong to
+                // whole row segments, so the raw accumulators change hands through LDS first: per fragment row i and
+                // half hh, the wave writes the 8 c rows 4 q + 2 hh + rr (q = 0..3, rr = 0, 1) x 128 columns as fp32 into
+                // its own piece of LDS (row 2 q + rr, row stride 544 bytes: the four row pairs of a write land on
+                // different banks) and reads them back as 16 bytes per lane (piece p = lane + 64 t: row p / 32, columns
+                // 4 (p % 32) ..+3); scale, bias, old value and the one rounding follow in the order of the other epilogues.
+                // One wave's LDS operations are carried out in order, so no barrier is needed around the exchange.  Bias and
+                // accumulation are run-time branches here (one copy of this code per kernel instance).
+                uint8_t* es = lds + 2 * STAGE + wave * EPI32_STAGE;
+                const uint32_t wr_ofs = (uint32_t)(2 * ekg) * EPI32_ROW + (uint32_t)el16 * 4u;
+#pragma unroll
+                for (int i = 0; i < NF; ++i) {
+#pragma unroll
+                    for (int hh = 0; hh < 2; ++hh) {
+#pragma unroll
+                        for (int j = 0; j < NJ; ++j) {
+#pragma unroll
+                            for (int rr = 0; rr < 2; ++rr)
+                                *reinterpret_cast<float*>(es + wr_ofs + rr * EPI32_ROW + j * 64) = acc[i][j][2 * hh + rr];
+                        }
+#pragma unroll
+                        for (int t4 = 0; t4 < 4; ++t4) {
+                            const int p = e_lane + 64 * t4;
+                            const int prow = p / 32, pcol = 4 * (p % 32);   // staged row 2 q + rr, first of four columns
+                            const v4fl raw = *reinterpret_cast<const v4fl*>(es + prow * EPI32_ROW + pcol * 4);
+                            const int crow = row0 + 16 * i + 4 * (prow / 2) + 2 * hh + (prow % 2);
+                            const int ccol = m_blk + wm * WTM + pcol;
+                            OutT* dst = c + (int64_t)crow * ldc + ccol;
+                            float v[4];
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                v[e] = raw[e] * scale;
+                                if (g.bias) v[e] = v[e] + load_bias(g.bias, g.bias_is_bf16, ccol + e);
+                            }
+                            if (g.accumulate) {
+                                float o0, o1, o2, o3;
+                                PairIo<OutT>::load((const LLMQ_GLOBAL OutT*)dst, o0, o1);
+                                PairIo<OutT>::load((const LLMQ_GLOBAL OutT*)(dst + 2), o2, o3);
+                                v[0] = v[0] + o0;
+                                v[1] = v[1] + o1;
+                                v[2] = v[2] + o2;
+                                v[3] = v[3] + o3;
+                            }
+                            if constexpr (std::is_same_v<OutT, uint16_t>) {
+                                const f32x2_t lo2 = {v[0], v[1]}, hi2 = {v[2], v[3]};
+                                typedef int v2i_g __attribute__((ext_vector_type(2)));
+                                const v2i_g packed = {__builtin_bit_cast(int, __builtin_convertvector(lo2, bf16x2_t)),
+                                                      __builtin_bit_cast(int, __builtin_convertvector(hi2, bf16x2_t))};
+                                *(LLMQ_GLOBAL v2i_g*)dst = packed;
+                            } else {
+                                const v4fl out4 = {v[0], v[1], v[2], v[3]};
+                                *(LLMQ_GLOBAL v4fl*)dst = out4;
+                            }
+                        }
+                    }
+                }
             } else if constexpr (KMA) {
                 // acc[i][j][r] is c row 16 i + 4 ekg + r, column 16 j + el16 of the wave tile.  Per fragment row i the
                 // wave writes its 16 x 128 outputs as bf16 into its own piece of LDS ([16 rows][256 bytes], the 32-byte
@@ -1371,6 +1432,9 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         constexpr std::false_type no{};
         if constexpr (SEG) {
             rows(no, no);
+        } else if constexpr (KMA && STAGE32) {
+            rows(no, no);
+            pending_stores = false;  // old values may have been loaded: the next tile's first barrier waits for everything
         } else if constexpr (NJ != 8 || KMA) {
             if (g.bias) rows(yes, no);
             else rows(no, no);
@@ -1851,8 +1915,9 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
 
 // Operands stored K-major (the reference's modes TT: b [K, N]; NN: a [K, M]; NT: both): the four-wave kernel's KMB / KMA
 // instances, whole tiles only.
-template <int B_FMT, bool KMA, bool KMB>
+template <typename OutT, int B_FMT, bool KMA, bool KMB>
 static int gemm_dispatch_kmajor(GemmArgs g, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+    constexpr bool kBf16 = std::is_same_v<OutT, uint16_t>;
     static_assert(KMA || KMB, "mode TN goes through gemm_dispatch");
     const char* mode = KMA ? (KMB ? "NT" : "NN") : "TT";
     LLMQ_REQUIRE(g.M > 0 && g.N > 0 && g.K > 0, "matmul: M, N, K must be positive (got %d, %d, %d)", g.M, g.N, g.K);
@@ -1863,11 +1928,10 @@ static int gemm_dispatch_kmajor(GemmArgs g, void* workspace, size_t workspace_by
     LLMQ_REQUIRE(aligned16(g.a) && aligned16(g.b) && aligned16(g.c) && aligned16(g.bias) && aligned16(workspace),
                  "matmul: all pointers must be 16-byte aligned");
     LLMQ_REQUIRE(workspace != nullptr || workspace_bytes == 0, "matmul: workspace size given without a workspace");
-    const bool m224 = !KMA && g.M % 256 != 0 && g.M % 224 == 0 && !g.accumulate;
+    const bool m224 = kBf16 && !KMA && g.M % 256 != 0 && g.M % 224 == 0 && !g.accumulate;
     LLMQ_REQUIRE(g.N % 256 == 0 && g.K % 256 == 0 && (g.M % 256 == 0 || m224) && cus % xcds == 0,
-                 "matmul: a K-major operand (mode %s) needs N %% 256 == 0, K %% 256 == 0 and M %% 256 == 0 (mode TT without "
-                 "accumulation also M %% 224 == 0); got M, N, K = %d, %d, %d", mode, g.M, g.N, g.K);
-    LLMQ_REQUIRE(!KMA || !g.accumulate, "matmul: mode %s (first operand K-major) does not accumulate into c", mode);
+                 "matmul: a K-major operand (mode %s) needs N %% 256 == 0, K %% 256 == 0 and M %% 256 == 0 (mode TT with bf16 output "
+                 "and without accumulation also M %% 224 == 0); got M, N, K = %d, %d, %d", mode, g.M, g.N, g.K);
     // the copies of a K-major operand address it as "tile base + 32-bit lane offset", and that offset walks the
     // whole K extent of the operand
     LLMQ_REQUIRE(!KMB || (int64_t)g.K * g.N < ((int64_t)1 << 31), "matmul: the K-major second operand must be smaller than 2 GiB "
@@ -1876,7 +1940,7 @@ static int gemm_dispatch_kmajor(GemmArgs g, void* workspace, size_t workspace_by
                  "(K * M = %lld bytes)", (long long)((int64_t)g.K * g.M));
     const int tiles = (g.N / 256) * (m224 ? g.M / 224 : g.M / 256);
     const bool cached_out = ((int64_t)g.M + g.N) * g.K + (int64_t)g.N * g.M * 2 <= ((int64_t)224 << 20);
-    if constexpr (!KMA) {
+    if constexpr (!KMA && kBf16) {
         if (m224) {
             const int grid = tiles < cus ? (tiles + xcds - 1) / xcds * xcds : cus;
             hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, B_FMT, false, 7, true, false, true>), dim3((unsigned)grid),
@@ -1895,18 +1959,35 @@ static int gemm_dispatch_kmajor(GemmArgs g, void* workspace, size_t workspace_by
     g.k_len = plan.k_len;
     g.part_per_xcd = plan.part_per_xcd;
     g.partial = reinterpret_cast<float*>(workspace);
-    if (cached_out)
-        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, B_FMT, false, 8, false, false, KMB, KMA>), dim3((unsigned)plan.grid),
+    // The K-major first operand has two epilogues: bf16 output without accumulation goes out as packed bf16 through
+    // LDS; fp32 output and accumulation take the fp32-staged one.  A K-major second operand alone changes nothing about
+    // the epilogue (the lane owns adjacent columns as in mode TN).
+    const bool general = KMA && (!kBf16 || g.accumulate);
+    if constexpr (KMA) {
+        if (general) {
+            hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<OutT, B_FMT, false, 8, true, false, KMB, true, false, true>),
+                               dim3((unsigned)plan.grid), dim3(256), 0, stream, g);
+        }
+    }
+    if constexpr (kBf16) {
+        if (!general) {
+            if (cached_out)
+                hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, B_FMT, false, 8, false, false, KMB, KMA>), dim3((unsigned)plan.grid),
+                                   dim3(256), 0, stream, g);
+            else
+                hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, B_FMT, false, 8, true, false, KMB, KMA>), dim3((unsigned)plan.grid),
+                                   dim3(256), 0, stream, g);
+        }
+    } else if constexpr (!KMA) {
+        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<float, B_FMT, false, 8, true, false, KMB, false>), dim3((unsigned)plan.grid),
                            dim3(256), 0, stream, g);
-    else
-        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, B_FMT, false, 8, true, false, KMB, KMA>), dim3((unsigned)plan.grid),
-                           dim3(256), 0, stream, g);
+    }
     LLMQ_HIP_TRY(hipGetLastError());
     if (plan.rem_split > 1) {
         hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<float, B_FMT, true, 8, true, false, KMB, KMA>), dim3((unsigned)plan.grid),
                            dim3(256), 0, stream, g);
         LLMQ_HIP_TRY(hipGetLastError());
-        hipLaunchKernelGGL((w4_segment_reduce_kernel<uint16_t>), dim3((unsigned)(xcds * plan.rem_max * 32)), dim3(256), 0, stream,
+        hipLaunchKernelGGL((w4_segment_reduce_kernel<OutT>), dim3((unsigned)(xcds * plan.rem_max * 32)), dim3(256), 0, stream,
                            g, plan.grid / xcds, plan.rem_max);
         LLMQ_HIP_TRY(hipGetLastError());
     }
@@ -1915,21 +1996,39 @@ static int gemm_dispatch_kmajor(GemmArgs g, void* workspace, size_t workspace_by
 
 }  // namespace llmq
 
+namespace llmq {
+// One call of the reference's matmul with an operand mode (EMMTranspose numbering: TT = 0, TN = 1, NT = 2, NN = 3).
+template <typename OutT>
+static int gemm_with_mode(GemmArgs g, void* workspace, size_t workspace_bytes, int mode, int b_format, hipStream_t st) {
+    LLMQ_REQUIRE(b_format == 0 || b_format == 1, "matmul: unknown fp8 format %d of the second operand", b_format);
+    if (mode == LLMQ_MODE_TN)
+        return b_format ? gemm_dispatch<OutT, 1>(g, workspace, workspace_bytes, st) : gemm_dispatch<OutT, 0>(g, workspace, workspace_bytes, st);
+    if (mode == LLMQ_MODE_TT)
+        return b_format ? gemm_dispatch_kmajor<OutT, 1, false, true>(g, workspace, workspace_bytes, st)
+                        : gemm_dispatch_kmajor<OutT, 0, false, true>(g, workspace, workspace_bytes, st);
+    if (mode == LLMQ_MODE_NN)
+        return b_format ? gemm_dispatch_kmajor<OutT, 1, true, false>(g, workspace, workspace_bytes, st)
+                        : gemm_dispatch_kmajor<OutT, 0, true, false>(g, workspace, workspace_bytes, st);
+    LLMQ_REQUIRE(mode == LLMQ_MODE_NT, "matmul: unknown operand mode %d (TT = 0, TN = 1, NT = 2, NN = 3)", mode);
+    return b_format ? gemm_dispatch_kmajor<OutT, 1, true, true>(g, workspace, workspace_bytes, st)
+                    : gemm_dispatch_kmajor<OutT, 0, true, true>(g, workspace, workspace_bytes, st);
+}
+}  // namespace llmq
+
 extern "C" int llmq_gemm_e4m3_bf16_mode(uint16_t* c, const uint8_t* a, const uint8_t* b, const uint16_t* bias_or_null,
                                         const float* sa_or_null, const float* sb_or_null, void* workspace_or_null,
                                         size_t workspace_bytes, int M, int N, int K, int mode, int b_format, int accumulate,
                                         void* stream) {
-    using namespace llmq;
-    LLMQ_REQUIRE(b_format == 0 || b_format == 1, "matmul: unknown fp8 format %d of the second operand", b_format);
-    GemmArgs g{c, a, b, bias_or_null, sa_or_null, sb_or_null, M, N, K, 1, accumulate, 8, nullptr, 0, 1, 0, 8, 0};
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    if (mode == LLMQ_MODE_TN)
-        return b_format ? gemm_dispatch<uint16_t, 1>(g, workspace_or_null, workspace_bytes, st)
-                        : gemm_dispatch<uint16_t, 0>(g, workspace_or_null, workspace_bytes, st);
-    if (mode == LLMQ_MODE_TT) return b_format ? gemm_dispatch_kmajor<1, false, true>(g, workspace_or_null, workspace_bytes, st) : gemm_dispatch_kmajor<0, false, true>(g, workspace_or_null, workspace_bytes, st);
-    if (mode == LLMQ_MODE_NN) return b_format ? gemm_dispatch_kmajor<1, true, false>(g, workspace_or_null, workspace_bytes, st) : gemm_dispatch_kmajor<0, true, false>(g, workspace_or_null, workspace_bytes, st);
-    LLMQ_REQUIRE(mode == LLMQ_MODE_NT, "matmul: unknown operand mode %d (TT = 0, TN = 1, NT = 2, NN = 3)", mode);
-    return b_format ? gemm_dispatch_kmajor<1, true, true>(g, workspace_or_null, workspace_bytes, st) : gemm_dispatch_kmajor<0, true, true>(g, workspace_or_null, workspace_bytes, st);
+    llmq::GemmArgs g{c, a, b, bias_or_null, sa_or_null, sb_or_null, M, N, K, 1, accumulate, 8, nullptr, 0, 1, 0, 8, 0};
+    return llmq::gemm_with_mode<uint16_t>(g, workspace_or_null, workspace_bytes, mode, b_format, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int llmq_gemm_e4m3_f32_mode(float* c, const uint8_t* a, const uint8_t* b, const void* bias_or_null, int bias_is_bf16,
+                                       const float* sa_or_null, const float* sb_or_null, void* workspace_or_null,
+                                       size_t workspace_bytes, int M, int N, int K, int mode, int b_format, int accumulate,
+                                       void* stream) {
+    llmq::GemmArgs g{c, a, b, bias_or_null, sa_or_null, sb_or_null, M, N, K, bias_is_bf16, accumulate, 8, nullptr, 0, 1, 0, 8, 0};
+    return llmq::gemm_with_mode<float>(g, workspace_or_null, workspace_bytes, mode, b_format, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int llmq_gemm_tn_e4m3_bf16(uint16_t* c, const uint8_t* a, const uint8_t* b, const uint16_t* bias_or_null,

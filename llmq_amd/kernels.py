@@ -128,21 +128,27 @@ def matmul(c, a, b, bias, scale_a, scale_b, M, N, K, accumulate=False, stream=0,
     if b_kmajor or a_kmajor:
         # the reference's modes TT (b stored [K, N] row-major, e.g. the output gradient dY[BT, OC] as the second operand
         # of the weight gradient without its transposed copy), NN (a stored [K, M], e.g. the weight W[OC, C] as the
-        # first operand of the dgrad) and NT (both); bf16 output, whole 256-tiles only
-        if c.dtype != torch.bfloat16:
-            raise ValueError("matmul: K-major operands are served with bf16 output only")
+        # first operand of the dgrad) and NT (both); whole 256-tiles only
         pa = _dev(a, "a", (torch.float8_e4m3fn, torch.uint8))
         pb = _dev(b, "b", (torch.float8_e4m3fn, torch.float8_e5m2, torch.uint8))
+        pc = _dev(c, "c", (torch.bfloat16, torch.float32))
         if a.numel() != M * K or b.numel() != N * K or c.numel() != N * M:
             raise ValueError("operand sizes do not match M, N, K")
-        pbias = _dev(bias, "bias", (torch.bfloat16,), optional=True)
         if bias is not None and bias.numel() != M:
             raise ValueError("bias must have M elements")
-        capi.check(L.llmq_gemm_e4m3_bf16_mode(
-            _dev(c, "c", (torch.bfloat16,)), pa, pb, pbias, _dev(scale_a, "scale_a", (torch.float32,), optional=True),
-            _dev(scale_b, "scale_b", (torch.float32,), optional=True), pws, ws_bytes, M, N, K,
-            (2 if b_kmajor else 3) if a_kmajor else 0,      # EMMTranspose: TT = 0, TN = 1, NT = 2, NN = 3
-            int(bool(b_e5m2) or b.dtype == torch.float8_e5m2), int(accumulate), _stream(stream)), L)
+        sa = _dev(scale_a, "scale_a", (torch.float32,), optional=True)
+        sb = _dev(scale_b, "scale_b", (torch.float32,), optional=True)
+        mode = (2 if b_kmajor else 3) if a_kmajor else 0      # EMMTranspose: TT = 0, TN = 1, NT = 2, NN = 3
+        fmt = int(bool(b_e5m2) or b.dtype == torch.float8_e5m2)
+        if c.dtype == torch.bfloat16:
+            pbias = _dev(bias, "bias", (torch.bfloat16,), optional=True)
+            capi.check(L.llmq_gemm_e4m3_bf16_mode(pc, pa, pb, pbias, sa, sb, pws, ws_bytes, M, N, K, mode, fmt, int(accumulate),
+                                                  _stream(stream)), L)
+        else:
+            pbias = _dev(bias, "bias", (torch.bfloat16, torch.float32), optional=True)
+            is_bf16 = int(bias is not None and bias.dtype == torch.bfloat16)
+            capi.check(L.llmq_gemm_e4m3_f32_mode(pc, pa, pb, pbias, is_bf16, sa, sb, pws, ws_bytes, M, N, K, mode, fmt,
+                                                 int(accumulate), _stream(stream)), L)
         return
     pa = _dev(a, "a", (torch.float8_e4m3fn, torch.uint8))   # e5m2 is supported for b only (kernels.h:92-94)
     pb = _dev(b, "b", (torch.float8_e4m3fn, torch.float8_e5m2, torch.uint8))

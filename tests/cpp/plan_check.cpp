@@ -27,15 +27,21 @@ int main() {
     // Qwen2.5-1.5B (1536 / 8960): small weights -> copying dgrad
     expect_plan("1.5B down", 16384, 8960, 1536, BF, BF, false, false, false, W::BothInPlace);
     expect_plan("1.5B gate+up", 16384, 1536, 17920, BF, BF, false, false, false, W::GradInPlace);
-    // accumulation: NT does not accumulate -> TT while C <= 8192, else the copies
+    // accumulation (gradient-accumulation micro-steps) and fp32 weight gradients are served in place as well
     expect_plan("accumulate, small C", 8192, 3584, 37888, BF, BF, true, false, true, W::GradInPlace);
-    expect_plan("accumulate, large C", 8192, 18944, 3584, BF, BF, true, false, true, W::Copies);
-    // fp32 weight gradient / fp32 dinp are not served in place
-    expect_plan("fp32 dweight", 8192, 18944, 3584, BF, F32, false, false, true, W::Copies);
+    expect_plan("accumulate, large C", 8192, 18944, 3584, BF, BF, true, false, true, W::BothInPlace);
+    expect_plan("fp32 dweight", 8192, 18944, 3584, BF, F32, false, false, true, W::BothInPlace);
+    expect_plan("fp32 dweight, accumulate", 8192, 18944, 3584, BF, F32, true, false, true, W::BothInPlace);
+    expect_plan("fp32 dweight, gate+up", 8192, 3584, 37888, BF, F32, true, false, true, W::GradInPlace);
+    expect_plan("1.5B down, fp32 dweight, accumulate", 16384, 8960, 1536, BF, F32, true, false, false, W::BothInPlace);
+    // an fp32 dinp is not served in place
     expect_plan("fp32 dinp", 8192, 18944, 3584, F32, BF, false, false, false, W::BothInPlace);
-    // Qwen2.5-0.5B (C = 896 = 4 x 224): only the gradient in place, on 224-wide tiles, and not when accumulating
+    // Qwen2.5-0.5B (C = 896 = 4 x 224): only the gradient in place, on 224-wide tiles (bf16 output without accumulation)
     expect_plan("0.5B gate+up", 8192, 896, 9728, BF, BF, false, false, false, W::GradInPlace);
     expect_plan("0.5B gate+up, accumulate", 8192, 896, 9728, BF, BF, true, false, false, W::Copies);
+    expect_plan("0.5B gate+up, fp32 dweight", 8192, 896, 9728, BF, F32, false, false, false, W::Copies);
+    // 0.5B down (C = 4864 = 19 x 256, OC = 896): OC off the 256 lattice -> copies
+    expect_plan("0.5B down, fp32 dweight", 8192, 4864, 896, BF, F32, false, false, false, W::Copies);
     // off the 256 lattice: nothing
     expect_plan("OC = 1152", 1024, 896, 1152, BF, BF, false, false, false, W::Copies);
     expect_plan("BT = 1000", 1000, 1024, 1024, BF, BF, false, true, false, W::Copies);

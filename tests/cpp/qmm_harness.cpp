@@ -39,8 +39,9 @@ static Tensor make(ETensorDType dt, void* p, std::vector<long> shape, float* sta
     return t;
 }
 
+// old: values c held before an accumulating matmul (empty: none), decoded to double
 static void check_gemm(const char* name, const std::vector<uint16_t>& got_bf16, const std::vector<float>& got_f32, int N, int M,
-                       const uint8_t* a, const uint8_t* b, int K, float scale) {
+                       const uint8_t* a, const uint8_t* b, int K, float scale, const std::vector<double>& old = {}) {
     const int S = 20000;
     std::vector<int32_t> in(S), im(S);
     uint64_t s = 88172645463325252ull;
@@ -52,8 +53,8 @@ static void check_gemm(const char* name, const std::vector<uint16_t>& got_bf16, 
     for (int i = 0; i < S; ++i) {
         const std::size_t o = (std::size_t)in[i] * M + im[i];
         const double g = bf16 ? (double)orc_bf16_to_f32(got_bf16[o]) : (double)got_f32[o];
-        const double ref = ex[i] * scale, err = std::fabs(g - ref);
-        const double bound = (bf16 ? std::ldexp(std::fabs(ref), -8) : 0.0) + std::ldexp(scale * sa[i], -11) + 1e-38;
+        const double ref = ex[i] * scale + (old.empty() ? 0.0 : old[o]), err = std::fabs(g - ref);
+        const double bound = std::ldexp(std::fabs(ref), bf16 ? -8 : -23) + std::ldexp(scale * sa[i], -11) + 1e-38;
         worst = std::fmax(worst, err / bound); maxabs = std::fmax(maxabs, err); e2 += err * err; r2 += ref * ref;
     }
     const double fro = std::sqrt(e2 / r2);
@@ -67,19 +68,21 @@ int main(int argc, char** argv) {
     const bool reuse_inp = argc > 4 && std::atoi(argv[4]) != 0;
     const bool fuse = argc > 5 && std::atoi(argv[5]) != 0;   // gradient quantize + transpose from one read
     // 1: bf16 weight gradient; 2: also ask for operands in their stored layouts (matmul modes NN / TT / NT) where the
-    // plan expects them to pay; 3: wherever the shapes are served
+    // plan expects them to pay; 3: wherever the shapes are served; 4 / 5: as 2 / 3 with an fp32 weight gradient
     const int dw_mode = argc > 6 ? std::atoi(argv[6]) : 0;
-    const bool dw_bf16 = dw_mode >= 1, direct = dw_mode >= 2, wherever = dw_mode == 3;
+    const bool dw_bf16 = dw_mode >= 1 && dw_mode <= 3, direct = dw_mode >= 2, wherever = dw_mode == 3 || dw_mode == 5;
+    // gradient accumulation: dweight starts from given values and the weight-gradient matmul adds to them
+    const bool accumulate = argc > 7 && std::atoi(argv[7]) != 0;
     const int B = 1, T = BT;
-    std::printf("qmm_harness BT=%d C=%d OC=%d reuse_inp=%d fuse=%d dweight=%s direct_grad_layout=%d wherever_served=%d\n", BT, C, OC,
-                (int)reuse_inp, (int)fuse, dw_bf16 ? "bf16" : "fp32", (int)direct, (int)wherever);
+    std::printf("qmm_harness BT=%d C=%d OC=%d reuse_inp=%d fuse=%d dweight=%s direct_grad_layout=%d wherever_served=%d accumulate=%d\n", BT, C, OC,
+                (int)reuse_inp, (int)fuse, dw_bf16 ? "bf16" : "fp32", (int)direct, (int)wherever, (int)accumulate);
     hipStream_t stream; HIP_OK(hipStreamCreate(&stream));
     QmmRunState rs; HIP_OK(hipGetDeviceProperties(&rs.DeviceProp, 0));
     rs.FuseGradTranspose = fuse;
     rs.DirectGradLayout = direct;
     rs.DirectGradLayoutWhereverServed = wherever;
     const QmmRunState::DirectPlan plan =
-        direct ? QmmRunState::direct_layout_plan(B, T, C, OC, ETensorDType::BF16, dw_bf16 ? ETensorDType::BF16 : ETensorDType::FP32, false,
+        direct ? QmmRunState::direct_layout_plan(B, T, C, OC, ETensorDType::BF16, dw_bf16 ? ETensorDType::BF16 : ETensorDType::FP32, accumulate,
                                                  wherever)
                : QmmRunState::DirectPlan{};
     std::printf("stored-layout plan: dgrad in place %d, wgrad %s\n", (int)plan.DgradInPlace,
@@ -125,7 +128,22 @@ int main(int argc, char** argv) {
     HIP_OK(hipMemcpy(dbias.Data, hdb0.data(), (std::size_t)OC * 2, hipMemcpyHostToDevice));
     const int bias_scratch = get_bias_backward_scratch_size(ETensorDType::FP8_E4M3, OC, rs.DeviceProp);   // dtype of the gradient it sums
     Tensor bias_buffer = make(ETensorDType::FP32, dalloc<float>((std::size_t)bias_scratch / 4), {bias_scratch / 4});
-    backward_qmm(dinp, dweight, dbias, dout, inp, weight, bias_buffer, false, rs, B, T, C, OC, reuse_inp, stream);
+    // the weight gradient an accumulating micro-step starts from
+    std::vector<double> dw_old;
+    if (accumulate) {
+        std::vector<uint16_t> h0((std::size_t)OC * C);
+        orc_fill_normal_bf16(h0.data(), h0.size(), 7, 5, 0.f, 1e-3f);
+        dw_old.resize(h0.size());
+        for (std::size_t i = 0; i < h0.size(); ++i) dw_old[i] = (double)orc_bf16_to_f32(h0[i]);
+        if (dw_bf16) {
+            HIP_OK(hipMemcpy(dweight.Data, h0.data(), h0.size() * 2, hipMemcpyHostToDevice));
+        } else {
+            std::vector<float> f0(h0.size());
+            for (std::size_t i = 0; i < h0.size(); ++i) f0[i] = orc_bf16_to_f32(h0[i]);
+            HIP_OK(hipMemcpy(dweight.Data, f0.data(), f0.size() * 4, hipMemcpyHostToDevice));
+        }
+    }
+    backward_qmm(dinp, dweight, dbias, dout, inp, weight, bias_buffer, accumulate, rs, B, T, C, OC, reuse_inp, stream);
     HIP_OK(hipStreamSynchronize(stream));
     EXPECT(rs.Top == 0 && rs.Live.empty(), "temporary stack not unwound");
     EXPECT(rs.HighWater == rs.Capacity, "backward_temp_bytes (%zu) != high-water mark (%zu)", rs.Capacity, rs.HighWater);
@@ -160,7 +178,7 @@ int main(int argc, char** argv) {
     orc_transpose_u8(gqt.data(), gq.data(), BT, OC);
     check_gemm("forward", hy, {}, BT, OC, wq.data(), xq.data(), C, sw * sx);
     check_gemm("dgrad", hdx, {}, BT, C, wqt.data(), gq.data(), OC, sw * sg);
-    check_gemm("wgrad", hdw16, hdw, OC, C, xqt.data(), gqt.data(), BT, sx * sg);
+    check_gemm("wgrad", hdw16, hdw, OC, C, xqt.data(), gqt.data(), BT, sx * sg, dw_old);
 
     {   // dbias += sx*sg * column sums of the quantized gradient (llama_model.cpp:334-336)
         std::vector<uint16_t> hdb(OC), want(hdb0);
@@ -270,9 +288,9 @@ int main(int argc, char** argv) {
     catch (const std::invalid_argument&) { threw = true; }
     EXPECT(threw, "matmul with K %% 16 != 0 (operand rows not 16-byte aligned) must throw std::invalid_argument");
     threw = false;
-    try { matmul(out, weight, inp.Quant, no_bias, nullptr, nullptr, nullptr, workspace, OC, BT, C, EMMTranspose::NN, true, stream); }
+    try { matmul(out, weight, inp.Quant, no_bias, nullptr, nullptr, nullptr, workspace, OC, BT, C + 16, EMMTranspose::NN, false, stream); }
     catch (const std::invalid_argument&) { threw = true; }
-    EXPECT(threw, "FP8 matmul in mode NN with accumulation (not served) must throw std::invalid_argument");
+    EXPECT(threw, "FP8 matmul in mode NN off the 256 lattice (not served) must throw std::invalid_argument");
     threw = false;
     try { quantize_with_abs_max(out, nullptr, inp.Value, stats, 8, rs.DeviceProp, stream); }
     catch (const std::invalid_argument&) { threw = true; }

@@ -21,7 +21,13 @@ BIN = os.path.join(HERE, "cpp", "build", "qmm_harness")
                                   ("1024", "1024", "1536", "0", "0", "1"), ("1024", "1024", "1536", "0", "0", "2"),
                                   ("1024", "1024", "1536", "0", "0", "3"), ("1024", "768", "9216", "0", "0", "2"),
                                   ("1024", "768", "9216", "0", "0", "3"), ("2048", "896", "768", "1", "0", "2"),
-                                  ("1024", "896", "1152", "0", "1", "2"), ("512", "1536", "512", "1", "1", "3")])
+                                  ("1024", "896", "1152", "0", "1", "2"), ("512", "1536", "512", "1", "1", "3"),
+                                  # fp32 weight gradients and gradient accumulation with the stored layouts ("4" / "5":
+                                  # fp32 dweight; last argument: accumulate): NN + NT into fp32; NT accumulating into
+                                  # bf16; TT accumulating into fp32 (OC = 9216); accumulation on the copying route
+                                  ("1024", "1024", "1536", "0", "0", "5"), ("1024", "1024", "1536", "0", "0", "3", "1"),
+                                  ("1024", "768", "9216", "0", "0", "4", "1"), ("1024", "1024", "1536", "0", "0", "5", "1"),
+                                  ("1024", "896", "1152", "0", "0", "1", "1")])
 def test_qmm_harness(args):
     assert os.path.exists(BIN), "build it with `make -C tests/cpp` (done by __graft_entry__.build())"
     r = subprocess.run([BIN, *args], capture_output=True, text=True, timeout=150)
@@ -39,4 +45,9 @@ PLANS = {("1024", "1024", "1536", "0", "0", "2"): "dgrad in place 0, wgrad both 
          ("1024", "768", "9216", "0", "0", "3"): "dgrad in place 1, wgrad both in place (NT)",
          ("2048", "896", "768", "1", "0", "2"): "dgrad in place 0, wgrad gradient in place (TT)",
          ("1024", "896", "1152", "0", "1", "2"): "dgrad in place 0, wgrad copies",
-         ("512", "1536", "512", "1", "1", "3"): "dgrad in place 1, wgrad both in place (NT)"}
+         ("512", "1536", "512", "1", "1", "3"): "dgrad in place 1, wgrad both in place (NT)",
+         ("1024", "1024", "1536", "0", "0", "5"): "dgrad in place 1, wgrad both in place (NT)",
+         ("1024", "1024", "1536", "0", "0", "3", "1"): "dgrad in place 1, wgrad both in place (NT)",
+         ("1024", "768", "9216", "0", "0", "4", "1"): "dgrad in place 0, wgrad gradient in place (TT)",
+         ("1024", "1024", "1536", "0", "0", "5", "1"): "dgrad in place 1, wgrad both in place (NT)",
+         ("1024", "896", "1152", "0", "0", "1", "1"): None}

@@ -736,7 +736,7 @@ def test_gemm_operands_in_k_major_layout(K, O, mnk, mode):
     bias = O.f32_to_bf16(biasv.astype(np.float32))
     old = O.f32_to_bf16(oldv.astype(np.float32)).reshape(N, M)
     mt = M % 64 == 0
-    cases = [(False, False), (True, False)] + ([(True, True)] if M % 256 == 0 and not a_km else [])
+    cases = [(False, False), (True, False)] + ([(True, True)] if M % 256 == 0 else [])
     for use_bias, use_old in cases:
         want = O.gemm_tn(a, b, sa=s, sb=s, bias=bias if use_bias else None, c_old=old if use_old else None, mt=mt)
         c = dev_bf16(old).reshape(N, M).clone() if use_old else torch.full((N, M), float("nan"), dtype=torch.bfloat16, device="cuda")
@@ -773,13 +773,65 @@ def test_gemm_operands_in_k_major_layout(K, O, mnk, mode):
 
 
 @pytest.mark.parametrize("mode", ["TT", "NN", "NT"])
+@pytest.mark.parametrize("mnk", [(256, 256, 256), (512, 768, 512), (1024, 2048, 1024), (4352, 4352, 1024), (4608, 4096, 512)])
+def test_gemm_k_major_fp32_output_and_accumulation(K, O, mnk, mode):
+    """The K-major modes with fp32 output and with accumulation into c (the reference's matmul takes every mode with
+    either, src/kernels/matmul.cpp:66-92: fp32 weight gradients, gradient-accumulation micro-steps).  With a K-major
+    first operand these go through the fp32-staged epilogue.  Integer operands -> bit exact against the oracle (bias,
+    old values, both output types, with and without a workspace, i.e. with the last round cut where the plan cuts it);
+    random codes -> bit-identical to mode TN on the transposed copies under the same plan, launch after launch."""
+    M, N, Kd = mnk
+    a_km, b_km = mode[0] == "N", mode[1] == "T"
+    lay_a = (lambda x: np.ascontiguousarray(x.T)) if a_km else (lambda x: x)
+    lay_b = (lambda x: np.ascontiguousarray(x.T)) if b_km else (lambda x: x)
+    a, _ = O.fill_int_e4m3(M * Kd, 919, 0)
+    b, _ = O.fill_int_e4m3(N * Kd, 919, 1)
+    a, b = a.reshape(M, Kd), b.reshape(N, Kd)
+    s = float(np.sqrt(np.float32(4.0 / Kd)))
+    _, biasv = O.fill_int_e4m3(M, 919, 2)
+    _, oldv = O.fill_int_e4m3(N * M, 919, 3)
+    bias = O.f32_to_bf16(biasv.astype(np.float32))
+    oldf = oldv.astype(np.float32).reshape(N, M)
+    for out_f32, use_bias, use_old, with_ws in [(True, False, False, False), (True, True, True, True), (True, False, True, False),
+                                                (False, True, True, False), (False, False, True, True)]:
+        old = (oldf if out_f32 else O.f32_to_bf16(oldf).reshape(N, M)) if use_old else None
+        want = O.gemm_tn(a, b, sa=s, sb=s, bias=bias if use_bias else None, c_old=old, out_f32=out_f32, mt=True)
+        dt = torch.float32 if out_f32 else torch.bfloat16
+        if use_old:
+            c = (torch.from_numpy(old).cuda() if out_f32 else dev_bf16(old)).reshape(N, M).clone()
+        else:
+            c = torch.full((N, M), float("nan"), dtype=dt, device="cuda")
+        K.matmul(c, dev_u8(lay_a(a)), dev_u8(lay_b(b)), dev_bf16(bias) if use_bias else None, dev_scalar(s), dev_scalar(s), M, N, Kd,
+                 accumulate=use_old, a_kmajor=a_km, b_kmajor=b_km, workspace=workspace() if with_ws else None)
+        got = c.cpu().numpy() if out_f32 else host_bits(c)
+        assert np.array_equal(got, want), (out_f32, use_bias, use_old, with_ws)
+    rng = np.random.default_rng(M + N)
+    ar = rng.integers(0, 256, (M, Kd)).astype(np.uint8)
+    br = rng.integers(0, 256, (N, Kd)).astype(np.uint8)
+    ar[(ar & 0x7F) == 0x7F] ^= 1
+    br[(br & 0x7F) == 0x7F] ^= 1
+    start = torch.from_numpy(rng.standard_normal((N, M)).astype(np.float32)).cuda()
+    set_variant((3, 0))                       # mode TN on the four-wave kernel: the same sums in the same order
+    try:
+        c_tn = start.clone()
+        mm(K, c_tn, dev_u8(ar), dev_u8(br), None, dev_scalar(0.37), dev_scalar(1.0 / 448), M, N, Kd, accumulate=True, workspace=workspace())
+        for _ in range(3):
+            c_km = start.clone()
+            mm(K, c_km, dev_u8(lay_a(ar)), dev_u8(lay_b(br)), None, dev_scalar(0.37), dev_scalar(1.0 / 448), M, N, Kd, accumulate=True,
+               a_kmajor=a_km, b_kmajor=b_km, workspace=workspace())
+            assert torch.equal(c_tn.view(torch.int32), c_km.view(torch.int32))
+    finally:
+        set_variant((0, 0))
+
+
+@pytest.mark.parametrize("mode", ["TT", "NN", "NT"])
 @pytest.mark.parametrize("cut", [0, 2, 4])
 @pytest.mark.parametrize("mnk", [(4352, 4352, 1024), (4608, 4096, 512), (4352, 4096, 1536), (8192, 4864, 512)])
 def test_gemm_k_major_last_round_cut(K, O, mnk, mode, cut):
     """K-major operands with a workspace: the tiles left over after the full rounds are cut into K segments (a
     second launch of the same operand mode writing raw fp32 tiles, summed in a fixed order by the reduction kernel),
     as in mode TN.  cut = 2, 4: forced; 0: whatever the plan decides with the workspace given.  Integer operands ->
-    bit exact against the oracle, with bias and (mode TT) accumulation; random codes bit-identical to mode TN under
+    bit exact against the oracle, with bias and accumulation; random codes bit-identical to mode TN under
     the same plan, and on repeated launches."""
     M, N, Kd = mnk
     variant = (3, cut)          # mode TN on the four-wave kernel as well: the same sums in the same order
@@ -802,7 +854,7 @@ def test_gemm_k_major_last_round_cut(K, O, mnk, mode, cut):
     br[(br & 0x7F) == 0x7F] ^= 1
     set_variant(variant)
     try:
-        for use_bias, use_old in [(False, False), (True, False)] + ([] if a_km else [(True, True)]):
+        for use_bias, use_old in [(False, False), (True, False), (True, True)]:
             want = O.gemm_tn(a, b, sa=s, sb=s, bias=bias if use_bias else None, c_old=old if use_old else None, mt=True)
             c = dev_bf16(old).reshape(N, M).clone() if use_old else torch.full((N, M), float("nan"), dtype=torch.bfloat16, device="cuda")
             mm(K, c, dev_u8(lay_a(a)), dev_u8(lay_b(b)), dev_bf16(bias) if use_bias else None, dev_scalar(s), dev_scalar(s), M, N, Kd,
@@ -957,11 +1009,12 @@ def test_gemm_k_major_operand_rejects_what_it_cannot_serve(K):
     c = torch.zeros((256, 256), dtype=torch.bfloat16, device="cuda")
     with pytest.raises(ValueError, match="mode TT"):
         K.matmul(c, a, b, None, None, None, 256, 256, 384, b_kmajor=True)      # K % 256 != 0
-    with pytest.raises(ValueError, match="does not accumulate"):
-        K.matmul(c, torch.zeros((512, 256), dtype=torch.uint8, device="cuda"), torch.zeros((256, 512), dtype=torch.uint8, device="cuda"),
-                 None, None, None, 256, 256, 512, accumulate=True, a_kmajor=True)
-    with pytest.raises(ValueError, match="bf16 output"):
-        K.matmul(c.float(), a, b, None, None, None, 256, 256, 384, b_kmajor=True)
+    with pytest.raises(ValueError, match="mode NN"):
+        K.matmul(torch.zeros((256, 224), device="cuda"), torch.zeros((256, 224), dtype=torch.uint8, device="cuda"),
+                 torch.zeros((256, 256), dtype=torch.uint8, device="cuda"), None, None, None, 224, 256, 256, a_kmajor=True)   # needs M % 256 == 0
+    with pytest.raises(ValueError, match="mode TT"):
+        K.matmul(torch.zeros((256, 224), device="cuda"), torch.zeros((224, 256), dtype=torch.uint8, device="cuda"),
+                 torch.zeros((256, 256), dtype=torch.uint8, device="cuda"), None, None, None, 224, 256, 256, b_kmajor=True)   # 224-wide tiles: bf16 only
     # a bias that is too short would be read out of bounds by the epilogue: refused by the wrapper in every operand mode
     short_bias = torch.zeros(128, dtype=torch.bfloat16, device="cuda")
     with pytest.raises(ValueError, match="bias must have M elements"):
