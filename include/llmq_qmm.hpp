@@ -64,7 +64,11 @@ struct QmmRunState {
                          (wherever_served || ((long)C * OC >= (48L << 20) && BT >= 8192 && BT <= 16384));
         const bool bf16_dw = dweight_dtype == ETensorDType::BF16;
         if ((bf16_dw || dweight_dtype == ETensorDType::FP32) && OC % 256 == 0 && BT % 256 == 0 && BT * OC < lim) {
-            if (tiles && BT * C < lim && (wherever_served || OC <= 8192)) p.Wgrad = EWgrad::BothInPlace;
+            // accumulating into c with both operands K-major costs the fp32-staged epilogue a read of the old values in
+            // 8- or 16-byte pieces: measured ahead of the copies on the 1.5B layers (184 against 238 us, 436 against 485 us
+            // into fp32), behind them on the 7B ones (533 against 512 us): taken for weights up to 32 M elements
+            const bool nt_pays = !accumulate || (long)C * OC <= (32L << 20);
+            if (tiles && BT * C < lim && (wherever_served || (OC <= 8192 && nt_pays))) p.Wgrad = EWgrad::BothInPlace;
             else if ((C % 256 == 0 || (C % 224 == 0 && bf16_dw && !accumulate)) && (wherever_served || C <= 8192)) p.Wgrad = EWgrad::GradInPlace;
         }
         return p;

@@ -29,9 +29,10 @@ int main() {
     expect_plan("1.5B gate+up", 16384, 1536, 17920, BF, BF, false, false, false, W::GradInPlace);
     // accumulation (gradient-accumulation micro-steps) and fp32 weight gradients are served in place as well
     expect_plan("accumulate, small C", 8192, 3584, 37888, BF, BF, true, false, true, W::GradInPlace);
-    expect_plan("accumulate, large C", 8192, 18944, 3584, BF, BF, true, false, true, W::BothInPlace);
+    expect_plan("accumulate, large C and large weight", 8192, 18944, 3584, BF, BF, true, false, true, W::Copies);
+    expect_plan("accumulate, large weight, wherever served", 8192, 18944, 3584, BF, BF, true, true, true, W::BothInPlace);
     expect_plan("fp32 dweight", 8192, 18944, 3584, BF, F32, false, false, true, W::BothInPlace);
-    expect_plan("fp32 dweight, accumulate", 8192, 18944, 3584, BF, F32, true, false, true, W::BothInPlace);
+    expect_plan("fp32 dweight, accumulate", 8192, 18944, 3584, BF, F32, true, false, true, W::Copies);
     expect_plan("fp32 dweight, gate+up", 8192, 3584, 37888, BF, F32, true, false, true, W::GradInPlace);
     expect_plan("1.5B down, fp32 dweight, accumulate", 16384, 8960, 1536, BF, F32, true, false, false, W::BothInPlace);
     // an fp32 dinp is not served in place
