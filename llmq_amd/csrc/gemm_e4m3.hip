@@ -13,8 +13,9 @@
 //     operand modes and the K segments of a cut last round;
 //   * gemm_tn_e4m3_pipe_kernel: 256 x 256 tile with 8 waves of 128 x 64 or 128 x 128 tile with 4 waves
 //     of 64 x 64, v_mfma_f32_32x32x64_f8f6f4; the other shapes on the 128 lattice, and the split-K path;
-//   * gemm_tn_e4m3_edge_kernel: 64 x 64 tile with predicated loads and stores: shapes off the lattice (any M, N; K a
-//     multiple of 16) and the last N % tile rows of the others.
+//   * gemm_tn_e4m3_edge_kernel: 64 x 64 tile with predicated loads and stores: small shapes off the lattice (any M, N; K
+//     a multiple of 16) and the last N % tile rows of the others; large shapes off the lattice run on RAGGED instances
+//     of the four-wave kernel (last tile row / column moved back into the matrix, K tail masked in the copies).
 // Common to the tiled kernels:
 //   * one workgroup computes a tile of c, K is walked in steps of 128 bytes;
 //   * both operand tiles are staged in LDS, double buffered, by 16-byte-per-lane direct-to-LDS loads
@@ -86,9 +87,11 @@ __device__ __forceinline__ void xcd_tile_range(int total, int xcds, int xcd, int
 
 // Logical tile number -> tile origin: groups of `group` tile-rows, column-major inside a group.
 // Tiles are 256 rows (n) by BM columns (m).
-template <int BM = 256>
+// RAGGED: N and M need not be multiples of the tile: the tile counts round up and the last tile row / column is
+// moved back so that it ends with the matrix (its first rows / columns then repeat those of its neighbour).
+template <int BM = 256, bool RAGGED = false>
 __device__ __forceinline__ void decode_tile256(const GemmArgs& g, int logical, int& n_blk, int& m_blk) {
-    const int tiles_n = g.N / 256, tiles_m = g.M / BM;
+    const int tiles_n = RAGGED ? (g.N + 255) / 256 : g.N / 256, tiles_m = RAGGED ? (g.M + BM - 1) / BM : g.M / BM;
     const int per_group = g.group * tiles_m;
     const int gid = logical / per_group;
     const int first_n = gid * g.group;
@@ -96,6 +99,10 @@ __device__ __forceinline__ void decode_tile256(const GemmArgs& g, int logical, i
     const int in_group = logical % per_group;
     n_blk = (first_n + in_group % gsz) * 256;
     m_blk = (in_group / gsz) * BM;
+    if constexpr (RAGGED) {
+        if (n_blk > g.N - 256) n_blk = g.N - 256;
+        if (m_blk > g.M - BM) m_blk = g.M - BM;
+    }
 }
 
 #define LLMQ_GLOBAL __attribute__((address_space(1)))
@@ -613,8 +620,9 @@ __device__ __forceinline__ int frag_swizzle(int row) {
 // fragment row into a private 4 KiB piece of LDS, read back as 16 bytes per lane and row.  bf16 output without
 // accumulation (the old values of c would have to be fetched in the scattered layout).
 template <typename OutT, int B_FMT, bool SEG, int NJ = 8, bool STREAM_OUT = true, bool ODDK = false, bool KMB = false,
-          bool KMA = false, bool FUSE_EPI = false, bool STAGE32 = false>
+          bool KMA = false, bool FUSE_EPI = false, bool STAGE32 = false, bool RAGGED = false>
 __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
+    static_assert(!RAGGED || (NJ == 8 && !SEG && !KMA && !KMB && !FUSE_EPI), "ragged shapes: full-width tiles of K-contiguous operands");
     static_assert(!(SEG && ODDK), "K segments are whole pairs of K-steps");
     static_assert(!STAGE32 || (KMA && !SEG && NJ == 8), "the fp32-staged epilogue belongs to the K-major first operand");
     static_assert(!FUSE_EPI || (NJ == 8 && !SEG && !KMA && std::is_same_v<OutT, uint16_t>),
@@ -646,12 +654,14 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     // XCD's last, partial round are left to a second launch of this kernel (SEG) that cuts each of them
     // into S segments of K (slot s: tile s / S, segment s % S) and writes raw accumulators as a 256 x 256
     // fp32 tile to g.partial for the reduction kernel below: the round then costs 1 / S of a tile.
-    const int total = (g.N / BLK) * (g.M / BLKM);
+    const int total = RAGGED ? ((g.N + BLK - 1) / BLK) * ((g.M + BLKM - 1) / BLKM) : (g.N / BLK) * (g.M / BLKM);
     const int xcd = blockIdx.x % g.xcds, slot = blockIdx.x / g.xcds;
     int xcd_first, xcd_count;
     xcd_tile_range(total, g.xcds, xcd, xcd_first, xcd_count);
     const int tile_stride = gridDim.x / g.xcds;
-    int my_tiles, k_first = 0, k_total = g.K;
+    // RAGGED: K is a multiple of 16 only; the stream walks K rounded up to whole steps and the copies of a tile's last
+    // step leave the chunks beyond K to zeros (issue_copy)
+    int my_tiles, k_first = 0, k_total = RAGGED ? (g.K + kBK - 1) / kBK * kBK : g.K;
     if constexpr (SEG) {
         const int rem = xcd_count % tile_stride;
         my_tiles = slot < rem * g.rem_split ? 1 : 0;
@@ -663,7 +673,7 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         if (g.rem_split > 1) my_tiles = xcd_count / tile_stride;
     }
     if (my_tiles <= 0) return;  // uniform for the whole workgroup, before any barrier
-    auto decode = [&](int logical, int& n_blk, int& m_blk) { decode_tile256<BLKM>(g, logical, n_blk, m_blk); };
+    auto decode = [&](int logical, int& n_blk, int& m_blk) { decode_tile256<BLKM, RAGGED>(g, logical, n_blk, m_blk); };
     // The output factor sa * sb is read here, once, before the copy stream starts.  Read in the epilogue it would be
     // two global loads per tile, and the wait the compiler puts behind each of them (it counts only the loads it
     // knows about, so it waits for "all": vmcnt(0)) would also drain the copies of the next tile's first two K-steps
@@ -741,6 +751,11 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     tile_bases(xcd_first + slot);
     // after the copies of one K-step; past the last tile the stream re-reads that tile's first K-steps
     // (harmless, and no step needs a special case)
+    // RAGGED: in a tile's last, partial K-step (K % 128 != 0) the lanes whose 16-byte chunk lies beyond K write zeros
+    // instead of copying (tail_mask: lanes with a chunk inside K)
+    [[maybe_unused]] const uint64_t tail_mask = __ballot(ld_chunk * 16 < (g.K % kBK == 0 ? kBK : g.K % kBK));
+    [[maybe_unused]] uint64_t copy_mask = ~0ull;   // lane mask of the copies issued next
+    [[maybe_unused]] const uint32_t lane16 = (uint32_t)(lane * 16);
     auto advance_copy = [&]() {
         copy_k0 += kBK;
         vp += p_step;
@@ -768,6 +783,7 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
             if (copy_tile + 1 < my_tiles) ++copy_tile;
             tile_bases(xcd_first + slot + copy_tile * tile_stride);
         }
+        if constexpr (RAGGED) copy_mask = copy_k0 + kBK > g.K ? tail_mask : ~0ull;
     };
     // Copy number c of a K-step, c = 0 .. COPIES-1: first the b-rows slabs, then the a-rows slabs, as two asm
     // statements.  set_m0 computes the LDS destination of the wave's part of the slab into M0 and hands it to the
@@ -801,18 +817,44 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
             lane_ofs = KMA ? (((it >> 1) & 1) ? vq_hi : vq) : (NJ == 7 && it == 3) ? vq3 : (NJ == 7 && it == 6) ? vq6 : vq;
         }
     };
+    // RAGGED: every copy runs under a lane mask -- all lanes, or in a tile's last, partial K-step the lanes whose chunk
+    // lies inside K.  The other lanes neither read global memory nor write LDS; they then store 16 zero bytes to the
+    // place the copy would have filled for them (M0 + 16 * lane, the destination rule of the copy instruction itself).
+    // Every wave has lanes inside K (a wave covers whole rows), so the copy instruction always executes and the counter
+    // bookkeeping of the K-steps holds.  One asm statement with its own branch: a branch of the compiler's between
+    // the write of M0 and the copy makes it save and restore M0 right in front of the copy (too close for the
+    // hardware; the hazard scan of the build rejects it).
+    const v4i zero16 = {0, 0, 0, 0};
+    auto masked_copy = [&](uint32_t lane_ofs, const uint8_t* src, uint32_t tok) {
+        uint32_t tmp;
+        asm volatile(
+            "s_mov_b64 exec, %3\n\t"
+            "global_load_lds_dwordx4 %1, %2\n\t"
+            "s_cmp_eq_u64 %3, -1\n\t"
+            "s_cbranch_scc1 1f\n\t"
+            "s_not_b64 exec, exec\n\t"
+            "v_add_u32 %0, m0, %4\n\t"
+            "ds_write_b128 %0, %5\n\t"
+            "s_mov_b64 exec, -1\n"
+            "1:"
+            : "=&v"(tmp)
+            : "v"(lane_ofs), "s"(src), "s"(copy_mask), "v"(lane16), "v"(zero16), "{m0}"(tok)
+            : "memory", "scc");
+    };
     auto issue_copy = [&](int c, uint32_t tok) {
         const uint8_t* src;
         uint32_t lane_ofs;
         copy_src(c, src, lane_ofs);
-        asm volatile("global_load_lds_dwordx4 %0, %1" : : "v"(lane_ofs), "s"(src), "{m0}"(tok) : "memory");
+        if constexpr (RAGGED) masked_copy(lane_ofs, src, tok);
+        else asm volatile("global_load_lds_dwordx4 %0, %1" : : "v"(lane_ofs), "s"(src), "{m0}"(tok) : "memory");
     };
     auto issue_copy_nop = [&](auto c_tag, auto stage_tag) {
         const uint8_t* src;
         uint32_t lane_ofs;
         copy_src(decltype(c_tag)::value, src, lane_ofs);
         const uint32_t tok = set_m0(c_tag, stage_tag);
-        asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(lane_ofs), "s"(src), "{m0}"(tok) : "memory");
+        if constexpr (RAGGED) masked_copy(lane_ofs, src, tok);   // the write of exec sits between the write of M0 and the copy
+        else asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(lane_ofs), "s"(src), "{m0}"(tok) : "memory");
     };
 
     const int sw = frag_swizzle(l16);
@@ -1208,6 +1250,13 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
             ldc = g.M;
             c = reinterpret_cast<OutT*>(g.c);
         }
+        // RAGGED: a tile moved back to end with the matrix leaves the rows / columns it shares with its neighbour to
+        // that neighbour (with accumulation they must be written once)
+        [[maybe_unused]] int n_own = n_blk, m_own = m_blk;
+        if constexpr (RAGGED) {
+            if (n_blk % BLK) n_own = (n_blk / BLK + 1) * BLK;
+            if (m_blk % BLKM) m_own = (m_blk / BLKM + 1) * BLKM;
+        }
         const int e_lane = opaque(threadIdx.x) % 64;
         const int el16 = e_lane % 16, ekg = e_lane / 16;
         const int m_lane = m_blk + wm * WTM + (NJ == 7 ? 6 : NJ) * el16;
@@ -1379,11 +1428,18 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
                     row[r] = scalar_ptr((LLMQ_GLOBAL char*)(c + (int64_t)(row0 + 16 * i + r) * ldc)) + lane_bytes;
+                // RAGGED: does this lane own its 8 columns of the fragment row's c rows (see n_own / m_own)
+                bool mine[4] = {true, true, true, true};
+                if constexpr (RAGGED) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) mine[r] = m_lane >= m_own && row0 + 16 * i + r + 4 * ekg >= n_own;
+                }
                 // the old values of the fragment row's four c rows are requested together
-                float old[4][8];
+                float old[4][8] = {};
                 if constexpr (ACC) {
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
+                        if (!mine[r]) continue;
                         if constexpr (std::is_same_v<OutT, uint16_t>) {
                             const v4i w = *(const LLMQ_GLOBAL v4i*)row[r];
 #pragma unroll
@@ -1410,6 +1466,7 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
                         if constexpr (BIAS) v[j] = v[j] + bias_v[j];
                         if constexpr (ACC) v[j] = v[j] + old[r][j];
                     }
+                    if (!mine[r]) continue;
                     if constexpr (std::is_same_v<OutT, uint16_t>) {
                         v4i packed;
 #pragma unroll
@@ -1448,7 +1505,8 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         } else {
             if (g.bias) rows(yes, no);
             else rows(no, no);
-            pending_stores = true;
+            // RAGGED: a wave may skip stores it does not own, so their number is not known to the relaxed wait
+            pending_stores = !RAGGED;
         }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the surplus copies issued during the last tile
@@ -1721,6 +1779,22 @@ static void launch_w4(bool odd_k, int grid, const GemmArgs& g, hipStream_t strea
                            dim3((unsigned)grid), dim3(256), 0, stream, g);
 }
 
+// Shapes off the tile lattice on the four-wave kernel (RAGGED instances): M and N from 256 up that need not be multiples
+// of the tile (M a multiple of 8: the lane's 8 adjacent outputs start 16-byte aligned for bf16), K any multiple of 16
+// from three K-steps up.  One persistent launch, whole 256 x 256 tiles, no cut of the last round.
+template <typename OutT, int B_FMT>
+static void launch_w4_ragged(const GemmArgs& g, int cus, int xcds, hipStream_t stream) {
+    const int tiles = ((g.N + 255) / 256) * ((g.M + 255) / 256);
+    const int grid = tiles < cus ? (tiles + xcds - 1) / xcds * xcds : cus;
+    const int steps = (g.K + kBK - 1) / kBK;
+    if (steps % 2)
+        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<OutT, B_FMT, false, 8, true, true, false, false, false, false, true>),
+                           dim3((unsigned)grid), dim3(256), 0, stream, g);
+    else
+        hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<OutT, B_FMT, false, 8, true, false, false, false, false, false, true>),
+                           dim3((unsigned)grid), dim3(256), 0, stream, g);
+}
+
 template <typename OutT, int B_FMT>
 static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     LLMQ_REQUIRE(g.M > 0 && g.N > 0 && g.K > 0, "matmul: M, N, K must be positive (got %d, %d, %d)", g.M, g.N, g.K);
@@ -1755,6 +1829,19 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
     if (!on_lattice) {
         LLMQ_REQUIRE(force_tile == 0 && force_splits == 0,
                      "matmul: M, N, K = %d, %d, %d are off the lattice of the forced kernel variant", g.M, g.N, g.K);
+        // Large enough for whole (moved-back) tiles of the four-wave kernel, and enough of them: that kernel; else the
+        // 64 x 64 kernel.  Measured: 3584 x 8200 x 3600 94 against 322 us, 1000 x 8192 x 3584 (128 tiles) 48 against 74 us,
+        // 4360 x 4100 x 656 35 against 49 us; 1000 x 1000 x 400 (16 tiles) 14 against 7 us.
+        const int64_t ragged_tiles = (int64_t)((g.N + 255) / 256) * ((g.M + 255) / 256);
+        if (g.M >= 256 && g.N >= 256 && g.M % 8 == 0 && g.K >= 3 * kBK && cus % xcds == 0 && ragged_tiles >= cus / 4 &&
+            g_gemm_persist != 0) {
+            g.group = 8;
+            g.rem_split = 1;
+            g.part_per_xcd = 0;
+            launch_w4_ragged<OutT, B_FMT>(g, cus, xcds, stream);
+            LLMQ_HIP_TRY(hipGetLastError());
+            return LLMQ_OK;
+        }
         return launch_edge(0);
     }
     const int n_tail = g.N % (g.M % 128 == 0 ? 128 : 256);

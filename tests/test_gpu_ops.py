@@ -88,8 +88,11 @@ def test_matmul_mode_tt_reads_the_first_operand_in_k_major_storage(P, O):
     exact, sumabs = O.gemm_exact(b, a)
     extra = bias.float().cpu().numpy().astype(np.float64)[None, :]
     gemm_check(c.float().cpu().numpy(), exact, sumabs, np.float32(0.25 * 0.125), True, extra=extra)
-    with pytest.raises(ValueError):                                            # fp32 output is not served in this mode
-        P.matmul(torch.empty((M, N), device="cuda"), at, bd, None, None, None, 0, ws, P.MODE_TT, False)
+    c32 = torch.full((M, N), float("nan"), device="cuda")                      # fp32 output in the same mode, accumulating
+    c32.copy_(extra_old := torch.randn((M, N), device="cuda"))
+    P.matmul(c32, at, bd, bias, sa, sb, 0, ws, P.MODE_TT, True)
+    gemm_check(c32.cpu().numpy(), exact, sumabs, np.float32(0.25 * 0.125), False,
+               extra=extra + extra_old.cpu().numpy().astype(np.float64))
     with pytest.raises(ValueError):                                            # a is [K, M]: handing over [M, K] mismatches c
         P.matmul(c, ad, bd, None, None, None, 0, ws, P.MODE_TT, False)
 
@@ -113,8 +116,9 @@ def test_matmul_modes_with_b_in_k_major_storage(P, O, mode):
     exact, sumabs = O.gemm_exact(b, a)
     extra = bias.float().cpu().numpy().astype(np.float64)[None, :]
     gemm_check(c.float().cpu().numpy(), exact, sumabs, np.float32(0.25 * 0.125), True, extra=extra)
-    with pytest.raises(ValueError):                      # these two modes do not accumulate
-        P.matmul(c, ad, bd, None, sa, sb, 0, ws, P.MODE_NN if mode == "NN" else P.MODE_TN, True)
+    old = c.clone()                                      # the same modes accumulating into c
+    P.matmul(c, ad, bd, None, sa, sb, 0, ws, P.MODE_NN if mode == "NN" else P.MODE_TN, True)
+    gemm_check(c.float().cpu().numpy(), exact, sumabs, np.float32(0.25 * 0.125), True, extra=old.float().cpu().numpy().astype(np.float64))
 
 
 def test_backward_bias_through_ops(P):
