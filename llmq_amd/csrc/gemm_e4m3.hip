@@ -755,7 +755,6 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     // instead of copying (tail_mask: lanes with a chunk inside K)
     [[maybe_unused]] const uint64_t tail_mask = __ballot(ld_chunk * 16 < (g.K % kBK == 0 ? kBK : g.K % kBK));
     [[maybe_unused]] uint64_t copy_mask = ~0ull;   // lane mask of the copies issued next
-    [[maybe_unused]] const uint32_t lane16 = (uint32_t)(lane * 16);
     auto advance_copy = [&]() {
         copy_k0 += kBK;
         vp += p_step;
@@ -824,21 +823,26 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     // bookkeeping of the K-steps holds.  One asm statement with its own branch: a branch of the compiler's between
     // the write of M0 and the copy makes it save and restore M0 right in front of the copy (too close for the
     // hardware; the hazard scan of the build rejects it).
-    const v4i zero16 = {0, 0, 0, 0};
     auto masked_copy = [&](uint32_t lane_ofs, const uint8_t* src, uint32_t tok) {
-        uint32_t tmp;
+        uint32_t addr, zero;   // live inside the statement only: lane number * 16 + M0, and 0
         asm volatile(
-            "s_mov_b64 exec, %3\n\t"
-            "global_load_lds_dwordx4 %1, %2\n\t"
-            "s_cmp_eq_u64 %3, -1\n\t"
+            "s_mov_b64 exec, %4\n\t"
+            "global_load_lds_dwordx4 %2, %3\n\t"
+            "s_cmp_eq_u64 %4, -1\n\t"
             "s_cbranch_scc1 1f\n\t"
             "s_not_b64 exec, exec\n\t"
-            "v_add_u32 %0, m0, %4\n\t"
-            "ds_write_b128 %0, %5\n\t"
+            "v_mbcnt_lo_u32_b32 %0, -1, 0\n\t"
+            "v_mbcnt_hi_u32_b32 %0, -1, %0\n\t"
+            "v_mov_b32 %1, 0\n\t"
+            "v_lshl_add_u32 %0, %0, 4, m0\n\t"
+            "ds_write_b32 %0, %1\n\t"
+            "ds_write_b32 %0, %1 offset:4\n\t"
+            "ds_write_b32 %0, %1 offset:8\n\t"
+            "ds_write_b32 %0, %1 offset:12\n\t"
             "s_mov_b64 exec, -1\n"
             "1:"
-            : "=&v"(tmp)
-            : "v"(lane_ofs), "s"(src), "s"(copy_mask), "v"(lane16), "v"(zero16), "{m0}"(tok)
+            : "=&v"(addr), "=&v"(zero)
+            : "v"(lane_ofs), "s"(src), "s"(copy_mask), "{m0}"(tok)
             : "memory", "scc");
     };
     auto issue_copy = [&](int c, uint32_t tok) {
