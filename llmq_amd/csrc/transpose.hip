@@ -7,7 +7,7 @@
 // Fast path (rows % 16 == 0 and cols % 16 == 0): a workgroup moves a [256 rows] x [128 cols] tile.
 // Each lane reads 16 bytes from each of four consecutive rows (8 lanes cover a 128-byte row segment),
 // transposes the four 4x4 byte blocks in registers with byte-permute instructions, writes the
-// resulting dwords into an LDS tile laid out [col][row] (stride 65 dwords), and the tile is then
+// resulting dwords into an LDS tile laid out [col][row] (stride 65 dwords, see the kernel), and the tile is then
 // written out as 16-byte pieces, 256 contiguous bytes per transposed row.
 // Any other shape takes a simple bounds-checked 64 x 64 tile kernel.
 #include "common.hpp"
@@ -42,6 +42,12 @@ __global__ __launch_bounds__(256) void transpose_u8_kernel(uint8_t* __restrict__
     const int chunk = t % 8;  // 16-column chunk
     const int q = t / 8;      // row quad within a pass (32 per pass, 2 passes)
     const int col = c0 + 16 * chunk;
+    // LDS has 64 banks of 4 bytes and the row stride is 65 dwords: the dword written by lane (chunk, q) lands on bank
+    // 16 chunk + q + const (mod 64), so chunks c and c + 4 would share banks (a two-way conflict on every write).
+    // Flipping bit 3 of the row-quad index for the upper four chunks gives them the other half of each group of 16
+    // banks; the reads below undo it.  Measured: the conflict counter goes from 0.67 to 0.50 of the LDS cycles (the
+    // rest are the four-dword reads); the kernel's rate does not change, it is bound by its global access pattern.
+    const int wr_flip = (chunk >> 2) * 8;
 
     uint4 v[2][4];
 #pragma unroll
@@ -68,7 +74,7 @@ __global__ __launch_bounds__(256) void transpose_u8_kernel(uint8_t* __restrict__
             uint32_t o[4];
             transpose4x4(w[0][k], w[1][k], w[2][k], w[3][k], o);
 #pragma unroll
-            for (int b = 0; b < 4; ++b) tile[(16 * chunk + 4 * k + b) * kTrStride + rq] = o[b];
+            for (int b = 0; b < 4; ++b) tile[(16 * chunk + 4 * k + b) * kTrStride + (rq ^ wr_flip)] = o[b];
         }
     }
     __syncthreads();
@@ -79,7 +85,7 @@ __global__ __launch_bounds__(256) void transpose_u8_kernel(uint8_t* __restrict__
         const int c = item / 16, p = item % 16;
         const int r = r0 + 16 * p;
         if (c0 + c < cols && r < rows) {
-            const uint32_t* s = &tile[c * kTrStride + 4 * p];
+            const uint32_t* s = &tile[c * kTrStride + 4 * (p ^ ((c >> 6) * 2))];
             *reinterpret_cast<uint4*>(dst + (int64_t)(c0 + c) * rows + r) = make_uint4(s[0], s[1], s[2], s[3]);
         }
     }
