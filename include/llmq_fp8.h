@@ -334,9 +334,11 @@ int llmq_rope_backward_bf16(uint16_t* dinp, const uint16_t* dout, const uint16_t
 int llmq_precompute_freqs_cis_f16(uint16_t* freqs_cis_host, int dim, int end, float theta);
 
 /*
- * fp32 overloads of the producers above (a model kept in fp32 whose matmuls run in FP8): the same arithmetic without the
+ * fp32 overloads of the producers above (a model kept in fp32 whose matmuls run in FP8): the same formulas without the
  * roundings to bf16, fp32 tensors throughout; abs_max_or_null as above, bit-identical to llmq_abs_max_f32 of the tensor
- * written.  C must be a multiple of 4 (RMSNorm: at most 8192), head_dim a multiple of 8; the rope table is fp32
+ * written.  The fp32 outputs agree with the reference's to a few fp32 ulp, not bit for bit: its float instantiations are
+ * compiled with multiply-add contraction and use an exponential and a reciprocal that are not specified to the bit,
+ * while these kernels evaluate every product and sum as written (no contraction).  C must be a multiple of 4 (RMSNorm: at most 8192), head_dim a multiple of 8; the rope table is fp32
  * [T, head_dim] of (cos, sin) pairs.  In fp32 RMSNorm the normalised value s * x is the fp32 product itself.
  * Replace the float overloads: swiglu_forward / swiglu_backward  src/kernels/kernels.h:157,164 (src/kernels/swiglu.cu:
  *           304-346,374-401; tested by src/testing/test-swiglu.cu:83-156), rope_forward / rope_backward and
