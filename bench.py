@@ -21,7 +21,8 @@ One JSON line is printed:
   gemm_error      max-abs and relative-Frobenius error of each of the six GEMMs against the exact product of the same
                   e4m3 operands (sampled outputs; computed with the CPU oracle beside the CPU baseline)
 Extra fields: roofline.mfma_only_ceiling_TFLOPs (register-only matrix-instruction loops: what the chip sustains
-under its power limit), roofline.traffic (hardware-counter bytes per GEMM launch, from profiles/), hip_graph_replay
+under its power limit), roofline.sensors_under_step_load (the driver's package power and shader clock, sampled while the
+steps run once more after the timed region), roofline.traffic (hardware-counter bytes per GEMM launch, from profiles/), hip_graph_replay
 (the same step replayed from a HIP graph), fused_quantize_transpose_step (the step with the single-read
 quantize + transposed-copy extension), direct_gradient_layout_step (the step with the backward matmuls reading
 weights, activations and output gradients in their stored layouts, matmul modes NN / NT / TT, instead of transposed
@@ -219,9 +220,13 @@ def main():
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     record[0] = 2
-    for _ in range(args.steps):
+    sensors = SensorSampler(enabled=not args.hbm_kernels_only)   # package power and shader clock while the second pass runs (never during the timed one)
+    for i_step in range(max(args.steps, 150 if sensors.available else 0)):   # 0.6 s of load: the sensors need it
+        if i_step == args.steps:
+            record[0] = 0       # events only around the first args.steps steps
         step()
     torch.cuda.synchronize()
+    sensor_report = sensors.stop()
     record[0] = 0
 
     # Samples for the error report (gemm_error): operands, scales and sampled outputs of the six GEMMs are taken
@@ -578,7 +583,8 @@ def main():
                    "tokens": BT, "gemm_flop_per_step": gemm_flop},
         "roofline": {"bound": "mfma", "kernel": "gemm_tn_e4m3_w4_kernel", "achieved": gemm_tflops_kernel,
                      "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": gemm_tflops_kernel / FP8_PEAK_TFLOPS,
-                     "traffic": measured_traffic(), "mfma_only_ceiling_TFLOPs": ceiling,
+                     "traffic": measured_traffic(), "sensors_under_step_load": sensor_report,
+                     "mfma_only_ceiling_TFLOPs": ceiling,
                      "frac_of_mfma_only_ceiling": gemm_tflops_kernel / max(ceiling["random_operands"], ceiling["random_operands_16x16x128"]),
                      "mean_launch_ms": ks["gemm"]["mean_ms"], "launches": ks["gemm"]["launches"],
                      "achieved_at_median_launch": tflops_median, "achieved_at_best_launch": tflops_best,
@@ -732,6 +738,65 @@ def secondary_path_steps(K, torch, dev, ws, iters=20):
         }
         del L
     return report
+
+
+class SensorSampler:
+    """Reads the driver's package power and shader clock (hwmon power1_input / power1_cap, pp_dpm_sclk under
+    /sys/class/drm/card*/device) every 10 ms from a thread until stop(); figures from the second half of the samples.
+    Absent files (another driver, no permission) give {"available": False}."""
+
+    def __init__(self, enabled=True):
+        import glob
+        import threading
+        self.available = False
+        if not enabled:
+            return
+        pw = glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input")
+        cap = glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_cap")
+        ck = glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk")
+        self.files = (pw[0], ck[0]) if len(pw) == 1 and len(ck) == 1 else None
+        self.cap = None
+        self.samples, self.halt, self.thread = [], False, None
+        if self.files is None:
+            return
+        try:
+            self.cap = int(open(cap[0]).read()) / 1e6 if cap else None
+            self.idle = self.read()
+        except (OSError, ValueError):
+            return
+        self.available = True
+        self.thread = threading.Thread(target=self.run, daemon=True)
+        self.thread.start()
+
+    def read(self):
+        import re
+        watts = int(open(self.files[0]).read()) / 1e6
+        m = re.search(r"(\d+)Mhz \*", open(self.files[1]).read())
+        return watts, (int(m.group(1)) if m else None)
+
+    def run(self):
+        while not self.halt:
+            try:
+                self.samples.append(self.read())
+            except (OSError, ValueError):
+                pass
+            time.sleep(0.01)
+
+    def stop(self):
+        if not self.available:
+            return {"available": False}
+        self.halt = True
+        self.thread.join()
+        late = self.samples[len(self.samples) // 2:]
+        watts = sorted(w for w, _ in late)
+        mhz = sorted(c for _, c in late if c)
+        if not watts or not mhz:
+            return {"available": False}
+        return {"available": True, "what": "hwmon power1_input and pp_dpm_sclk sampled every 10 ms while the steps of the "
+                "second (untimed) pass run; second half of the samples",
+                "samples": len(late), "power_W_median": watts[len(watts) // 2], "power_W_max": watts[-1],
+                "power_cap_W": self.cap, "sclk_MHz_median": mhz[len(mhz) // 2], "sclk_MHz_min": mhz[0],
+                "first_sample_right_after_the_timed_steps": {"power_W": self.idle[0], "sclk_MHz": self.idle[1]}}
 
 
 def measured_traffic():

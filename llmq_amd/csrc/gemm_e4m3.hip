@@ -617,8 +617,13 @@ __device__ __forceinline__ int frag_swizzle(int row) {
 // a lane 8 adjacent columns of c (it is made by the copy addressing of a K-contiguous a; a transposing read hands 16
 // adjacent columns to 16 adjacent lanes): a lane then owns columns 16 j + l16, and the epilogue goes through LDS --
 // scale, bias and the rounding to bf16 where the accumulators are, 16 rows x 128 columns of bf16 per wave and
-// fragment row into a private 4 KiB piece of LDS, read back as 16 bytes per lane and row.  bf16 output without
-// accumulation (the old values of c would have to be fetched in the scattered layout).
+// fragment row into a private 4 KiB piece of LDS, read back as 16 bytes per lane and row.  That epilogue serves bf16
+// output without accumulation (the old values of c would have to be fetched in the scattered layout); fp32 output and
+// accumulation take the STAGE32 instances, whose epilogue hands the raw fp32 accumulators through LDS first.
+// FUSE_EPI: the epilogue of full-width bf16 tiles without bias and accumulation runs under the matrix instructions of
+// the tile's last and the next tile's first K-step (see k_step).
+// RAGGED: M, N and K need not be multiples of the tile: edge tiles are moved back to end with the matrix, K is walked
+// in whole steps with the copies of the last one masked (see masked_copy and the epilogue's ownership test).
 template <typename OutT, int B_FMT, bool SEG, int NJ = 8, bool STREAM_OUT = true, bool ODDK = false, bool KMB = false,
           bool KMA = false, bool FUSE_EPI = false, bool STAGE32 = false, bool RAGGED = false>
 __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {

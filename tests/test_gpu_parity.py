@@ -620,7 +620,8 @@ def test_gemm_matches_swapped_operand_transpose(K, O):
 
 GENERAL_SHAPES = [(144, 272, 400), (1152, 8192, 896), (896, 2048, 896), (1024, 512, 896), (512, 256, 384),
                   (256, 1000, 512), (3584, 300, 256), (8, 8, 16), (1, 1, 16), (130, 70, 48), (200, 264, 1024), (448, 520, 640),
-                  (2112, 2064, 656), (2112, 4104, 528), (1000, 4104, 400)]
+                  (2112, 2064, 656), (2112, 4104, 528), (1000, 4104, 400), (2056, 2049, 400), (2296, 2303, 496),
+                  (4104, 1025, 640)]
 
 
 @pytest.mark.parametrize("mnk", GENERAL_SHAPES)
@@ -629,9 +630,10 @@ def test_gemm_general_shapes(K, O, mnk):
     (src/kernels/matmul.cpp:55-57, 160-184).  Here: M, K off the 128 lattice or N below 128 -> the general-shape
     kernel; a ragged N on top of regular M, K -> tiled kernels for the rows before the last N % 128, general-shape
     kernel for those; K an odd multiple of 128 -> the four-wave kernel's odd-K instances ((1152, 8192, 896) and
-    (896, 2048, 896) on its 192- and 224-wide tiles, (1024, 512, 896) on the full tile); the last three shapes (64 and
-    more 256 x 256 tiles, M and N off the lattice, K tails of 16 bytes, even and odd K-step counts) -> the four-wave
-    kernel's ragged instances.  Integer operands -> bit
+    (896, 2048, 896) on its 192- and 224-wide tiles, (1024, 512, 896) on the full tile); the last six shapes (64 and
+    more 256 x 256 tiles; M 8 or 248 past a tile boundary, N 1 or 255 past one, so that moved-back tiles overlap their
+    neighbours by almost a whole tile or by one row; K tails of 16 and 112 bytes and none; even and odd K-step counts)
+    -> the four-wave kernel's ragged instances.  Integer operands -> bit
     exact against the oracle for bf16 / fp32 output with bias and accumulation; random codes within the tolerance."""
     M, N, Kd = mnk
     a, _ = O.fill_int_e4m3(M * Kd, 2024, 0)
