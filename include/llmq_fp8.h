@@ -123,9 +123,10 @@ int llmq_transpose_u8(uint8_t* dst, const uint8_t* src, int rows, int cols, void
  * scalars or NULL (= 1).  bias is bf16[M] or NULL.  Any M, N >= 1; K must be a multiple of 16 (16-byte aligned
  * operand rows, the rule of the reference's default backend, src/kernels/matmul.cpp:55-57).  The fast kernels take
  * K % 128 == 0 with M % 128 == 0 (bf16 output without accumulation: also M % 224 == 0 or M % 192 == 0) and all but
- * the last N % 128 rows of c.  Other shapes with M, N >= 256, M % 8 == 0, K >= 384 and at least 64 tiles of 256 x 256
- * run on instances of the same kernel with moved-back edge tiles at about three quarters of its rate; a slow
- * general-shape kernel serves the N % 128 remainder rows and every shape that is left.
+ * the last N % 128 rows of c.  Other shapes with M % 8 == 0 run on ragged instances of the same kernels (256 x 256
+ * tiles with moved-back edge tiles for large outputs with K >= 384, at about three quarters of the lattice rate;
+ * 128 x 128 tiles with clamped rows otherwise); a slow general-shape kernel serves the N % 128 remainder rows of a
+ * regular M, K, shapes with M % 8 != 0 and outputs smaller than one 128 x 128 tile.
  * Replaces: matmul(nv_bfloat16* c, const __nv_fp8_e4m3* a, const __nv_fp8_e4m3* b,
  *           const nv_bfloat16* bias, const float* scale_a, const float* scale_b, cublasLtHandle_t,
  *           std::byte* ws, size_t ws_size, int M, int N, int K, EMMTranspose::TN, bool accumulate,

@@ -172,8 +172,15 @@ __device__ __forceinline__ void static_for(F&& f) {
 // operand stream then runs across tile boundaries: the copies of the next tile's first two K-steps are
 // issued during the last two K-steps of the current tile, so the epilogue of a tile overlaps with the
 // fetch of the next one and no pipeline fill or workgroup launch sits between tiles.  Needs K >= 256.
-template <int BLK_N, int BLK_M, int WV_N, int WV_M, typename OutT, bool SPLIT, bool PERSIST, int B_FMT>
+// RAGGED: M, N and K need not be multiples of the tile (M a multiple of 8, K of 16).  Tile counts round up; a lane whose
+// operand row lies beyond the matrix copies the matrix's last row instead (its products land in accumulators that are
+// never stored), a lane whose 16-byte chunk lies beyond K copies a chunk of zeros, and the epilogue stores only what
+// lies inside c.  Every lane still issues every copy, so the counters of the K loop hold as they are.
+static __device__ uint4 ragged_zero_chunk;  // never written: 16 zero bytes in global memory
+
+template <int BLK_N, int BLK_M, int WV_N, int WV_M, typename OutT, bool SPLIT, bool PERSIST, int B_FMT, bool RAGGED = false>
 __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(GemmArgs g) {
+    static_assert(!RAGGED || (!SPLIT && !PERSIST), "ragged shapes: one tile per workgroup, no K split");
     constexpr int T = WV_N * WV_M * 64;
     constexpr int WT_N = BLK_N / WV_N, WT_M = BLK_M / WV_M;
     constexpr int NI = WT_N / 32, NJ = WT_M / 32;
@@ -192,7 +199,8 @@ __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(Gemm
     const int wn = wave / WV_M, wm = wave % WV_M;
     const int l32 = lane % 32, kg = lane / 32;
 
-    const int tiles_n = g.N / BLK_N, tiles_m = g.M / BLK_M;
+    const int tiles_n = RAGGED ? (g.N + BLK_N - 1) / BLK_N : g.N / BLK_N;
+    const int tiles_m = RAGGED ? (g.M + BLK_M - 1) / BLK_M : g.M / BLK_M;
     // Tile order: XCD x (workgroups are dealt to XCDs round-robin) owns a contiguous range of the
     // "logical" tile sequence, which walks column-major groups of g.group tile-rows.
     const int total = tiles_n * tiles_m;
@@ -228,31 +236,48 @@ __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(Gemm
     // global source of every direct-to-LDS copy this lane issues for one K-step
     const uint8_t* p_src;
     const uint8_t* q_src[Q_ITERS];
+    [[maybe_unused]] const uint8_t* p_rag[P_ITERS];  // RAGGED: one source per copy (rows are clamped one by one)
+    [[maybe_unused]] int lane_k = 0;                 // RAGGED: offset of this lane's chunk within a K-step
     auto set_sources = [&](int nb, int mb) {
         const int t_id = PERSIST ? opaque(threadIdx.x) : tid;
         const int ld_row = t_id / 8;
         const int ld_chunk = (t_id & 7) ^ ((ld_row >> 1) & 7);
         p_src = g.b + (int64_t)nb * g.K + (int64_t)ld_row * g.K + ld_chunk * 16 + k_begin;
+        if constexpr (RAGGED) {
+            lane_k = ld_chunk * 16;
+#pragma unroll
+            for (int it = 0; it < P_ITERS; ++it) {
+                int row = nb + it * (T / 8) + ld_row;
+                row = row < g.N ? row : g.N - 1;
+                p_rag[it] = g.b + (int64_t)row * g.K + ld_chunk * 16;
+            }
+        }
 #pragma unroll
         for (int it = 0; it < Q_ITERS; ++it) {
             const int rho = it * (T / 8) + ld_row;
             const int w = rho / WT_M, rw = rho % WT_M;
             const int grow = w * WT_M + NJ * (rw % 32) + rw / 32;
-            q_src[it] = g.a + (int64_t)mb * g.K + (int64_t)grow * g.K + ld_chunk * 16 + k_begin;
+            int row = mb + grow;
+            if constexpr (RAGGED) row = row < g.M ? row : g.M - 1;
+            q_src[it] = g.a + (int64_t)row * g.K + ld_chunk * 16 + k_begin;
         }
     };
     set_sources(n_blk, m_blk);
     auto issue_loads = [&](int stage_ofs, int k0) {
         uint8_t* base = lds + stage_ofs + wave * 1024;
+        [[maybe_unused]] const bool beyond_k = RAGGED && k0 + lane_k >= g.K;
+        [[maybe_unused]] const uint8_t* zeros = reinterpret_cast<const uint8_t*>(&ragged_zero_chunk);
 #pragma unroll
         for (int it = 0; it < P_ITERS; ++it) {
             const uint8_t* src = p_src + (int64_t)it * (T / 8) * g.K + k0;
+            if constexpr (RAGGED) src = beyond_k ? zeros : p_rag[it] + k0;
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                              (__attribute__((address_space(3))) void*)(base + it * T * 16), 16, 0, 0);
         }
 #pragma unroll
         for (int it = 0; it < Q_ITERS; ++it) {
             const uint8_t* src = q_src[it] + k0;
+            if constexpr (RAGGED) src = beyond_k ? zeros : src;
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                              (__attribute__((address_space(3))) void*)(base + P_BYTES + it * T * 16), 16,
                                              0, 0);
@@ -283,7 +308,7 @@ __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(Gemm
     };
     clear_acc();
 
-    const int KT = k_count / kBK;
+    const int KT = RAGGED ? (k_count + kBK - 1) / kBK : k_count / kBK;
     issue_loads(0, 0);
     if (KT > 1) {
         issue_loads(STAGE, kBK);
@@ -366,12 +391,17 @@ __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(Gemm
         const int m_lane = mb + wm * WT_M + NJ * el32;
         // byte offset of the lane inside a group of rows; below 2^32 (4 rows of at most 2^27 elements)
         const uint32_t lane_bytes = ((uint32_t)(4 * ekg) * (uint32_t)g.M + (uint32_t)m_lane) * (uint32_t)sizeof(T);
+        // RAGGED: the lane's pair of columns lies inside c as a whole or not at all (M is even); its rows are tested one by one
+        const bool col_inside = !RAGGED || m_lane < g.M;
         float bias0 = 0.f, bias1 = 0.f;
         if constexpr (BIAS) {
-            bias0 = load_bias(g.bias, g.bias_is_bf16, m_lane);
-            bias1 = load_bias(g.bias, g.bias_is_bf16, m_lane + 1);
+            if (col_inside) {
+                bias0 = load_bias(g.bias, g.bias_is_bf16, m_lane);
+                bias1 = load_bias(g.bias, g.bias_is_bf16, m_lane + 1);
+            }
         }
         const int row0 = nb + wn * WT_N;  // wave-uniform
+        auto inside = [&](int i, int r) { return !RAGGED || (col_inside && row0 + i * 32 + 8 * (r / 4) + (r % 4) + 4 * ekg < g.N); };
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
             float o0[16], o1[16];
@@ -379,11 +409,13 @@ __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(Gemm
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     LLMQ_GLOBAL char* row = scalar_ptr((LLMQ_GLOBAL char*)(out + (int64_t)(row0 + i * 32 + 8 * (r / 4) + (r % 4)) * g.M));
-                    PairIo<T>::load(row + lane_bytes, o0[r], o1[r]);
+                    o0[r] = o1[r] = 0.f;
+                    if (inside(i, r)) PairIo<T>::load(row + lane_bytes, o0[r], o1[r]);
                 }
             }
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
+                if (!inside(i, r)) continue;
                 LLMQ_GLOBAL char* row = scalar_ptr((LLMQ_GLOBAL char*)(out + (int64_t)(row0 + i * 32 + 8 * (r / 4) + (r % 4)) * g.M));
                 float v0 = acc[i][0][r] * scale, v1 = acc[i][1][r] * scale;
                 if constexpr (BIAS) {
@@ -409,8 +441,10 @@ __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(Gemm
         const int m_wave = mb + wm * WT_M;
         float bias0 = 0.f, bias1 = 0.f;
         if constexpr (BIAS) {
-            bias0 = load_bias(g.bias, g.bias_is_bf16, m_wave + NJ * el32);
-            bias1 = load_bias(g.bias, g.bias_is_bf16, m_wave + NJ * el32 + 1);
+            if (!RAGGED || m_wave + NJ * el32 < g.M) {
+                bias0 = load_bias(g.bias, g.bias_is_bf16, m_wave + NJ * el32);
+                bias1 = load_bias(g.bias, g.bias_is_bf16, m_wave + NJ * el32 + 1);
+            }
         }
         uint8_t* tile = lds + 2 * STAGE + wave * EPI_BYTES;
         // register r of a fragment is tile row 8*(r/4) + 4*kg + r%4, stored at row position (row ^ kg)
@@ -440,6 +474,8 @@ __global__ __launch_bounds__(WV_N* WV_M * 64) void gemm_tn_e4m3_pipe_kernel(Gemm
 #pragma unroll
             for (int p = 0; p < 4; ++p) {
                 LLMQ_GLOBAL char* row = scalar_ptr((LLMQ_GLOBAL char*)(out + (int64_t)(row0 + i * 32 + p * 8) * g.M));
+                // RAGGED: the lane's 8 columns lie inside c as a whole or not at all (M is a multiple of 8)
+                if (RAGGED && (row0 + i * 32 + p * 8 + (r_row ^ ekg) >= g.N || m_wave + r_chunk * 8 >= g.M)) continue;
                 __builtin_nontemporal_store(piece[p], (LLMQ_GLOBAL v4i*)(row + lane_bytes));
             }
         }
@@ -1661,7 +1697,8 @@ static int launch_pipe(const GemmArgs& g, int splits, int persistent_grid, hipSt
 // Kernel selection overrides, 0 / -1 = automatic.  They exist only in the test-aid build of this file
 // (LLMQ_TEST_HOOKS), where the parity tests force every kernel instantiation in turn; in the product library
 // they are constants and the dispatch below is a function of its arguments alone.  tile: 1 = 256 x 256 tile with
-// 8 waves, 2 = 128 x 128 tile with 4 waves, 3 = four-wave kernel, 4 / 5 = its 224- / 192-wide tiles.  splits:
+// 8 waves, 2 = 128 x 128 tile with 4 waves, 3 = four-wave kernel, 4 / 5 = its 224- / 192-wide tiles; for shapes off the
+// lattice only 2 and 3 (the ragged instances of those kernels) and 6 = the 64 x 64 kernel.  splits:
 // forced number of K splits (needs a workspace).  persist: -1 = automatic, 0 = never, 1 = whenever possible.
 // fuse: -1 = automatic, 0 = the four-wave kernel's epilogue always after the K loop, 1 = under the last K-step wherever
 // that instance exists (full-width bf16 tiles without bias and accumulation).
@@ -1804,6 +1841,32 @@ static void launch_w4_ragged(const GemmArgs& g, int cus, int xcds, hipStream_t s
                            dim3((unsigned)grid), dim3(256), 0, stream, g);
 }
 
+// Shapes off the tile lattice on 128 x 128 tiles (RAGGED instance of the 8-wave kernel family's four-wave configuration):
+// any N, M a multiple of 8, K a multiple of 16.  One tile per workgroup, two workgroups per compute unit.
+template <typename OutT, int B_FMT>
+static int launch_pipe_ragged(const GemmArgs& g, hipStream_t stream) {
+    const int64_t tiles = (int64_t)((g.N + 127) / 128) * ((g.M + 127) / 128);
+    LLMQ_REQUIRE(tiles < ((int64_t)1 << 31), "matmul: too many tiles (%lld)", (long long)tiles);
+    hipLaunchKernelGGL((gemm_tn_e4m3_pipe_kernel<128, 128, 2, 2, OutT, false, false, B_FMT, true>), dim3((unsigned)tiles),
+                       dim3(256), 0, stream, g);
+    LLMQ_HIP_TRY(hipGetLastError());
+    return LLMQ_OK;
+}
+
+// Which of the two ragged tilings is faster, from estimated times in microseconds: rounds of tiles over the chip (one
+// 256 x 256 tile per compute unit, or two co-resident 128 x 128 tiles) times the K-steps of a tile at the measured cost
+// of a step (1.4 / 1.0 us) plus a measured per-round cost (8 / 3 us: prologue, epilogue and the masked last step of the
+// ragged four-wave instance).  Checked against a sweep of 60 shapes (M, N from 1000 to 16392, K from 400 to 8208): the
+// estimate is within 10 % of the measured time and picks the faster kernel except where the two are within 5 %.
+// Examples (us, 128 x 128 / four-wave): 1000 x 8192 x 3584 30 / 44, 2056 x 4100 x 3600 64 / 46, 4360 x 4100 x 656 28 / 33,
+// 3584 x 8200 x 3600 131 / 90, 8200 x 8200 x 8208 649 / 448, 3000 x 16392 x 656 63 / 71.
+static bool ragged_prefers_four_wave(int M, int N, int K, int cus) {
+    const double steps = (double)((K + kBK - 1) / kBK);
+    const int64_t t256 = (int64_t)((N + 255) / 256) * ((M + 255) / 256), t128 = (int64_t)((N + 127) / 128) * ((M + 127) / 128);
+    const double r256 = (double)((t256 + cus - 1) / cus), r128 = (double)((t128 + 2 * cus - 1) / (2 * cus));
+    return r256 * (1.4 * steps + 8.0) < r128 * (1.0 * steps + 3.0);
+}
+
 template <typename OutT, int B_FMT>
 static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     LLMQ_REQUIRE(g.M > 0 && g.N > 0 && g.K > 0, "matmul: M, N, K must be positive (got %d, %d, %d)", g.M, g.N, g.K);
@@ -1836,20 +1899,35 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
     const bool m_narrow = narrow_out && (g.M % 224 == 0 || g.M % 192 == 0);  // served by 256-row tiles only
     const bool on_lattice = g.K % kBK == 0 && (g.M % 128 == 0 || m_narrow) && g.N >= (g.M % 128 == 0 ? 128 : 256);
     if (!on_lattice) {
-        LLMQ_REQUIRE(force_tile == 0 && force_splits == 0,
+        // Three kernels serve shapes off the lattice: the four-wave kernel's ragged instances (whole 256 x 256 tiles,
+        // moved back at the edges: M, N >= 256, K >= 384) and the ragged instance of the 128 x 128 tiles, whichever the
+        // estimate above expects to be faster, both for M a multiple of 8 (the lane's 8 adjacent bf16 outputs start
+        // 16-byte aligned); the 64 x 64 kernel for the rest (M % 8 != 0, or less than one 128 x 128 tile of outputs).
+        LLMQ_REQUIRE(force_splits == 0 && (force_tile == 0 || force_tile == 2 || force_tile == 3 || force_tile == 6),
                      "matmul: M, N, K = %d, %d, %d are off the lattice of the forced kernel variant", g.M, g.N, g.K);
-        // Large enough for whole (moved-back) tiles of the four-wave kernel, and enough of them: that kernel; else the
-        // 64 x 64 kernel.  Measured: 3584 x 8200 x 3600 94 against 322 us, 1000 x 8192 x 3584 (128 tiles) 48 against 74 us,
-        // 4360 x 4100 x 656 35 against 49 us; 1000 x 1000 x 400 (16 tiles) 14 against 7 us.
-        const int64_t ragged_tiles = (int64_t)((g.N + 255) / 256) * ((g.M + 255) / 256);
-        if (g.M >= 256 && g.N >= 256 && g.M % 8 == 0 && g.K >= 3 * kBK && cus % xcds == 0 && ragged_tiles >= cus / 4 &&
-            g_gemm_persist != 0) {
+        const bool w4_fits = g.M >= 256 && g.N >= 256 && g.M % 8 == 0 && g.K >= 3 * kBK && cus % xcds == 0;
+        const bool pipe_fits = g.M % 8 == 0;
+        int pick = 6;
+        if (force_tile != 0) {
+            LLMQ_REQUIRE(force_tile == 6 || (force_tile == 3 ? w4_fits : pipe_fits),
+                         "matmul: M, N, K = %d, %d, %d do not fit the forced ragged kernel", g.M, g.N, g.K);
+            pick = force_tile;
+        } else if (w4_fits && g_gemm_persist != 0 && (!pipe_fits || ragged_prefers_four_wave(g.M, g.N, g.K, cus))) {
+            pick = 3;
+        } else if (pipe_fits && (int64_t)g.M * g.N >= 128 * 128) {
+            pick = 2;
+        }
+        if (pick == 3) {
             g.group = 8;
             g.rem_split = 1;
             g.part_per_xcd = 0;
             launch_w4_ragged<OutT, B_FMT>(g, cus, xcds, stream);
             LLMQ_HIP_TRY(hipGetLastError());
             return LLMQ_OK;
+        }
+        if (pick == 2) {
+            g.group = 8;
+            return launch_pipe_ragged<OutT, B_FMT>(g, stream);
         }
         return launch_edge(0);
     }

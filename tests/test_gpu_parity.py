@@ -624,6 +624,53 @@ GENERAL_SHAPES = [(144, 272, 400), (1152, 8192, 896), (896, 2048, 896), (1024, 5
                   (4104, 1025, 640)]
 
 
+RAGGED_SHAPES = [(264, 300, 384), (1000, 1000, 400), (1000, 520, 1040), (512, 776, 3600), (1000, 8192, 3584), (2056, 4100, 1552),
+                 (4360, 4100, 656), (3584, 8200, 3600), (1032, 72, 48), (136, 5000, 112)]
+
+
+@pytest.mark.parametrize("mnk", RAGGED_SHAPES)
+def test_gemm_off_lattice_kernels_agree(K, O, mnk):
+    """Shapes off the tile lattice have three kernels: the ragged instances of the four-wave kernel (moved-back 256 x 256
+    tiles, masked last K-step) and of the 128 x 128 tiles (clamped rows, zero chunks beyond K), and the 64 x 64 kernel.
+    The dispatch picks by estimated time; here each is forced in turn (test-aid build) on integer operands and all must
+    give the same bits for bf16 and fp32 output, with bias and with accumulation -- and the first shape's bits are the
+    oracle's.  (test_gemm_general_shapes compares the automatic choice with the oracle on further shapes.)"""
+    M, N, Kd = mnk
+    a, _ = O.fill_int_e4m3(M * Kd, 77, 0)
+    b, _ = O.fill_int_e4m3(N * Kd, 77, 1)
+    a, b = a.reshape(M, Kd), b.reshape(N, Kd)
+    s = float(np.sqrt(np.float32(4.0 / Kd)))
+    _, biasv = O.fill_int_e4m3(M, 77, 2)
+    _, oldv = O.fill_int_e4m3(N * M, 77, 3)
+    bias = O.f32_to_bf16(biasv.astype(np.float32))
+    old = O.f32_to_bf16(oldv.astype(np.float32)).reshape(N, M)
+    old32 = oldv.astype(np.float32).reshape(N, M)
+    four_wave = M >= 256 and N >= 256 and Kd >= 384
+    results = {}
+    try:
+        for tile in (6, 2) + ((3,) if four_wave else ()):
+            set_variant((tile, 0))
+            results[tile] = [host_bits(run_gemm(K, a, b, M, N, Kd, s, s)),
+                             host_bits(run_gemm(K, a, b, M, N, Kd, s, s, bias)),
+                             host_bits(run_gemm(K, a, b, M, N, Kd, s, s, bias, old)),
+                             run_gemm(K, a, b, M, N, Kd, s, s, out_f32=True).cpu().numpy(),
+                             run_gemm(K, a, b, M, N, Kd, None, None, bias, old32, out_f32=True).cpu().numpy()]
+    finally:
+        set_variant((0, 0))
+    for tile in results:
+        for i, (x, y) in enumerate(zip(results[6], results[tile])):
+            assert np.array_equal(x, y), (tile, i)
+    if mnk == RAGGED_SHAPES[0]:
+        assert np.array_equal(results[6][2], O.gemm_tn(a, b, sa=s, sb=s, bias=bias, c_old=old))
+    if four_wave:
+        set_variant((3, 0))
+        try:
+            with pytest.raises(ValueError):   # two K-steps: fewer than the ragged four-wave instances walk
+                run_gemm(K, a[:, :256].copy(), b[:, :256].copy(), M, N, 256, s, s)
+        finally:
+            set_variant((0, 0))
+
+
 @pytest.mark.parametrize("mnk", GENERAL_SHAPES)
 def test_gemm_general_shapes(K, O, mnk):
     """The reference's default backend serves every FP8 shape with 16-byte aligned rows
