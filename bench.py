@@ -220,7 +220,7 @@ def main():
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     record[0] = 2
-    sensors = SensorSampler(enabled=not args.hbm_kernels_only)   # package power and shader clock while the second pass runs (never during the timed one)
+    sensors = SensorSampler(enabled=not args.hbm_kernels_only and args.steps >= 20)   # package power and shader clock while the second pass runs (never during the timed one)
     for i_step in range(max(args.steps, 150 if sensors.available else 0)):   # 0.6 s of load: the sensors need it
         if i_step == args.steps:
             record[0] = 0       # events only around the first args.steps steps
