@@ -1714,8 +1714,11 @@ constexpr int g_gemm_tile = 0, g_gemm_splits = 0, g_gemm_persist = -1, g_gemm_fu
 // w4_segment_reduce_kernel: the round then takes 1 / rem_split of a tile's time, at the price of two more
 // launches.  The decision uses measured figures (microseconds): a tile of depth K on an otherwise idle
 // chip takes about K / 164 (twice as fast as in a full round); the operand bytes of the round stream at
-// about 3.5 TB/s from memory (10 TB/s when both operands fit the 256 MB last-level cache) whichever way
-// the round is organised; the extra launches cost about 20, a partial tile 0.03 in the reduction.
+// about 6 TB/s (10 TB/s when both operands fit the 256 MB last-level cache) whichever way the round is
+// organised; the extra launches cost about 20, a partial tile 0.03 in the reduction.  Measured against it
+// (us, whole launch, uncut / cut): 18944 x 3584 x 8192 (12 tiles left over) 388 / 362 with 4 segments;
+// 3584 x 37888 x 8192 (24 left over) 758 / 742 with 3 to 5 segments; 18944 x 8192 x 3584 (64 left over, at most 2
+// segments fit the workspace) 382 / 387: the first two are cut, the third is not.
 struct W4Plan {
     int grid, rem_split, k_len, part_per_xcd, rem_max;
 };
@@ -1731,7 +1734,7 @@ static W4Plan plan_w4(int tiles256, int cus, int xcds, int M, int N, int K, int 
     const int pairs = K / (2 * kBK);  // segments are whole pairs of K-steps
     const int64_t ws_tiles = (int64_t)(workspace_bytes / (size_t)(256 * 256 * 4));
     const int rem_total = xr * rem_hi + (xcds - xr) * rem_lo;
-    const double stream_us = (double)rem_total * 512.0 * K / (((double)M + N) * K <= 192e6 ? 10e6 : 3.5e6);
+    const double stream_us = (double)rem_total * 512.0 * K / (((double)M + N) * K <= 192e6 ? 10e6 : 6e6);
     const double tile_us = (double)K / 164.0;
     const double whole_us = tile_us > stream_us ? tile_us : stream_us;
     int best = 1;
