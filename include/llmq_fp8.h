@@ -152,9 +152,10 @@ int llmq_gemm_tn_e4m3_bf16(uint16_t* c, const uint8_t* a, const uint8_t* b, cons
  *   NN  a[K, M], b[N, K]            (a K-major: the weight W[OC, C] in its stored layout as the first operand of the dgrad)
  *   NT  a[K, M], b[K, N]            (both K-major: activation X[BT, C] and gradient dY[BT, OC] of the weight gradient)
  * so that the transposed copies the reference's FP8 path materialises (src/models/llama_model.cpp:309-339; its own
- * kernels take TN only) are not needed.  The K-major modes serve M, N and K multiples of 256 (TT with bf16 output and
- * without accumulation also M a multiple of 224) and K-major operands below 2 GiB, with bias and accumulation in every
- * mode (llmq_gemm_e4m3_f32_mode: the same with fp32 output, src/kernels/kernels.h:72-78).  Other
+ * kernels take TN only) are not needed.  The K-major modes serve M, N and K multiples of 256 (with bf16 output and
+ * without accumulation also M a multiple of 224 in modes TT and NN, of 192 in mode NN) and K-major operands below
+ * 2 GiB, with bias and accumulation in every mode (llmq_gemm_e4m3_f32_mode: the same with fp32 output,
+ * src/kernels/kernels.h:72-78).  Other
  * shapes return LLMQ_ERR_INVALID_ARGUMENT before anything is launched and the caller takes the transposing route.
  * b_format: 0 = e4m3, 1 = e5m2.  The workspace serves the cut of the last round of tiles as in mode TN (the K-major
  * modes have no split-K for few-tile outputs).  Results are bit-identical to mode TN on the transposed copies whenever

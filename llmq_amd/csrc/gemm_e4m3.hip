@@ -669,17 +669,19 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     static_assert(!FUSE_EPI || (NJ == 8 && !SEG && !KMA && std::is_same_v<OutT, uint16_t>),
                   "the epilogue under the last K-step is written for full-width bf16 tiles of K-contiguous a");
     static_assert(!((KMB || KMA) && ODDK), "the K-major operand modes are built for even K-step counts");
-    static_assert(!KMA || (NJ == 8 && (SEG || STAGE32 || std::is_same_v<OutT, uint16_t>)),
-                  "the K-major first operand is built for 256-wide tiles; fp32 output as K segments or through the fp32-staged epilogue");
+    static_assert(!KMA || (NJ == 8 && (SEG || STAGE32 || std::is_same_v<OutT, uint16_t>)) ||
+                      (NJ < 8 && !SEG && !STAGE32 && !KMB && std::is_same_v<OutT, uint16_t>),
+                  "the K-major first operand: fp32 output as K segments or through the fp32-staged epilogue; narrow tiles "
+                  "for bf16 output of mode NN");
     constexpr int BLK = 256, T = 256, WT = 128, NF = 8;
     constexpr int WTM = 16 * NJ, BLKM = 2 * WTM;  // columns (first-operand rows) per wave and per tile
     constexpr int P_BYTES = BLK * kBK, STAGE = 2 * P_BYTES;
     constexpr int ITERS = BLK * 8 / T;    // 16-byte copies per lane and K-step, b rows
-    constexpr int ITERS_Q = BLKM * 8 / T;  // the same for the a rows (= NJ)
+    constexpr int ITERS_Q = KMA ? 8 : BLKM * 8 / T;  // the same for the a rows (= NJ; a K-major a tile: 8 slabs of 16 k rows)
     static_assert(NJ == 8 || ((NJ == 7 || NJ == 6) && !SEG && std::is_same_v<OutT, uint16_t>), "unsupported tile width");
     typedef float v4f __attribute__((ext_vector_type(4)));
 
-    constexpr int EPI_STAGE = 16 * WTM * 2;  // KMA: one fragment row of a wave's outputs as bf16
+    constexpr int EPI_STAGE = 16 * 256;  // KMA: one fragment row of a wave's outputs as bf16, rows of 256 bytes
     constexpr int EPI32_ROW = 4 * WTM + 32;  // STAGE32: half a fragment row (8 c rows) of raw accumulators, rows padded by 32 bytes
     constexpr int EPI32_STAGE = 8 * EPI32_ROW;
     __shared__ __attribute__((aligned(16))) uint8_t lds[2 * STAGE + (KMA ? 4 * (STAGE32 ? EPI32_STAGE : EPI_STAGE) : 0)];
@@ -755,9 +757,12 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
         const int l = ld_row % 16;
         return ld_row < 16 ? frag_step(2 * it) * l : frag_row(2 * it + 1) - frag_row(2 * it) + frag_step(2 * it + 1) * l;
     };
-    const uint32_t q_lane = KMA ? (uint32_t)kb_row * (uint32_t)g.M + (uint32_t)kb_chunk * 16u
+    // A K-major a tile of a narrow instance is 2 NJ chunks wide: a lane whose chunk lies beyond that copies a chunk
+    // 2 (8 - NJ) to the left instead (inside the tile, so inside the matrix; it lands in a place no fragment reads)
+    auto inside_tile = [](int chunk) { return chunk < 2 * NJ ? chunk : chunk - 2 * (8 - NJ); };
+    const uint32_t q_lane = KMA ? (uint32_t)kb_row * (uint32_t)g.M + (uint32_t)inside_tile(kb_chunk) * 16u
                                 : (uint32_t)slab_lane_rows(0) * (uint32_t)g.K + (uint32_t)ld_chunk * 16u;
-    const uint32_t q_lane_hi = (uint32_t)kb_row * (uint32_t)g.M + (uint32_t)(kb_chunk ^ 8) * 16u;  // KMA, slabs 2, 3, 6, 7
+    const uint32_t q_lane_hi = (uint32_t)kb_row * (uint32_t)g.M + (uint32_t)inside_tile(kb_chunk ^ 8) * 16u;  // KMA, slabs 2, 3, 6, 7
     const uint32_t q_step = KMA ? (uint32_t)kBK * (uint32_t)g.M : (uint32_t)kBK;
     const uint32_t q_lane_3 = (uint32_t)slab_lane_rows(NJ == 7 ? 3 : 0) * (uint32_t)g.K + (uint32_t)ld_chunk * 16u;
     const uint32_t q_lane_6 = (uint32_t)slab_lane_rows(NJ == 7 ? 6 : 0) * (uint32_t)g.K + (uint32_t)ld_chunk * 16u;
@@ -936,10 +941,18 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
     // ways, with the wave's column half wm in the place of its row half wn
     const uint32_t ka_base = (uint32_t)((32 * kg + l16 / 2) * 256 + (l16 & 1) * 8) + (uint32_t)(((8 * wm) ^ ((kg & 1) << 3)) * 16) +
                              (uint32_t)((l16 / 2) * 16);
+    // Narrow tiles: the wave half wm starts at chunk NJ wm, which is no power of two, so fragment j's chunk NJ wm + j is
+    // xor-ed with the lane's swizzle explicitly (one more vector instruction per fragment read)
+    [[maybe_unused]] const uint32_t ka_row = (uint32_t)((32 * kg + l16 / 2) * 256 + (l16 & 1) * 8);
+    [[maybe_unused]] const uint32_t ka_swz = (uint32_t)(((l16 / 2) | ((kg & 1) << 3)) * 16);
+    auto frag_a_ofs = [&](int j) -> uint32_t {  // byte offset, within the a half of a stage, of the first read of fragment j
+        if constexpr (NJ == 8) return (uint32_t)(opaque((int)ka_base) ^ (16 * j));
+        else return (uint32_t)opaque((int)ka_row) + ((uint32_t)((NJ * wm + j) * 16) ^ (uint32_t)opaque((int)ka_swz));
+    };
     typedef __attribute__((address_space(3))) v2i_lds* lds_v2i_a;
     auto read_frag_a = [&](const uint8_t* stage, int j) -> v8i {
         if constexpr (KMA) {
-            const uint8_t* p = stage + P_BYTES + (opaque((int)ka_base) ^ (16 * j));
+            const uint8_t* p = stage + P_BYTES + frag_a_ofs(j);
             const v2i_lds r0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_a)(p));
             const v2i_lds r1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_a)(p + 2048));
             const v2i_lds r2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_a)(p + 4096));
@@ -1147,7 +1160,9 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
                     // previous tile's epilogue) sit that epilogue's stores; the counter retires in issue
                     // order, so allowing as many outstanding operations as there were stores is enough.
                     if (pending_stores) {
-                        if constexpr (sizeof(OutT) == 2 && NJ != 7) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(32 + kYoung) : "memory");
+                        // stores of a bf16 epilogue per lane and tile: 32 (one per c row), 64 with the two-piece rows of
+                        // the 224-wide tile of a K-contiguous a
+                        if constexpr (sizeof(OutT) == 2 && (NJ != 7 || KMA)) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(32 + kYoung) : "memory");
                         else asm volatile("s_waitcnt vmcnt(63) lgkmcnt(0)" ::: "memory");
                     } else {
                         asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kYoung) : "memory");
@@ -1161,8 +1176,8 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
                 if constexpr (KMA) {
                     // the eight transposing reads of the next step's first two a fragments, two between each write of M0
                     // and its copy
-                    const uint8_t* pa0 = nxt + P_BYTES + opaque((int)ka_base);
-                    const uint8_t* pa1 = nxt + P_BYTES + (opaque((int)ka_base) ^ 16);
+                    const uint8_t* pa0 = nxt + P_BYTES + frag_a_ofs(0);
+                    const uint8_t* pa1 = nxt + P_BYTES + frag_a_ofs(1);
                     uint32_t tok = set_m0(std::integral_constant<int, 0>{}, refill);
                     const v2i_lds a00 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_a)(pa0));
                     const v2i_lds a01 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_a)(pa0 + 2048));
@@ -1421,6 +1436,7 @@ __global__ __launch_bounds__(256) void gemm_tn_e4m3_w4_kernel(GemmArgs g) {
                     for (int q = 0; q < 4; ++q) {
                         const v4i packed = *reinterpret_cast<const v4i*>(es + q * 1024 + (rd_ofs ^ (uint32_t)(32 * q)));
                         LLMQ_GLOBAL char* row_ptr = scalar_ptr((LLMQ_GLOBAL char*)(c + (int64_t)(row0 + 16 * i + 4 * q) * ldc));
+                        if (NJ < 8 && e_lane % 16 >= 2 * NJ) continue;  // narrow tiles: the wave half is 16 NJ columns wide
                         if constexpr (STREAM_OUT) __builtin_nontemporal_store(packed, (LLMQ_GLOBAL v4i*)(row_ptr + out_bytes));
                         else *(LLMQ_GLOBAL v4i*)(row_ptr + out_bytes) = packed;
                     }
@@ -2105,23 +2121,51 @@ static int gemm_dispatch_kmajor(GemmArgs g, void* workspace, size_t workspace_by
     LLMQ_REQUIRE(aligned16(g.a) && aligned16(g.b) && aligned16(g.c) && aligned16(g.bias) && aligned16(workspace),
                  "matmul: all pointers must be 16-byte aligned");
     LLMQ_REQUIRE(workspace != nullptr || workspace_bytes == 0, "matmul: workspace size given without a workspace");
-    const bool m224 = kBf16 && !KMA && g.M % 256 != 0 && g.M % 224 == 0 && !g.accumulate;
+    // Narrow tiles (bf16 output without accumulation): mode TT on 224-wide tiles for an M that only 224 divides; mode NN
+    // on 224- or 192-wide tiles for such an M, and for an M that 256 divides as well when whole rounds of narrow tiles
+    // beat the rounds of full tiles by the margin mode TN asks for (M = 3584, N = 8192: 512 tiles of 224 in two rounds
+    // instead of 448 of 256 in 1.75; measured on 3584 x 8192 x 37888: 742 -> 7xx us).
+    const bool narrow_ok = kBf16 && !g.accumulate && !(KMA && KMB);
+    int narrow_nj = 0;
+    if (narrow_ok && g.M % 256 != 0) {
+        if (g.M % 224 == 0) narrow_nj = 7;
+        else if (KMA && g.M % 192 == 0) narrow_nj = 6;
+    } else if (narrow_ok && KMA && g.N % 256 == 0 && g_gemm_tile == 0) {
+        const int64_t tn = g.N / 256, t256 = tn * (g.M / 256), rem256 = t256 % cus;
+        if (t256 >= cus && (rem256 == 0 || rem256 > cus / xcds)) {
+            auto rounds = [&](int64_t tiles) { return (double)((tiles + cus - 1) / cus); };
+            double best = rounds(t256) * 8.0;
+            if (g.M % 224 == 0 && rounds(tn * (g.M / 224)) * 7.0 * 1.08 < best) {
+                best = rounds(tn * (g.M / 224)) * 7.0 * 1.08;
+                narrow_nj = 7;
+            }
+            if (g.M % 192 == 0 && rounds(tn * (g.M / 192)) * 6.0 * 1.12 < best) narrow_nj = 6;
+        }
+    }
+    const bool m224 = narrow_nj != 0;
     LLMQ_REQUIRE(g.N % 256 == 0 && g.K % 256 == 0 && (g.M % 256 == 0 || m224) && cus % xcds == 0,
-                 "matmul: a K-major operand (mode %s) needs N %% 256 == 0, K %% 256 == 0 and M %% 256 == 0 (mode TT with bf16 output "
-                 "and without accumulation also M %% 224 == 0); got M, N, K = %d, %d, %d", mode, g.M, g.N, g.K);
+                 "matmul: a K-major operand (mode %s) needs N %% 256 == 0, K %% 256 == 0 and M %% 256 == 0 (with bf16 output and "
+                 "without accumulation also M %% 224 == 0 in modes TT and NN, M %% 192 == 0 in mode NN); got M, N, K = %d, %d, %d",
+                 mode, g.M, g.N, g.K);
     // the copies of a K-major operand address it as "tile base + 32-bit lane offset", and that offset walks the
     // whole K extent of the operand
     LLMQ_REQUIRE(!KMB || (int64_t)g.K * g.N < ((int64_t)1 << 31), "matmul: the K-major second operand must be smaller than 2 GiB "
                  "(K * N = %lld bytes)", (long long)((int64_t)g.K * g.N));
     LLMQ_REQUIRE(!KMA || (int64_t)g.K * g.M < ((int64_t)1 << 31), "matmul: the K-major first operand must be smaller than 2 GiB "
                  "(K * M = %lld bytes)", (long long)((int64_t)g.K * g.M));
-    const int tiles = (g.N / 256) * (m224 ? g.M / 224 : g.M / 256);
+    const int tiles = (g.N / 256) * (narrow_nj ? g.M / (32 * narrow_nj) : g.M / 256);
     const bool cached_out = ((int64_t)g.M + g.N) * g.K + (int64_t)g.N * g.M * 2 <= ((int64_t)224 << 20);
-    if constexpr (!KMA && kBf16) {
-        if (m224) {
+    if constexpr (kBf16 && !(KMA && KMB)) {
+        if (narrow_nj) {
             const int grid = tiles < cus ? (tiles + xcds - 1) / xcds * xcds : cus;
-            hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, B_FMT, false, 7, true, false, true>), dim3((unsigned)grid),
-                               dim3(256), 0, stream, g);
+            g.rem_split = 1;
+            g.part_per_xcd = 0;
+            if (narrow_nj == 7)
+                hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, B_FMT, false, 7, true, false, KMB, KMA>), dim3((unsigned)grid),
+                                   dim3(256), 0, stream, g);
+            else if constexpr (KMA)
+                hipLaunchKernelGGL((gemm_tn_e4m3_w4_kernel<uint16_t, B_FMT, false, 6, true, false, KMB, KMA>), dim3((unsigned)grid),
+                                   dim3(256), 0, stream, g);
             LLMQ_HIP_TRY(hipGetLastError());
             return LLMQ_OK;
         }
