@@ -2122,9 +2122,11 @@ static int gemm_dispatch_kmajor(GemmArgs g, void* workspace, size_t workspace_by
                  "matmul: all pointers must be 16-byte aligned");
     LLMQ_REQUIRE(workspace != nullptr || workspace_bytes == 0, "matmul: workspace size given without a workspace");
     // Narrow tiles (bf16 output without accumulation): mode TT on 224-wide tiles for an M that only 224 divides; mode NN
-    // on 224- or 192-wide tiles for such an M, and for an M that 256 divides as well when whole rounds of narrow tiles
-    // beat the rounds of full tiles by the margin mode TN asks for (M = 3584, N = 8192: 512 tiles of 224 in two rounds
-    // instead of 448 of 256 in 1.75; measured on 3584 x 8192 x 37888: 742 -> 7xx us).
+    // on 224- or 192-wide tiles for such an M, and on 192-wide tiles for an M that 256 divides as well when whole rounds of
+    // them beat the rounds of full tiles by the margin mode TN asks for (1536 x 16384 x 17920: 512 tiles of 192 in two
+    // rounds instead of 384 of 256 in 1.5; measured 384 -> 343 us).  Not so the 224-wide tile: its rows of a K-major a
+    // start at multiples of 224 bytes, off the 128-byte lines of the memory system three times out of four, and the
+    // launch fetches 1.7 times the bytes of the full tiles (3584 x 8192 x 37888: 3.09 against 1.79 GB) for 1 % of time.
     const bool narrow_ok = kBf16 && !g.accumulate && !(KMA && KMB);
     int narrow_nj = 0;
     if (narrow_ok && g.M % 256 != 0) {
@@ -2134,12 +2136,7 @@ static int gemm_dispatch_kmajor(GemmArgs g, void* workspace, size_t workspace_by
         const int64_t tn = g.N / 256, t256 = tn * (g.M / 256), rem256 = t256 % cus;
         if (t256 >= cus && (rem256 == 0 || rem256 > cus / xcds)) {
             auto rounds = [&](int64_t tiles) { return (double)((tiles + cus - 1) / cus); };
-            double best = rounds(t256) * 8.0;
-            if (g.M % 224 == 0 && rounds(tn * (g.M / 224)) * 7.0 * 1.08 < best) {
-                best = rounds(tn * (g.M / 224)) * 7.0 * 1.08;
-                narrow_nj = 7;
-            }
-            if (g.M % 192 == 0 && rounds(tn * (g.M / 192)) * 6.0 * 1.12 < best) narrow_nj = 6;
+            if (g.M % 192 == 0 && rounds(tn * (g.M / 192)) * 6.0 * 1.12 < rounds(t256) * 8.0) narrow_nj = 6;
         }
     }
     const bool m224 = narrow_nj != 0;
