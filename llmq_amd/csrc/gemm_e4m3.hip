@@ -1875,7 +1875,7 @@ static int launch_pipe_ragged(const GemmArgs& g, hipStream_t stream) {
 // Which of the two ragged tilings is faster, from estimated times in microseconds: rounds of tiles over the chip (one
 // 256 x 256 tile per compute unit, or two co-resident 128 x 128 tiles) times the K-steps of a tile at the measured cost
 // of a step (1.4 / 1.0 us) plus a measured per-round cost (8 / 3 us: prologue, epilogue and the masked last step of the
-// ragged four-wave instance).  Checked against a sweep of 60 shapes (M, N from 1000 to 16392, K from 400 to 8208): the
+// ragged four-wave instance).  Checked against a sweep of 42 shapes (M, N from 1000 to 16392, K from 400 to 8208): the
 // estimate is within 10 % of the measured time and picks the faster kernel except where the two are within 5 %.
 // Examples (us, 128 x 128 / four-wave): 1000 x 8192 x 3584 30 / 44, 2056 x 4100 x 3600 64 / 46, 4360 x 4100 x 656 28 / 33,
 // 3584 x 8200 x 3600 131 / 90, 8200 x 8200 x 8208 649 / 448, 3000 x 16392 x 656 63 / 71.
@@ -1931,7 +1931,7 @@ static int gemm_dispatch(GemmArgs g, void* workspace, size_t workspace_bytes, hi
             LLMQ_REQUIRE(force_tile == 6 || (force_tile == 3 ? w4_fits : pipe_fits),
                          "matmul: M, N, K = %d, %d, %d do not fit the forced ragged kernel", g.M, g.N, g.K);
             pick = force_tile;
-        } else if (w4_fits && g_gemm_persist != 0 && (!pipe_fits || ragged_prefers_four_wave(g.M, g.N, g.K, cus))) {
+        } else if (w4_fits && g_gemm_persist != 0 && ragged_prefers_four_wave(g.M, g.N, g.K, cus)) {
             pick = 3;
         } else if (pipe_fits && (int64_t)g.M * g.N >= 128 * 128) {
             pick = 2;
