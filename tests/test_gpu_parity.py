@@ -764,7 +764,7 @@ def test_gemm_swept_shapes_exact_and_inside_their_rows(K, O, mnk):
 
 @pytest.mark.parametrize("mode", ["TT", "NN", "NT"])
 @pytest.mark.parametrize("mnk", [(256, 256, 256), (512, 768, 512), (448, 512, 768), (1024, 2048, 1024), (2304, 512, 2816),
-                                 (3584, 4096, 512), (576, 768, 512), (3584, 8192, 512), (1536, 16384, 256)])
+                                 (3584, 4096, 512), (576, 768, 512), (1536, 16384, 256)])
 def test_gemm_operands_in_k_major_layout(K, O, mnk, mode):
     """Modes TT / NN / NT of the reference's matmul signature (src/kernels/kernels.h:22, matmul.cpp:66-67): b stored
     [K, N] and / or a stored [K, M] row-major, read through transposing LDS reads instead of a materialised transpose
@@ -779,6 +779,8 @@ def test_gemm_operands_in_k_major_layout(K, O, mnk, mode):
         pytest.skip("two K-major operands are served on 256-wide tiles only")
     if not a_km and M % 256 and M % 224:
         pytest.skip("mode TT has 256- and 224-wide tiles")
+    if mnk == (1536, 16384, 256) and mode != "NN":
+        pytest.skip("this shape is here for mode NN's automatic choice of 192-wide tiles")
     lay_a = (lambda x: np.ascontiguousarray(x.T)) if a_km else (lambda x: x)      # [K, M]: what the caller holds
     lay_b = (lambda x: np.ascontiguousarray(x.T)) if b_km else (lambda x: x)      # [K, N]
     a, _ = O.fill_int_e4m3(M * Kd, 606, 0)
